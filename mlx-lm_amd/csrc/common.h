@@ -1,0 +1,107 @@
+// Shared device helpers for the gfx950 kernels: element types, 64-lane wave
+// reductions, block reductions through LDS and the error channel that every
+// extern "C" entry point uses.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#define WAVE 64
+
+// element type codes shared with the Python side
+#define DT_F32 0
+#define DT_BF16 1
+
+struct bf16 {
+  uint16_t bits;
+};
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16 v) {
+  return __uint_as_float(((uint32_t)v.bits) << 16);
+}
+__device__ __forceinline__ float bits_to_f32(uint16_t b) {
+  return __uint_as_float(((uint32_t)b) << 16);
+}
+
+// round to nearest even, NaN kept quiet
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+template <typename T>
+__device__ __forceinline__ T from_f32(float v);
+template <>
+__device__ __forceinline__ float from_f32<float>(float v) {
+  return v;
+}
+template <>
+__device__ __forceinline__ bf16 from_f32<bf16>(float v) {
+  bf16 r;
+  r.bits = f32_to_bf16_bits(v);
+  return r;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; `red` is LDS of at least 17 floats.
+// Every thread gets the result.  Safe to call repeatedly with the same `red`.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nw = (blockDim.x + 63) >> 6;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < nw; ++i) t += red[i];
+  return t;
+}
+__device__ __forceinline__ float block_max(float v, float* red) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nw = (blockDim.x + 63) >> 6;
+  v = wave_max(v);
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float t = red[0];
+  for (int i = 1; i < nw; ++i) t = fmaxf(t, red[i]);
+  return t;
+}
+
+// ---------------------------------------------------------------------------
+// host side: one error string per thread, returned codes are 0 (ok) or 1.
+
+static thread_local char g_err[512];
+
+#define FAIL(...)                               \
+  do {                                          \
+    snprintf(g_err, sizeof(g_err), __VA_ARGS__); \
+    return 1;                                   \
+  } while (0)
+
+#define CHECK_LAUNCH(name)                                                    \
+  do {                                                                        \
+    hipError_t e_ = hipGetLastError();                                        \
+    if (e_ != hipSuccess) FAIL("%s: launch failed: %s", name, hipGetErrorString(e_)); \
+  } while (0)
+
+#define DEFINE_LAST_ERROR(fn) \
+  extern "C" const char* fn() { return g_err; }

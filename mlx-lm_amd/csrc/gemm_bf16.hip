@@ -1,0 +1,277 @@
+// Linear layer on bfloat16 operands with MFMA and 32-bit accumulation:
+//   out[m, n] = epilogue( sum_k A[m, k] * W[n, k] + bias[n] )
+// A is [M, K] activations, W is [N, K] (the [out, in] layout of a linear
+// layer), both contiguous along k, which is what both MFMA operands want.
+// Epilogues: plain, tanh-GELU, or accumulate into a 32-bit residual stream.
+// Replaces nn.Linear calls of the reference (mlx_lm/models/gpt2.py:41-42,52,
+// 68,76-80) and the tied head (mlx_lm/models/gpt2.py:167).
+//
+// Two kernels:
+//  * gemm_bf16_tile: 128x128x64 block tile, 4 waves in 2x2, each wave a 64x64
+//    tile of four v_mfma_f32_32x32x16_bf16 accumulators.  Any M, N; K % 8 == 0.
+//  * gemm_bf16_skinny: M <= 64 rows (decode).  A block of four waves owns 16
+//    output features and splits K among its waves; W streams from HBM once
+//    as the MFMA A-operand, the activations are the B-operand.
+#include "common.h"
+
+#define FLAG_GELU 1
+#define FLAG_ACCUMULATE 2
+#define FLAG_OUT_F32 4
+
+struct GemmArgs {
+  const uint16_t* A;
+  const uint16_t* W;
+  const float* bias;
+  void* out;
+  int M, N, K;
+  int lda, ldw, ldo;
+  int flags;
+};
+
+__device__ __forceinline__ float gelu_tanh(float x) {
+  const float c = 0.7978845608028654f;  // sqrt(2/pi)
+  const float u = c * (x + 0.044715f * x * x * x);
+  return 0.5f * x * (1.0f + tanhf(u));
+}
+
+__device__ __forceinline__ void store_out(const GemmArgs& p, int m, int n, float v) {
+  if (p.bias) v += p.bias[n];
+  if (p.flags & FLAG_GELU) v = gelu_tanh(v);
+  const size_t idx = (size_t)m * p.ldo + n;
+  if (p.flags & FLAG_ACCUMULATE) {
+    float* o = (float*)p.out;
+    o[idx] += v;
+  } else if (p.flags & FLAG_OUT_F32) {
+    ((float*)p.out)[idx] = v;
+  } else {
+    ((uint16_t*)p.out)[idx] = f32_to_bf16_bits(v);
+  }
+}
+
+// ---------------------------------------------------------------------------
+
+#define BM 128
+#define BN 128
+#define BK 64
+#define LDS_STRIDE (BK + 8)  // 144 bytes a row: 16-byte reads of 16 rows hit distinct banks
+
+__global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(GemmArgs p) {
+  __shared__ __attribute__((aligned(16))) uint16_t As[BM * LDS_STRIDE];
+  __shared__ __attribute__((aligned(16))) uint16_t Bs[BN * LDS_STRIDE];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.y * BM;
+  const int n0 = blockIdx.x * BN;
+
+  f32x16_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // each thread moves four 16-byte pieces of A and of W per k-block
+  uint4 ra[4], rb[4];
+  const uint4 zero4 = make_uint4(0, 0, 0, 0);
+
+  auto load_global = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = tid + 256 * i;
+      const int row = c >> 3;
+      const int kc = (c & 7) * 8;
+      const int gk = k0 + kc;
+      const int gm = m0 + row, gn = n0 + row;
+      ra[i] = (gm < p.M && gk < p.K) ? *(const uint4*)(p.A + (size_t)gm * p.lda + gk) : zero4;
+      rb[i] = (gn < p.N && gk < p.K) ? *(const uint4*)(p.W + (size_t)gn * p.ldw + gk) : zero4;
+    }
+  };
+  auto store_lds = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = tid + 256 * i;
+      const int row = c >> 3;
+      const int kc = (c & 7) * 8;
+      *(uint4*)(As + row * LDS_STRIDE + kc) = ra[i];
+      *(uint4*)(Bs + row * LDS_STRIDE + kc) = rb[i];
+    }
+  };
+
+  load_global(0);
+  store_lds();
+  __syncthreads();
+
+  const int frag_row = lane & 31;
+  const int frag_k = (lane >> 5) * 8;
+
+  for (int k0 = 0; k0 < p.K; k0 += BK) {
+    const bool more = (k0 + BK) < p.K;
+    if (more) load_global(k0 + BK);
+#pragma unroll
+    for (int ks = 0; ks < BK; ks += 16) {
+      bf16x8_t a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        a[i] = *(const bf16x8_t*)(As + (wm * 64 + i * 32 + frag_row) * LDS_STRIDE + ks + frag_k);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        b[j] = *(const bf16x8_t*)(Bs + (wn * 64 + j * 32 + frag_row) * LDS_STRIDE + ks + frag_k);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+    if (more) {
+      store_lds();
+      __syncthreads();
+    }
+  }
+
+  // accumulator r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+      if (n >= p.N) continue;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (m < p.M) store_out(p, m, n, acc[i][j][r]);
+      }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Skinny kernel: out^T tile = W[16 features, K] x A^T[K, up to 64 rows].
+// Lane l of a wave reads 32 contiguous bytes of W row (l % 16) per 64-wide
+// k-block, at k offset (l / 16) * 16, and feeds them to two 16x16x32 MFMAs;
+// the activation fragment uses the same k offsets, so the products pair up.
+
+#define SK_WAVES 4
+#define SK_MAXM 64
+
+template <int MT>  // number of 16-row groups of activations (1..4)
+__global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(GemmArgs p) {
+  __shared__ float red[SK_WAVES][MT][64 * 4];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int n0 = blockIdx.x * 16;
+  const int wrow = n0 + (lane & 15);
+  const int koff = (lane >> 4) * 16;
+  const bool wvalid = wrow < p.N;
+  const uint16_t* wp = p.W + (size_t)(wvalid ? wrow : 0) * p.ldw + koff;
+
+  f32x4_t acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+  const uint4 zero4 = make_uint4(0, 0, 0, 0);
+  union Frag {
+    uint4 u;
+    bf16x8_t v;
+  };
+
+  for (int k0 = wave * 64; k0 < p.K; k0 += SK_WAVES * 64) {
+    const int k = k0 + koff;  // this lane covers k .. k+15
+    Frag w0, w1;
+    w0.u = (wvalid && k < p.K) ? *(const uint4*)(wp + k0) : zero4;
+    w1.u = (wvalid && k + 8 < p.K) ? *(const uint4*)(wp + k0 + 8) : zero4;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const int m = t * 16 + (lane & 15);
+      const bool av = m < p.M;
+      const uint16_t* ap = p.A + (size_t)(av ? m : 0) * p.lda + k;
+      Frag a0, a1;
+      a0.u = (av && k < p.K) ? *(const uint4*)(ap) : zero4;
+      a1.u = (av && k + 8 < p.K) ? *(const uint4*)(ap + 8) : zero4;
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0.v, a0.v, acc[t], 0, 0, 0);
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1.v, a1.v, acc[t], 0, 0, 0);
+    }
+  }
+
+  // sum the waves' partial tiles in a fixed order
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][t][lane * 4 + r] = acc[t][r];
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      // accumulator r: feature row 4*(lane/16) + r, activation column lane%16
+      const int m = t * 16 + (lane & 15);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < SK_WAVES; ++w) v += red[w][t][lane * 4 + r];
+        const int n = n0 + 4 * (lane >> 4) + r;
+        if (m < p.M && n < p.N) store_out(p, m, n, v);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+
+DEFINE_LAST_ERROR(mlxlm_last_error)
+
+static int check_args(const GemmArgs& p) {
+  if (p.M < 0 || p.N <= 0 || p.K <= 0) FAIL("gemm_bf16: bad sizes M=%d N=%d K=%d", p.M, p.N, p.K);
+  if (p.K % 8 != 0) FAIL("gemm_bf16: K=%d must be a multiple of 8", p.K);
+  if (p.lda % 8 != 0 || p.ldw % 8 != 0)
+    FAIL("gemm_bf16: row strides lda=%d ldw=%d must be multiples of 8", p.lda, p.ldw);
+  if (p.lda < p.K || p.ldw < p.K || p.ldo < p.N)
+    FAIL("gemm_bf16: row strides smaller than the rows (lda=%d ldw=%d ldo=%d)", p.lda, p.ldw, p.ldo);
+  if (!p.A || !p.W || !p.out) FAIL("gemm_bf16: null pointer");
+  if (((uintptr_t)p.A | (uintptr_t)p.W) & 15) FAIL("gemm_bf16: A and W must be 16-byte aligned");
+  if ((p.flags & FLAG_ACCUMULATE) && (p.flags & FLAG_GELU))
+    FAIL("gemm_bf16: GELU and accumulate cannot be combined");
+  return 0;
+}
+
+// variant: 0 = choose, 1 = tile kernel, 2 = skinny kernel
+extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* bias, int M, int N,
+                         int K, int lda, int ldw, int ldo, int flags, int variant,
+                         hipStream_t stream) {
+  GemmArgs p;
+  p.A = (const uint16_t*)A;
+  p.W = (const uint16_t*)W;
+  p.bias = bias;
+  p.out = out;
+  p.M = M, p.N = N, p.K = K;
+  p.lda = lda, p.ldw = ldw, p.ldo = ldo;
+  p.flags = flags;
+  if (check_args(p)) return 1;
+  if (M == 0) return 0;
+  if (variant == 0) variant = (M <= SK_MAXM) ? 2 : 1;
+  if (variant == 2) {
+    if (M > SK_MAXM) FAIL("gemm_bf16: the skinny kernel takes at most %d rows, got %d", SK_MAXM, M);
+    dim3 grid((N + 15) / 16), block(256);
+    const int mt = (M + 15) / 16;
+    if (mt == 1)
+      hipLaunchKernelGGL(gemm_bf16_skinny_kernel<1>, grid, block, 0, stream, p);
+    else if (mt == 2)
+      hipLaunchKernelGGL(gemm_bf16_skinny_kernel<2>, grid, block, 0, stream, p);
+    else if (mt == 3)
+      hipLaunchKernelGGL(gemm_bf16_skinny_kernel<3>, grid, block, 0, stream, p);
+    else
+      hipLaunchKernelGGL(gemm_bf16_skinny_kernel<4>, grid, block, 0, stream, p);
+  } else if (variant == 1) {
+    dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM), block(256);
+    hipLaunchKernelGGL(gemm_bf16_tile_kernel, grid, block, 0, stream, p);
+  } else {
+    FAIL("gemm_bf16: unknown variant %d", variant);
+  }
+  CHECK_LAUNCH("gemm_bf16");
+  return 0;
+}

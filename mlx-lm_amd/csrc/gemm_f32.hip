@@ -1,0 +1,182 @@
+// Linear layer in true 32-bit: float operands, float products and sums
+// (v_mfma_f32_32x32x2_f32; no reduced-precision matrix mode, no splitting).
+//   out[m, n] = epilogue( sum_k A[m, k] * W[n, k] + bias[n] )
+// A is [M, K], W is [N, K], both contiguous along k.  Epilogues: plain,
+// tanh-GELU, or accumulate into the residual stream.  Any M, N; K % 4 == 0.
+// The 32-bit twin of gemm_bf16.hip; replaces the same nn.Linear calls
+// (mlx_lm/models/gpt2.py:41-42,52,68,76-80,167).
+#include "common.h"
+
+#define FLAG_GELU 1
+#define FLAG_ACCUMULATE 2
+
+struct GemmArgs {
+  const float* A;
+  const float* W;
+  const float* bias;
+  float* out;
+  int M, N, K;
+  int lda, ldw, ldo;
+  int flags;
+};
+
+__device__ __forceinline__ float gelu_tanh(float x) {
+  const float c = 0.7978845608028654f;  // sqrt(2/pi)
+  const float u = c * (x + 0.044715f * x * x * x);
+  return 0.5f * x * (1.0f + tanhf(u));
+}
+
+#define BK 16
+#define LDS_STRIDE (BK + 1)
+
+// WM x WN waves of 64x64 (BIG) or 32x32 (small) wave tiles
+template <int TM, int TN>  // 32x32 MFMA tiles per wave along m and n
+__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs p) {
+  constexpr int BM_ = 2 * TM * 32;
+  constexpr int BN_ = 2 * TN * 32;
+  __shared__ float As[BM_ * LDS_STRIDE];
+  __shared__ float Bs[BN_ * LDS_STRIDE];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.y * BM_;
+  const int n0 = blockIdx.x * BN_;
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // a k-block of a tile is BM_ x 16 floats = BM_*4 pieces of 16 bytes
+  constexpr int PA = (BM_ * 4) / 256;
+  constexpr int PB = (BN_ * 4) / 256;
+  float4 ra[PA], rb[PB];
+  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+
+  auto load_global = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < PA; ++i) {
+      const int c = tid + 256 * i;
+      const int row = c >> 2, gk = k0 + (c & 3) * 4, gm = m0 + row;
+      ra[i] = (gm < p.M && gk < p.K) ? *(const float4*)(p.A + (size_t)gm * p.lda + gk) : zero4;
+    }
+#pragma unroll
+    for (int i = 0; i < PB; ++i) {
+      const int c = tid + 256 * i;
+      const int row = c >> 2, gk = k0 + (c & 3) * 4, gn = n0 + row;
+      rb[i] = (gn < p.N && gk < p.K) ? *(const float4*)(p.W + (size_t)gn * p.ldw + gk) : zero4;
+    }
+  };
+  auto store_lds = [&]() {
+#pragma unroll
+    for (int i = 0; i < PA; ++i) {
+      const int c = tid + 256 * i;
+      float* d = As + (c >> 2) * LDS_STRIDE + (c & 3) * 4;
+      d[0] = ra[i].x, d[1] = ra[i].y, d[2] = ra[i].z, d[3] = ra[i].w;
+    }
+#pragma unroll
+    for (int i = 0; i < PB; ++i) {
+      const int c = tid + 256 * i;
+      float* d = Bs + (c >> 2) * LDS_STRIDE + (c & 3) * 4;
+      d[0] = rb[i].x, d[1] = rb[i].y, d[2] = rb[i].z, d[3] = rb[i].w;
+    }
+  };
+
+  load_global(0);
+  store_lds();
+  __syncthreads();
+
+  const int frag_row = lane & 31;
+  const int frag_k = lane >> 5;
+
+  for (int k0 = 0; k0 < p.K; k0 += BK) {
+    const bool more = (k0 + BK) < p.K;
+    if (more) load_global(k0 + BK);
+#pragma unroll
+    for (int ks = 0; ks < BK; ks += 2) {
+      float a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        a[i] = As[(wm * TM * 32 + i * 32 + frag_row) * LDS_STRIDE + ks + frag_k];
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        b[j] = Bs[(wn * TN * 32 + j * 32 + frag_row) * LDS_STRIDE + ks + frag_k];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+    if (more) {
+      store_lds();
+      __syncthreads();
+    }
+  }
+
+  // accumulator r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + wn * TN * 32 + j * 32 + (lane & 31);
+      if (n >= p.N) continue;
+      const float bias = p.bias ? p.bias[n] : 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * TM * 32 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (m >= p.M) continue;
+        float v = acc[i][j][r] + bias;
+        if (p.flags & FLAG_GELU) v = gelu_tanh(v);
+        float* o = p.out + (size_t)m * p.ldo + n;
+        if (p.flags & FLAG_ACCUMULATE)
+          *o += v;
+        else
+          *o = v;
+      }
+    }
+}
+
+DEFINE_LAST_ERROR(mlxlm_last_error)
+
+// variant: 0 = choose, 1 = 128x128 block tile, 2 = 64x64 block tile
+extern "C" int gemm_f32(void* out, const void* A, const void* W, const float* bias, int M, int N,
+                        int K, int lda, int ldw, int ldo, int flags, int variant,
+                        hipStream_t stream) {
+  GemmArgs p;
+  p.A = (const float*)A;
+  p.W = (const float*)W;
+  p.bias = bias;
+  p.out = (float*)out;
+  p.M = M, p.N = N, p.K = K;
+  p.lda = lda, p.ldw = ldw, p.ldo = ldo;
+  p.flags = flags;
+  if (M < 0 || N <= 0 || K <= 0) FAIL("gemm_f32: bad sizes M=%d N=%d K=%d", M, N, K);
+  if (K % 4 != 0) FAIL("gemm_f32: K=%d must be a multiple of 4", K);
+  if (lda % 4 != 0 || ldw % 4 != 0)
+    FAIL("gemm_f32: row strides lda=%d ldw=%d must be multiples of 4", lda, ldw);
+  if (lda < K || ldw < K || ldo < N)
+    FAIL("gemm_f32: row strides smaller than the rows (lda=%d ldw=%d ldo=%d)", lda, ldw, ldo);
+  if (!A || !W || !out) FAIL("gemm_f32: null pointer");
+  if (((uintptr_t)A | (uintptr_t)W) & 15) FAIL("gemm_f32: A and W must be 16-byte aligned");
+  if ((flags & FLAG_ACCUMULATE) && (flags & FLAG_GELU))
+    FAIL("gemm_f32: GELU and accumulate cannot be combined");
+  if (M == 0) return 0;
+  if (variant == 0) variant = (M <= 64 || (size_t)M * N < (size_t)128 * 128 * 128) ? 2 : 1;
+  if (variant == 1) {
+    dim3 grid((N + 127) / 128, (M + 127) / 128), block(256);
+    hipLaunchKernelGGL((gemm_f32_kernel<2, 2>), grid, block, 0, stream, p);
+  } else if (variant == 2) {
+    dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
+    hipLaunchKernelGGL((gemm_f32_kernel<1, 1>), grid, block, 0, stream, p);
+  } else {
+    FAIL("gemm_f32: unknown variant %d", variant);
+  }
+  CHECK_LAUNCH("gemm_f32");
+  return 0;
+}

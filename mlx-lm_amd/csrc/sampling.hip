@@ -1,0 +1,352 @@
+// Sampling from rows of 32-bit logits, one block per row, everything in 32-bit.
+//
+// sample_rows does, in the reference's order (mlx_lm/sample_utils.py:46-67 and
+// mlx_lm/generate.py:411-412):
+//   logprobs = logits - logsumexp(logits)
+//   temp == 0: token = argmax(logprobs)
+//   else: top_p -> min_p -> xtc -> top_k filters, then a draw from
+//         softmax(filtered / temp).
+// Every filter of the reference keeps the tokens whose log-probability lies
+// on one side of a threshold, so the kept set is always
+//   { lo <= lp <= hi } plus the xtc special tokens above hi,
+// and each filter only moves lo or hi.  Thresholds that the reference finds by
+// sorting (top_p: sample_utils.py:204-237, top_k: 129-151, the min_p floor:
+// 154-201) are found here by bisection over the ordered bit patterns of the
+// floats, each probe being one block-wide sum or count.  Tokens that tie with
+// a threshold are all kept.  The draw is Gumbel-max with uniforms hashed from
+// (seed, counter, token id), so a row's result does not depend on the rows
+// beside it (the reference draws with mx.random.categorical,
+// sample_utils.py:279-281).
+//
+// apply_logit_bias and apply_penalties are the logits processors of
+// mlx_lm/sample_utils.py:72-126,284-369, run before sample_rows.
+#include "common.h"
+
+#define SAMPLE_THREADS 1024
+
+struct SampleArgs {
+  int* tokens;            // [R]
+  float* token_logprob;   // [R]
+  float* logprobs;        // [R, ld_logprobs] or null
+  const float* logits;    // [R, ld]
+  const float* temp;      // [R]
+  const float* top_p;     // [R]
+  const float* min_p;     // [R]
+  const int* min_keep;    // [R]
+  const int* top_k;       // [R]
+  const float* xtc_prob;  // [R]
+  const float* xtc_thr;   // [R]
+  const unsigned long long* seed;  // [R]
+  const int* counter;     // [R]
+  const int* xtc_special; // [n_special]
+  int n_special;
+  int vocab, ld, ld_logprobs;
+};
+
+__device__ __forceinline__ unsigned int ordered_key(float f) {
+  const unsigned int b = __float_as_uint(f);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+__device__ __forceinline__ float key_to_float(unsigned int k) {
+  const unsigned int b = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+  return __uint_as_float(b);
+}
+
+__device__ __forceinline__ unsigned long long mix64(unsigned long long x) {
+  x ^= x >> 30;
+  x *= 0xBF58476D1CE4E5B9ull;
+  x ^= x >> 27;
+  x *= 0x94D049BB133111EBull;
+  x ^= x >> 31;
+  return x;
+}
+// uniform in (0, 1), 24 bits, from (seed, counter, index)
+__device__ __forceinline__ float uniform01(unsigned long long seed, unsigned int counter,
+                                           unsigned int index) {
+  unsigned long long x = mix64(seed + 0x9E3779B97F4A7C15ull * (unsigned long long)(counter + 1u));
+  x = mix64(x ^ (0xD1B54A32D192ED03ull * (unsigned long long)(index + 1u)));
+  return ((float)(unsigned int)(x >> 40) + 0.5f) * (1.0f / 16777216.0f);
+}
+
+struct Kept {
+  float lo, hi;
+  const int* special;
+  int n_special;
+  __device__ __forceinline__ bool operator()(int i, float lp) const {
+    if (!(lp >= lo)) return false;
+    if (lp <= hi) return true;
+    for (int s = 0; s < n_special; ++s)
+      if (special[s] == i) return true;
+    return false;
+  }
+};
+
+// (value, index) argmax over the block; ties go to the lowest index
+__device__ __forceinline__ void block_argmax(float& v, int& idx, float* redv, int* redi) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nw = (blockDim.x + 63) >> 6;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(v, o, WAVE);
+    const int oi = __shfl_xor(idx, o, WAVE);
+    if (ov > v || (ov == v && oi < idx)) v = ov, idx = oi;
+  }
+  __syncthreads();
+  if (lane == 0) redv[wave] = v, redi[wave] = idx;
+  __syncthreads();
+  v = redv[0], idx = redi[0];
+  for (int w = 1; w < nw; ++w)
+    if (redv[w] > v || (redv[w] == v && redi[w] < idx)) v = redv[w], idx = redi[w];
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(SampleArgs a) {
+  __shared__ float red[32];
+  __shared__ int redi[32];
+  const int r = blockIdx.x;
+  const int V = a.vocab;
+  const float* x = a.logits + (size_t)r * a.ld;
+  const int tid = threadIdx.x, nt = blockDim.x;
+
+  // log-sum-exp
+  float mx = -INFINITY;
+  for (int i = tid; i < V; i += nt) mx = fmaxf(mx, x[i]);
+  mx = block_max(mx, red);
+  float se = 0.f;
+  for (int i = tid; i < V; i += nt) se += expf(x[i] - mx);
+  se = block_sum(se, red);
+  const float lse = mx + logf(se);
+
+  if (a.logprobs) {
+    float* lp = a.logprobs + (size_t)r * a.ld_logprobs;
+    for (int i = tid; i < V; i += nt) lp[i] = x[i] - lse;
+  }
+
+  const float temp = a.temp[r];
+  if (temp == 0.f) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = tid; i < V; i += nt) {
+      const float v = x[i];
+      if (v > bv) bv = v, bi = i;
+    }
+    block_argmax(bv, bi, red, redi);
+    if (tid == 0) a.tokens[r] = bi, a.token_logprob[r] = bv - lse;
+    return;
+  }
+
+  Kept kept;
+  kept.lo = -INFINITY, kept.hi = INFINITY;
+  kept.special = a.xtc_special, kept.n_special = 0;
+  const float lp_max = mx - lse;
+
+  // top_p: keep lp >= v*, v* the smallest value whose ascending cumulative
+  // probability H(v) = sum_{lp_j <= v} p_j exceeds 1 - top_p.
+  const float top_p = a.top_p[r];
+  if (top_p > 0.f && top_p < 1.f) {
+    const float need = 1.f - top_p;
+    unsigned int lo = 0u, hi = ordered_key(lp_max);  // H(hi) = 1 > need
+    while (lo < hi) {
+      const unsigned int mid = lo + ((hi - lo) >> 1);
+      const float c = key_to_float(mid);
+      float s = 0.f;
+      for (int i = tid; i < V; i += nt) {
+        const float lp = x[i] - lse;
+        if (lp <= c) s += expf(lp);
+      }
+      s = block_sum(s, red);
+      if (s > need)
+        hi = mid;
+      else
+        lo = mid + 1u;
+    }
+    kept.lo = fmaxf(kept.lo, key_to_float(lo));
+  }
+
+  // k-th largest value among the kept tokens, -inf if fewer than k are kept
+  auto kth_largest = [&](int k) -> float {
+    float cnt_all = 0.f;
+    for (int i = tid; i < V; i += nt) cnt_all += kept(i, x[i] - lse) ? 1.f : 0.f;
+    cnt_all = block_sum(cnt_all, red);
+    if (cnt_all < (float)k) return -INFINITY;
+    unsigned int lo = 0u, hi = ordered_key(lp_max);  // largest c with count(lp >= c) >= k
+    while (lo < hi) {
+      const unsigned int mid = lo + ((hi - lo + 1u) >> 1);
+      const float c = key_to_float(mid);
+      float cnt = 0.f;
+      for (int i = tid; i < V; i += nt) {
+        const float lp = x[i] - lse;
+        cnt += (lp >= c && kept(i, lp)) ? 1.f : 0.f;
+      }
+      cnt = block_sum(cnt, red);
+      if (cnt >= (float)k)
+        lo = mid;
+      else
+        hi = mid - 1u;
+    }
+    return key_to_float(lo);
+  };
+
+  // min_p: drop lp < max + log(min_p), but never one of the min_keep best
+  const float min_p = a.min_p[r];
+  if (min_p != 0.f) {
+    float floor_lp = lp_max + logf(min_p);
+    const int mk = a.min_keep[r];
+    if (mk > 1) floor_lp = fminf(floor_lp, kth_largest(mk));
+    kept.lo = fmaxf(kept.lo, floor_lp);
+  }
+
+  // xtc: with probability xtc_prob drop every token whose (renormalised)
+  // probability is above the threshold, except the least likely of them and
+  // the special tokens
+  const float xtc_prob = a.xtc_prob[r];
+  if (xtc_prob > 0.f) {
+    const float u = uniform01(a.seed[r], (unsigned int)a.counter[r], 0xfffffffeu);
+    if (!(u > xtc_prob)) {
+      float z = 0.f;
+      for (int i = tid; i < V; i += nt) {
+        const float lp = x[i] - lse;
+        if (kept(i, lp)) z += expf(lp);
+      }
+      z = block_sum(z, red);
+      const float thr = a.xtc_thr[r];
+      float least = INFINITY;
+      for (int i = tid; i < V; i += nt) {
+        const float lp = x[i] - lse;
+        if (kept(i, lp) && expf(lp) / z > thr) least = fminf(least, lp);
+      }
+      least = -block_max(-least, red);
+      kept.hi = least;
+      kept.n_special = a.n_special;
+    }
+  }
+
+  const int top_k = a.top_k[r];
+  if (top_k > 0) kept.lo = fmaxf(kept.lo, kth_largest(top_k));
+
+  // Gumbel-max draw from softmax(lp / temp) over the kept tokens
+  const float inv_temp = 1.f / temp;
+  const unsigned long long seed = a.seed[r];
+  const unsigned int counter = (unsigned int)a.counter[r];
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = tid; i < V; i += nt) {
+    const float lp = x[i] - lse;
+    if (!kept(i, lp)) continue;
+    const float u = uniform01(seed, counter, (unsigned int)i);
+    const float g = -logf(-logf(u));
+    const float v = lp * inv_temp + g;
+    if (v > bv) bv = v, bi = i;
+  }
+  block_argmax(bv, bi, red, redi);
+  if (tid == 0) {
+    a.tokens[r] = bi;
+    a.token_logprob[r] = x[bi] - lse;
+  }
+}
+
+// ---------------------------------------------------------------------------
+
+// logits[row, idx[j]] += val[j] for j in [offsets[row], offsets[row+1])
+__global__ __launch_bounds__(256) void logit_bias_kernel(float* logits, int ld,
+                                                         const int* offsets, const int* idx,
+                                                         const float* val) {
+  const int r = blockIdx.x;
+  float* x = logits + (size_t)r * ld;
+  // duplicates in one row are applied one after the other by one thread
+  for (int j = offsets[r] + threadIdx.x; j < offsets[r + 1]; j += blockDim.x) {
+    bool first = true;
+    for (int k = offsets[r]; k < j; ++k)
+      if (idx[k] == idx[j]) first = false;
+    if (!first) continue;
+    float v = x[idx[j]];
+    for (int k = j; k < offsets[r + 1]; ++k)
+      if (idx[k] == idx[j]) v += val[k];
+    x[idx[j]] = v;
+  }
+}
+
+// Repetition, presence and frequency penalties over the tail of each row's
+// token history; hist[offsets[row] .. offsets[row+1]) is that history, oldest
+// first, and each penalty looks at its own last `*_ctx` tokens of it.
+__global__ __launch_bounds__(256) void penalties_kernel(float* logits, int ld, const int* offsets,
+                                                        const int* hist, const float* rep,
+                                                        const int* rep_ctx, const float* pres,
+                                                        const int* pres_ctx, const float* freq,
+                                                        const int* freq_ctx) {
+  const int r = blockIdx.x;
+  float* x = logits + (size_t)r * ld;
+  const int b = offsets[r], e = offsets[r + 1];
+  const int rep_b = max(b, e - rep_ctx[r]);
+  const int pres_b = max(b, e - pres_ctx[r]);
+  const int freq_b = max(b, e - freq_ctx[r]);
+  for (int j = b + threadIdx.x; j < e; j += blockDim.x) {
+    const int t = hist[j];
+    bool first = true;
+    for (int k = b; k < j; ++k)
+      if (hist[k] == t) first = false;
+    if (!first) continue;
+    bool in_rep = false, in_pres = false;
+    int n_freq = 0;
+    for (int k = j; k < e; ++k) {
+      if (hist[k] != t) continue;
+      if (k >= rep_b) in_rep = true;
+      if (k >= pres_b) in_pres = true;
+      if (k >= freq_b) ++n_freq;
+    }
+    float v = x[t];
+    const float rp = rep[r];
+    if (in_rep && rp != 0.f && rp != 1.f) v = v < 0.f ? v * rp : v / rp;
+    if (in_pres) v -= pres[r];
+    v -= freq[r] * (float)n_freq;
+    x[t] = v;
+  }
+}
+
+DEFINE_LAST_ERROR(mlxlm_last_error)
+
+extern "C" int sample_rows(int* tokens, float* token_logprob, float* logprobs, int ld_logprobs,
+                           const float* logits, int ld, int n_rows, int vocab, const float* temp,
+                           const float* top_p, const float* min_p, const int* min_keep,
+                           const int* top_k, const float* xtc_prob, const float* xtc_thr,
+                           const unsigned long long* seed, const int* counter,
+                           const int* xtc_special, int n_special, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (vocab <= 0 || ld < vocab) FAIL("sample_rows: bad vocab %d / row stride %d", vocab, ld);
+  if (!tokens || !token_logprob || !logits || !temp || !top_p || !min_p || !min_keep || !top_k ||
+      !xtc_prob || !xtc_thr || !seed || !counter)
+    FAIL("sample_rows: null pointer");
+  if (logprobs && ld_logprobs < vocab) FAIL("sample_rows: logprobs row stride %d too small", ld_logprobs);
+  if (n_special > 0 && !xtc_special) FAIL("sample_rows: special tokens missing");
+  SampleArgs a;
+  a.tokens = tokens, a.token_logprob = token_logprob, a.logprobs = logprobs, a.logits = logits;
+  a.temp = temp, a.top_p = top_p, a.min_p = min_p, a.min_keep = min_keep, a.top_k = top_k;
+  a.xtc_prob = xtc_prob, a.xtc_thr = xtc_thr, a.seed = seed, a.counter = counter;
+  a.xtc_special = xtc_special, a.n_special = n_special;
+  a.vocab = vocab, a.ld = ld, a.ld_logprobs = ld_logprobs;
+  hipLaunchKernelGGL(sample_rows_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, a);
+  CHECK_LAUNCH("sample_rows");
+  return 0;
+}
+
+extern "C" int apply_logit_bias(float* logits, int ld, int n_rows, const int* offsets,
+                                const int* idx, const float* val, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (!logits || !offsets || !idx || !val) FAIL("apply_logit_bias: null pointer");
+  hipLaunchKernelGGL(logit_bias_kernel, dim3(n_rows), dim3(256), 0, stream, logits, ld, offsets, idx,
+                     val);
+  CHECK_LAUNCH("apply_logit_bias");
+  return 0;
+}
+
+extern "C" int apply_penalties(float* logits, int ld, int n_rows, const int* offsets,
+                               const int* hist, const float* rep, const int* rep_ctx,
+                               const float* pres, const int* pres_ctx, const float* freq,
+                               const int* freq_ctx, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (!logits || !offsets || !hist || !rep || !rep_ctx || !pres || !pres_ctx || !freq || !freq_ctx)
+    FAIL("apply_penalties: null pointer");
+  hipLaunchKernelGGL(penalties_kernel, dim3(n_rows), dim3(256), 0, stream, logits, ld, offsets, hist,
+                     rep, rep_ctx, pres, pres_ctx, freq, freq_ctx);
+  CHECK_LAUNCH("apply_penalties");
+  return 0;
+}

@@ -1,0 +1,313 @@
+"""Python faces of the HIP kernels: argument checks, pointers, launch.
+
+Each function takes torch tensors that live on the GPU, checks on the host
+what the kernel assumes about them (shape, dtype, contiguity) and launches on
+torch's current stream.  Nothing here computes on the CPU or through a torch
+operator; a missing library raises.
+"""
+
+import ctypes
+
+import torch
+
+from . import build
+
+_c_int = ctypes.c_int
+_c_float = ctypes.c_float
+_c_size_t = ctypes.c_size_t
+_vp = ctypes.c_void_p
+
+DT = {torch.float32: 0, torch.bfloat16: 1}
+
+GEMM_GELU = 1
+GEMM_ACCUMULATE = 2
+GEMM_OUT_F32 = 4
+
+
+def _stream():
+    return _vp(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return _vp(t.data_ptr()) if t is not None else _vp(0)
+
+
+def _need(cond, msg):
+    if not cond:
+        raise ValueError(msg)
+
+
+def _dev(t, name, dtype=None):
+    _need(t.is_cuda, f"{name} must be on the GPU")
+    _need(t.is_contiguous(), f"{name} must be contiguous")
+    if dtype is not None:
+        _need(t.dtype == dtype, f"{name} must be {dtype}, is {t.dtype}")
+
+
+def _rows2d(t, name):
+    """A 2-D tensor whose rows are contiguous; returns its row stride."""
+    _need(t.is_cuda, f"{name} must be on the GPU")
+    _need(t.dim() == 2 and t.stride(1) == 1, f"{name} must be 2-D with contiguous rows")
+    return t.stride(0)
+
+
+# ---------------------------------------------------------------------------
+
+
+def embed_gather_add(out, table, ids, add_table=None, add_ids=None):
+    """``out[t] = table[ids[t]] (+ add_table[add_ids[t]])`` into float32 ``out``."""
+    lib = build.load("embed")
+    n, width = out.shape
+    _dev(out, "out", torch.float32)
+    _dev(table, "table")
+    _dev(ids, "ids", torch.int32)
+    _need(table.dtype in DT, f"table dtype {table.dtype} not supported")
+    _need(table.shape[1] == width and ids.numel() >= n, "embed_gather_add: shapes disagree")
+    if add_table is not None:
+        _dev(add_table, "add_table", table.dtype)
+        _dev(add_ids, "add_ids", torch.int32)
+        _need(add_table.shape[1] == width and add_ids.numel() >= n, "embed_gather_add: shapes disagree")
+    rc = lib.embed_gather_add(
+        _ptr(out), _ptr(table), _ptr(ids), _ptr(add_table), _ptr(add_ids),
+        _c_int(n), _c_int(width), _c_int(DT[table.dtype]), _stream(),
+    )
+    build.check(lib, rc, "embed_gather_add")
+    return out
+
+
+def layernorm(out, x, gamma, beta, eps, rows=None):
+    """LayerNorm of float32 rows of ``x`` (all, or those listed in ``rows``) into ``out``."""
+    lib = build.load("norm")
+    n, width = out.shape
+    _dev(out, "out")
+    _dev(x, "x", torch.float32)
+    _need(out.dtype in DT, f"out dtype {out.dtype} not supported")
+    _need(x.shape[-1] == width, "layernorm: widths disagree")
+    if rows is None:
+        _need(x.shape[0] >= n, "layernorm: fewer input rows than output rows")
+    else:
+        _dev(rows, "rows", torch.int32)
+        _need(rows.numel() >= n, "layernorm: fewer row indices than output rows")
+    for name, v in (("gamma", gamma), ("beta", beta)):
+        if v is not None:
+            _dev(v, name, torch.float32)
+            _need(v.numel() == width, f"layernorm: {name} has {v.numel()} elements, width is {width}")
+    rc = lib.layernorm(
+        _ptr(out), _ptr(x), _ptr(rows), _ptr(gamma), _ptr(beta), _c_float(eps),
+        _c_int(n), _c_int(width), _c_int(DT[out.dtype]), _stream(),
+    )
+    build.check(lib, rc, "layernorm")
+    return out
+
+
+def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0):
+    """``out = epilogue(a @ w.T + bias)``.
+
+    ``a`` is ``[M, K]``, ``w`` is ``[N, K]``, both float32 or both bfloat16;
+    ``bias`` float32.  ``accumulate`` adds into a float32 ``out`` (the residual
+    stream); otherwise ``out`` is float32 or the operands' dtype.
+    """
+    lda, ldw, ldo = _rows2d(a, "a"), _rows2d(w, "w"), _rows2d(out, "out")
+    M, K = a.shape
+    N = w.shape[0]
+    _need(w.shape[1] == K, f"linear: a is [{M},{K}] but w is {list(w.shape)}")
+    _need(tuple(out.shape) == (M, N), f"linear: out is {list(out.shape)}, want [{M},{N}]")
+    _need(a.dtype == w.dtype and a.dtype in DT, "linear: a and w must share float32 or bfloat16")
+    if bias is not None:
+        _dev(bias, "bias", torch.float32)
+        _need(bias.numel() == N, "linear: bias length")
+    flags = 0
+    if gelu:
+        flags |= GEMM_GELU
+    if accumulate:
+        _need(out.dtype == torch.float32, "linear: accumulate needs a float32 out")
+        flags |= GEMM_ACCUMULATE
+    if a.dtype == torch.float32:
+        _need(out.dtype == torch.float32, "linear: float32 operands give a float32 out")
+        lib = build.load("gemm_f32")
+        fn = lib.gemm_f32
+    else:
+        if out.dtype == torch.float32:
+            flags |= GEMM_OUT_F32
+        else:
+            _need(out.dtype == torch.bfloat16, "linear: out must be float32 or bfloat16")
+        lib = build.load("gemm_bf16")
+        fn = lib.gemm_bf16
+    rc = fn(
+        _ptr(out), _ptr(a), _ptr(w), _ptr(bias), _c_int(M), _c_int(N), _c_int(K),
+        _c_int(lda), _c_int(ldw), _c_int(ldo), _c_int(flags), _c_int(variant), _stream(),
+    )
+    build.check(lib, rc, "linear")
+    return out
+
+
+# ---------------------------------------------------------------------------
+
+
+class PagedKV:
+    """Keys and values of one cache slot: two views ``[n_pages, Hkv, page, hd]``."""
+
+    __slots__ = ("k", "v", "page_stride", "n_kv_heads", "head_dim", "page_size")
+
+    def __init__(self, k, v):
+        _need(k.shape == v.shape and k.dim() == 4, "PagedKV: k and v must be [pages, heads, page, dim]")
+        _need(k.dtype == v.dtype and k.dtype in DT, "PagedKV: dtype")
+        for t in (k, v):
+            _need(t.is_cuda and t.stride(3) == 1 and t.stride(2) == t.shape[3]
+                  and t.stride(1) == t.shape[2] * t.shape[3], "PagedKV: a page must be contiguous")
+        _need(k.stride(0) == v.stride(0), "PagedKV: k and v page strides differ")
+        self.k, self.v = k, v
+        self.page_stride = k.stride(0)
+        _, self.n_kv_heads, self.page_size, self.head_dim = k.shape
+
+
+def _attn_common(qkv_like, kv, block_table, token_req, positions):
+    _dev(block_table, "block_table", torch.int32)
+    _dev(token_req, "token_req", torch.int32)
+    _dev(positions, "positions", torch.int32)
+    _need(block_table.dim() == 2, "block_table must be [requests, max_blocks]")
+    _need(qkv_like.dtype == kv.k.dtype, "queries and cache must share a dtype")
+
+
+def kv_write(k_src, v_src, kv, block_table, token_req, positions):
+    """Scatter rows of ``k_src``/``v_src`` ``[T, Hkv*hd]`` into their pages."""
+    lib = build.load("attention")
+    ld = _rows2d(k_src, "k_src")
+    _need(_rows2d(v_src, "v_src") == ld, "kv_write: k and v row strides differ")
+    n = k_src.shape[0]
+    _need(k_src.shape == v_src.shape and k_src.shape[1] == kv.n_kv_heads * kv.head_dim,
+          "kv_write: source width must be n_kv_heads*head_dim")
+    _attn_common(k_src, kv, block_table, token_req, positions)
+    _need(token_req.numel() >= n and positions.numel() >= n, "kv_write: per-token arrays too short")
+    rc = lib.kv_write(
+        _ptr(k_src), _ptr(v_src), _c_int(ld), _ptr(kv.k), _ptr(kv.v), _c_size_t(kv.page_stride),
+        _ptr(block_table), _c_int(block_table.shape[1]), _ptr(token_req), _ptr(positions),
+        _c_int(n), _c_int(kv.n_kv_heads), _c_int(kv.head_dim), _c_int(kv.page_size),
+        _c_int(DT[k_src.dtype]), _stream(),
+    )
+    build.check(lib, rc, "kv_write")
+
+
+def attn_tile(out, q, kv, block_table, token_req, positions, tiles, n_tiles, n_heads, scale, window=0):
+    """Attention for tiles of up to 16 consecutive queries of one request each.
+
+    ``tiles`` is int32 ``[n_tiles, 2]``: first flat row and number of rows.
+    """
+    lib = build.load("attention")
+    ldq, ldo = _rows2d(q, "q"), _rows2d(out, "out")
+    _need(q.shape[1] == n_heads * kv.head_dim, "attn_tile: q width must be n_heads*head_dim")
+    _need(out.shape[1] == n_heads * kv.head_dim and out.dtype == q.dtype, "attn_tile: out shape/dtype")
+    _attn_common(q, kv, block_table, token_req, positions)
+    _dev(tiles, "tiles", torch.int32)
+    _need(tiles.numel() >= 2 * n_tiles, "attn_tile: tile list too short")
+    rc = lib.attn_tile(
+        _ptr(out), _ptr(q), _c_int(ldq), _c_int(ldo), _ptr(kv.k), _ptr(kv.v),
+        _c_size_t(kv.page_stride), _ptr(block_table), _c_int(block_table.shape[1]),
+        _ptr(token_req), _ptr(positions), _ptr(tiles), _c_int(n_tiles), _c_int(n_heads),
+        _c_int(kv.n_kv_heads), _c_int(kv.head_dim), _c_int(kv.page_size), _c_int(window),
+        _c_float(scale), _c_int(DT[q.dtype]), _stream(),
+    )
+    build.check(lib, rc, "attn_tile")
+    return out
+
+
+ATTN_ROW_MAX_HEAD_DIM = 144  # beyond this the per-wave key tiles do not fit in LDS
+
+
+def attn_row(out, q, kv, block_table, token_req, positions, rows, n_rows, n_heads, scale,
+             window=0, n_splits=1, part_o=None, part_ml=None):
+    """Attention for single query rows, keys split ``n_splits`` ways."""
+    lib = build.load("attention")
+    ldq, ldo = _rows2d(q, "q"), _rows2d(out, "out")
+    _need(q.shape[1] == n_heads * kv.head_dim, "attn_row: q width must be n_heads*head_dim")
+    _need(out.shape[1] == n_heads * kv.head_dim and out.dtype == q.dtype, "attn_row: out shape/dtype")
+    _need(kv.head_dim <= ATTN_ROW_MAX_HEAD_DIM,
+          f"attn_row: head_dim {kv.head_dim} above {ATTN_ROW_MAX_HEAD_DIM}; use attn_tile")
+    _attn_common(q, kv, block_table, token_req, positions)
+    _dev(rows, "rows", torch.int32)
+    _need(rows.numel() >= n_rows, "attn_row: row list too short")
+    if n_splits > 1:
+        _dev(part_o, "part_o", torch.float32)
+        _dev(part_ml, "part_ml", torch.float32)
+        _need(part_o.numel() >= n_rows * n_heads * n_splits * kv.head_dim, "attn_row: part_o too small")
+        _need(part_ml.numel() >= n_rows * n_heads * n_splits * 2, "attn_row: part_ml too small")
+    rc = lib.attn_row(
+        _ptr(out), _ptr(q), _c_int(ldq), _c_int(ldo), _ptr(kv.k), _ptr(kv.v),
+        _c_size_t(kv.page_stride), _ptr(block_table), _c_int(block_table.shape[1]),
+        _ptr(token_req), _ptr(positions), _ptr(rows), _c_int(n_rows), _c_int(n_heads),
+        _c_int(kv.n_kv_heads), _c_int(kv.head_dim), _c_int(kv.page_size), _c_int(window),
+        _c_float(scale), _c_int(n_splits), _ptr(part_o), _ptr(part_ml), _c_int(DT[q.dtype]),
+        _stream(),
+    )
+    build.check(lib, rc, "attn_row")
+    return out
+
+
+# ---------------------------------------------------------------------------
+
+
+def sample_rows(tokens, token_logprob, logits, temp, top_p, min_p, min_keep, top_k, xtc_prob,
+                xtc_thr, seed, counter, xtc_special=None, logprobs=None):
+    """Sample one token from each row of float32 ``logits``; see csrc/sampling.hip."""
+    lib = build.load("sampling")
+    ld = _rows2d(logits, "logits")
+    n, vocab = logits.shape
+    _need(logits.dtype == torch.float32, "sample_rows: logits must be float32")
+    _dev(tokens, "tokens", torch.int32)
+    _dev(token_logprob, "token_logprob", torch.float32)
+    for name, t, dt in (("temp", temp, torch.float32), ("top_p", top_p, torch.float32),
+                        ("min_p", min_p, torch.float32), ("min_keep", min_keep, torch.int32),
+                        ("top_k", top_k, torch.int32), ("xtc_prob", xtc_prob, torch.float32),
+                        ("xtc_thr", xtc_thr, torch.float32), ("seed", seed, torch.int64),
+                        ("counter", counter, torch.int32)):
+        _dev(t, name, dt)
+        _need(t.numel() >= n, f"sample_rows: {name} shorter than the rows")
+    _need(tokens.numel() >= n and token_logprob.numel() >= n, "sample_rows: outputs too short")
+    n_special = 0
+    if xtc_special is not None and xtc_special.numel() > 0:
+        _dev(xtc_special, "xtc_special", torch.int32)
+        n_special = xtc_special.numel()
+    ld_lp = 0
+    if logprobs is not None:
+        ld_lp = _rows2d(logprobs, "logprobs")
+        _need(logprobs.dtype == torch.float32 and logprobs.shape[0] >= n and logprobs.shape[1] >= vocab,
+              "sample_rows: logprobs shape/dtype")
+    rc = lib.sample_rows(
+        _ptr(tokens), _ptr(token_logprob), _ptr(logprobs), _c_int(ld_lp), _ptr(logits), _c_int(ld),
+        _c_int(n), _c_int(vocab), _ptr(temp), _ptr(top_p), _ptr(min_p), _ptr(min_keep), _ptr(top_k),
+        _ptr(xtc_prob), _ptr(xtc_thr), _ptr(seed), _ptr(counter),
+        _ptr(xtc_special if n_special else None), _c_int(n_special), _stream(),
+    )
+    build.check(lib, rc, "sample_rows")
+
+
+def apply_logit_bias(logits, offsets, idx, val):
+    lib = build.load("sampling")
+    ld = _rows2d(logits, "logits")
+    _need(logits.dtype == torch.float32, "apply_logit_bias: logits must be float32")
+    _dev(offsets, "offsets", torch.int32)
+    _dev(idx, "idx", torch.int32)
+    _dev(val, "val", torch.float32)
+    _need(offsets.numel() == logits.shape[0] + 1, "apply_logit_bias: offsets length")
+    rc = lib.apply_logit_bias(_ptr(logits), _c_int(ld), _c_int(logits.shape[0]), _ptr(offsets),
+                              _ptr(idx), _ptr(val), _stream())
+    build.check(lib, rc, "apply_logit_bias")
+
+
+def apply_penalties(logits, offsets, hist, rep, rep_ctx, pres, pres_ctx, freq, freq_ctx):
+    lib = build.load("sampling")
+    ld = _rows2d(logits, "logits")
+    n = logits.shape[0]
+    _need(logits.dtype == torch.float32, "apply_penalties: logits must be float32")
+    _dev(offsets, "offsets", torch.int32)
+    _dev(hist, "hist", torch.int32)
+    _need(offsets.numel() == n + 1, "apply_penalties: offsets length")
+    for name, t, dt in (("rep", rep, torch.float32), ("pres", pres, torch.float32),
+                        ("freq", freq, torch.float32), ("rep_ctx", rep_ctx, torch.int32),
+                        ("pres_ctx", pres_ctx, torch.int32), ("freq_ctx", freq_ctx, torch.int32)):
+        _dev(t, name, dt)
+        _need(t.numel() >= n, f"apply_penalties: {name} shorter than the rows")
+    rc = lib.apply_penalties(_ptr(logits), _c_int(ld), _c_int(n), _ptr(offsets), _ptr(hist),
+                             _ptr(rep), _ptr(rep_ctx), _ptr(pres), _ptr(pres_ctx), _ptr(freq),
+                             _ptr(freq_ctx), _stream())
+    build.check(lib, rc, "apply_penalties")

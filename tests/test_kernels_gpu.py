@@ -1,0 +1,468 @@
+"""Each HIP kernel alone against a plain torch reference, at sizes of its own."""
+
+import math
+
+import pytest
+import torch
+
+import plain_gpt2 as plain
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+def _k():
+    from mlx_lm_amd.ops import kernels
+
+    return kernels
+
+
+def _rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+# ---------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width", [48, 1600, 200])
+def test_embed_gather_add(dtype, width):
+    k = _k()
+    V, P, T = 301, 77, 53
+    table = _rand((V, width), dtype, 1)
+    pos_table = _rand((P, width), dtype, 2)
+    g = torch.Generator().manual_seed(3)
+    ids = torch.randint(0, V, (T,), generator=g, dtype=torch.int32).to(DEV)
+    pos = torch.randint(0, P, (T,), generator=g, dtype=torch.int32).to(DEV)
+    out = torch.empty(T, width, dtype=torch.float32, device=DEV)
+    k.embed_gather_add(out, table, ids, pos_table, pos)
+    want = table.float()[ids.long()] + pos_table.float()[pos.long()]
+    assert torch.equal(out, want)
+    k.embed_gather_add(out, table, ids)
+    assert torch.equal(out, table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width,eps", [(64, 1e-5), (1600, 1e-6), (200, 1e-3)])
+def test_layernorm(out_dtype, width, eps):
+    k = _k()
+    R = 37
+    x = _rand((R, width), torch.float32, 4, 3.0) + 1.5
+    x[5] = x[5] * 1e-3  # a low-variance row, where eps matters
+    gamma = 1 + _rand((width,), torch.float32, 5, 0.1)
+    beta = _rand((width,), torch.float32, 6, 0.1)
+    out = torch.empty(R, width, dtype=out_dtype, device=DEV)
+    k.layernorm(out, x, gamma, beta, eps)
+    want = plain.layer_norm(x.double().cpu(), gamma.double().cpu(), beta.double().cpu(), eps)
+    tol = 2e-5 if out_dtype == torch.float32 else 2e-2
+    assert torch.allclose(out.double().cpu(), want, atol=tol, rtol=tol)
+    # gathered rows
+    rows = torch.tensor([7, 0, 36, 7], dtype=torch.int32, device=DEV)
+    out2 = torch.empty(4, width, dtype=out_dtype, device=DEV)
+    k.layernorm(out2, x, gamma, beta, eps, rows=rows)
+    assert torch.equal(out2, out[rows.long()])
+
+
+GEMM_SHAPES = [
+    (1, 48, 64),
+    (7, 1000, 96),
+    (16, 80, 200),
+    (33, 257, 384),
+    (64, 4800, 1600),
+    (130, 300, 72),
+    (300, 513, 1608),
+]
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+@pytest.mark.parametrize("mode", ["plain", "gelu", "accumulate"])
+def test_gemm_f32(M, N, K, mode):
+    k = _k()
+    a = _rand((M, K), torch.float32, 10)
+    w = _rand((N, K), torch.float32, 11, 0.1)
+    bias = _rand((N,), torch.float32, 12)
+    ref = plain.linear(a.double().cpu(), w.double().cpu(), bias.double().cpu())
+    for variant in (1, 2):
+        if mode == "accumulate":
+            out = _rand((M, N), torch.float32, 13)
+            want = out.double().cpu() + ref
+            k.linear(out, a, w, bias, accumulate=True, variant=variant)
+        else:
+            out = torch.empty(M, N, dtype=torch.float32, device=DEV)
+            k.linear(out, a, w, bias, gelu=(mode == "gelu"), variant=variant)
+            want = plain.gelu_tanh(ref) if mode == "gelu" else ref
+        err = (out.double().cpu() - want).abs().max().item()
+        assert err < 1e-5 * math.sqrt(K) * 4, (variant, err)
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+@pytest.mark.parametrize("mode", ["plain", "gelu", "accumulate", "f32out"])
+def test_gemm_bf16(M, N, K, mode):
+    k = _k()
+    a = _rand((M, K), torch.bfloat16, 10)
+    w = _rand((N, K), torch.bfloat16, 11, 0.1)
+    bias = _rand((N,), torch.float32, 12)
+    ref = plain.linear(a.double().cpu(), w.double().cpu(), bias.double().cpu())
+    variants = (1, 2) if M <= 64 else (1,)
+    for variant in variants:
+        if mode == "accumulate":
+            out = _rand((M, N), torch.float32, 13)
+            want = out.double().cpu() + ref
+            k.linear(out, a, w, bias, accumulate=True, variant=variant)
+            tol = 1e-4 * math.sqrt(K)
+        elif mode == "f32out":
+            out = torch.empty(M, N, dtype=torch.float32, device=DEV)
+            k.linear(out, a, w, bias, variant=variant)
+            want = ref
+            tol = 1e-4 * math.sqrt(K)
+        else:
+            out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+            k.linear(out, a, w, bias, gelu=(mode == "gelu"), variant=variant)
+            want = plain.gelu_tanh(ref) if mode == "gelu" else ref
+            tol = None
+        got = out.double().cpu()
+        if tol is None:
+            # one bfloat16 rounding of the exact value
+            assert torch.allclose(got, want, rtol=2**-7, atol=1e-3), (variant, (got - want).abs().max())
+        else:
+            assert (got - want).abs().max().item() < tol, (variant, (got - want).abs().max())
+
+
+def test_gemm_refuses_bad_sizes():
+    k = _k()
+    a = torch.zeros(4, 20, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(8, 20, dtype=torch.bfloat16, device=DEV)
+    out = torch.zeros(4, 8, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        k.linear(out, a, w)
+    with pytest.raises(ValueError):
+        k.linear(out, a.float(), w)
+
+
+# ---------------------------------------------------------------------------
+# paged attention
+
+
+class PagedCase:
+    """Random requests with a scrambled page assignment and a ragged step."""
+
+    def __init__(self, dtype, n_heads, n_kv_heads, head_dim, page_size, ctx_lens, q_lens, seed,
+                 window=0):
+        from mlx_lm_amd.ops.kernels import PagedKV
+
+        g = torch.Generator().manual_seed(seed)
+        self.dtype, self.H, self.Hkv, self.hd, self.ps = dtype, n_heads, n_kv_heads, head_dim, page_size
+        self.window = window
+        R = len(ctx_lens)
+        self.total = [c + q for c, q in zip(ctx_lens, q_lens)]
+        max_blocks = max((t + page_size - 1) // page_size for t in self.total) + 1
+        n_pages = sum((t + page_size - 1) // page_size for t in self.total) + 3
+        perm = torch.randperm(n_pages, generator=g).tolist()
+        self.block_table = torch.full((R, max_blocks), -1, dtype=torch.int32)
+        pool = torch.full((n_pages, 2, n_kv_heads, page_size, head_dim), float("nan")).to(dtype)
+        self.k_full, self.v_full = [], []
+        nxt = 0
+        for r in range(R):
+            kf = torch.randn(self.total[r], n_kv_heads, head_dim, generator=g).to(dtype)
+            vf = torch.randn(self.total[r], n_kv_heads, head_dim, generator=g).to(dtype)
+            self.k_full.append(kf)
+            self.v_full.append(vf)
+            for b in range((self.total[r] + page_size - 1) // page_size):
+                self.block_table[r, b] = perm[nxt]
+                nxt += 1
+            # tokens already in the cache; this step's tokens go through kv_write
+            for p in range(ctx_lens[r]):
+                page = self.block_table[r, p // page_size]
+                pool[page, 0, :, p % page_size] = kf[p]
+                pool[page, 1, :, p % page_size] = vf[p]
+        self.pool = pool.to(DEV)
+        self.kv = PagedKV(self.pool[:, 0], self.pool[:, 1])
+        token_req, positions = [], []
+        for r in range(R):
+            for i in range(q_lens[r]):
+                token_req.append(r)
+                positions.append(ctx_lens[r] + i)
+        self.T = len(token_req)
+        self.token_req = torch.tensor(token_req, dtype=torch.int32, device=DEV)
+        self.positions = torch.tensor(positions, dtype=torch.int32, device=DEV)
+        self.q = torch.randn(self.T, n_heads * head_dim, generator=g).to(dtype)
+        self.k_new = torch.stack([self.k_full[r][p] for r, p in zip(token_req, positions)]).reshape(self.T, -1)
+        self.v_new = torch.stack([self.v_full[r][p] for r, p in zip(token_req, positions)]).reshape(self.T, -1)
+        self.block_table_dev = self.block_table.to(DEV)
+        self.ctx_lens, self.q_lens = ctx_lens, q_lens
+        self.scale = head_dim**-0.5
+
+    def reference(self):
+        out = torch.empty(self.T, self.H * self.hd, dtype=torch.float64)
+        t = 0
+        for r, (c, n) in enumerate(zip(self.ctx_lens, self.q_lens)):
+            if n == 0:
+                continue
+            q = self.q[t : t + n].double().reshape(n, self.H, self.hd).permute(1, 0, 2)
+            kk = self.k_full[r][: c + n].double().permute(1, 0, 2)
+            vv = self.v_full[r][: c + n].double().permute(1, 0, 2)
+            mask = plain.causal_mask(n, c, self.window if self.window else None)
+            o = plain.attention(q, kk, vv, self.scale, mask)
+            out[t : t + n] = plain.merge_heads(o)
+            t += n
+        return out
+
+    def tiles(self, qt=16):
+        tiles, t = [], 0
+        for n in self.q_lens:
+            for s in range(0, n, qt):
+                tiles.append((t + s, min(qt, n - s)))
+            t += n
+        return torch.tensor(tiles, dtype=torch.int32, device=DEV)
+
+
+ATTN_CASES = [
+    # H, Hkv, hd, page, ctx_lens, q_lens, window
+    (4, 4, 16, 16, [0, 5, 40], [33, 1, 7], 0),
+    (3, 3, 32, 16, [0, 100, 17, 64], [90, 1, 2, 1], 0),
+    (6, 2, 48, 8, [3, 0, 250], [20, 70, 1], 0),
+    (5, 1, 80, 32, [130, 0], [1, 130], 0),
+    (2, 2, 128, 64, [200, 0], [3, 65], 0),
+    (4, 2, 64, 16, [0, 300, 90], [200, 1, 5], 37),
+    (25, 25, 64, 16, [511, 0], [1, 48], 0),
+]
+
+
+def _attn_tol(dtype):
+    return 2e-5 if dtype == torch.float32 else 1.6e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", ATTN_CASES)
+def test_kv_write_and_attn_tile(dtype, case):
+    k = _k()
+    H, Hkv, hd, ps, ctx, ql, window = case
+    c = PagedCase(dtype, H, Hkv, hd, ps, ctx, ql, seed=hd + H, window=window)
+    k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
+    torch.cuda.synchronize()
+    # every written token is where the table says, bit for bit
+    pool = c.pool.cpu()
+    for r in range(len(ctx)):
+        for p in range(c.total[r]):
+            page = c.block_table[r, p // ps]
+            assert torch.equal(pool[page, 0, :, p % ps], c.k_full[r][p])
+            assert torch.equal(pool[page, 1, :, p % ps], c.v_full[r][p])
+    tiles = c.tiles()
+    out = torch.full((c.T, H * hd), float("nan")).to(dtype).to(DEV)
+    k.attn_tile(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, tiles,
+                tiles.shape[0], H, c.scale, window)
+    want = c.reference()
+    err = (out.double().cpu() - want).abs().max().item()
+    assert err < _attn_tol(dtype), err
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", ATTN_CASES)
+@pytest.mark.parametrize("n_splits", [1, 3, 8])
+def test_attn_row(dtype, case, n_splits):
+    k = _k()
+    H, Hkv, hd, ps, ctx, ql, window = case
+    c = PagedCase(dtype, H, Hkv, hd, ps, ctx, ql, seed=hd + H + 1, window=window)
+    k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
+    rows = torch.arange(c.T, dtype=torch.int32, device=DEV)
+    part_o = torch.empty(c.T * H * n_splits * hd, dtype=torch.float32, device=DEV)
+    part_ml = torch.empty(c.T * H * n_splits * 2, dtype=torch.float32, device=DEV)
+    out = torch.full((c.T, H * hd), float("nan")).to(dtype).to(DEV)
+    k.attn_row(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, c.T, H,
+               c.scale, window, n_splits, part_o, part_ml)
+    want = c.reference()
+    err = (out.double().cpu() - want).abs().max().item()
+    assert err < _attn_tol(dtype), err
+
+
+def test_attn_far_key_stands_out():
+    """One key among hundreds carries the answer: a dropped tile or page shows."""
+    k = _k()
+    H, hd, ps = 2, 32, 16
+    for far in (0, 15, 16, 63, 64, 257, 400):
+        c = PagedCase(torch.float32, H, H, hd, ps, [401], [1], seed=far)
+        # the query points along key `far` of head 0 so that its score is 30:
+        # that key takes nearly all the weight
+        kf = c.k_full[0][far, 0].clone()
+        c.q[0, :hd] = kf * (30.0 / (c.scale * float(kf.norm() ** 2)))
+        k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
+        rows = torch.zeros(1, dtype=torch.int32, device=DEV)
+        want = c.reference()
+        for n_splits in (1, 4):
+            out = torch.empty(1, H * hd, dtype=torch.float32, device=DEV)
+            po = torch.empty(H * n_splits * hd, dtype=torch.float32, device=DEV)
+            pm = torch.empty(H * n_splits * 2, dtype=torch.float32, device=DEV)
+            k.attn_row(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, 1,
+                       H, c.scale, 0, n_splits, po, pm)
+            assert (out.double().cpu() - want).abs().max().item() < 2e-5
+            # and the answer is that key's value, to within the others' small weight
+            v_far = c.v_full[0][far, 0].double()
+            assert (out[0, :hd].double().cpu() - v_far).abs().max().item() < 0.1
+
+
+def test_attn_refuses_bad_head_dim():
+    k = _k()
+    from mlx_lm_amd.ops.kernels import PagedKV
+
+    pool = torch.zeros(4, 2, 1, 16, 24, device=DEV)
+    kv = PagedKV(pool[:, 0], pool[:, 1])
+    q = torch.zeros(1, 24, device=DEV)
+    z = torch.zeros(1, dtype=torch.int32, device=DEV)
+    bt = torch.zeros(1, 2, dtype=torch.int32, device=DEV)
+    with pytest.raises(RuntimeError, match="multiple of 16"):
+        k.attn_row(q.clone(), q, kv, bt, z, z, z, 1, 1, 1.0)
+
+
+# ---------------------------------------------------------------------------
+# sampling
+
+
+def _sample(logits, temp=0.0, top_p=0.0, min_p=0.0, min_keep=1, top_k=0, xtc_prob=0.0, xtc_thr=0.1,
+            seed=0, counter=0, special=None, want_logprobs=False):
+    k = _k()
+    n, V = logits.shape
+
+    def col(v, dt):
+        if isinstance(v, (list, tuple)):
+            return torch.tensor(v, dtype=dt, device=DEV)
+        return torch.full((n,), v, dtype=dt, device=DEV)
+
+    tokens = torch.empty(n, dtype=torch.int32, device=DEV)
+    tlp = torch.empty(n, dtype=torch.float32, device=DEV)
+    lp = torch.empty(n, V, dtype=torch.float32, device=DEV) if want_logprobs else None
+    sp = torch.tensor(special, dtype=torch.int32, device=DEV) if special else None
+    k.sample_rows(tokens, tlp, logits, col(temp, torch.float32), col(top_p, torch.float32),
+                  col(min_p, torch.float32), col(min_keep, torch.int32), col(top_k, torch.int32),
+                  col(xtc_prob, torch.float32), col(xtc_thr, torch.float32), col(seed, torch.int64),
+                  col(counter, torch.int32), sp, lp)
+    return tokens.cpu(), tlp.cpu(), (lp.cpu() if lp is not None else None)
+
+
+def test_sample_greedy_and_logprobs():
+    logits = _rand((9, 1000), torch.float32, 20, 3.0)
+    logits[3, 17] = logits[3, 500] = 50.0  # a tie goes to the lower index
+    tok, tlp, lp = _sample(logits, want_logprobs=True)
+    want_lp = plain.log_softmax(logits.double().cpu())
+    assert torch.equal(tok.long(), want_lp.argmax(-1))
+    assert tok[3] == 17
+    assert torch.allclose(lp.double(), want_lp, atol=1e-5)
+    assert torch.allclose(tlp.double(), want_lp.gather(1, tok.long()[:, None])[:, 0], atol=1e-5)
+
+
+def _support(probs_row, n=4000, **kw):
+    """Empirical distribution of n draws (n rows, one counter each)."""
+    V = probs_row.numel()
+    logits = torch.log(probs_row).float().to(DEV)[None].repeat(n, 1).contiguous()
+    tok, _, _ = _sample(logits, counter=list(range(n)), **kw)
+    return torch.bincount(tok.long(), minlength=V).double() / n
+
+
+def test_sample_temperature_distribution():
+    p = torch.tensor([0.5, 0.25, 0.125, 0.0625, 0.0625])
+    freq = _support(p, n=8000, temp=1.0, seed=5)
+    assert (freq - p.double()).abs().max() < 0.02
+    # temperature 0.5 squares the probabilities
+    q = p.double() ** 2
+    q = q / q.sum()
+    freq = _support(p, n=8000, temp=0.5, seed=6)
+    assert (freq - q).abs().max() < 0.02
+
+
+def test_sample_filters_match_reference_vectors():
+    # vectors of the reference's tests/test_sample_utils.py:19-105
+    p = torch.tensor([0.9, 1e-9, 1e-9, 0.1])
+    f = _support(p / p.sum(), n=500, temp=1.0, top_p=0.3, seed=1)
+    assert f[0] == 1.0
+    p = torch.tensor([1e-9, 0.5, 0.4, 0.1])
+    f = _support(p / p.sum(), n=6000, temp=1.0, top_p=0.6, seed=2)
+    assert f[0] == 0 and f[3] == 0 and abs(f[1] - 0.5556) < 0.03
+    f = _support(p / p.sum(), n=6000, temp=1.0, top_p=0.95, seed=3)
+    assert f[0] == 0 and abs(f[1] - 0.5) < 0.03 and abs(f[3] - 0.1) < 0.02
+    p = torch.tensor([0.6, 1e-9, 0.1, 0.3])
+    f = _support(p / p.sum(), n=6000, temp=1.0, top_k=2, seed=4)
+    assert f[1] == 0 and f[2] == 0 and abs(f[0] - 0.6667) < 0.03
+    p = torch.tensor([0.9, 1e-9, 1e-9, 0.1])
+    f = _support(p / p.sum(), n=500, temp=1.0, min_p=0.8, seed=5)
+    assert f[0] == 1.0
+    f = _support(p / p.sum(), n=4000, temp=1.0, min_p=0.05, seed=6)
+    assert abs(f[0] - 0.9) < 0.03 and f[1] == 0
+    # min_tokens_to_keep keeps the two best although min_p would drop one
+    f = _support(p / p.sum(), n=4000, temp=1.0, min_p=0.8, min_keep=2, seed=7)
+    assert abs(f[3] - 0.1) < 0.03 and f[1] == 0 and f[2] == 0
+
+
+def test_sample_filters_against_plain_on_random_rows():
+    g = torch.Generator().manual_seed(9)
+    V = 777
+    logits = (torch.randn(6, V, generator=g) * 2.5).float()
+    lp = plain.log_softmax(logits.double())
+    for kw, filt in [
+        (dict(top_p=0.7), lambda x: plain.top_p_filter(x, 0.7)),
+        (dict(top_k=13), lambda x: plain.top_k_filter(x, 13)),
+        (dict(min_p=0.2, min_keep=5), lambda x: plain.min_p_filter(x, 0.2, 5)),
+        (dict(top_p=0.9, min_p=0.05, top_k=20),
+         lambda x: plain.top_k_filter(plain.min_p_filter(plain.top_p_filter(x, 0.9), 0.05), 20)),
+        (dict(xtc_prob=1.0, xtc_thr=0.02, special=[int(lp[0].argmax())]),
+         lambda x: plain.xtc_filter(x, 0.02, [int(lp[0].argmax())])),
+    ]:
+        allowed = torch.isfinite(filt(lp.clone()))
+        seen = torch.zeros_like(allowed)
+        for counter in range(60):
+            tok, _, _ = _sample(logits.to(DEV), temp=1.5, seed=11, counter=counter, **kw)
+            seen[torch.arange(6), tok.long()] = True
+        assert not (seen & ~allowed).any(), kw
+        # small supports are covered completely
+        small = allowed.sum(-1) <= 6
+        assert torch.equal((seen & allowed)[small], allowed[small]), kw
+
+
+def test_sample_seed_and_batch_independence():
+    logits = _rand((5, 300), torch.float32, 30, 2.0)
+    a, _, _ = _sample(logits, temp=0.9, seed=[1, 2, 3, 4, 5], counter=[0, 1, 2, 3, 4])
+    b, _, _ = _sample(logits, temp=0.9, seed=[1, 2, 3, 4, 5], counter=[0, 1, 2, 3, 4])
+    assert torch.equal(a, b)
+    # row 2 alone gives the same token as row 2 in the batch
+    c, _, _ = _sample(logits[2:3].contiguous(), temp=0.9, seed=[3], counter=[2])
+    assert c[0] == a[2]
+    draws = {int(_sample(logits[:1].contiguous(), temp=2.0, seed=[7], counter=[i])[0][0]) for i in range(16)}
+    assert len(draws) > 1
+
+
+def test_logit_bias_and_penalties():
+    k = _k()
+    V = 50
+    logits = _rand((3, V), torch.float32, 40)
+    base = logits.double().cpu()
+    offsets = torch.tensor([0, 2, 2, 5], dtype=torch.int32, device=DEV)
+    idx = torch.tensor([0, 7, 3, 3, 9], dtype=torch.int32, device=DEV)
+    val = torch.tensor([2000.0, -1.0, 0.5, 0.25, 4.0], device=DEV)
+    x = logits.clone()
+    k.apply_logit_bias(x, offsets, idx, val)
+    want = base.clone()
+    want[0, 0] += 2000
+    want[0, 7] -= 1
+    want[2, 3] += 0.75
+    want[2, 9] += 4
+    assert torch.allclose(x.double().cpu(), want, atol=1e-4)
+
+    hist_rows = [[5, 6, 5, 7, 5], [], [1, 2, 3, 4, 1, 1, 9]]
+    hist = torch.tensor(sum(hist_rows, []), dtype=torch.int32, device=DEV)
+    offsets = torch.tensor([0, 5, 5, 12], dtype=torch.int32, device=DEV)
+    f32 = lambda v: torch.tensor(v, dtype=torch.float32, device=DEV)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    rep, pres, freq = [1.3, 1.3, 0.0], [0.5, 0.0, 0.25], [0.0, 0.1, 0.2]
+    rep_ctx, pres_ctx, freq_ctx = [20, 20, 20], [2, 20, 3], [20, 20, 4]
+    x = logits.clone()
+    k.apply_penalties(x, offsets, hist, f32(rep), i32(rep_ctx), f32(pres), i32(pres_ctx), f32(freq),
+                      i32(freq_ctx))
+    for r in range(3):
+        want = base[r].clone()
+        if rep[r]:
+            want = plain.repetition_penalty(want, hist_rows[r], rep[r], rep_ctx[r])
+        if pres[r]:
+            want = plain.presence_penalty(want, hist_rows[r], pres[r], pres_ctx[r])
+        if freq[r]:
+            want = plain.frequency_penalty(want, hist_rows[r], freq[r], freq_ctx[r])
+        assert torch.allclose(x[r].double().cpu(), want, atol=1e-5), r
