@@ -1,0 +1,275 @@
+"""Pages of keys and values for every live request, and slots of fixed-size state.
+
+The reference keeps one growing array per layer and request (``KVCache``,
+mlx_lm/models/cache.py:325-407) or per layer and batch (``BatchKVCache``,
+921-1139, batched by padding), sliding windows in ``RotatingKVCache``
+(410-591) and fixed-size state in ``ArraysCache`` (594-733).  Here memory is
+cut into pages of ``page_size`` tokens instead:
+
+* Cache slots (one per layer run that writes a cache) whose mixers want the
+  same thing -- same key heads, head size and window -- form a *group*.  A
+  group has one pool of pages; page ``p`` of the group is one page in every
+  slot of the group, so a request has one block table per group.
+* A request's block table lists, for block ``b`` (positions ``b*page_size ..``),
+  the page that holds it, or -1 once a window has passed it.
+* Pages are taken before a step runs (``reserve``) and counted as filled after
+  it (``commit``); they are given back when the request ends (``release``), is
+  cut short (``truncate``) or, in a windowed group, when every later query is
+  out of their reach.
+* Every request also gets a state slot: a row in each fixed-size state tensor
+  (zeroed when the request starts), whether or not any mixer asks for one.
+"""
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional
+
+from ..config.plan import CacheNeed, StateNeed
+from .pages import PagePool
+
+
+class OutOfPages(RuntimeError):
+    """Not enough free pages for what was asked."""
+
+
+class OutOfSlots(RuntimeError):
+    """Every state slot is taken."""
+
+
+@dataclass
+class RequestCache:
+    request_id: object
+    state_slot: int
+    length: int = 0  # tokens whose keys and values are in the pages
+    reserved: int = 0  # tokens that have pages (>= length)
+    blocks: List[List[int]] = field(default_factory=list)  # per group: page of each block or -1
+
+
+class _Group:
+    def __init__(self, need: CacheNeed, n_pages):
+        self.need = need
+        self.slots: List[int] = []
+        self.pool = PagePool(n_pages)
+        self.storage = None  # [n_slots, n_pages, 2, n_kv_heads, page_size, head_dim]
+
+
+class CacheManager:
+    """Pages, block tables and state slots for the requests that are live.
+
+    ``needs`` has one entry per cache slot: a ``CacheNeed``, a ``StateNeed`` or
+    ``None``.  ``n_pages`` is the number of pages of every group.  With
+    ``device`` set, storage is allocated there in ``dtype``; without, the
+    manager only does the bookkeeping (for tests and dry runs).
+    """
+
+    def __init__(self, needs, page_size, n_pages, max_requests, dtype=None, device=None):
+        if page_size <= 0 or page_size % 16:
+            raise ValueError(f"page_size must be a positive multiple of 16, got {page_size}")
+        if max_requests <= 0:
+            raise ValueError("max_requests must be positive")
+        self.page_size, self.n_pages, self.max_requests = page_size, n_pages, max_requests
+        self.dtype, self.device = dtype, device
+        self.groups: List[_Group] = []
+        self.slot_group: Dict[int, tuple] = {}  # cache slot -> (group index, index in the group)
+        self.state_needs: Dict[int, StateNeed] = {}
+        self.state_storage: Dict[int, object] = {}
+        by_need = {}
+        for slot, need in enumerate(needs):
+            if isinstance(need, CacheNeed):
+                if need not in by_need:
+                    by_need[need] = len(self.groups)
+                    self.groups.append(_Group(need, n_pages))
+                g = by_need[need]
+                self.slot_group[slot] = (g, len(self.groups[g].slots))
+                self.groups[g].slots.append(slot)
+            elif isinstance(need, StateNeed):
+                self.state_needs[slot] = need
+            elif need is not None:
+                raise TypeError(f"cache slot {slot}: unknown need {need!r}")
+        self._free_state_slots = list(range(max_requests - 1, -1, -1))
+        self.requests: Dict[object, RequestCache] = {}
+        if device is not None:
+            self._allocate()
+
+    def _allocate(self):
+        import torch
+
+        for g in self.groups:
+            n = g.need
+            g.storage = torch.zeros(
+                (len(g.slots), self.n_pages, 2, n.n_kv_heads, self.page_size, n.head_dim),
+                dtype=self.dtype,
+                device=self.device,
+            )
+        for slot, need in self.state_needs.items():
+            self.state_storage[slot] = torch.zeros(
+                (self.max_requests, *need.shape), dtype=getattr(torch, need.dtype), device=self.device
+            )
+
+    # -- sizes ---------------------------------------------------------------
+
+    def blocks_for(self, n_tokens):
+        return (n_tokens + self.page_size - 1) // self.page_size
+
+    def bytes_per_token(self):
+        """Bytes of keys and values that one token takes over all slots."""
+        import torch
+
+        size = torch.empty((), dtype=self.dtype).element_size() if self.dtype is not None else 0
+        return sum(2 * g.need.n_kv_heads * g.need.head_dim * len(g.slots) * size for g in self.groups)
+
+    def free_pages(self):
+        """Free pages of the group that has fewest."""
+        return min((g.pool.n_free for g in self.groups), default=self.n_pages)
+
+    def pages_needed(self, request_id, n_new):
+        """Pages that ``reserve(request_id, n_new)`` would take (the most over the groups)."""
+        rc = self.requests[request_id]
+        return max(0, self.blocks_for(rc.length + n_new) - self.blocks_for(rc.reserved))
+
+    # -- life of a request -----------------------------------------------------
+
+    def add(self, request_id):
+        if request_id in self.requests:
+            raise ValueError(f"request {request_id!r} is already live")
+        if not self._free_state_slots:
+            raise OutOfSlots(f"all {self.max_requests} request slots are taken")
+        slot = self._free_state_slots.pop()
+        rc = RequestCache(request_id, slot, blocks=[[] for _ in self.groups])
+        self.requests[request_id] = rc
+        for storage in self.state_storage.values():
+            storage[slot].zero_()
+        return rc
+
+    def reserve(self, request_id, n_new):
+        """Make sure positions ``length .. length+n_new-1`` have pages in every group.
+
+        All or nothing: if any group is short, nothing is taken and
+        ``OutOfPages`` is raised.
+        """
+        rc = self.requests[request_id]
+        if n_new < 0:
+            raise ValueError("cannot reserve a negative number of tokens")
+        want_blocks = self.blocks_for(rc.length + n_new)
+        taken = []
+        for gi, g in enumerate(self.groups):
+            extra = want_blocks - len(rc.blocks[gi])
+            pages = g.pool.take(extra) if extra > 0 else []
+            if pages is None:
+                for gj, got in taken:
+                    self.groups[gj].pool.give_back(got)
+                raise OutOfPages(
+                    f"request {request_id!r} needs {extra} more pages, {g.pool.n_free} are free"
+                )
+            taken.append((gi, pages))
+        for gi, pages in taken:
+            rc.blocks[gi].extend(pages)
+        rc.reserved = max(rc.reserved, rc.length + n_new)
+        return rc
+
+    def commit(self, request_id, n_new):
+        """Count ``n_new`` more tokens as stored; give back pages a window has passed."""
+        rc = self.requests[request_id]
+        if rc.length + n_new > rc.reserved:
+            raise ValueError(f"request {request_id!r}: committing tokens that were never reserved")
+        rc.length += n_new
+        for gi, g in enumerate(self.groups):
+            w = g.need.window
+            if w <= 0:
+                continue
+            # the next query sits at position >= length and sees keys > position - w
+            first_needed = max(0, rc.length - w + 1)
+            for b in range(first_needed // self.page_size):
+                if rc.blocks[gi][b] >= 0:
+                    g.pool.give_back([rc.blocks[gi][b]])
+                    rc.blocks[gi][b] = -1
+        return rc
+
+    def truncate(self, request_id, new_length):
+        """Forget the tokens from ``new_length`` on (``trim`` of mlx_lm/models/cache.py:378-381).
+
+        Whole pages beyond the new end go back.  A windowed group that has
+        already given back pages the shorter sequence would need again cannot
+        be truncated.
+        """
+        rc = self.requests[request_id]
+        if not (0 <= new_length <= rc.length):
+            raise ValueError(f"cannot truncate request {request_id!r} from {rc.length} to {new_length}")
+        keep = self.blocks_for(new_length)
+        for gi, g in enumerate(self.groups):
+            w = g.need.window
+            if w > 0:
+                first_needed = max(0, new_length - w + 1) // self.page_size
+                if any(p < 0 for p in rc.blocks[gi][first_needed:keep]):
+                    raise ValueError(
+                        f"request {request_id!r}: a window has already dropped pages that "
+                        f"length {new_length} needs"
+                    )
+        for gi, g in enumerate(self.groups):
+            tail = [p for p in rc.blocks[gi][keep:] if p >= 0]
+            g.pool.give_back(tail)
+            del rc.blocks[gi][keep:]
+        rc.length = new_length
+        rc.reserved = min(rc.reserved, keep * self.page_size)
+        rc.reserved = max(rc.reserved, rc.length)
+        return rc
+
+    def release(self, request_id):
+        """The request is over: all its pages and its state slot go back."""
+        rc = self.requests.pop(request_id)
+        for gi, g in enumerate(self.groups):
+            g.pool.give_back([p for p in rc.blocks[gi] if p >= 0])
+        self._free_state_slots.append(rc.state_slot)
+
+    def release_all(self):
+        for rid in list(self.requests):
+            self.release(rid)
+
+    # -- views for a step ------------------------------------------------------
+
+    def block_table(self, request_id, group):
+        return self.requests[request_id].blocks[group]
+
+    def kv(self, slot):
+        """``(keys, values)`` of cache slot ``slot``, each ``[n_pages, n_kv_heads, page, head_dim]``."""
+        g, i = self.slot_group[slot]
+        s = self.groups[g].storage[i]
+        return s[:, 0], s[:, 1]
+
+    def state(self, slot):
+        """State tensor of cache slot ``slot``: ``[max_requests, *shape]``."""
+        return self.state_storage[slot]
+
+    def poison_free_pages(self, value=float("nan")):
+        """Overwrite every page that no request holds (tests: stale pages must not matter)."""
+        import torch
+
+        for g in self.groups:
+            free = torch.tensor(sorted(g.pool._free), dtype=torch.long, device=g.storage.device)
+            if free.numel():
+                g.storage[:, free] = value
+
+    def check(self):
+        """No page lost, held twice or free while in a block table."""
+        for gi, g in enumerate(self.groups):
+            g.pool.check()
+            seen = {}
+            for rc in self.requests.values():
+                for p in rc.blocks[gi]:
+                    if p < 0:
+                        continue
+                    if p in seen:
+                        raise AssertionError(
+                            f"group {gi}: page {p} held by {seen[p]!r} and {rc.request_id!r}"
+                        )
+                    if not g.pool._held[p]:
+                        raise AssertionError(f"group {gi}: page {p} in a block table but free")
+                    seen[p] = rc.request_id
+            if len(seen) != g.pool.n_held:
+                raise AssertionError(
+                    f"group {gi}: {g.pool.n_held} pages held but {len(seen)} in block tables"
+                )
+        slots = [rc.state_slot for rc in self.requests.values()]
+        if len(set(slots)) != len(slots) or set(slots) & set(self._free_state_slots):
+            raise AssertionError("a state slot is held twice or both held and free")
+        if len(slots) + len(self._free_state_slots) != self.max_requests:
+            raise AssertionError("a state slot is lost")

@@ -1,0 +1,228 @@
+"""The step function: one batch of (request, its next tokens) through the model."""
+
+from dataclasses import dataclass
+from typing import List, Sequence
+
+import torch
+
+from ..cache import CacheManager
+from ..weights.loader import resolve_dtype
+from .context import ROW_KERNEL_MAX_Q, TILE_Q, AttentionPlan, Scratch, StepContext
+
+
+@dataclass
+class StepEntry:
+    """A request's share of a step: its next tokens and the places, among
+    these tokens, whose logits are wanted."""
+
+    request_id: object
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+class _HostRing:
+    """Pinned host buffers for the step's integer arrays, reused in turn.
+
+    A buffer is written again only after the copy that read it has finished.
+    """
+
+    def __init__(self, n=4):
+        self.bufs = [None] * n
+        self.events = [None] * n
+        self.i = 0
+
+    def get(self, n_ints):
+        self.i = (self.i + 1) % len(self.bufs)
+        if self.events[self.i] is not None:
+            self.events[self.i].synchronize()
+        b = self.bufs[self.i]
+        if b is None or b.numel() < n_ints:
+            b = torch.empty(max(n_ints, 4096), dtype=torch.int32, pin_memory=True)
+            self.bufs[self.i] = b
+        return b
+
+    def mark(self):
+        ev = self.events[self.i] or torch.cuda.Event()
+        ev.record()
+        self.events[self.i] = ev
+
+
+class Engine:
+    """A model, its cache and the step function over them.
+
+    ``step(entries)`` runs exactly the tokens it is given as one flat batch --
+    portions of prompts beside single decoded tokens, cut anywhere -- against
+    what earlier steps left in the cache, and returns float32 logits at the
+    wanted places.  The reference's forward takes a rectangle of tokens and
+    returns logits everywhere (mlx_lm/models/gpt2.py:161-168); callers there
+    slice or drop them (mlx_lm/generate.py:398,424-431,1244,1415).
+    """
+
+    def __init__(self, model, dtype="bfloat16", device="cuda:0", page_size=16, n_pages=None,
+                 max_tokens=None, max_requests=64):
+        if not torch.cuda.is_available():
+            raise RuntimeError("the engine needs a GPU: torch.cuda.is_available() is false")
+        self.model = model
+        self.decoder = model.decoder
+        self.dtype = resolve_dtype(dtype)
+        self.device = torch.device(device)
+        torch.cuda.set_device(self.device)
+        if n_pages is None:
+            if max_tokens is None:
+                raise ValueError("give the cache size as n_pages or max_tokens")
+            n_pages = (max_tokens + page_size - 1) // page_size
+        self.cache = CacheManager(self.decoder.cache_needs(), page_size, n_pages, max_requests,
+                                  dtype=self.dtype, device=self.device)
+        self.scratch = Scratch(self.device)
+        self._ring = _HostRing()
+        self._meta_dev = None
+        self._logits = None
+        self.steps = 0
+
+    # -- buffers ---------------------------------------------------------------
+
+    def logits_buffer(self, n_rows, vocab):
+        if self._logits is None or self._logits.shape[0] < n_rows or self._logits.shape[1] != vocab:
+            self._logits = torch.empty((max(n_rows, 8), vocab), dtype=torch.float32, device=self.device)
+        return self._logits[:n_rows]
+
+    # -- requests --------------------------------------------------------------
+
+    def add_request(self, request_id):
+        return self.cache.add(request_id)
+
+    def end_request(self, request_id):
+        self.cache.release(request_id)
+
+    def has_request(self, request_id):
+        return request_id in self.cache.requests
+
+    def context_len(self, request_id):
+        return self.cache.requests[request_id].length
+
+    # -- the step --------------------------------------------------------------
+
+    def _check(self, entries):
+        seen = set()
+        V, P = self.decoder.vocab_size, self.decoder.max_positions
+        for e in entries:
+            if e.request_id in seen:
+                raise ValueError(f"request {e.request_id!r} occurs twice in one step")
+            seen.add(e.request_id)
+            if e.request_id not in self.cache.requests:
+                raise KeyError(f"request {e.request_id!r} is not live")
+            n = len(e.tokens)
+            if n == 0:
+                raise ValueError(f"request {e.request_id!r} brings no tokens")
+            for t in e.tokens:
+                if not (0 <= int(t) < V):
+                    raise ValueError(f"token id {t} of request {e.request_id!r} is outside [0, {V})")
+            length = self.cache.requests[e.request_id].length
+            if length + n > P:
+                raise ValueError(
+                    f"request {e.request_id!r} would reach {length + n} tokens, the model "
+                    f"has {P} positions"
+                )
+            for w in e.want:
+                if not (0 <= int(w) < n):
+                    raise ValueError(f"wanted place {w} of request {e.request_id!r} is outside its {n} tokens")
+
+    def step(self, entries: List[StepEntry]):
+        """Run one batch; returns float32 logits ``[n_wanted, vocab]`` (``None`` if nothing is wanted).
+
+        The returned tensor is a view of a buffer that the next step overwrites.
+        """
+        if not entries:
+            return None
+        self._check(entries)
+        cm = self.cache
+        # pages first: all or nothing for the whole step
+        done = []
+        try:
+            for e in entries:
+                cm.reserve(e.request_id, len(e.tokens))
+                done.append(e)
+        except Exception:
+            for e in done:
+                rc = cm.requests[e.request_id]
+                cm.truncate(e.request_id, rc.length)  # gives back pages beyond what is stored
+            raise
+
+        ctx = self._build_context(entries)
+        self.scratch.reset()
+        logits = self.decoder.forward(ctx)
+        for e in entries:
+            cm.commit(e.request_id, len(e.tokens))
+        self.steps += 1
+        return logits
+
+    def _build_context(self, entries):
+        cm = self.cache
+        R = len(entries)
+        T = sum(len(e.tokens) for e in entries)
+        ctx = StepContext(self)
+        q_start = 0
+        token_ids, positions, token_req, wanted, slot_ids = [], [], [], [], []
+        tiles, rows, all_tiles = [], [], []
+        plan = AttentionPlan()
+        for r, e in enumerate(entries):
+            rc = cm.requests[e.request_id]
+            n = len(e.tokens)
+            ctx.q_starts.append(q_start)
+            ctx.q_lens.append(n)
+            ctx.context_lens.append(rc.length)
+            token_ids.extend(int(t) for t in e.tokens)
+            positions.extend(range(rc.length, rc.length + n))
+            token_req.extend([r] * n)
+            wanted.extend(q_start + int(w) for w in e.want)
+            slot_ids.append(rc.state_slot)
+            for s in range(0, n, TILE_Q):
+                all_tiles.extend((q_start + s, min(TILE_Q, n - s)))
+            if n <= ROW_KERNEL_MAX_Q:
+                rows.extend(range(q_start, q_start + n))
+                plan.max_row_context = max(plan.max_row_context, rc.length + n)
+            else:
+                for s in range(0, n, TILE_Q):
+                    tiles.extend((q_start + s, min(TILE_Q, n - s)))
+            q_start += n
+        plan.n_tiles, plan.n_rows, plan.n_all_tiles = len(tiles) // 2, len(rows), len(all_tiles) // 2
+
+        # block tables, one per group, padded to the longest of the step
+        tables = []
+        for gi in range(len(cm.groups)):
+            width = max(1, max(len(cm.requests[e.request_id].blocks[gi]) for e in entries))
+            flat = []
+            for e in entries:
+                b = cm.requests[e.request_id].blocks[gi]
+                flat.extend(b)
+                flat.extend([-1] * (width - len(b)))
+            tables.append((width, flat))
+
+        # everything in one pinned buffer and one copy; pieces start on 4-int boundaries
+        pieces = [token_ids, positions, token_req, wanted, slot_ids, tiles, rows, all_tiles]
+        pieces += [flat for _, flat in tables]
+        offsets, total = [], 0
+        for p in pieces:
+            offsets.append(total)
+            total += (len(p) + 3) // 4 * 4
+        host = self._ring.get(total)
+        for off, p in zip(offsets, pieces):
+            if p:
+                host[off : off + len(p)] = torch.tensor(p, dtype=torch.int32)
+        if self._meta_dev is None or self._meta_dev.numel() < total:
+            self._meta_dev = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
+        dev = self._meta_dev
+        dev[:total].copy_(host[:total], non_blocking=True)
+        self._ring.mark()
+
+        def piece(i, n):
+            return dev[offsets[i] : offsets[i] + n]
+
+        ctx.n_tokens, ctx.n_requests, ctx.n_wanted = T, R, len(wanted)
+        ctx.token_ids, ctx.positions, ctx.token_req = piece(0, T), piece(1, T), piece(2, T)
+        ctx.wanted_rows, ctx.slot_ids = piece(3, len(wanted)), piece(4, R)
+        plan.tiles, plan.rows, plan.all_tiles = piece(5, len(tiles)), piece(6, len(rows)), piece(7, len(all_tiles))
+        ctx.attention_plan = plan
+        for gi, (width, flat) in enumerate(tables):
+            ctx.block_tables.append(piece(8 + gi, len(flat)).view(R, width))
+        return ctx

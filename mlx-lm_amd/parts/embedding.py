@@ -1,0 +1,36 @@
+"""Token embedding: a row of the table for each token, written to the residual stream."""
+
+from ..ops import kernels
+from .base import Part, TensorSpec, register_embedding
+
+
+class TokenEmbedding(Part):
+    """``h[t] = table[ids[t]]``, plus a position term if the model has one.
+
+    mlx_lm/models/gpt2.py:119-120,132.
+    """
+
+    def __init__(self, vocab_size, width, weight_name="weight", prefix=""):
+        super().__init__(prefix)
+        if vocab_size <= 0 or width <= 0:
+            raise ValueError(f"embedding sizes must be positive, got {vocab_size} x {width}")
+        self.vocab_size, self.width = vocab_size, width
+        self.weight_name = self._name(weight_name)
+        self.table = None
+
+    def tensors(self):
+        return {self.weight_name: TensorSpec((self.vocab_size, self.width), "matrix")}
+
+    def load(self, tensors):
+        self.table = tensors[self.weight_name]
+
+    def forward(self, ctx, out, add=None):
+        """Fill float32 ``out [tokens, width]``; ``add`` is ``(table, index)`` or ``None``."""
+        if add is None:
+            kernels.embed_gather_add(out, self.table, ctx.token_ids)
+        else:
+            kernels.embed_gather_add(out, self.table, ctx.token_ids, add[0], add[1])
+        return out
+
+
+register_embedding("token", TokenEmbedding)

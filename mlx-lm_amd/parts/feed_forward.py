@@ -1,0 +1,47 @@
+"""Feed-forward parts."""
+
+from ..ops import kernels
+from .base import FeedForward, TensorSpec, register_feed_forward
+
+_TANH_GELU = ("gelu_new", "gelu_pytorch_tanh", "gelu_tanh", "gelu_approx")
+
+
+class GeluMLP(FeedForward):
+    """``residual += c_proj(gelu_tanh(c_fc(x)))``, dense, with biases.
+
+    mlx_lm/models/gpt2.py:71-80; the activation and the bias add are fused
+    into the first product, the residual add into the second.
+    """
+
+    def __init__(self, width, inner, activation="gelu_new", prefix=""):
+        super().__init__(prefix)
+        if activation not in _TANH_GELU:
+            raise ValueError(
+                f"activation '{activation}' is not implemented (only the tanh GELU: {_TANH_GELU})"
+            )
+        if width % 8 or inner % 8:
+            raise ValueError(f"feed-forward sizes must be multiples of 8, got {width} and {inner}")
+        self.width, self.inner = width, inner
+        self.fc_w = self.fc_b = self.proj_w = self.proj_b = None
+
+    def tensors(self):
+        n = self._name
+        return {
+            n("c_fc.weight"): TensorSpec((self.inner, self.width), "matrix"),
+            n("c_fc.bias"): TensorSpec((self.inner,), "vector"),
+            n("c_proj.weight"): TensorSpec((self.width, self.inner), "matrix"),
+            n("c_proj.bias"): TensorSpec((self.width,), "vector"),
+        }
+
+    def load(self, tensors):
+        n = self._name
+        self.fc_w, self.fc_b = tensors[n("c_fc.weight")], tensors[n("c_fc.bias")]
+        self.proj_w, self.proj_b = tensors[n("c_proj.weight")], tensors[n("c_proj.bias")]
+
+    def forward(self, ctx, x, residual):
+        act = ctx.scratch((x.shape[0], self.inner), ctx.dtype)
+        kernels.linear(act, x, self.fc_w, self.fc_b, gelu=True)
+        kernels.linear(residual, act, self.proj_w, self.proj_b, accumulate=True)
+
+
+register_feed_forward("gelu_mlp", GeluMLP)

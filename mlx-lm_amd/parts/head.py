@@ -1,0 +1,32 @@
+"""Output heads: from the final normed rows to float32 logits."""
+
+from ..ops import kernels
+from .base import Part, TensorSpec, register_head
+
+
+class LinearHead(Part):
+    """``logits = x @ weight.T``, no bias.
+
+    With ``weight_name`` set to the embedding table's name the head is tied:
+    there is one buffer, used by both (``wte.as_linear``,
+    mlx_lm/models/gpt2.py:167).
+    """
+
+    def __init__(self, vocab_size, width, weight_name, prefix=""):
+        super().__init__(prefix)
+        self.vocab_size, self.width = vocab_size, width
+        self.weight_name = weight_name  # a full name: the head may share another part's tensor
+        self.weight = None
+
+    def tensors(self):
+        return {self.weight_name: TensorSpec((self.vocab_size, self.width), "matrix")}
+
+    def load(self, tensors):
+        self.weight = tensors[self.weight_name]
+
+    def forward(self, ctx, x, out):
+        kernels.linear(out, x, self.weight)
+        return out
+
+
+register_head("linear", LinearHead)

@@ -1,0 +1,69 @@
+"""Shared by the tests: tiny configurations, model folders, traces."""
+
+import json
+import os
+
+import torch
+
+import plain_gpt2 as plain
+
+# Two tiny GPT-2 configurations that differ in every size and option, and a
+# third with sizes that are no powers of two anywhere.
+TINY_A = dict(model_type="gpt2", n_layer=2, n_embd=64, n_head=4, n_inner=256, vocab_size=512,
+              n_positions=128, n_ctx=128, layer_norm_epsilon=1e-5, activation_function="gelu_new")
+TINY_B = dict(model_type="gpt2", n_layer=3, n_embd=96, n_head=3, n_inner=384, vocab_size=1000,
+              n_positions=256, n_ctx=256, layer_norm_epsilon=1e-6, activation_function="gelu_new")
+TINY_C = dict(model_type="gpt2", n_layer=2, n_embd=240, n_head=5, n_inner=200, vocab_size=333,
+              n_positions=448, layer_norm_epsilon=3e-4, activation_function="gelu_pytorch_tanh")
+
+TINY = {"A": (TINY_A, 0, "a"), "B": (TINY_B, 1, "b"), "C": (TINY_C, 5, "b")}
+
+
+def sharpen(tensors, config, score_std):
+    """Scale every layer's query and key projections so that attention is
+    peaked: scores get a spread of about ``score_std`` (weights drawn with
+    std 0.02 give 0.0004 * n_embd), so a key that is dropped, doubled or taken
+    from a wrong page changes the output by far more than rounding."""
+    D = config["n_embd"]
+    factor = (score_std / (0.0004 * D)) ** 0.5
+    for i in range(config["n_layer"]):
+        w = tensors[f"h.{i}.attn.c_attn.weight"]  # Conv1D layout [in, 3D]
+        w[:, : 2 * D] *= factor
+        tensors[f"h.{i}.attn.c_attn.bias"][: 2 * D] *= factor
+    return tensors
+
+
+def make_folder(path, name, sharp=0.0, dtype="float32"):
+    """Write tiny model ``name`` to ``path``; returns (config, plain-layout float32 weights)."""
+    from safetensors.torch import load_file, save_file
+
+    from mlx_lm_amd.weights import write_model_folder
+
+    config, seed, scheme = TINY[name]
+    write_model_folder(path, dict(config), seed, scheme, dtype=dtype)
+    f = os.path.join(path, "model.safetensors")
+    tensors = load_file(f)
+    if sharp:
+        tensors = sharpen({k: v.clone() for k, v in tensors.items()}, config, sharp)
+        save_file(tensors, f)
+    weights = plain.from_checkpoint_layout({k: v.float() for k, v in tensors.items()}, config["n_layer"])
+    return config, weights
+
+
+def round_matrices_to_bf16(weights):
+    """What the engine's bfloat16 path holds: matrices rounded, vectors as they are."""
+    out = {}
+    for k, v in weights.items():
+        out[k] = v.to(torch.bfloat16).float() if v.dim() == 2 else v
+    return out
+
+
+def random_tokens(n, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def write_trace(path, steps):
+    with open(path, "w") as fh:
+        for s in steps:
+            fh.write(json.dumps(s) + "\n")

@@ -222,6 +222,25 @@ def conv1d_layout(weights, n_layer):
     return out
 
 
+def from_checkpoint_layout(tensors, n_layer):
+    """Checkpoint tensors to the names and layouts ``forward`` wants.
+
+    What the reference's ``sanitize`` does (mlx_lm/models/gpt2.py:170-196):
+    drop ``attn.bias``, transpose the four Conv1D matrices, prefix ``model.``.
+    """
+    out = {}
+    for k, v in tensors.items():
+        if k.endswith(".attn.bias"):
+            continue
+        out[k] = v
+    for i in range(n_layer):
+        for t in ("attn.c_attn", "attn.c_proj", "mlp.c_fc", "mlp.c_proj"):
+            key = f"h.{i}.{t}.weight"
+            if key in out:
+                out[key] = out[key].t().contiguous()
+    return {(k if k.startswith("model.") else "model." + k): v for k, v in out.items()}
+
+
 # ----------------------------------------------------------------------------
 # sampling (plain forms of mlx_lm/sample_utils.py)
 

@@ -1,0 +1,265 @@
+"""The engine against the plain implementation: whole, decoded, in portions, mixed."""
+
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import plain_gpt2 as plain
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+# max |engine - plain| as a fraction of max |plain logits|.  float32: the
+# engine sums in float32 where the plain implementation has float64.
+# bfloat16: activations are rounded to 8 bits of mantissa between the layers'
+# matrix products (the plain side gets the same bfloat16-rounded matrices).
+TOL = {"float32": 2e-5, "bfloat16": 2.5e-2}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    out = {}
+    for name in ("A", "B", "C"):
+        for sharp in (0.0, 8.0):
+            d = tmp_path_factory.mktemp(f"tiny{name}{int(sharp)}")
+            out[(name, sharp)] = (str(d),) + helpers.make_folder(str(d), name, sharp)
+    return out
+
+
+def _engine(folder, dtype, n_pages, page_size=16, max_requests=8):
+    from mlx_lm_amd.engine import Engine
+    from mlx_lm_amd.utils import load_model
+
+    model, _ = load_model(folder, dtype=dtype)
+    return Engine(model, dtype=dtype, page_size=page_size, n_pages=n_pages, max_requests=max_requests)
+
+
+def _plain_logits(weights, config, tokens, dtype):
+    w = helpers.round_matrices_to_bf16(weights) if dtype == "bfloat16" else weights
+    return plain.forward(w, config, tokens)
+
+
+def _close(got, want, dtype, what=""):
+    scale = want.abs().max().item()
+    err = (got.double().cpu() - want).abs().max().item()
+    assert err <= TOL[dtype] * scale, f"{what}: max error {err:.3e} against scale {scale:.3e}"
+
+
+def _run(engine, rid, tokens, cuts, want_all=True):
+    """Feed ``tokens`` in portions of the given sizes; logits at every position."""
+    from mlx_lm_amd.engine import StepEntry
+
+    engine.add_request(rid)
+    rows, i = [], 0
+    for n in cuts:
+        part = tokens[i : i + n]
+        rows.append(engine.step([StepEntry(rid, part, list(range(len(part))))]).clone())
+        i += n
+    assert i == len(tokens)
+    engine.end_request(rid)
+    return torch.cat(rows)
+
+
+def _cuts_changing(n):
+    sizes, out, i = [7, 2, 64, 3, 16, 2, 33, 5], [], 0
+    while n > 0:
+        s = min(sizes[i % len(sizes)], n)
+        if n - s == 1:  # never leave a single token for the end: portions go down to two
+            s += 1
+        out.append(s)
+        n -= s
+        i += 1
+    return out
+
+
+CASES = [("A", 0.0, 100), ("B", 0.0, 200), ("B", 8.0, 250), ("C", 8.0, 300), ("A", 8.0, 128)]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,sharp,n", CASES)
+def test_whole_decoded_and_portions(folders, dtype, name, sharp, n):
+    folder, config, weights = folders[(name, sharp)]
+    tokens = helpers.random_tokens(n, config["vocab_size"], seed=n)
+    want = _plain_logits(weights, config, tokens, dtype)
+    eng = _engine(folder, dtype, n_pages=(n + 15) // 16 + 2)
+    whole = _run(eng, "whole", tokens, [n])
+    _close(whole, want, dtype, "whole")
+    decoded = _run(eng, "decoded", tokens, [n - 32] + [1] * 32)
+    _close(decoded, want, dtype, "last 32 one by one")
+    portions = _run(eng, "portions", tokens, _cuts_changing(n))
+    _close(portions, want, dtype, "portions of changing size")
+    eng.cache.check()
+    assert eng.cache.free_pages() == eng.cache.n_pages
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_and_long_decode(folders, dtype):
+    """The first tokens of a sequence one by one, then decoding to the last position."""
+    folder, config, weights = folders[("B", 8.0)]
+    n = config["n_positions"]
+    tokens = helpers.random_tokens(n, config["vocab_size"], seed=77)
+    want = _plain_logits(weights, config, tokens, dtype)
+    eng = _engine(folder, dtype, n_pages=n // 16)
+    got = _run(eng, "r", tokens, [1] * n)
+    _close(got[:8], want[:8], dtype, "first tokens")
+    _close(got, want, dtype, "decoding every token")
+    # one more token does not fit the model's positions
+    from mlx_lm_amd.engine import StepEntry
+
+    eng.add_request("full")
+    eng.step([StepEntry("full", tokens, [])])
+    with pytest.raises(ValueError, match="positions"):
+        eng.step([StepEntry("full", [1], [0])])
+
+
+def _mixed_trace(config, seed, lengths, n_live=4):
+    """Steps that mix portions of some requests with decoded tokens of others.
+
+    Requests start when a place is free, run a few portions of changing size,
+    then go on token by token; ends of requests give pages back for the next.
+    """
+    g = torch.Generator().manual_seed(seed)
+    tokens = {f"r{i}": helpers.random_tokens(n, config["vocab_size"], seed * 100 + i) for i, n in enumerate(lengths)}
+    waiting = list(tokens)
+    live, fed, steps, step_no = [], {}, [], 0
+    while waiting or live:
+        while waiting and len(live) < n_live:
+            rid = waiting.pop(0)
+            live.append(rid)
+            fed[rid] = 0
+        entries, ended = [], []
+        for rid in list(live):
+            left = len(tokens[rid]) - fed[rid]
+            if torch.rand((), generator=g).item() < 0.15 and len(live) > 1:
+                continue  # left out of this step, goes on later
+            prompt_part = int(len(tokens[rid]) * 0.6)
+            if fed[rid] < prompt_part:
+                n = int(torch.randint(2, 40, (), generator=g))
+                n = min(n, prompt_part - fed[rid])
+                if prompt_part - fed[rid] - n == 1:
+                    n += 1
+            else:
+                n = 1
+            n = min(n, left)
+            part = tokens[rid][fed[rid] : fed[rid] + n]
+            entries.append({"id": rid, "tokens": part, "want": list(range(n))})
+            fed[rid] += n
+            if fed[rid] == len(tokens[rid]):
+                ended.append(rid)
+                live.remove(rid)
+        if entries:
+            steps.append({"step": step_no, "entries": entries, "end": ended})
+            step_no += 1
+    return tokens, steps
+
+
+def _held(lengths, n_live):
+    return sum(sorted(((n + 63) // 64 * 64 for n in lengths), reverse=True)[:n_live])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,sharp", [("A", 8.0), ("B", 8.0), ("C", 0.0)])
+def test_mixed_batches_with_few_pages(folders, dtype, name, sharp):
+    from mlx_lm_amd.engine import StepEntry
+
+    folder, config, weights = folders[(name, sharp)]
+    P = config["n_positions"]
+    lengths = [min(P, n) for n in (100, 37, 128, 64, 90, 17, 120, 75)]
+    tokens, steps = _mixed_trace(config, seed=3, lengths=lengths)
+    max_tokens = _held(lengths, 4)
+    eng = _engine(folder, dtype, n_pages=max_tokens // 16)
+    got = {rid: [] for rid in tokens}
+    used_pages = set()
+    for s in steps:
+        for e in s["entries"]:
+            if not eng.has_request(e["id"]):
+                eng.add_request(e["id"])
+        eng.cache.poison_free_pages()
+        logits = eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        i = 0
+        for e in s["entries"]:
+            got[e["id"]].append(logits[i : i + len(e["want"])].clone())
+            i += len(e["want"])
+            used_pages.update(eng.cache.block_table(e["id"], 0))
+        for rid in s["end"]:
+            eng.end_request(rid)
+        eng.cache.check()
+    assert any(len(s["entries"]) >= 3 for s in steps)
+    assert sum((n + 15) // 16 for n in lengths) > eng.cache.n_pages  # pages were used again
+    for rid, toks in tokens.items():
+        want = _plain_logits(weights, config, toks, dtype)
+        _close(torch.cat(got[rid]), want, dtype, f"mixed, request {rid}")
+
+
+@pytest.mark.parametrize("page_size", [16, 32, 64])
+def test_page_sizes_agree(folders, page_size):
+    folder, config, weights = folders[("B", 8.0)]
+    tokens = helpers.random_tokens(150, config["vocab_size"], seed=9)
+    want = _plain_logits(weights, config, tokens, "float32")
+    eng = _engine(folder, "float32", n_pages=4 * 64 // page_size, page_size=page_size)
+    got = _run(eng, "r", tokens, [70, 2, 1, 1, 50, 26])
+    _close(got, want, "float32", f"page size {page_size}")
+
+
+def test_out_of_pages_is_an_error_and_takes_nothing(folders):
+    from mlx_lm_amd.cache import OutOfPages
+    from mlx_lm_amd.engine import StepEntry
+
+    folder, config, _ = folders[("A", 0.0)]
+    eng = _engine(folder, "float32", n_pages=4)
+    eng.add_request("a")
+    eng.add_request("b")
+    eng.step([StepEntry("a", list(range(40)), [])])  # 3 pages
+    with pytest.raises(OutOfPages):
+        eng.step([StepEntry("a", [1], [0]), StepEntry("b", list(range(20)), [19])])
+    eng.cache.check()
+    assert eng.cache.free_pages() == 1
+    assert eng.context_len("a") == 40 and eng.context_len("b") == 0
+    out = eng.step([StepEntry("a", [1], [0]), StepEntry("b", list(range(10)), [9])])
+    assert out.shape == (2, config["vocab_size"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(folders, tmp_path, dtype):
+    """bin/trace_run as a user calls it: whole, decoded and mixed, from files."""
+    folder, config, weights = folders[("B", 8.0)]
+    lengths = [90, 40, 130, 64, 70]
+    tokens, steps = _mixed_trace(config, seed=11, lengths=lengths, n_live=3)
+    # a request whole, and the same one with its last 32 tokens one by one
+    whole = helpers.random_tokens(120, config["vocab_size"], seed=5)
+    base = len(steps)
+    steps.append({"step": base, "entries": [{"id": "w", "tokens": whole, "want": list(range(120))}], "end": ["w"]})
+    steps.append({"step": base + 1, "entries": [{"id": "d", "tokens": whole[:88], "want": list(range(88))}], "end": []})
+    for i in range(32):
+        steps.append({"step": base + 2 + i, "entries": [{"id": "d", "tokens": [whole[88 + i]], "want": [0]}],
+                      "end": ["d"] if i == 31 else []})
+    trace = tmp_path / "trace.jsonl"
+    helpers.write_trace(trace, steps)
+    out = tmp_path / "out"
+    with open(trace) as fh:
+        proc = subprocess.run(
+            [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+             "--out", str(out), "--max-tokens", str(_held(lengths + [128], 3))],
+            stdin=fh, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.split("\n") if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+    V = config["vocab_size"]
+    got = {}
+    for s in steps:
+        data = np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(-1, V)
+        i = 0
+        for e in s["entries"]:
+            got.setdefault(e["id"], []).append(torch.from_numpy(data[i : i + len(e["want"])].copy()))
+            i += len(e["want"])
+        assert i == data.shape[0]
+    tokens["w"] = whole
+    tokens["d"] = whole
+    for rid, toks in tokens.items():
+        want = _plain_logits(weights, config, toks, dtype)
+        _close(torch.cat(got[rid]), want, dtype, f"trace_run, request {rid}")
