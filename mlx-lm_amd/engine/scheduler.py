@@ -1,0 +1,289 @@
+"""Continuous batching above the step function.
+
+The reference's ``BatchGenerator`` (mlx_lm/generate.py:1565-1945) keeps a FIFO
+of prompts, a prefill batch and a generation batch, and runs them as two
+padded model calls per iteration.  Here one ``step`` holds both kinds of work:
+
+1. every decoding request brings its one next token;
+2. what is left of ``max_num_batched_tokens`` goes to requests that are still
+   reading their prompt, in order of admission, as portions of at most
+   ``prefill_step_size`` tokens;
+3. waiting requests are admitted, first come first served, while fewer than
+   ``max_num_seqs`` run and the pages for their whole prompt are free.
+
+When pages run out for a decoding request, the request admitted last is
+pre-empted: its pages are given back and it returns to the *front* of the
+waiting queue with everything it has generated kept; when it is admitted again
+it reads prompt and generated tokens as one prompt and goes on where it was
+(sampling is keyed by the index of the generated token, so the continuation
+does not change).  A request that could never fit the pool alone is refused
+when it is added.
+
+Decisions (``plan_step``) are pure bookkeeping on the host and can be tested
+without a GPU; ``step`` runs a plan through the engine and the sampler.
+"""
+
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Any, Callable, List, Optional, Sequence
+
+from .step import StepEntry
+
+
+@dataclass
+class Request:
+    """One generation request and its progress."""
+
+    request_id: Any
+    prompt: List[int]
+    max_tokens: int
+    sampler: Any = None
+    logits_processors: Optional[list] = None
+    stop_sequences: Sequence[Sequence[int]] = ()
+    seed: int = 0
+    want_logprobs: bool = False
+    # progress
+    generated: List[int] = field(default_factory=list)
+    num_computed: int = 0  # tokens of prompt+generated whose keys and values are in the cache
+    finish_reason: Optional[str] = None
+    preemptions: int = 0
+    order: int = 0
+
+    @property
+    def tokens(self):
+        return self.prompt + self.generated
+
+    @property
+    def num_tokens(self):
+        return len(self.prompt) + len(self.generated)
+
+    @property
+    def decoding(self):
+        """All but the newest token are computed: the next step brings one token."""
+        return self.num_computed == self.num_tokens - 1 and len(self.generated) > 0
+
+
+@dataclass
+class StepOutput:
+    """What a step produced for one request (cf. mlx_lm/generate.py:1321-1328)."""
+
+    request_id: Any
+    token: int
+    logprob: float
+    finish_reason: Optional[str] = None
+    logprobs: Any = None  # float32 [vocab] device tensor when the request asked for it
+
+
+@dataclass
+class PlannedEntry:
+    request: Request
+    n_tokens: int
+    samples: bool  # the portion ends at the request's newest token: its logits are wanted
+
+
+@dataclass
+class SchedulerStats:
+    steps: int = 0
+    prompt_tokens: int = 0
+    generation_tokens: int = 0
+    preemptions: int = 0
+    pages_high_water: int = 0
+
+
+def stops(tokens, stop_sequences):
+    """True if ``tokens`` ends with one of the stop sequences.
+
+    The reference matches with a trie over token ids (mlx_lm/generate.py:
+    887-956); a suffix comparison finds the same matches.
+    """
+    for s in stop_sequences:
+        n = len(s)
+        if n and len(tokens) >= n and list(tokens[-n:]) == list(s):
+            return True
+    return False
+
+
+class Scheduler:
+    """Admits requests, cuts prompts into portions, decodes, finishes and frees."""
+
+    def __init__(self, engine, sample: Callable, max_num_seqs=32, max_num_batched_tokens=2048,
+                 prefill_step_size=2048):
+        if max_num_seqs <= 0 or max_num_batched_tokens <= 0 or prefill_step_size <= 0:
+            raise ValueError("max_num_seqs, max_num_batched_tokens and prefill_step_size must be positive")
+        self.engine = engine
+        self.cache = engine.cache
+        self.sample = sample
+        self.max_positions = engine.decoder.max_positions
+        self.max_num_seqs = min(max_num_seqs, self.cache.max_requests)
+        self.max_num_batched_tokens = max_num_batched_tokens
+        self.prefill_step_size = prefill_step_size
+        self.waiting = deque()
+        self.running: List[Request] = []
+        self.stats = SchedulerStats()
+        self._order = 0
+
+    # -- requests ----------------------------------------------------------------
+
+    def add(self, request: Request):
+        if not request.prompt:
+            raise ValueError("a request needs a prompt of at least one token")
+        if request.max_tokens < 0:
+            raise ValueError("max_tokens must not be negative")
+        if len(request.prompt) > self.max_positions:
+            raise ValueError(
+                f"the prompt has {len(request.prompt)} tokens, the model has {self.max_positions} positions"
+            )
+        most = min(len(request.prompt) + request.max_tokens, self.max_positions)
+        if self.cache.blocks_for(most) > self.cache.n_pages:
+            raise ValueError(
+                f"request {request.request_id!r} can reach {most} tokens, the cache holds "
+                f"{self.cache.n_pages * self.cache.page_size}"
+            )
+        if any(r.request_id == request.request_id for r in list(self.waiting) + self.running):
+            raise ValueError(f"request id {request.request_id!r} is in use")
+        request.order = self._order
+        self._order += 1
+        self.waiting.append(request)
+        return request
+
+    def abort(self, request_id):
+        """Take a request out, wherever it is (``remove`` of mlx_lm/generate.py:1777-1802)."""
+        for r in list(self.waiting):
+            if r.request_id == request_id:
+                self.waiting.remove(r)
+                return r
+        for r in self.running:
+            if r.request_id == request_id:
+                self._drop(r)
+                return r
+        raise KeyError(f"request {request_id!r} is not known")
+
+    @property
+    def has_work(self):
+        return bool(self.waiting or self.running)
+
+    def _drop(self, r):
+        self.running.remove(r)
+        if self.engine.has_request(r.request_id):
+            self.engine.end_request(r.request_id)
+
+    def _preempt(self, r):
+        self._drop(r)
+        r.num_computed = 0
+        r.preemptions += 1
+        self.stats.preemptions += 1
+        self.waiting.appendleft(r)
+
+    # -- decisions ---------------------------------------------------------------
+
+    def _pages_for(self, r, n_new):
+        if self.engine.has_request(r.request_id):
+            return self.cache.pages_needed(r.request_id, n_new)
+        return self.cache.blocks_for(n_new)
+
+    def plan_step(self):
+        """Decide what the next step runs; may pre-empt.  Returns ``[PlannedEntry]``."""
+        free = self.cache.free_pages()
+        budget = self.max_num_batched_tokens
+        plan = []
+
+        # 1. one token for every decoding request; pre-empt from the newest if pages run short
+        decoding = [r for r in self.running if r.decoding]
+        decoding.sort(key=lambda r: r.order)
+        while decoding:
+            need = sum(self._pages_for(r, 1) for r in decoding)
+            if need <= free and len(decoding) <= budget:
+                break
+            victim = max(self.running, key=lambda r: r.order)
+            if victim in decoding:
+                decoding.remove(victim)
+            self._preempt(victim)
+            free = self.cache.free_pages()
+        for r in decoding:
+            free -= self._pages_for(r, 1)
+            budget -= 1
+            plan.append(PlannedEntry(r, 1, True))
+
+        # 2. requests still reading their prompt, in order of admission
+        for r in sorted((r for r in self.running if not r.decoding), key=lambda r: r.order):
+            if budget <= 0:
+                break
+            left = r.num_tokens - r.num_computed
+            n = min(left, budget, self.prefill_step_size)
+            while n > 0 and self._pages_for(r, n) > free:
+                n = self._fit(r, n, free)
+            if n <= 0:
+                continue
+            free -= self._pages_for(r, n)
+            budget -= n
+            plan.append(PlannedEntry(r, n, n == left))
+
+        # 3. admit waiting requests while their whole prompt fits
+        while self.waiting and len(self.running) < self.max_num_seqs and budget > 0:
+            r = self.waiting[0]
+            whole = self.cache.blocks_for(min(r.num_tokens + 1, self.max_positions))
+            if whole > free:
+                break
+            self.waiting.popleft()
+            self.engine.add_request(r.request_id)
+            self.running.append(r)
+            n = min(r.num_tokens, budget, self.prefill_step_size)
+            free -= whole
+            budget -= n
+            plan.append(PlannedEntry(r, n, n == r.num_tokens))
+        return plan
+
+    def _fit(self, r, n, free):
+        """The longest portion of at most ``n`` tokens whose pages are free."""
+        ps = self.cache.page_size
+        if self.engine.has_request(r.request_id):
+            rc = self.cache.requests[r.request_id]
+            room = self.cache.blocks_for(rc.reserved) * ps - rc.length
+        else:
+            room = 0
+        return min(n - 1, room + free * ps)
+
+    # -- running a plan ------------------------------------------------------------
+
+    def step(self):
+        """Plan, run and sample one step; returns the ``StepOutput`` of every sampled token."""
+        plan = self.plan_step()
+        if not plan:
+            if self.has_work and not self.running:
+                raise RuntimeError("requests are waiting but none can be admitted")
+            return []
+        entries = []
+        for p in plan:
+            r = p.request
+            toks = r.tokens[r.num_computed : r.num_computed + p.n_tokens]
+            entries.append(StepEntry(r.request_id, toks, [p.n_tokens - 1] if p.samples else []))
+        logits = self.engine.step(entries)
+        for p in plan:
+            r = p.request
+            if not r.generated:
+                self.stats.prompt_tokens += p.n_tokens
+            r.num_computed += p.n_tokens
+        self.stats.steps += 1
+        self.stats.pages_high_water = max(
+            self.stats.pages_high_water, max((g.pool.high_water for g in self.cache.groups), default=0)
+        )
+        sampled = [p.request for p in plan if p.samples]
+        if not sampled:
+            return []
+        results = self.sample(logits, sampled)
+        outputs = []
+        for r, (token, logprob, logprobs) in zip(sampled, results):
+            r.generated.append(int(token))
+            self.stats.generation_tokens += 1
+            # "length" at max_tokens or when the model's positions are used up;
+            # "stop" is checked second and wins (mlx_lm/generate.py:1501-1514)
+            reason = None
+            if len(r.generated) >= r.max_tokens or r.num_tokens >= self.max_positions:
+                reason = "length"
+            if stops(r.generated, r.stop_sequences):
+                reason = "stop"
+            r.finish_reason = reason
+            outputs.append(StepOutput(r.request_id, int(token), float(logprob), reason, logprobs))
+            if reason is not None:
+                self._drop(r)
+        return outputs
