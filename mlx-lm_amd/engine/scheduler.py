@@ -9,7 +9,8 @@ padded model calls per iteration.  Here one ``step`` holds both kinds of work:
    reading their prompt, in order of admission, as portions of at most
    ``prefill_step_size`` tokens;
 3. waiting requests are admitted, first come first served, while fewer than
-   ``max_num_seqs`` run and the pages for their whole prompt are free.
+   ``max_num_seqs`` run and the pages for their whole prompt are free; those
+   pages are taken at admission, so reading a prompt never stalls half-way.
 
 When pages run out for a decoding request, the request admitted last is
 pre-empted: its pages are given back and it returns to the *front* of the
@@ -226,6 +227,9 @@ class Scheduler:
                 break
             self.waiting.popleft()
             self.engine.add_request(r.request_id)
+            # the whole prompt's pages are taken now, so a request that was
+            # admitted can always finish reading its prompt
+            self.cache.reserve(r.request_id, min(r.num_tokens + 1, self.max_positions))
             self.running.append(r)
             n = min(r.num_tokens, budget, self.prefill_step_size)
             free -= whole

@@ -1,0 +1,159 @@
+"""The cache manager's bookkeeping (no GPU): no page lost, held twice or freed twice."""
+
+import random
+
+import pytest
+
+from mlx_lm_amd.cache import CacheManager, OutOfPages, OutOfSlots, PagePool
+from mlx_lm_amd.config import CacheNeed, StateNeed
+
+
+def test_page_pool_is_lifo_and_strict():
+    pool = PagePool(4)
+    assert pool.take(2) == [0, 1] and pool.n_free == 2
+    pool.give_back([0])
+    assert pool.take(1) == [0]  # the page just given back comes out first
+    assert pool.take(3) is None and pool.n_free == 2  # nothing taken when short
+    with pytest.raises(ValueError, match="not held"):
+        pool.give_back([3])
+    pool.give_back([1])
+    with pytest.raises(ValueError, match="not held"):
+        pool.give_back([1])
+    with pytest.raises(ValueError, match="not of this pool"):
+        pool.give_back([9])
+    pool.check()
+    assert pool.high_water == 2
+
+
+def _manager(n_pages=8, window=0, max_requests=4):
+    needs = [CacheNeed(2, 16, 0), CacheNeed(2, 16, 0), CacheNeed(2, 16, window), None, StateNeed((3,))]
+    return CacheManager(needs, 16, n_pages, max_requests)
+
+
+def test_groups_follow_needs():
+    cm = _manager(window=40)
+    assert len(cm.groups) == 2 and cm.groups[0].slots == [0, 1] and cm.groups[1].slots == [2]
+    assert cm.slot_group[2] == (1, 0) and 4 in cm.state_needs and 3 not in cm.slot_group
+    assert len(_manager(window=0).groups) == 1
+
+
+def test_reserve_commit_release():
+    cm = _manager()
+    a = cm.add("a")
+    cm.reserve("a", 17)
+    assert a.blocks[0] == [0, 1] and a.length == 0 and cm.free_pages() == 6
+    cm.commit("a", 17)
+    cm.reserve("a", 15)  # fits the second page
+    assert cm.free_pages() == 6 and cm.pages_needed("a", 16) == 1
+    cm.commit("a", 15)
+    with pytest.raises(ValueError, match="never reserved"):
+        cm.commit("a", 1)
+    b = cm.add("b")
+    with pytest.raises(OutOfPages):
+        cm.reserve("b", 16 * 7)
+    assert b.blocks[0] == [] and cm.free_pages() == 6  # all or nothing
+    cm.release("a")
+    assert cm.free_pages() == 8
+    cm.reserve("b", 5)
+    assert b.blocks[0] == [1]  # used again at once
+    cm.check()
+    with pytest.raises(ValueError, match="already live"):
+        cm.add("b")
+
+
+def test_state_slots():
+    cm = _manager(max_requests=2)
+    s0, s1 = cm.add("a").state_slot, cm.add("b").state_slot
+    assert {s0, s1} == {0, 1}
+    with pytest.raises(OutOfSlots):
+        cm.add("c")
+    cm.release("a")
+    assert cm.add("c").state_slot == s0
+    cm.check()
+
+
+def test_window_gives_pages_back_as_it_passes():
+    cm = _manager(n_pages=8, window=20)
+    rc = cm.add("a")
+    cm.reserve("a", 40)
+    cm.commit("a", 40)
+    # the next query is at 40 and sees keys 21..40: block 0 (0..15) is out of reach
+    assert rc.blocks[1] == [-1, 1, 2] and rc.blocks[0] == [0, 1, 2]
+    assert cm.groups[1].pool.n_free == 6
+    for _ in range(30):
+        cm.reserve("a", 1)
+        cm.commit("a", 1)
+    assert rc.length == 70 and [p >= 0 for p in rc.blocks[1]] == [False, False, False, True, True]
+    cm.check()
+    with pytest.raises(ValueError, match="window"):
+        cm.truncate("a", 30)
+    cm.truncate("a", 68)  # the query at 68 sees keys from 49 on: block 3 is still there
+    assert len(rc.blocks[0]) == 5 and rc.length == 68
+    with pytest.raises(ValueError, match="window"):
+        cm.truncate("a", 66)  # would need key 47 again, whose page is gone
+    cm.release("a")
+    assert cm.free_pages() == 8
+
+
+def test_truncate_gives_whole_pages_back():
+    cm = _manager()
+    rc = cm.add("a")
+    cm.reserve("a", 50)
+    cm.commit("a", 50)
+    cm.truncate("a", 33)
+    assert rc.length == 33 and len(rc.blocks[0]) == 3 and cm.free_pages() == 5
+    cm.truncate("a", 32)
+    assert len(rc.blocks[0]) == 2
+    cm.reserve("a", 20)
+    assert len(rc.blocks[0]) == 4
+    cm.check()
+
+
+@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("window", [0, 24])
+def test_random_orders_keep_every_page_accounted(seed, window):
+    rng = random.Random(seed)
+    cm = _manager(n_pages=12, window=window, max_requests=5)
+    live, n = {}, 0
+    for _ in range(600):
+        op = rng.random()
+        if op < 0.2 and len(live) < 5:
+            rid = f"r{n}"
+            n += 1
+            cm.add(rid)
+            live[rid] = 0
+        elif op < 0.75 and live:
+            rid = rng.choice(list(live))
+            k = rng.choice([1, 1, 1, 2, 7, 16, 33])
+            try:
+                cm.reserve(rid, k)
+            except OutOfPages:
+                before = [g.pool.n_free for g in cm.groups]
+                cm.check()
+                assert before == [g.pool.n_free for g in cm.groups]
+                continue
+            if rng.random() < 0.9:
+                cm.commit(rid, k)
+                live[rid] += k
+        elif op < 0.85 and live:
+            rid = rng.choice(list(live))
+            if window == 0:
+                new = rng.randint(0, live[rid])
+                cm.truncate(rid, new)
+                live[rid] = new
+        elif live:
+            rid = rng.choice(list(live))
+            cm.release(rid)
+            del live[rid]
+        cm.check()
+        for rid, length in live.items():
+            rc = cm.requests[rid]
+            assert rc.length == length
+            # every position a later query can see has a page
+            lo = 0 if window == 0 else max(0, length - window + 1)
+            for gi, g in enumerate(cm.groups):
+                first = 0 if g.need.window == 0 else lo // 16
+                assert all(p >= 0 for p in rc.blocks[gi][first : cm.blocks_for(length)])
+    cm.release_all()
+    assert all(g.pool.n_free == 12 for g in cm.groups)
+    cm.check()

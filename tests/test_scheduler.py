@@ -1,0 +1,190 @@
+"""The scheduler's decisions with a stand-in engine (no GPU)."""
+
+import random
+from types import SimpleNamespace
+
+import pytest
+
+from mlx_lm_amd.cache import CacheManager
+from mlx_lm_amd.config import CacheNeed
+from mlx_lm_amd.engine.scheduler import Request, Scheduler, stops
+
+
+class FakeEngine:
+    """Keeps the real cache bookkeeping, runs no model; records what each step held."""
+
+    def __init__(self, n_pages, max_positions=256, max_requests=8, page_size=16):
+        self.cache = CacheManager([CacheNeed(2, 16, 0)], page_size, n_pages, max_requests)
+        self.decoder = SimpleNamespace(max_positions=max_positions)
+        self.log = []
+
+    def add_request(self, rid):
+        return self.cache.add(rid)
+
+    def end_request(self, rid):
+        self.cache.release(rid)
+
+    def has_request(self, rid):
+        return rid in self.cache.requests
+
+    def step(self, entries):
+        for e in entries:
+            self.cache.reserve(e.request_id, len(e.tokens))
+        rows = []
+        for e in entries:
+            start = self.cache.requests[e.request_id].length
+            self.cache.commit(e.request_id, len(e.tokens))
+            rows += [(e.request_id, start + w, tuple(e.tokens)) for w in e.want]
+        self.log.append([(e.request_id, len(e.tokens), list(e.want)) for e in entries])
+        self.cache.check()
+        return rows
+
+
+def token_for(rid, index):
+    return (hash((rid, index)) % 997) + 1
+
+
+def fake_sample(rows, requests):
+    assert len(rows) == len(requests)
+    out = []
+    for (rid, pos, _), r in zip(rows, requests):
+        assert rid == r.request_id and pos == r.num_tokens - 1  # the row of the newest token
+        out.append((token_for(rid, len(r.generated)), -1.0, None))
+    return out
+
+
+def run_all(sched, limit=10000):
+    done = {}
+    for _ in range(limit):
+        if not sched.has_work:
+            return done
+        for o in sched.step():
+            done.setdefault(o.request_id, []).append(o)
+    raise AssertionError("the scheduler did not finish")
+
+
+def test_portions_under_a_token_budget_beside_decoding():
+    eng = FakeEngine(n_pages=64)
+    s = Scheduler(eng, fake_sample, max_num_seqs=4, max_num_batched_tokens=40, prefill_step_size=32)
+    s.add(Request("a", list(range(1, 71)), 3))
+    s.step()
+    assert eng.log[-1] == [("a", 32, [])]
+    s.add(Request("b", list(range(1, 11)), 5))
+    s.step()  # a goes on with 32 more, b gets the 8 left of the budget
+    assert eng.log[-1] == [("a", 32, []), ("b", 8, [])]
+    outs = s.step()  # a's last 6 (sampled), b's last 2 (sampled)
+    assert eng.log[-1] == [("a", 6, [5]), ("b", 2, [1])]
+    assert [o.request_id for o in outs] == ["a", "b"] and outs[0].token == token_for("a", 0)
+    s.add(Request("c", list(range(1, 60)), 2))
+    s.step()  # decoding tokens first, then c's first portion in the same step
+    assert eng.log[-1] == [("a", 1, [0]), ("b", 1, [0]), ("c", 32, [])]
+    done = run_all(s)
+    assert [o.finish_reason for o in done["c"]] == [None, "length"]
+    assert eng.cache.free_pages() == 64 and not eng.cache.requests
+
+
+def test_max_tokens_stop_and_positions():
+    eng = FakeEngine(n_pages=64, max_positions=40)
+    s = Scheduler(eng, fake_sample)
+    for rid, n, mt in (("a", 5, 2), ("b", 7, 3), ("c", 3, 4), ("d", 9, 5)):
+        s.add(Request(rid, list(range(1, n + 1)), mt))
+    s.add(Request("stop", [1, 2, 3], 50, stop_sequences=[[token_for("stop", 1), token_for("stop", 2)]]))
+    s.add(Request("long", list(range(1, 31)), 100))
+    done = run_all(s)
+    assert [len(done[r]) for r in "abcd"] == [2, 3, 4, 5]  # per-request max_tokens
+    assert all(done[r][-1].finish_reason == "length" for r in "abcd")
+    assert [o.finish_reason for o in done["stop"]] == [None, None, "stop"]  # the stopping token is reported
+    assert len(done["long"]) == 40 - 30 and done["long"][-1].finish_reason == "length"
+    # tokens are those of a request run alone, whatever shared its steps
+    assert [o.token for o in done["d"]] == [token_for("d", i) for i in range(5)]
+    assert stops([4, 5, 6], [[5, 6]]) and not stops([5, 6, 4], [[5, 6]]) and not stops([6], [[5, 6]])
+
+
+def test_admission_waits_for_pages_and_keeps_order():
+    eng = FakeEngine(n_pages=6)
+    s = Scheduler(eng, fake_sample, max_num_seqs=8)
+    s.add(Request("a", list(range(1, 50)), 4))  # 4 pages
+    s.add(Request("b", list(range(1, 40)), 4))  # 3 pages: has to wait
+    s.add(Request("c", [1, 2], 4))  # would fit, but b is first
+    first = s.step()
+    assert [r.request_id for r in s.running] == ["a"] and [r.request_id for r in s.waiting] == ["b", "c"]
+    done = run_all(s)
+    done["a"] = first + done["a"]
+    assert sorted(done) == ["a", "b", "c"] and all(len(v) == 4 for v in done.values())
+    first_step = {rid: next(i for i, st in enumerate(eng.log) if any(e[0] == rid for e in st)) for rid in "abc"}
+    assert first_step["a"] < first_step["b"] <= first_step["c"]
+
+
+def test_preemption_when_pages_run_out():
+    eng = FakeEngine(n_pages=5, max_positions=200)
+    s = Scheduler(eng, fake_sample, max_num_seqs=4)
+    s.add(Request("old", list(range(1, 31)), 40))  # 2 pages, grows to 5
+    s.add(Request("new", list(range(1, 17)), 40))  # 2 pages with its first token
+    done = run_all(s)
+    assert s.stats.preemptions >= 1
+    pre = [r for r in ("old", "new")]
+    assert len(done["old"]) == 40 and len(done["new"]) == 40
+    # the pre-empted request went on where it was: same tokens as alone
+    for rid in pre:
+        assert [o.token for o in done[rid]] == [token_for(rid, i) for i in range(40)]
+    # the newer request was the victim and re-read prompt + generated as one prompt
+    reread = [st for st in eng.log if any(e[0] == "new" and e[1] > 16 for e in st)]
+    assert reread
+    assert eng.cache.free_pages() == 5
+
+
+def test_what_cannot_fit_is_refused_at_once():
+    eng = FakeEngine(n_pages=4, max_positions=100)
+    s = Scheduler(eng, fake_sample)
+    with pytest.raises(ValueError, match="cache holds"):
+        s.add(Request("big", list(range(1, 60)), 30))
+    with pytest.raises(ValueError, match="positions"):
+        s.add(Request("long", list(range(1, 120)), 1))
+    with pytest.raises(ValueError, match="at least one token"):
+        s.add(Request("empty", [], 1))
+    s.add(Request("ok", [1, 2, 3], 2))
+    with pytest.raises(ValueError, match="in use"):
+        s.add(Request("ok", [1], 1))
+
+
+def test_abort_frees_everything():
+    eng = FakeEngine(n_pages=16)
+    s = Scheduler(eng, fake_sample, max_num_batched_tokens=16, prefill_step_size=16)
+    s.add(Request("a", list(range(1, 60)), 5))
+    s.add(Request("b", list(range(1, 20)), 5))
+    s.step()
+    s.abort("a")  # mid-prompt
+    s.abort("b")  # still waiting or just admitted
+    assert not s.has_work and eng.cache.free_pages() == 16
+    with pytest.raises(KeyError):
+        s.abort("a")
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_random_load_every_request_finishes_with_its_own_tokens(seed):
+    rng = random.Random(seed)
+    P = 128
+    eng = FakeEngine(n_pages=rng.choice([8, 12, 30]), max_positions=P, max_requests=6)
+    s = Scheduler(eng, fake_sample, max_num_seqs=rng.choice([2, 4, 6]),
+                  max_num_batched_tokens=rng.choice([8, 33, 256]), prefill_step_size=rng.choice([5, 64]))
+    want, done, added = {}, {}, 0
+    for _ in range(3000):
+        if added < 25 and rng.random() < 0.3:
+            n, mt = rng.randint(1, 100), rng.randint(1, 40)
+            rid = f"r{added}"
+            s.add(Request(rid, [rng.randint(1, 900) for _ in range(n)], mt))
+            want[rid] = min(mt, max(1, P - n))
+            added += 1
+        if s.has_work:
+            for o in s.step():
+                done.setdefault(o.request_id, []).append(o)
+        elif added == 25:
+            break
+        assert len(s.running) <= s.max_num_seqs
+        assert all(sum(e[1] for e in st) <= s.max_num_batched_tokens for st in eng.log[-1:])
+    assert sorted(done) == sorted(want)
+    for rid, outs in done.items():
+        assert len(outs) == want[rid], rid
+        assert [o.token for o in outs] == [token_for(rid, i) for i in range(len(outs))]
+        assert outs[-1].finish_reason == "length" and all(o.finish_reason is None for o in outs[:-1])
+    assert eng.cache.free_pages() == eng.cache.n_pages
