@@ -90,7 +90,7 @@ class StepContext:
     device arrays over the tokens; ``slot_ids`` gives each request's state
     slot; ``wanted_rows`` the flat rows whose logits are asked for.  The host
     lists ``q_starts``/``q_lens``/``context_lens`` (tokens before this step)
-    say where each request's run lies.
+    say where each request's run lies, ``state_slots`` is ``slot_ids`` on the host.
     """
 
     def __init__(self, engine):
@@ -102,7 +102,7 @@ class StepContext:
         self.token_ids = self.positions = self.token_req = None
         self.slot_ids = self.wanted_rows = None
         self.block_tables = []
-        self.q_starts, self.q_lens, self.context_lens = [], [], []
+        self.q_starts, self.q_lens, self.context_lens, self.state_slots = [], [], [], []
         self.attention_plan = AttentionPlan()
         self._views = {}
 

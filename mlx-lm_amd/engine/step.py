@@ -176,6 +176,7 @@ class Engine:
             token_req.extend([r] * n)
             wanted.extend(q_start + int(w) for w in e.want)
             slot_ids.append(rc.state_slot)
+            ctx.state_slots.append(rc.state_slot)
             for s in range(0, n, TILE_Q):
                 all_tiles.extend((q_start + s, min(TILE_Q, n - s)))
             if n <= ROW_KERNEL_MAX_Q:

@@ -1,0 +1,404 @@
+"""Each part alone against the plain implementation, and toy parts defined here
+that are registered, built and stepped without touching the framework's files."""
+
+import json
+import math
+import os
+from dataclasses import dataclass
+
+import pytest
+import torch
+
+import helpers
+import plain_gpt2 as plain
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+TOL = {"float32": 2e-5, "bfloat16": 2.5e-2}
+
+
+def _close(got, want, dtype, what=""):
+    scale = max(want.abs().max().item(), 1e-6)
+    err = (got.double().cpu() - want).abs().max().item()
+    assert err <= TOL[dtype] * scale, f"{what}: max error {err:.3e} against scale {scale:.3e}"
+
+
+@pytest.fixture(scope="module")
+def folder_b(tmp_path_factory):
+    d = str(tmp_path_factory.mktemp("partsB"))
+    config, weights = helpers.make_folder(d, "B", 8.0)
+    return d, config, weights
+
+
+def _engine(folder, dtype, n_pages=32):
+    from mlx_lm_amd.engine import Engine
+    from mlx_lm_amd.utils import load_model
+
+    model, _ = load_model(folder, dtype=dtype)
+    return Engine(model, dtype=dtype, page_size=16, n_pages=n_pages, max_requests=4)
+
+
+def _context(engine, entries):
+    """Pages and a step context for ``entries`` without running the model."""
+    for e in entries:
+        if not engine.has_request(e.request_id):
+            engine.add_request(e.request_id)
+        engine.cache.reserve(e.request_id, len(e.tokens))
+    ctx = engine._build_context(entries)
+    engine.scratch.reset()
+    return ctx
+
+
+def _commit(engine, entries):
+    for e in entries:
+        engine.cache.commit(e.request_id, len(e.tokens))
+
+
+def _w(weights, dtype):
+    w = helpers.round_matrices_to_bf16(weights) if dtype == "bfloat16" else weights
+    return {k: v.double() for k, v in w.items()}
+
+
+def _act(x, dtype):
+    return x.to(torch.bfloat16 if dtype == "bfloat16" else torch.float32).to(DEV)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_parts_alone(folder_b, dtype):
+    from mlx_lm_amd.engine import StepEntry
+
+    folder, config, weights = folder_b
+    w = _w(weights, dtype)
+    eng = _engine(folder, dtype)
+    dec = eng.decoder
+    D, H, V = config["n_embd"], config["n_head"], config["vocab_size"]
+    eps = config["layer_norm_epsilon"]
+    g = torch.Generator().manual_seed(1)
+
+    # embedding with learned positions, the second request starting at position 30
+    first = [StepEntry("b", helpers.random_tokens(30, V, 2), [])]
+    ctx = _context(eng, first)
+    _commit(eng, first)
+    toks_a, toks_b = helpers.random_tokens(21, V, 3), helpers.random_tokens(5, V, 4)
+    entries = [StepEntry("a", toks_a, [0, 20]), StepEntry("b", toks_b, [4])]
+    ctx = _context(eng, entries)
+    h = ctx.scratch((26, D), "float32")
+    dec.embedding.forward(ctx, h, dec.embedding_positions.embedding_term(ctx))
+    want = torch.cat([
+        plain.add_learned_positions(plain.embed_tokens(w["model.wte.weight"], torch.tensor(toks_a)), w["model.wpe.weight"], 0),
+        plain.add_learned_positions(plain.embed_tokens(w["model.wte.weight"], torch.tensor(toks_b)), w["model.wpe.weight"], 30),
+    ])
+    _close(h, want, "float32", "embedding")  # exact sums of stored values
+
+    # norm, on all rows and on the wanted rows only
+    x = (torch.randn(26, D, generator=g) * 2 + 0.5)
+    norm = dec.layers[1].ffn_norm
+    y = norm.forward(ctx, x.to(DEV))
+    want = plain.layer_norm(x.double(), w["model.h.1.ln_2.weight"], w["model.h.1.ln_2.bias"], eps)
+    _close(y, want, dtype, "layernorm")
+    y = norm.forward(ctx, x.to(DEV), rows=ctx.wanted_rows, n_rows=ctx.n_wanted)
+    _close(y, want[[0, 20, 25]], dtype, "layernorm on wanted rows")
+
+    # feed-forward adds into the residual stream
+    xin = _act(torch.randn(26, D, generator=g), dtype)
+    res0 = torch.randn(26, D, generator=g)
+    res = res0.clone().to(DEV)
+    dec.layers[2].ffn.forward(ctx, xin, res)
+    want = res0.double() + plain.mlp(xin.double().cpu(), w, "model.h.2.mlp.")
+    _close(res, want, dtype, "feed-forward")
+
+    # head
+    xin = _act(torch.randn(3, D, generator=g), dtype)
+    logits = torch.empty(3, V, dtype=torch.float32, device=DEV)
+    dec.head.forward(ctx, xin, logits)
+    _close(logits, plain.tied_head(xin.double().cpu(), w["model.wte.weight"]), dtype, "head")
+    eng.cache.release_all()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_part_and_block_in_portions(folder_b, dtype):
+    from mlx_lm_amd.engine import StepEntry
+
+    folder, config, weights = folder_b
+    w = _w(weights, dtype)
+    eng = _engine(folder, dtype)
+    dec = eng.decoder
+    D, H = config["n_embd"], config["n_head"]
+    g = torch.Generator().manual_seed(2)
+    n = 75
+    x = _act(torch.randn(n, D, generator=g), dtype)
+    res0 = torch.randn(n, D, generator=g)
+    want = res0.double() + plain.self_attention(x.double().cpu(), w, "model.h.1.attn.", H)
+    attn = dec.layers[1].mixer
+    got, i = [], 0
+    for cut in (37, 2, 1, 20, 1, 14):  # tiles, short portions and single rows
+        e = [StepEntry("r", [0] * cut, [])]
+        ctx = _context(eng, e)
+        res = res0[i : i + cut].clone().to(DEV)
+        attn.forward(ctx, x[i : i + cut], res, ctx.cache_view(1), True)
+        got.append(res.clone())
+        _commit(eng, e)
+        i += cut
+    _close(torch.cat(got), want, dtype, "attention part in portions")
+    eng.cache.release_all()
+
+    # a whole block
+    h0 = torch.randn(n, D, generator=g)
+    e = [StepEntry("s", [0] * n, [])]
+    ctx = _context(eng, e)
+    h = h0.clone().to(DEV)
+    dec.layers[0].forward(ctx, h, ctx.cache_view(0), True)
+    _close(h, plain.block(h0.double(), w, 0, H, config["layer_norm_epsilon"]), dtype, "block")
+    eng.cache.release_all()
+    eng.cache.check()
+
+
+# ---------------------------------------------------------------------------
+# toy parts: a mixer with state of its own, a rotating position encoding, grouped
+# key heads, a window, a layer that runs twice and a layer that reads another's cache
+
+
+def _register_toys():
+    from mlx_lm_amd.config import BaseModelArgs, LayerSpec, ModelPlan, PartSpec, RunEntry, StateNeed, register_model
+    from mlx_lm_amd.parts import (DecoderModel, Mixer, PositionEncoding, TensorSpec, register_mixer,
+                                  register_position_encoding)
+
+    class DecayMixer(Mixer):
+        """``s_t = decay * s_{t-1} + x_t``; adds ``s_t`` to the residual.  Its state
+        ``s`` lives in the request's state slot between steps."""
+
+        def __init__(self, width, prefix=""):
+            super().__init__(prefix)
+            self.width = width
+
+        def cache_need(self):
+            return StateNeed((self.width,), "float32")
+
+        def tensors(self):
+            return {self._name("decay"): TensorSpec((self.width,), "vector")}
+
+        def load(self, tensors):
+            self.decay = tensors[self._name("decay")]
+
+        def forward(self, ctx, x, residual, cache, writes_cache=True):
+            for start, n, slot in zip(ctx.q_starts, ctx.q_lens, ctx.state_slots):
+                s = cache.state[slot]
+                for t in range(start, start + n):
+                    s = self.decay * s + x[t].float()
+                    residual[t] += s
+                cache.state[slot] = s
+
+    class PairRotation(PositionEncoding):
+        """Rotates pairs of head columns by ``position * theta^(-2i/d)`` (written with torch ops)."""
+
+        def __init__(self, head_dim, theta, prefix=""):
+            super().__init__(prefix)
+            self.head_dim, self.theta = head_dim, theta
+
+        def rotate(self, ctx, q, k):
+            half = self.head_dim // 2
+            freq = self.theta ** (-torch.arange(half, device=q.device, dtype=torch.float32) / half)
+            ang = ctx.positions.float()[:, None] * freq[None]
+            cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+            for t in (q, k):
+                v = t.float().reshape(t.shape[0], -1, self.head_dim)
+                a, b = v[..., :half], v[..., half:]
+                out = torch.cat([a * cos - b * sin, a * sin + b * cos], -1)
+                t.copy_(out.reshape(t.shape).to(t.dtype))
+
+    register_mixer("toy_decay", DecayMixer)
+    register_position_encoding("toy_pair_rotation", PairRotation)
+
+    @dataclass
+    class ToyArgs(BaseModelArgs):
+        model_type: str
+        width: int
+        vocab: int
+        max_len: int
+        heads: int
+        kv_heads: int
+        head_dim: int
+        window: int
+        inner: int
+        eps: float
+        theta: float
+
+    class ToyModel:
+        def __init__(self, args):
+            self.args, self.model_type = args, args.model_type
+            self.decoder = DecoderModel(self.plan(args))
+
+        @property
+        def layers(self):
+            return self.decoder.layers
+
+        @staticmethod
+        def plan(a):
+            def norm(p):
+                return PartSpec("layernorm", {"width": a.width, "eps": a.eps}, p)
+
+            def attention(p, window):
+                return PartSpec("attention", {
+                    "width": a.width, "n_heads": a.heads, "n_kv_heads": a.kv_heads, "head_dim": a.head_dim,
+                    "window": window, "bias": False, "qkv_name": "qkv", "out_name": "o",
+                    "position": PartSpec("toy_pair_rotation", {"head_dim": a.head_dim, "theta": a.theta})}, p)
+
+            def ffn(p):
+                return PartSpec("gelu_mlp", {"width": a.width, "inner": a.inner}, p)
+
+            mixers = [attention("l0.mix.", 0), attention("l1.mix.", a.window),
+                      PartSpec("toy_decay", {"width": a.width}, "l2.mix.")]
+            layers = [LayerSpec("pre_norm", norm(f"l{i}.n1."), m, norm(f"l{i}.n2."), ffn(f"l{i}.ff."))
+                      for i, m in enumerate(mixers)]
+            # layer 0 runs twice (two cache slots); the last run of layer 1 reads the
+            # keys and values that its first run wrote
+            schedule = [RunEntry(0, 0), RunEntry(1, 1), RunEntry(2, 2), RunEntry(0, 3),
+                        RunEntry(1, 1, writes_cache=False)]
+            return ModelPlan(
+                width=a.width, vocab_size=a.vocab, max_positions=a.max_len,
+                embedding=PartSpec("token", {"vocab_size": a.vocab, "width": a.width}, "emb."),
+                embedding_positions=None, layers=layers, schedule=schedule,
+                final_norm=norm("nf."), head=PartSpec("linear", {"vocab_size": a.vocab, "width": a.width,
+                                                                  "weight_name": "head.weight"}))
+
+    register_model("toy_hybrid", ToyModel, ToyArgs)
+    return ToyModel, ToyArgs
+
+
+TOY = dict(model_type="toy_hybrid", width=80, vocab=211, max_len=160, heads=6, kv_heads=2, head_dim=32,
+           window=24, inner=120, eps=1e-4, theta=100.0)
+
+
+def _toy_folder(path):
+    from safetensors.torch import save_file
+
+    ToyModel, ToyArgs = _register_toys()
+    model = ToyModel(ToyArgs.from_dict(TOY))
+    g = torch.Generator().manual_seed(7)
+    tensors = {}
+    for name, spec in model.decoder.expected_tensors().items():
+        if name.endswith("decay"):
+            t = 0.5 + 0.4 * torch.rand(spec.shape, generator=g)
+        elif spec.role == "vector":
+            t = 1.0 + 0.1 * torch.randn(spec.shape, generator=g) if "weight" in name else 0.05 * torch.randn(spec.shape, generator=g)
+        else:
+            t = torch.randn(spec.shape, generator=g) * (0.25 if "qkv" in name else 0.05)
+        tensors[name] = t
+    os.makedirs(path, exist_ok=True)
+    json.dump(TOY, open(os.path.join(path, "config.json"), "w"))
+    save_file(tensors, os.path.join(path, "model.safetensors"))
+    return tensors
+
+
+def _toy_plain(t, ids):
+    """The toy model on one whole sequence, from the plain parts."""
+    a = TOY
+    w = {k: v.double() for k, v in t.items()}
+    L = len(ids)
+    H, Hkv, hd = a["heads"], a["kv_heads"], a["head_dim"]
+    pos = torch.arange(L, dtype=torch.float64)
+    half = hd // 2
+    freq = a["theta"] ** (-torch.arange(half, dtype=torch.float64) / half)
+    ang = pos[:, None] * freq[None]
+
+    def rotate(v):  # [heads, L, hd]
+        x, y = v[..., :half], v[..., half:]
+        return torch.cat([x * ang.cos() - y * ang.sin(), x * ang.sin() + y * ang.cos()], -1)
+
+    def ln(x, p):
+        return plain.layer_norm(x, w[p + "weight"], w[p + "bias"], a["eps"])
+
+    def ffn(x, p):
+        return plain.mlp(x, w, p)
+
+    kv_store = {}
+
+    def attention(x, p, window, slot, writes):
+        qkv = plain.linear(x, w[p + "qkv.weight"])
+        q = qkv[:, : H * hd].reshape(L, H, hd).permute(1, 0, 2)
+        if writes:
+            k = qkv[:, H * hd : (H + Hkv) * hd].reshape(L, Hkv, hd).permute(1, 0, 2)
+            v = qkv[:, (H + Hkv) * hd :].reshape(L, Hkv, hd).permute(1, 0, 2)
+            kv_store[slot] = (rotate(k), v)
+        k, v = kv_store[slot]
+        o = plain.attention(rotate(q), k, v, hd**-0.5, plain.causal_mask(L, 0, window or None))
+        return plain.linear(plain.merge_heads(o), w[p + "o.weight"])
+
+    def decay(x, p):
+        s, out = torch.zeros(a["width"], dtype=torch.float64), []
+        for i in range(L):
+            s = w[p + "decay"] * s + x[i]
+            out.append(s)
+        return torch.stack(out)
+
+    h = plain.embed_tokens(w["emb.weight"], torch.tensor(ids))
+    runs = [(0, 0, True), (1, 1, True), (2, 2, True), (0, 3, True), (1, 1, False)]
+    for layer, slot, writes in runs:
+        p = f"l{layer}."
+        x = ln(h, p + "n1.")
+        if layer == 2:
+            h = h + decay(x, p + "mix.")
+        else:
+            h = h + attention(x, p + "mix.", a["window"] if layer == 1 else 0, slot, writes)
+        h = h + ffn(ln(h, p + "n2."), p + "ff.")
+    return plain.tied_head(ln(h, "nf."), w["head.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype):
+    from mlx_lm_amd.engine import Engine, StepEntry
+    from mlx_lm_amd.utils import load_model
+
+    tensors = _toy_folder(str(tmp_path))
+    model, config = load_model(str(tmp_path), dtype=dtype)  # found by config.json's model_type
+    assert model.model_type == "toy_hybrid" and len(model.layers) == 3
+    cm_needs = model.decoder.cache_needs()
+    assert len(cm_needs) == 4 and cm_needs[2].shape == (80,) and cm_needs[1].window == 24
+    eng = Engine(model, dtype=dtype, page_size=16, n_pages=14, max_requests=3)
+    assert len(eng.cache.groups) == 2  # all keys, and a window of them: pages of their own
+
+    ref = helpers.round_matrices_to_bf16(tensors) if dtype == "bfloat16" else tensors
+    seqs = {"a": helpers.random_tokens(150, TOY["vocab"], 1), "b": helpers.random_tokens(61, TOY["vocab"], 2)}
+    want = {k: _toy_plain(ref, v) for k, v in seqs.items()}
+    # the bfloat16 tolerance is wider here: the toy mixers written with torch ops round again
+    tol = dict(TOL, bfloat16=6e-2)
+
+    def check(got, rid, what):
+        scale = want[rid].abs().max().item()
+        err = (got.double().cpu() - want[rid]).abs().max().item()
+        assert err <= tol[dtype] * scale, f"{what}: {err:.3e} against {scale:.3e}"
+
+    # whole
+    eng.add_request("a")
+    check(eng.step([StepEntry("a", seqs["a"], list(range(150)))]), "a", "whole")
+    eng.end_request("a")
+    # in portions, the two requests mixed, pages of the windowed group coming back on the way
+    fed = {"a": 0, "b": 0}
+    got = {"a": [], "b": []}
+    cuts = {"a": [40, 2, 1, 1, 30, 1, 1, 17, 3, 54], "b": [1, 1, 25, 2, 1, 31]}
+    eng.add_request("a")
+    eng.add_request("b")
+    for i in range(10):
+        entries = []
+        for rid in ("a", "b"):
+            if i < len(cuts[rid]):
+                n = cuts[rid][i]
+                entries.append(StepEntry(rid, seqs[rid][fed[rid] : fed[rid] + n], list(range(n))))
+                fed[rid] += n
+        eng.cache.poison_free_pages()
+        out = eng.step(entries)
+        j = 0
+        for e in entries:
+            got[e.request_id].append(out[j : j + len(e.tokens)].clone())
+            j += len(e.tokens)
+        eng.cache.check()
+    for rid in ("a", "b"):
+        check(torch.cat(got[rid]), rid, f"portions, request {rid}")
+    # the window let pages go: the windowed group holds fewer than the full group
+    full, windowed = eng.cache.groups
+    if full.need.window:
+        full, windowed = windowed, full
+    assert windowed.pool.n_held < full.pool.n_held
+    eng.end_request("a")
+    eng.end_request("b")
+    assert eng.cache.free_pages() == 14
