@@ -42,6 +42,7 @@ class RequestCache:
     length: int = 0  # tokens whose keys and values are in the pages
     reserved: int = 0  # tokens that have pages (>= length)
     blocks: List[List[int]] = field(default_factory=list)  # per group: page of each block or -1
+    serial: int = 0  # unique over the manager's life, unlike the id
 
 
 class _Group:
@@ -134,7 +135,8 @@ class CacheManager:
         if not self._free_state_slots:
             raise OutOfSlots(f"all {self.max_requests} request slots are taken")
         slot = self._free_state_slots.pop()
-        rc = RequestCache(request_id, slot, blocks=[[] for _ in self.groups])
+        self._serial = getattr(self, "_serial", 0) + 1
+        rc = RequestCache(request_id, slot, blocks=[[] for _ in self.groups], serial=self._serial)
         self.requests[request_id] = rc
         for storage in self.state_storage.values():
             storage[slot].zero_()

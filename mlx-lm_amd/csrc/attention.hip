@@ -435,14 +435,20 @@ static int fill_args(AttnArgs& p, const char* who, void* out, const void* q, int
   return 0;
 }
 
-template <typename K>
-static int allow_lds(const char* who, K kernel, size_t bytes) {
+// Kernels that want more than 64 KB of LDS have to be told so once per size.
+static int allow_lds(const char* who, const void* kernel, size_t bytes) {
+  static const void* seen[8];
+  static size_t granted[8];
+  static int n_seen = 0;
   if (bytes > 160 * 1024) FAIL("%s: needs %zu bytes of LDS, more than a CU has", who, bytes);
-  if (bytes > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)kernel,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e != hipSuccess) FAIL("%s: cannot get %zu bytes of LDS: %s", who, bytes, hipGetErrorString(e));
-  }
+  if (bytes <= 64 * 1024) return 0;
+  int i = 0;
+  while (i < n_seen && seen[i] != kernel) ++i;
+  if (i < n_seen && granted[i] >= bytes) return 0;
+  hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e != hipSuccess) FAIL("%s: cannot get %zu bytes of LDS: %s", who, bytes, hipGetErrorString(e));
+  if (i == n_seen && n_seen < 8) seen[n_seen++] = kernel;
+  if (i < 8) granted[i] = bytes;
   return 0;
 }
 
@@ -462,10 +468,10 @@ extern "C" int attn_tile(void* out, const void* q, int ldq, int ldo, const void*
   const size_t lds = sizeof(float) * ((size_t)QT * head_dim + (size_t)KT * (head_dim + 1) + QT * KT);
   dim3 grid(n_tiles, n_heads), block(256);
   if (dtype == DT_F32) {
-    if (allow_lds("attn_tile", attn_tile_kernel<float>, lds)) return 1;
+    if (allow_lds("attn_tile", (const void*)attn_tile_kernel<float>, lds)) return 1;
     hipLaunchKernelGGL(attn_tile_kernel<float>, grid, block, lds, stream, p);
   } else {
-    if (allow_lds("attn_tile", attn_tile_kernel<bf16>, lds)) return 1;
+    if (allow_lds("attn_tile", (const void*)attn_tile_kernel<bf16>, lds)) return 1;
     hipLaunchKernelGGL(attn_tile_kernel<bf16>, grid, block, lds, stream, p);
   }
   CHECK_LAUNCH("attn_tile");
@@ -494,12 +500,12 @@ extern "C" int attn_row(void* out, const void* q, int ldq, int ldo, const void* 
       sizeof(float) * ((size_t)head_dim + 4 * (size_t)KT * (head_dim + 1) + 4 * KT + 8 + 4 * (size_t)head_dim);
   dim3 grid(n_rows, n_heads, n_splits), block(256);
   if (dtype == DT_F32) {
-    if (allow_lds("attn_row", attn_row_kernel<float>, lds)) return 1;
+    if (allow_lds("attn_row", (const void*)attn_row_kernel<float>, lds)) return 1;
     hipLaunchKernelGGL(attn_row_kernel<float>, grid, block, lds, stream, p);
     if (n_splits > 1)
       hipLaunchKernelGGL(attn_merge_kernel<float>, dim3(n_rows, n_heads), dim3(64), 0, stream, p);
   } else {
-    if (allow_lds("attn_row", attn_row_kernel<bf16>, lds)) return 1;
+    if (allow_lds("attn_row", (const void*)attn_row_kernel<bf16>, lds)) return 1;
     hipLaunchKernelGGL(attn_row_kernel<bf16>, grid, block, lds, stream, p);
     if (n_splits > 1)
       hipLaunchKernelGGL(attn_merge_kernel<bf16>, dim3(n_rows, n_heads), dim3(64), 0, stream, p);

@@ -1,0 +1,111 @@
+"""Decode steps recorded once as a HIP graph and replayed.
+
+A step in which every request brings exactly one token and wants its logits
+has the same launches every time: only the contents of the integer arrays
+(token ids, positions, block tables, state slots) change.  Such a step is run
+once eagerly, then captured with its host-to-device copy into a graph; later
+steps of the same batch size fill the pinned host array and replay.  This
+takes the place of the reference's one-step-ahead ``mx.async_eval`` pipelining
+(mlx_lm/generate.py:446-451,1449-1456) as the cure for launch latency.
+"""
+
+import numpy as np
+import torch
+
+from .context import AttentionPlan, StepContext
+
+
+def _pad4(n):
+    return (n + 3) // 4 * 4
+
+
+class DecodeGraph:
+    """The recorded decode step for one batch size."""
+
+    def __init__(self, engine, batch):
+        self.engine, self.batch = engine, batch
+        cm = engine.cache
+        B = batch
+        self.max_blocks = cm.blocks_for(engine.decoder.max_positions)
+        sizes = [B] * 6 + [2 * B] + [B * self.max_blocks] * len(cm.groups)
+        self.offsets, total = [], 0
+        for s in sizes:
+            self.offsets.append(total)
+            total += _pad4(s)
+        self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+        self.host_np = self.host.numpy()
+        self.dev = torch.zeros(total, dtype=torch.int32, device=engine.device)
+        ar = np.arange(B, dtype=np.int32)
+        for i in (2, 3, 5):  # token_req, wanted rows, attention rows: row r is request r
+            self.host_np[self.offsets[i] : self.offsets[i] + B] = ar
+        tiles = np.stack([ar, np.ones(B, dtype=np.int32)], 1).reshape(-1)
+        self.host_np[self.offsets[6] : self.offsets[6] + 2 * B] = tiles
+        self._row_keys = [[None] * B for _ in cm.groups]
+        self.graph = None
+        self.logits = None
+        self._keep = None  # buffers the recorded launches point into
+        self._copied = None
+
+    def _piece(self, i, n):
+        return self.dev[self.offsets[i] : self.offsets[i] + n]
+
+    def _context(self):
+        eng, B = self.engine, self.batch
+        ctx = StepContext(eng)
+        ctx.n_tokens = ctx.n_requests = ctx.n_wanted = B
+        ctx.token_ids, ctx.positions, ctx.token_req = self._piece(0, B), self._piece(1, B), self._piece(2, B)
+        ctx.wanted_rows, ctx.slot_ids = self._piece(3, B), self._piece(4, B)
+        plan = AttentionPlan()
+        plan.rows, plan.n_rows = self._piece(5, B), B
+        plan.all_tiles, plan.n_all_tiles = self._piece(6, 2 * B), B
+        plan.tiles, plan.n_tiles = self._piece(6, 0), 0
+        plan.max_row_context = eng.decoder.max_positions
+        ctx.attention_plan = plan
+        for gi in range(len(eng.cache.groups)):
+            ctx.block_tables.append(self._piece(7 + gi, B * self.max_blocks).view(B, self.max_blocks))
+        return ctx
+
+    def _fill(self, entries):
+        cm = self.engine.cache
+        if self._copied is not None:
+            self._copied.synchronize()  # the last replay's copy has read the host array
+        h, off, B = self.host_np, self.offsets, self.batch
+        for r, e in enumerate(entries):
+            rc = cm.requests[e.request_id]
+            h[off[0] + r] = int(e.tokens[0])
+            h[off[1] + r] = rc.length
+            h[off[4] + r] = rc.state_slot
+            for gi in range(len(cm.groups)):
+                blocks = rc.blocks[gi]
+                key = (rc.serial, len(blocks))
+                if self._row_keys[gi][r] != key:
+                    base = off[7 + gi] + r * self.max_blocks
+                    # pages a window has let go (-1) are never read; page 0 keeps the entry valid
+                    h[base : base + len(blocks)] = [p if p >= 0 else 0 for p in blocks]
+                    self._row_keys[gi][r] = key
+
+    def run(self, entries):
+        eng = self.engine
+        self._fill(entries)
+        if self.graph is None:
+            ctx = self._context()
+            # once eagerly: libraries load, scratch memory grows to what the step needs
+            self.dev.copy_(self.host, non_blocking=True)
+            eng.scratch.reset()
+            eng.decoder.forward(ctx)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            eng.scratch.frozen = True
+            try:
+                with torch.cuda.graph(graph):
+                    self.dev.copy_(self.host, non_blocking=True)
+                    eng.scratch.reset()
+                    self.logits = eng.decoder.forward(ctx)
+            finally:
+                eng.scratch.frozen = False
+            self.graph = graph
+            self._keep = (eng.scratch.buffer, eng._logits)
+            self._copied = torch.cuda.Event()
+        self.graph.replay()
+        self._copied.record()
+        return self.logits

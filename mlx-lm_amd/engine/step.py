@@ -59,7 +59,7 @@ class Engine:
     """
 
     def __init__(self, model, dtype="bfloat16", device="cuda:0", page_size=16, n_pages=None,
-                 max_tokens=None, max_requests=64):
+                 max_tokens=None, max_requests=64, use_graphs=True):
         if not torch.cuda.is_available():
             raise RuntimeError("the engine needs a GPU: torch.cuda.is_available() is false")
         self.model = model
@@ -78,6 +78,9 @@ class Engine:
         self._meta_dev = None
         self._logits = None
         self.steps = 0
+        # decode steps are recorded as graphs where every part launches kernels only
+        self.use_graphs = use_graphs and all(getattr(p, "graph_safe", False) for p in self.decoder.parts())
+        self._graphs = {}
 
     # -- buffers ---------------------------------------------------------------
 
@@ -148,9 +151,17 @@ class Engine:
                 cm.truncate(e.request_id, rc.length)  # gives back pages beyond what is stored
             raise
 
-        ctx = self._build_context(entries)
-        self.scratch.reset()
-        logits = self.decoder.forward(ctx)
+        if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+            graph = self._graphs.get(len(entries))
+            if graph is None:
+                from .graph import DecodeGraph
+
+                graph = self._graphs[len(entries)] = DecodeGraph(self, len(entries))
+            logits = graph.run(entries)
+        else:
+            ctx = self._build_context(entries)
+            self.scratch.reset()
+            logits = self.decoder.forward(ctx)
         for e in entries:
             cm.commit(e.request_id, len(e.tokens))
         self.steps += 1

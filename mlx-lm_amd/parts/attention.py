@@ -20,6 +20,7 @@ class CausalSelfAttention(Mixer):
     before the cache write.
     """
 
+
     def __init__(self, width, n_heads, head_dim, n_kv_heads=None, scale=None, bias=True, window=0,
                  position=None, qkv_name="c_attn", out_name="c_proj", prefix=""):
         super().__init__(prefix)
@@ -42,6 +43,8 @@ class CausalSelfAttention(Mixer):
             build_part(POSITION_ENCODINGS, "position encoding", position) if position is not None else None
         )
         self.qkv_w = self.qkv_b = self.out_w = self.out_b = None
+        # launches kernels only (a step of such parts can be recorded), unless the position hook does more
+        self.graph_safe = self.position is None or getattr(self.position, "graph_safe", False)
 
     def cache_need(self):
         return CacheNeed(self.n_kv_heads, self.head_dim, self.window)

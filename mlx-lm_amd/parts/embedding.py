@@ -10,6 +10,8 @@ class TokenEmbedding(Part):
     mlx_lm/models/gpt2.py:119-120,132.
     """
 
+    graph_safe = True  # launches kernels only: a step of such parts can be recorded
+
     def __init__(self, vocab_size, width, weight_name="weight", prefix=""):
         super().__init__(prefix)
         if vocab_size <= 0 or width <= 0:

@@ -13,6 +13,8 @@ class GeluMLP(FeedForward):
     into the first product, the residual add into the second.
     """
 
+    graph_safe = True  # launches kernels only: a step of such parts can be recorded
+
     def __init__(self, width, inner, activation="gelu_new", prefix=""):
         super().__init__(prefix)
         if activation not in _TANH_GELU:

@@ -12,6 +12,8 @@ class LinearHead(Part):
     mlx_lm/models/gpt2.py:167).
     """
 
+    graph_safe = True  # launches kernels only: a step of such parts can be recorded
+
     def __init__(self, vocab_size, width, weight_name, prefix=""):
         super().__init__(prefix)
         self.vocab_size, self.width = vocab_size, width

@@ -12,6 +12,8 @@ class LayerNorm(Norm):
     computes in float32, writes the compute dtype.
     """
 
+    graph_safe = True  # launches kernels only: a step of such parts can be recorded
+
     def __init__(self, width, eps, bias=True, prefix=""):
         super().__init__(prefix)
         self.width, self.eps, self.has_bias = width, float(eps), bias

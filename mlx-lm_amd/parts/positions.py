@@ -6,6 +6,8 @@ from .base import PositionEncoding, TensorSpec, register_position_encoding
 class NoPositions(PositionEncoding):
     """Nothing is added and nothing is rotated."""
 
+    graph_safe = True  # launches kernels only: a step of such parts can be recorded
+
     def __init__(self, prefix=""):
         super().__init__(prefix)
 
@@ -18,6 +20,8 @@ class LearnedPositions(PositionEncoding):
     A position at or beyond the table's end is refused by the engine before
     anything runs (the reference does not check it).
     """
+
+    graph_safe = True  # launches kernels only: a step of such parts can be recorded
 
     def __init__(self, max_positions, width, weight_name="weight", prefix=""):
         super().__init__(prefix)

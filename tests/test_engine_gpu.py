@@ -263,3 +263,55 @@ def test_trace_run_program(folders, tmp_path, dtype):
     for rid, toks in tokens.items():
         want = _plain_logits(weights, config, toks, dtype)
         _close(torch.cat(got[rid]), want, dtype, f"trace_run, request {rid}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recorded_decode_steps_equal_eager_ones(folders, dtype):
+    """Decode steps replayed from a graph, with the program's own eager work between the
+    replays (portions of other prompts, requests ending, pages used again), against
+    the same trace run eagerly and against the plain implementation."""
+    from mlx_lm_amd.engine import Engine, StepEntry
+    from mlx_lm_amd.utils import load_model
+
+    folder, config, weights = folders[("B", 8.0)]
+    V = config["vocab_size"]
+    model, _ = load_model(folder, dtype=dtype)
+    seqs = {r: helpers.random_tokens(n, V, seed=60 + i) for i, (r, n) in enumerate(
+        [("a", 120), ("b", 75), ("c", 200), ("d", 64)])}
+    results = {}
+    for use_graphs in (True, False):
+        eng = Engine(model, dtype=dtype, page_size=16, n_pages=30, max_requests=4, use_graphs=use_graphs)
+        assert eng.use_graphs == use_graphs
+        got = {r: [] for r in seqs}
+        fed = dict.fromkeys(seqs, 0)
+        for r in ("a", "b", "c"):
+            eng.add_request(r)
+            n = len(seqs[r]) // 2
+            got[r].append(eng.step([StepEntry(r, seqs[r][:n], list(range(n)))]).clone())
+            fed[r] = n
+        live = ["a", "b", "c"]
+        step = 0
+        while live:
+            step += 1
+            out = eng.step([StepEntry(r, [seqs[r][fed[r]]], [0]) for r in live])  # recorded
+            for i, r in enumerate(live):
+                got[r].append(out[i : i + 1].clone())
+                fed[r] += 1
+            for r in list(live):
+                if fed[r] == len(seqs[r]):
+                    eng.end_request(r)
+                    live.remove(r)
+            if step == 20:  # eager work between replays: a new request's prompt, in two portions
+                eng.add_request("d")
+                got["d"].append(eng.step([StepEntry("d", seqs["d"][:40], list(range(40)))]).clone())
+                got["d"].append(eng.step([StepEntry("d", seqs["d"][40:63], list(range(23)))]).clone())
+                fed["d"] = 63
+                live.append("d")
+            eng.cache.check()
+        if use_graphs:
+            assert sorted(eng._graphs) == [1, 2, 3, 4] and all(g.graph is not None for g in eng._graphs.values())
+        results[use_graphs] = {r: torch.cat(v) for r, v in got.items()}
+    for r, toks in seqs.items():
+        want = _plain_logits(weights, config, toks, dtype)
+        _close(results[True][r], want, dtype, f"recorded, request {r}")
+        assert torch.equal(results[True][r], results[False][r]), r
