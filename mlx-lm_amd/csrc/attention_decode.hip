@@ -1,0 +1,240 @@
+// Decode attention for bfloat16 caches: one query row per block, keys streamed
+// from the pages straight into registers (no LDS staging), for head sizes 32,
+// 64 and 128.  Same contract as attn_row in attention.hip (same arguments,
+// same partial buffers, same merge); this is the kernel that serving uses,
+// attn_row stays as the general one (any head size, float caches).
+//
+// Replaces scaled_dot_product_attention with one query per sequence
+// (mlx_lm/models/base.py:132-139 with mask=None, mlx_lm/generate.py:1414).
+//
+// Work split: grid (rows, heads, n_splits), 256 threads.  The row's keys
+// [k_lo, k_hi) are cut into tiles of 64; the tiles are dealt to the splits in
+// runs and, inside a block, to the four waves in turn.  A wave reads a tile as
+// CPK-lane groups: lane l holds 16 bytes (8 columns) l % CPK of key l / CPK of
+// each load, where CPK = head_dim / 8 lanes cover one key.  One load
+// instruction therefore reads 64 / CPK whole keys that lie back to back in a
+// page.  Scores: 8 products per lane, summed over the CPK lanes of the key by
+// xor shuffles.  The weighted sum keeps, per lane, the 8 columns of *its* keys
+// and is only joined over the lane groups (and then the waves) at the end.
+#include "common.h"
+
+struct DecodeArgs {
+  uint16_t* out;
+  const uint16_t* q;
+  const uint16_t* k_pages;
+  const uint16_t* v_pages;
+  const int* block_table;
+  const int* token_req;
+  const int* positions;
+  const int* rows;
+  float* part_o;
+  float* part_ml;
+  size_t page_stride;
+  int ldq, ldo, max_blocks;
+  int n_heads, n_kv_heads, page_size, window, n_splits;
+  float scale;
+};
+
+#define TILE 64
+
+__device__ __forceinline__ void unpack8(const uint4& v, float* f) {
+  f[0] = __uint_as_float(v.x << 16), f[1] = __uint_as_float(v.x & 0xffff0000u);
+  f[2] = __uint_as_float(v.y << 16), f[3] = __uint_as_float(v.y & 0xffff0000u);
+  f[4] = __uint_as_float(v.z << 16), f[5] = __uint_as_float(v.z & 0xffff0000u);
+  f[6] = __uint_as_float(v.w << 16), f[7] = __uint_as_float(v.w & 0xffff0000u);
+}
+
+template <int CPK>  // lanes per key: head_dim = 8 * CPK
+__global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs p) {
+  constexpr int HD = 8 * CPK;
+  constexpr int KPL = 64 / CPK;    // keys per load instruction
+  constexpr int NL = TILE / KPL;   // loads per tile (= CPK)
+  __shared__ float Ms[4], Ls[4];
+  __shared__ float Os[4][HD];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int item = blockIdx.x, h = blockIdx.y, split = blockIdx.z;
+  const int row = p.rows[item];
+  const int kv_head = h / (p.n_heads / p.n_kv_heads);
+  const int pos = p.positions[row];
+  const int* table = p.block_table + (size_t)p.token_req[row] * p.max_blocks;
+  const int sub = lane % CPK;  // which 8 columns of the key
+  const int kin = lane / CPK;  // which key of a load
+
+  float qf[8];
+  {
+    const uint4 qv = *(const uint4*)(p.q + (size_t)row * p.ldq + h * HD + sub * 8);
+    unpack8(qv, qf);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) qf[i] *= p.scale;
+  }
+
+  const int k_hi = pos + 1;
+  const int k_lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+  const int kt0 = (k_lo / TILE) * TILE;
+  const int n_tiles = (k_hi - kt0 + TILE - 1) / TILE;
+  const int per_split = (n_tiles + p.n_splits - 1) / p.n_splits;
+  const int t_begin = split * per_split;
+  const int t_end = min(n_tiles, t_begin + per_split);
+
+  float m = -INFINITY, l = 0.f, o[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = 0.f;
+
+  const size_t head_off = (size_t)kv_head * p.page_size * HD;
+
+  for (int t = t_begin + wave; t < t_end; t += 4) {
+    const int kt = kt0 + t * TILE;
+    uint4 kv[NL], vv[NL];
+    // all loads of the tile first; addresses of keys outside [k_lo, k_hi) are
+    // pulled inside (their scores are masked below)
+#pragma unroll
+    for (int j = 0; j < NL; ++j) {
+      int key = kt + j * KPL + kin;
+      key = min(max(key, k_lo), k_hi - 1);
+      const int page = table[key / p.page_size];
+      const size_t off = (size_t)page * p.page_stride + head_off +
+                         (size_t)(key % p.page_size) * HD + sub * 8;
+      kv[j] = *(const uint4*)(p.k_pages + off);
+      vv[j] = *(const uint4*)(p.v_pages + off);
+    }
+    float s[NL];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < NL; ++j) {
+      float kf[8];
+      unpack8(kv[j], kf);
+      float d = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) d += qf[i] * kf[i];
+#pragma unroll
+      for (int x = 1; x < CPK; x <<= 1) d += __shfl_xor(d, x, WAVE);
+      const int key = kt + j * KPL + kin;
+      s[j] = (key >= k_lo && key < k_hi) ? d : -INFINITY;
+      tmax = fmaxf(tmax, s[j]);
+    }
+#pragma unroll
+    for (int x = CPK; x < 64; x <<= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, x, WAVE));
+    const float m_new = fmaxf(m, tmax);  // finite: every tile holds at least one live key
+    const float alpha = __expf(m - m_new);
+    l *= alpha;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] *= alpha;
+#pragma unroll
+    for (int j = 0; j < NL; ++j) {
+      const float pj = __expf(s[j] - m_new);  // exp(-inf) = 0 for masked keys
+      float vf[8];
+      unpack8(vv[j], vf);
+      if (sub == 0) l += pj;  // one lane of the key's group counts it
+#pragma unroll
+      for (int i = 0; i < 8; ++i) o[i] += pj * vf[i];
+    }
+    m = m_new;
+  }
+
+  // join the lane groups: lanes with the same `sub` hold the same columns
+#pragma unroll
+  for (int x = CPK; x < 64; x <<= 1) {
+    l += __shfl_xor(l, x, WAVE);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] += __shfl_xor(o[i], x, WAVE);
+  }
+#pragma unroll
+  for (int x = 1; x < CPK; x <<= 1) l += __shfl_xor(l, x, WAVE);
+
+  if (lane == 0) Ms[wave] = m, Ls[wave] = l;
+  if (lane < CPK) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) Os[wave][lane * 8 + i] = o[i];
+  }
+  __syncthreads();
+
+  const float M = fmaxf(fmaxf(Ms[0], Ms[1]), fmaxf(Ms[2], Ms[3]));
+  float w[4], L = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    w[i] = (Ms[i] == -INFINITY) ? 0.f : __expf(Ms[i] - M);
+    L += Ls[i] * w[i];
+  }
+  if (tid < HD) {
+    const float acc = Os[0][tid] * w[0] + Os[1][tid] * w[1] + Os[2][tid] * w[2] + Os[3][tid] * w[3];
+    if (p.n_splits == 1) {
+      p.out[(size_t)row * p.ldo + h * HD + tid] = f32_to_bf16_bits(acc / L);
+    } else {
+      const size_t base = ((size_t)item * p.n_heads + h) * p.n_splits + split;
+      p.part_o[base * HD + tid] = acc;
+      if (tid == 0) p.part_ml[base * 2] = M, p.part_ml[base * 2 + 1] = L;
+    }
+  }
+}
+
+// grid (rows, heads), HD threads: join the splits
+template <int CPK>
+__global__ void attn_decode_merge_kernel(DecodeArgs p) {
+  constexpr int HD = 8 * CPK;
+  const int item = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
+  const int row = p.rows[item];
+  const size_t base = ((size_t)item * p.n_heads + h) * p.n_splits;
+  float M = -INFINITY;
+  for (int s = 0; s < p.n_splits; ++s) M = fmaxf(M, p.part_ml[(base + s) * 2]);
+  float L = 0.f, acc = 0.f;
+  for (int s = 0; s < p.n_splits; ++s) {
+    const float ms = p.part_ml[(base + s) * 2];
+    if (ms == -INFINITY) continue;
+    const float w = __expf(ms - M);
+    L += p.part_ml[(base + s) * 2 + 1] * w;
+    acc += p.part_o[(base + s) * HD + d] * w;
+  }
+  p.out[(size_t)row * p.ldo + h * HD + d] = f32_to_bf16_bits(acc / L);
+}
+
+DEFINE_LAST_ERROR(mlxlm_last_error)
+
+template <int CPK>
+static void launch(const DecodeArgs& p, int n_rows, hipStream_t stream) {
+  hipLaunchKernelGGL(attn_decode_kernel<CPK>, dim3(n_rows, p.n_heads, p.n_splits), dim3(256), 0, stream, p);
+  if (p.n_splits > 1)
+    hipLaunchKernelGGL(attn_decode_merge_kernel<CPK>, dim3(n_rows, p.n_heads), dim3(8 * CPK), 0, stream, p);
+}
+
+// Same arguments as attn_row; bfloat16 only, head_dim 32, 64 or 128, and pages
+// that hold whole loads (page_size a multiple of 512 / head_dim keys).
+extern "C" int attn_decode(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                           const void* v_pages, size_t page_stride, const int* block_table,
+                           int max_blocks, const int* token_req, const int* positions,
+                           const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
+                           int page_size, int window, float scale, int n_splits, float* part_o,
+                           float* part_ml, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (head_dim != 32 && head_dim != 64 && head_dim != 128)
+    FAIL("attn_decode: head_dim %d is not 32, 64 or 128 (attn_row takes the others)", head_dim);
+  const int kpl = 512 / head_dim;
+  if (page_size <= 0 || page_size % kpl != 0)
+    FAIL("attn_decode: page_size %d must be a multiple of %d for head_dim %d", page_size, kpl, head_dim);
+  if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads != 0)
+    FAIL("attn_decode: %d query heads cannot be grouped over %d key heads", n_heads, n_kv_heads);
+  if (!out || !q || !k_pages || !v_pages || !block_table || !token_req || !positions || !rows)
+    FAIL("attn_decode: null pointer");
+  if (ldq % 8 != 0 || ((uintptr_t)q & 15)) FAIL("attn_decode: queries must be 16-byte aligned rows");
+  if (page_stride % 8 != 0 || (((uintptr_t)k_pages | (uintptr_t)v_pages) & 15))
+    FAIL("attn_decode: pages must be 16-byte aligned");
+  if (window < 0) FAIL("attn_decode: window %d must not be negative", window);
+  if (n_splits < 1 || n_splits > 65535) FAIL("attn_decode: n_splits %d out of range", n_splits);
+  if (n_splits > 1 && (!part_o || !part_ml)) FAIL("attn_decode: splits need the partial buffers");
+  DecodeArgs p;
+  p.out = (uint16_t*)out, p.q = (const uint16_t*)q;
+  p.k_pages = (const uint16_t*)k_pages, p.v_pages = (const uint16_t*)v_pages;
+  p.block_table = block_table, p.token_req = token_req, p.positions = positions, p.rows = rows;
+  p.part_o = part_o, p.part_ml = part_ml, p.page_stride = page_stride;
+  p.ldq = ldq, p.ldo = ldo, p.max_blocks = max_blocks;
+  p.n_heads = n_heads, p.n_kv_heads = n_kv_heads, p.page_size = page_size;
+  p.window = window, p.n_splits = n_splits, p.scale = scale;
+  if (head_dim == 32)
+    launch<4>(p, n_rows, stream);
+  else if (head_dim == 64)
+    launch<8>(p, n_rows, stream);
+  else
+    launch<16>(p, n_rows, stream);
+  CHECK_LAUNCH("attn_decode");
+  return 0;
+}

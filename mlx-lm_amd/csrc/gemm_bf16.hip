@@ -18,6 +18,11 @@
 #define FLAG_ACCUMULATE 2
 #define FLAG_OUT_F32 4
 
+// Out-of-range loads read a clamped address and are zeroed afterwards with this
+// constant: selecting between an address and a zero kept in a variable turns
+// the load into a flat load through scratch memory.
+#define ZERO4 make_uint4(0u, 0u, 0u, 0u)
+
 struct GemmArgs {
   const uint16_t* A;
   const uint16_t* W;
@@ -76,7 +81,6 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(GemmArgs p) {
 
   // each thread moves four 16-byte pieces of A and of W per k-block
   uint4 ra[4], rb[4];
-  const uint4 zero4 = make_uint4(0, 0, 0, 0);
 
   auto load_global = [&](int k0) {
 #pragma unroll
@@ -86,8 +90,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(GemmArgs p) {
       const int kc = (c & 7) * 8;
       const int gk = k0 + kc;
       const int gm = m0 + row, gn = n0 + row;
-      ra[i] = (gm < p.M && gk < p.K) ? *(const uint4*)(p.A + (size_t)gm * p.lda + gk) : zero4;
-      rb[i] = (gn < p.N && gk < p.K) ? *(const uint4*)(p.W + (size_t)gn * p.ldw + gk) : zero4;
+      const int ck = min(gk, p.K - 8);
+      const uint4 ta = *(const uint4*)(p.A + (size_t)min(gm, p.M - 1) * p.lda + ck);
+      const uint4 tb = *(const uint4*)(p.W + (size_t)min(gn, p.N - 1) * p.ldw + ck);
+      ra[i] = (gm < p.M && gk < p.K) ? ta : ZERO4;
+      rb[i] = (gn < p.N && gk < p.K) ? tb : ZERO4;
     }
   };
   auto store_lds = [&]() {
@@ -168,13 +175,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(GemmArgs p) {
   const int wrow = n0 + (lane & 15);
   const int koff = (lane >> 4) * 16;
   const bool wvalid = wrow < p.N;
-  const uint16_t* wp = p.W + (size_t)(wvalid ? wrow : 0) * p.ldw + koff;
+  const uint16_t* wrow_p = p.W + (size_t)(wvalid ? wrow : 0) * p.ldw;
 
   f32x4_t acc[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
-  const uint4 zero4 = make_uint4(0, 0, 0, 0);
   union Frag {
     uint4 u;
     bf16x8_t v;
@@ -183,16 +189,20 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(GemmArgs p) {
   for (int k0 = wave * 64; k0 < p.K; k0 += SK_WAVES * 64) {
     const int k = k0 + koff;  // this lane covers k .. k+15
     Frag w0, w1;
-    w0.u = (wvalid && k < p.K) ? *(const uint4*)(wp + k0) : zero4;
-    w1.u = (wvalid && k + 8 < p.K) ? *(const uint4*)(wp + k0 + 8) : zero4;
+    const uint4 t0 = *(const uint4*)(wrow_p + min(k, p.K - 8));
+    const uint4 t1 = *(const uint4*)(wrow_p + min(k + 8, p.K - 8));
+    w0.u = (wvalid && k < p.K) ? t0 : ZERO4;
+    w1.u = (wvalid && k + 8 < p.K) ? t1 : ZERO4;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
       const int m = t * 16 + (lane & 15);
       const bool av = m < p.M;
-      const uint16_t* ap = p.A + (size_t)(av ? m : 0) * p.lda + k;
+      const uint16_t* arow = p.A + (size_t)(av ? m : 0) * p.lda;
       Frag a0, a1;
-      a0.u = (av && k < p.K) ? *(const uint4*)(ap) : zero4;
-      a1.u = (av && k + 8 < p.K) ? *(const uint4*)(ap + 8) : zero4;
+      const uint4 u0 = *(const uint4*)(arow + min(k, p.K - 8));
+      const uint4 u1 = *(const uint4*)(arow + min(k + 8, p.K - 8));
+      a0.u = (av && k < p.K) ? u0 : ZERO4;
+      a1.u = (av && k + 8 < p.K) ? u1 : ZERO4;
       acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0.v, a0.v, acc[t], 0, 0, 0);
       acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1.v, a1.v, acc[t], 0, 0, 0);
     }

@@ -1,0 +1,287 @@
+// Linear layer for decode steps: at most 16 rows of activations against a
+// bfloat16 weight matrix that streams from HBM exactly once.
+//   out[m, n] = epilogue( sum_k A[m, k] * W[n, k] + bias[n] )
+// with two fusions that save a launch and a round trip through memory each:
+//  * prologue: A may be given as the float32 residual stream plus LayerNorm
+//    parameters; every block then norms the (few) rows itself into LDS
+//    (mlx_lm/models/gpt2.py:104,106: ln_1 / ln_2 before c_attn / c_fc);
+//  * epilogue: output columns from `q_width` on may be scattered straight
+//    into the pages of the key/value cache (mlx_lm/models/cache.py:352-354)
+//    instead of the output matrix.
+// Otherwise the epilogues of gemm_bf16.hip: plain, tanh-GELU, accumulate into
+// the float32 residual stream, float32 out.
+//
+// A block of eight waves owns 16 output features.  The activations (normed or
+// copied) sit in LDS as the MFMA B-operand; each wave takes every eighth
+// 64-wide k-block of the 16 weight rows as the A-operand of two
+// v_mfma_f32_16x16x32_bf16 (lane l reads 32 contiguous bytes of row l % 16 at
+// k offset (l / 16) * 16).  Weight loads run two passes of four k-blocks ahead
+// of the MFMAs; the eight partial tiles are summed in a fixed order.
+#include "common.h"
+
+#define FLAG_GELU 1
+#define FLAG_ACCUMULATE 2
+#define FLAG_OUT_F32 4
+#define FLAG_KV 8
+
+#define NW 8        // waves per block
+#define U 4         // k-blocks per pass and wave
+#define LN_MAX_V 16 // float4 per lane a normed row may take (K <= 4096)
+#define ZERO4 make_uint4(0u, 0u, 0u, 0u)  // a constant, not a variable: see load_pass
+
+struct DecodeGemmArgs {
+  const uint16_t* W;
+  const float* bias;
+  void* out;
+  const uint16_t* A;   // [M, K] activations, or null when X is given
+  const float* X;      // [M, K] residual stream to be normed
+  const float* gamma;
+  const float* beta;
+  float eps;
+  int M, N, K, lda, ldx, ldw, ldo, flags;
+  int a_stride;        // LDS row stride in elements
+  // key/value scatter
+  uint16_t* k_pages;
+  uint16_t* v_pages;
+  size_t page_stride;
+  const int* block_table;
+  const int* token_req;
+  const int* positions;
+  int max_blocks, q_width, kv_width, head_dim, page_size;
+};
+
+__device__ __forceinline__ float gelu_tanh(float x) {
+  const float c = 0.7978845608028654f;
+  const float u = c * (x + 0.044715f * x * x * x);
+  return 0.5f * x * (1.0f + tanhf(u));
+}
+
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+}
+
+union Frag {
+  uint4 u;
+  bf16x8_t v;
+};
+
+// LV: float4 per lane that a normed row takes (8: K <= 2048, 16: K <= 4096); 0: no norm
+template <int LV>
+__global__ __launch_bounds__(NW * 64, (LV <= 8 ? 2 : 1)) void gemm_bf16_decode_kernel(DecodeGemmArgs p) {
+  constexpr bool LN = LV > 0;
+  constexpr int NV = LN ? LV : 1;
+  extern __shared__ __attribute__((aligned(16))) uint16_t As[];  // [M][a_stride]
+  __shared__ float red[NW][256];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n0 = blockIdx.x * 16;
+  const int koff = (lane >> 4) * 16;
+  const bool wvalid = n0 + (lane & 15) < p.N;
+  const uint16_t* wrow = p.W + (size_t)(wvalid ? n0 + (lane & 15) : 0) * p.ldw;
+  const int n_chunks = (p.K + 63) / 64;
+
+  // Loads are never predicated on their address (a select between an address
+  // and a dummy makes them flat loads, which also count as LDS traffic): every
+  // address is pulled into range and the value is zeroed afterwards, with a
+  // constant (a zero that lives in a variable is a second address to select).
+  auto load_pass = [&](Frag (&w)[U][2], int pass) {
+    if (wave + NW * pass * U >= n_chunks) return;  // the whole pass lies beyond K (uniform)
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = wave + NW * (pass * U + u);
+      const int k = min(c, n_chunks - 1) * 64 + koff;
+      const uint4 t0 = *(const uint4*)(wrow + min(k, p.K - 8));
+      const uint4 t1 = *(const uint4*)(wrow + min(k + 8, p.K - 8));
+      const bool live = wvalid && c < n_chunks;
+      w[u][0].u = (live && k < p.K) ? t0 : ZERO4;
+      w[u][1].u = (live && k + 8 < p.K) ? t1 : ZERO4;
+    }
+  };
+
+  Frag w0[U][2], w1[U][2];
+  load_pass(w0, 0);  // in flight while the activations are prepared
+
+  // ---- activations into LDS ------------------------------------------------
+  if (LN) {
+    for (int r = wave; r < p.M; r += NW) {
+      const float* x = p.X + (size_t)r * p.ldx;
+      float4 v[NV];
+      float s = 0.f;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int k = (lane + 64 * i) * 4;
+        const float4 t = *(const float4*)(x + min(k, p.K - 4));
+        v[i] = k < p.K ? t : make_float4(0.f, 0.f, 0.f, 0.f);
+        s += v[i].x + v[i].y + v[i].z + v[i].w;
+      }
+      const float mean = wave_sum(s) / (float)p.K;
+      float q = 0.f;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int k = (lane + 64 * i) * 4;
+        if (k < p.K) {
+          const float a = v[i].x - mean, b = v[i].y - mean, c = v[i].z - mean, d = v[i].w - mean;
+          q += a * a + b * b + c * c + d * d;
+        }
+      }
+      const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)p.K + p.eps);
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int k = (lane + 64 * i) * 4;
+        if (k < p.K) {
+          const float4 g = *(const float4*)(p.gamma + k);
+          const float4 b = *(const float4*)(p.beta + k);
+          uint2 o;
+          o.x = pack2((v[i].x - mean) * rstd * g.x + b.x, (v[i].y - mean) * rstd * g.y + b.y);
+          o.y = pack2((v[i].z - mean) * rstd * g.z + b.z, (v[i].w - mean) * rstd * g.w + b.w);
+          *(uint2*)(As + r * p.a_stride + k) = o;
+        }
+      }
+    }
+  } else {
+    const int per_row = p.K / 8;
+    for (int c = tid; c < p.M * per_row; c += NW * 64) {
+      const int r = c / per_row, k = (c - r * per_row) * 8;
+      *(uint4*)(As + r * p.a_stride + k) = *(const uint4*)(p.A + (size_t)r * p.lda + k);
+    }
+  }
+  __syncthreads();
+
+  // ---- main loop: two passes of loads ahead of the MFMAs --------------------
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+  const bool avalid = (lane & 15) < p.M;
+  const uint16_t* arow = As + min(lane & 15, p.M - 1) * p.a_stride;
+
+  auto compute_pass = [&](Frag (&w)[U][2], int pass) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = wave + NW * (pass * U + u);
+      if (c < n_chunks) {  // uniform over the wave
+        const int k = c * 64 + koff;
+        Frag a0, a1;
+        const uint4 t0 = *(const uint4*)(arow + min(k, p.K - 8));
+        const uint4 t1 = *(const uint4*)(arow + min(k + 8, p.K - 8));
+        a0.u = (avalid && k < p.K) ? t0 : ZERO4;
+        a1.u = (avalid && k + 8 < p.K) ? t1 : ZERO4;
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][0].v, a0.v, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][1].v, a1.v, acc, 0, 0, 0);
+      }
+    }
+  };
+
+  const int n_pass = (n_chunks + NW * U - 1) / (NW * U);
+  for (int pass = 0; pass < n_pass; pass += 2) {
+    load_pass(w1, pass + 1);
+    compute_pass(w0, pass);
+    load_pass(w0, pass + 2);
+    compute_pass(w1, pass + 1);
+  }
+
+  // ---- sum the waves' tiles in a fixed order, then the epilogue ---------------
+#pragma unroll
+  for (int r = 0; r < 4; ++r) red[wave][lane * 4 + r] = acc[r];
+  __syncthreads();
+  if (tid < 256) {
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) v += red[w][tid];
+    // element tid = 4 * L + r of the MFMA tile: feature 4 * (L / 16) + r, row L % 16
+    const int L = tid >> 2, r = tid & 3;
+    const int n = n0 + 4 * (L >> 4) + r;
+    const int m = L & 15;
+    if (m < p.M && n < p.N) {
+      if (p.bias) v += p.bias[n];
+      if (p.flags & FLAG_GELU) v = gelu_tanh(v);
+      if ((p.flags & FLAG_KV) && n >= p.q_width) {
+        const int c = n - p.q_width;
+        const bool is_v = c >= p.kv_width;
+        const int cc = is_v ? c - p.kv_width : c;
+        const int head = cc / p.head_dim, d = cc - head * p.head_dim;
+        const int pos = p.positions[m];
+        const int page = p.block_table[(size_t)p.token_req[m] * p.max_blocks + pos / p.page_size];
+        const size_t dst = (size_t)page * p.page_stride +
+                           ((size_t)head * p.page_size + pos % p.page_size) * p.head_dim + d;
+        (is_v ? p.v_pages : p.k_pages)[dst] = f32_to_bf16_bits(v);
+      } else {
+        const size_t idx = (size_t)m * p.ldo + n;
+        if (p.flags & FLAG_ACCUMULATE)
+          ((float*)p.out)[idx] += v;
+        else if (p.flags & FLAG_OUT_F32)
+          ((float*)p.out)[idx] = v;
+        else
+          ((uint16_t*)p.out)[idx] = f32_to_bf16_bits(v);
+      }
+    }
+  }
+}
+
+DEFINE_LAST_ERROR(mlxlm_last_error)
+
+#define MAX_LDS_BYTES (120 * 1024)
+
+// LDS row stride: rows of 16-byte reads from 16 lanes must fall on distinct
+// banks, which holds when the stride in 32-bit words is 4 mod 32.
+static int a_stride_for(int K) { return K + ((8 - K % 64) + 64) % 64; }
+
+// 1 if gemm_bf16_decode takes these sizes (the caller falls back otherwise)
+extern "C" int gemm_bf16_decode_takes(int M, int K, int with_norm) {
+  if (M < 1 || M > 16 || K % 8 != 0) return 0;
+  if (with_norm && (K > LN_MAX_V * 256 || K % 4 != 0)) return 0;
+  return (size_t)M * a_stride_for(K) * 2 <= MAX_LDS_BYTES;
+}
+
+extern "C" int gemm_bf16_decode(
+    void* out, const void* A, int lda, const float* X, int ldx, const float* gamma,
+    const float* beta, float eps, const void* W, const float* bias, int M, int N, int K, int ldw,
+    int ldo, int flags, void* k_pages, void* v_pages, size_t page_stride, const int* block_table,
+    int max_blocks, const int* token_req, const int* positions, int q_width, int kv_width,
+    int head_dim, int page_size, hipStream_t stream) {
+  if (M == 0) return 0;
+  const bool ln = X != nullptr;
+  if (!gemm_bf16_decode_takes(M, K, ln))
+    FAIL("gemm_bf16_decode: M=%d K=%d%s is outside what this kernel takes", M, K, ln ? " with norm" : "");
+  if (N <= 0) FAIL("gemm_bf16_decode: bad N=%d", N);
+  if ((A == nullptr) == (X == nullptr)) FAIL("gemm_bf16_decode: give activations or a residual stream to norm");
+  if (!W || !out) FAIL("gemm_bf16_decode: null pointer");
+  if (ldw % 8 != 0 || ldw < K || ((uintptr_t)W & 15)) FAIL("gemm_bf16_decode: W rows must be 16-byte aligned");
+  if (A && (lda % 8 != 0 || lda < K || ((uintptr_t)A & 15))) FAIL("gemm_bf16_decode: A rows must be 16-byte aligned");
+  if (X && (ldx % 4 != 0 || ldx < K || ((uintptr_t)X & 15))) FAIL("gemm_bf16_decode: X rows must be 16-byte aligned");
+  if (X && (!gamma || !beta || ((uintptr_t)gamma & 15) || ((uintptr_t)beta & 15)))
+    FAIL("gemm_bf16_decode: the norm needs scale and shift, 16-byte aligned");
+  if ((flags & FLAG_ACCUMULATE) && (flags & (FLAG_GELU | FLAG_KV)))
+    FAIL("gemm_bf16_decode: accumulate cannot be combined with GELU or the cache scatter");
+  if (flags & FLAG_KV) {
+    if (!k_pages || !v_pages || !block_table || !token_req || !positions)
+      FAIL("gemm_bf16_decode: the cache scatter needs pages, block table, token_req and positions");
+    if (head_dim <= 0 || page_size <= 0 || kv_width % head_dim != 0 || q_width + 2 * kv_width != N)
+      FAIL("gemm_bf16_decode: q_width %d + 2 * kv_width %d must be N=%d, kv_width a multiple of head_dim %d",
+           q_width, kv_width, N, head_dim);
+    if (flags & (FLAG_OUT_F32 | FLAG_GELU)) FAIL("gemm_bf16_decode: the cache scatter writes bfloat16, no GELU");
+    if (ldo < q_width) FAIL("gemm_bf16_decode: ldo=%d smaller than q_width=%d", ldo, q_width);
+  } else if (ldo < N) {
+    FAIL("gemm_bf16_decode: ldo=%d smaller than N=%d", ldo, N);
+  }
+  DecodeGemmArgs p;
+  p.W = (const uint16_t*)W, p.bias = bias, p.out = out, p.A = (const uint16_t*)A, p.X = X;
+  p.gamma = gamma, p.beta = beta, p.eps = eps;
+  p.M = M, p.N = N, p.K = K, p.lda = lda, p.ldx = ldx, p.ldw = ldw, p.ldo = ldo, p.flags = flags;
+  p.a_stride = a_stride_for(K);
+  p.k_pages = (uint16_t*)k_pages, p.v_pages = (uint16_t*)v_pages, p.page_stride = page_stride;
+  p.block_table = block_table, p.token_req = token_req, p.positions = positions;
+  p.max_blocks = max_blocks, p.q_width = q_width, p.kv_width = kv_width;
+  p.head_dim = head_dim, p.page_size = page_size;
+  const size_t lds = (size_t)M * p.a_stride * 2;
+  const int which = !ln ? 0 : (K <= 2048 ? 1 : 2);
+  void (*kernels[3])(DecodeGemmArgs) = {gemm_bf16_decode_kernel<0>, gemm_bf16_decode_kernel<8>,
+                                        gemm_bf16_decode_kernel<LN_MAX_V>};
+  static size_t granted[3] = {0, 0, 0};
+  if (lds + sizeof(float) * NW * 256 > 64 * 1024 && granted[which] < lds) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernels[which],
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) FAIL("gemm_bf16_decode: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    granted[which] = lds;
+  }
+  hipLaunchKernelGGL(kernels[which], dim3((N + 15) / 16), dim3(NW * 64), lds, stream, p);
+  CHECK_LAUNCH("gemm_bf16_decode");
+  return 0;
+}

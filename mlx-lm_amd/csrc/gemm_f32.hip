@@ -10,6 +10,11 @@
 #define FLAG_GELU 1
 #define FLAG_ACCUMULATE 2
 
+// Out-of-range loads read a clamped address and are zeroed afterwards with this
+// constant: selecting between an address and a zero kept in a variable turns
+// the load into a flat load through scratch memory.
+#define ZERO4 make_float4(0.f, 0.f, 0.f, 0.f)
+
 struct GemmArgs {
   const float* A;
   const float* W;
@@ -56,20 +61,21 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs p) {
   constexpr int PA = (BM_ * 4) / 256;
   constexpr int PB = (BN_ * 4) / 256;
   float4 ra[PA], rb[PB];
-  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
 
   auto load_global = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < PA; ++i) {
       const int c = tid + 256 * i;
       const int row = c >> 2, gk = k0 + (c & 3) * 4, gm = m0 + row;
-      ra[i] = (gm < p.M && gk < p.K) ? *(const float4*)(p.A + (size_t)gm * p.lda + gk) : zero4;
+      const float4 t = *(const float4*)(p.A + (size_t)min(gm, p.M - 1) * p.lda + min(gk, p.K - 4));
+      ra[i] = (gm < p.M && gk < p.K) ? t : ZERO4;
     }
 #pragma unroll
     for (int i = 0; i < PB; ++i) {
       const int c = tid + 256 * i;
       const int row = c >> 2, gk = k0 + (c & 3) * 4, gn = n0 + row;
-      rb[i] = (gn < p.N && gk < p.K) ? *(const float4*)(p.W + (size_t)gn * p.ldw + gk) : zero4;
+      const float4 t = *(const float4*)(p.W + (size_t)min(gn, p.N - 1) * p.ldw + min(gk, p.K - 4));
+      rb[i] = (gn < p.N && gk < p.K) ? t : ZERO4;
     }
   };
   auto store_lds = [&]() {

@@ -22,6 +22,7 @@ DT = {torch.float32: 0, torch.bfloat16: 1}
 GEMM_GELU = 1
 GEMM_ACCUMULATE = 2
 GEMM_OUT_F32 = 4
+GEMM_KV = 8
 
 
 def _stream():
@@ -100,19 +101,54 @@ def layernorm(out, x, gamma, beta, eps, rows=None):
     return out
 
 
-def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0):
+class NormedInput:
+    """The LayerNorm of float32 rows, not computed yet.
+
+    ``linear`` takes it as its input and, where its kernel can, norms the rows
+    itself while the first weights are on their way; anything else calls
+    ``materialize()`` and gets the tensor.
+    """
+
+    def __init__(self, alloc, x, gamma, beta, eps, dtype):
+        self.alloc, self.x, self.gamma, self.beta, self.eps, self.dtype = alloc, x, gamma, beta, eps, dtype
+        self.shape = tuple(x.shape)
+        self._out = None
+
+    def materialize(self):
+        if self._out is None:
+            self._out = self.alloc(self.shape, self.dtype)
+            layernorm(self._out, self.x, self.gamma, self.beta, self.eps)
+        return self._out
+
+
+class KVScatter:
+    """Where the key and value columns of a fused q/k/v projection go: the
+    pages of ``kv``, for each token at its request's position."""
+
+    def __init__(self, kv, block_table, token_req, positions, q_width):
+        self.kv, self.block_table, self.token_req, self.positions = kv, block_table, token_req, positions
+        self.q_width = q_width
+        self.kv_width = kv.n_kv_heads * kv.head_dim
+
+
+def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatter=None):
     """``out = epilogue(a @ w.T + bias)``.
 
-    ``a`` is ``[M, K]``, ``w`` is ``[N, K]``, both float32 or both bfloat16;
-    ``bias`` float32.  ``accumulate`` adds into a float32 ``out`` (the residual
-    stream); otherwise ``out`` is float32 or the operands' dtype.
+    ``a`` is ``[M, K]`` (or a ``NormedInput``), ``w`` is ``[N, K]``, both
+    float32 or both bfloat16; ``bias`` float32.  ``accumulate`` adds into a
+    float32 ``out`` (the residual stream); otherwise ``out`` is float32 or the
+    operands' dtype.  With ``scatter`` (a ``KVScatter``) the columns from
+    ``scatter.q_width`` on are also written to the key/value pages.  Up to 16
+    bfloat16 rows go to the decode kernel, which fuses the norm and the
+    scatter; everything else is composed from the general kernels.
     """
-    lda, ldw, ldo = _rows2d(a, "a"), _rows2d(w, "w"), _rows2d(out, "out")
+    lazy = a if isinstance(a, NormedInput) else None
     M, K = a.shape
     N = w.shape[0]
+    ldw, ldo = _rows2d(w, "w"), _rows2d(out, "out")
     _need(w.shape[1] == K, f"linear: a is [{M},{K}] but w is {list(w.shape)}")
     _need(tuple(out.shape) == (M, N), f"linear: out is {list(out.shape)}, want [{M},{N}]")
-    _need(a.dtype == w.dtype and a.dtype in DT, "linear: a and w must share float32 or bfloat16")
+    _need(a.dtype == w.dtype and w.dtype in DT, "linear: a and w must share float32 or bfloat16")
     if bias is not None:
         _dev(bias, "bias", torch.float32)
         _need(bias.numel() == N, "linear: bias length")
@@ -122,15 +158,48 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0):
     if accumulate:
         _need(out.dtype == torch.float32, "linear: accumulate needs a float32 out")
         flags |= GEMM_ACCUMULATE
-    if a.dtype == torch.float32:
+    if scatter is not None:
+        _need(not accumulate and not gelu and out.dtype == w.dtype, "linear: scatter goes with a plain epilogue")
+        _need(scatter.q_width + 2 * scatter.kv_width == N, "linear: scatter widths do not add up to N")
+        _need(scatter.kv.k.dtype == w.dtype, "linear: cache dtype differs from the projection's")
+    if w.dtype == torch.float32:
         _need(out.dtype == torch.float32, "linear: float32 operands give a float32 out")
+    elif out.dtype == torch.float32:
+        flags |= GEMM_OUT_F32
+    else:
+        _need(out.dtype == torch.bfloat16, "linear: out must be float32 or bfloat16")
+
+    if w.dtype == torch.bfloat16 and variant == 0 and 0 < M <= 16:
+        lib = build.load("gemm_bf16_decode")
+        if lib.gemm_bf16_decode_takes(_c_int(M), _c_int(K), _c_int(1 if lazy else 0)):
+            if lazy:
+                _dev(lazy.x, "x", torch.float32)
+                A, lda, X, ldx = None, 0, lazy.x, lazy.x.stride(0)
+                gamma, beta, eps = lazy.gamma, lazy.beta, lazy.eps
+            else:
+                A, lda, X, ldx, gamma, beta, eps = a, _rows2d(a, "a"), None, 0, None, None, 0.0
+            sc = scatter
+            rc = lib.gemm_bf16_decode(
+                _ptr(out), _ptr(A), _c_int(lda), _ptr(X), _c_int(ldx), _ptr(gamma), _ptr(beta),
+                _c_float(eps), _ptr(w), _ptr(bias), _c_int(M), _c_int(N), _c_int(K), _c_int(ldw),
+                _c_int(ldo), _c_int(flags | (GEMM_KV if sc else 0)),
+                _ptr(sc.kv.k if sc else None), _ptr(sc.kv.v if sc else None),
+                _c_size_t(sc.kv.page_stride if sc else 0), _ptr(sc.block_table if sc else None),
+                _c_int(sc.block_table.shape[1] if sc else 0), _ptr(sc.token_req if sc else None),
+                _ptr(sc.positions if sc else None), _c_int(sc.q_width if sc else 0),
+                _c_int(sc.kv_width if sc else 0), _c_int(sc.kv.head_dim if sc else 0),
+                _c_int(sc.kv.page_size if sc else 0), _stream(),
+            )
+            build.check(lib, rc, "linear")
+            return out
+
+    if lazy:
+        a = lazy.materialize()
+    lda = _rows2d(a, "a")
+    if w.dtype == torch.float32:
         lib = build.load("gemm_f32")
         fn = lib.gemm_f32
     else:
-        if out.dtype == torch.float32:
-            flags |= GEMM_OUT_F32
-        else:
-            _need(out.dtype == torch.bfloat16, "linear: out must be float32 or bfloat16")
         lib = build.load("gemm_bf16")
         fn = lib.gemm_bf16
     rc = fn(
@@ -138,6 +207,10 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0):
         _c_int(lda), _c_int(ldw), _c_int(ldo), _c_int(flags), _c_int(variant), _stream(),
     )
     build.check(lib, rc, "linear")
+    if scatter is not None:
+        q, kw = scatter.q_width, scatter.kv_width
+        kv_write(out[:, q : q + kw], out[:, q + kw :], scatter.kv, scatter.block_table,
+                 scatter.token_req, scatter.positions)
     return out
 
 
@@ -240,6 +313,39 @@ def attn_row(out, q, kv, block_table, token_req, positions, rows, n_rows, n_head
         _stream(),
     )
     build.check(lib, rc, "attn_row")
+    return out
+
+
+def attn_decode_takes(q_dtype, kv):
+    """Whether the register-streaming decode kernel takes this cache geometry."""
+    return (q_dtype == torch.bfloat16 and kv.head_dim in (32, 64, 128)
+            and kv.page_size % (512 // kv.head_dim) == 0)
+
+
+def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_heads, scale,
+                window=0, n_splits=1, part_o=None, part_ml=None):
+    """``attn_row`` for bfloat16 caches with head_dim 32, 64 or 128: keys stream into registers."""
+    lib = build.load("attention_decode")
+    ldq, ldo = _rows2d(q, "q"), _rows2d(out, "out")
+    _need(q.dtype == torch.bfloat16, "attn_decode: bfloat16 only")
+    _need(q.shape[1] == n_heads * kv.head_dim, "attn_decode: q width must be n_heads*head_dim")
+    _need(out.shape[1] == n_heads * kv.head_dim and out.dtype == q.dtype, "attn_decode: out shape/dtype")
+    _attn_common(q, kv, block_table, token_req, positions)
+    _dev(rows, "rows", torch.int32)
+    _need(rows.numel() >= n_rows, "attn_decode: row list too short")
+    if n_splits > 1:
+        _dev(part_o, "part_o", torch.float32)
+        _dev(part_ml, "part_ml", torch.float32)
+        _need(part_o.numel() >= n_rows * n_heads * n_splits * kv.head_dim, "attn_decode: part_o too small")
+        _need(part_ml.numel() >= n_rows * n_heads * n_splits * 2, "attn_decode: part_ml too small")
+    rc = lib.attn_decode(
+        _ptr(out), _ptr(q), _c_int(ldq), _c_int(ldo), _ptr(kv.k), _ptr(kv.v),
+        _c_size_t(kv.page_stride), _ptr(block_table), _c_int(block_table.shape[1]),
+        _ptr(token_req), _ptr(positions), _ptr(rows), _c_int(n_rows), _c_int(n_heads),
+        _c_int(kv.n_kv_heads), _c_int(kv.head_dim), _c_int(kv.page_size), _c_int(window),
+        _c_float(scale), _c_int(n_splits), _ptr(part_o), _ptr(part_ml), _stream(),
+    )
+    build.check(lib, rc, "attn_decode")
     return out
 
 

@@ -43,6 +43,7 @@ class CausalSelfAttention(Mixer):
             build_part(POSITION_ENCODINGS, "position encoding", position) if position is not None else None
         )
         self.qkv_w = self.qkv_b = self.out_w = self.out_b = None
+        self.accepts_lazy_input = True  # the fused projection can norm its input itself
         # launches kernels only (a step of such parts can be recorded), unless the position hook does more
         self.graph_safe = self.position is None or getattr(self.position, "graph_safe", False)
 
@@ -75,14 +76,19 @@ class CausalSelfAttention(Mixer):
     def forward(self, ctx, x, residual, cache, writes_cache=True):
         T = x.shape[0]
         qkv = ctx.scratch((T, self.q_width + 2 * self.kv_width), ctx.dtype)
-        kernels.linear(qkv, x, self.qkv_w, self.qkv_b)
         q = qkv[:, : self.q_width]
-        k = qkv[:, self.q_width : self.q_width + self.kv_width]
-        v = qkv[:, self.q_width + self.kv_width :]
-        if self.position is not None:
+        if self.position is None:
+            # keys and values go to their pages from the projection's epilogue
+            scatter = kernels.KVScatter(cache.kv, cache.block_table, ctx.token_req, ctx.positions,
+                                        self.q_width) if writes_cache else None
+            kernels.linear(qkv, x, self.qkv_w, self.qkv_b, scatter=scatter)
+        else:
+            kernels.linear(qkv, x, self.qkv_w, self.qkv_b)
+            k = qkv[:, self.q_width : self.q_width + self.kv_width]
+            v = qkv[:, self.q_width + self.kv_width :]
             self.position.rotate(ctx, q, k)
-        if writes_cache:
-            kernels.kv_write(k, v, cache.kv, cache.block_table, ctx.token_req, ctx.positions)
+            if writes_cache:
+                kernels.kv_write(k, v, cache.kv, cache.block_table, ctx.token_req, ctx.positions)
         out = ctx.scratch((T, self.q_width), ctx.dtype)
         self.attend(ctx, out, q, cache)
         kernels.linear(residual, out, self.out_w, self.out_b, accumulate=True)
@@ -104,8 +110,9 @@ class CausalSelfAttention(Mixer):
                 n = plan.n_rows * self.n_heads * n_splits
                 part_o = ctx.scratch((n * self.head_dim,), "float32")
                 part_ml = ctx.scratch((n * 2,), "float32")
-            kernels.attn_row(out, q, *args, plan.rows, plan.n_rows, self.n_heads, self.scale,
-                             self.window, n_splits, part_o, part_ml)
+            row_kernel = kernels.attn_decode if kernels.attn_decode_takes(q.dtype, cache.kv) else kernels.attn_row
+            row_kernel(out, q, *args, plan.rows, plan.n_rows, self.n_heads, self.scale,
+                       self.window, n_splits, part_o, part_ml)
 
 
 register_mixer("attention", CausalSelfAttention)

@@ -4,7 +4,9 @@ A part takes its sizes and constants as constructor parameters, declares the
 tensors it wants by name, and runs on a ``StepContext``.  It does not know
 which model it is in.  Five kinds of part exist:
 
-* ``Norm``             ``forward(ctx, x, rows=None, n_rows=None) -> y``
+* ``Norm``             ``forward(ctx, x, rows=None, n_rows=None, lazy=False) -> y``;
+                       with ``lazy`` it may return a ``NormedInput`` for a
+                       consumer that set ``accepts_lazy_input``
 * ``Mixer``            ``forward(ctx, x, residual, cache, writes_cache)`` adds
                        its output into ``residual``; ``cache_need()`` says
                        what cache slot it wants
@@ -54,7 +56,7 @@ class Part:
 
 
 class Norm(Part):
-    def forward(self, ctx, x, rows=None, n_rows=None):
+    def forward(self, ctx, x, rows=None, n_rows=None, lazy=False):
         raise NotImplementedError
 
 

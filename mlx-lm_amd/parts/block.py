@@ -19,8 +19,10 @@ class PreNormBlock(Block):
 
     def forward(self, ctx, h, cache, writes_cache=True):
         mark = ctx.scratch_mark()
-        self.mixer.forward(ctx, self.mixer_norm.forward(ctx, h), h, cache, writes_cache)
-        self.ffn.forward(ctx, self.ffn_norm.forward(ctx, h), h)
+        lazy = getattr(self.mixer, "accepts_lazy_input", False)
+        self.mixer.forward(ctx, self.mixer_norm.forward(ctx, h, lazy=lazy), h, cache, writes_cache)
+        lazy = getattr(self.ffn, "accepts_lazy_input", False)
+        self.ffn.forward(ctx, self.ffn_norm.forward(ctx, h, lazy=lazy), h)
         ctx.scratch_release(mark)
         return h
 

@@ -14,6 +14,7 @@ class GeluMLP(FeedForward):
     """
 
     graph_safe = True  # launches kernels only: a step of such parts can be recorded
+    accepts_lazy_input = True  # the first product can norm its input itself
 
     def __init__(self, width, inner, activation="gelu_new", prefix=""):
         super().__init__(prefix)

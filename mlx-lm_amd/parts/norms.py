@@ -29,7 +29,10 @@ class LayerNorm(Norm):
         self.weight = tensors[self._name("weight")]
         self.bias = tensors[self._name("bias")] if self.has_bias else None
 
-    def forward(self, ctx, x, rows=None, n_rows=None):
+    def forward(self, ctx, x, rows=None, n_rows=None, lazy=False):
+        if lazy and rows is None:
+            # the consumer's first matrix product may norm the rows itself
+            return kernels.NormedInput(ctx.scratch, x, self.weight, self.bias, self.eps, ctx.dtype)
         n = x.shape[0] if n_rows is None else n_rows
         out = ctx.scratch((n, self.width), ctx.dtype)
         kernels.layernorm(out, x, self.weight, self.bias, self.eps, rows=rows)

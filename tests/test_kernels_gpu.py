@@ -277,6 +277,48 @@ def test_attn_row(dtype, case, n_splits):
     assert err < _attn_tol(dtype), err
 
 
+@pytest.mark.parametrize("case", [c for c in ATTN_CASES if c[2] in (32, 64, 128)] + [
+    (8, 2, 32, 16, [700, 15, 16], [1, 1, 3], 0),
+    (4, 4, 128, 16, [63, 64, 1000], [1, 2, 1], 100),
+])
+@pytest.mark.parametrize("n_splits", [1, 3, 8])
+def test_attn_decode(case, n_splits):
+    k = _k()
+    H, Hkv, hd, ps, ctx, ql, window = case
+    c = PagedCase(torch.bfloat16, H, Hkv, hd, ps, ctx, ql, seed=hd + H + 2, window=window)
+    assert k.attn_decode_takes(torch.bfloat16, c.kv)
+    k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
+    rows = torch.arange(c.T, dtype=torch.int32, device=DEV)
+    part_o = torch.empty(c.T * H * n_splits * hd, dtype=torch.float32, device=DEV)
+    part_ml = torch.empty(c.T * H * n_splits * 2, dtype=torch.float32, device=DEV)
+    out = torch.full((c.T, H * hd), float("nan")).to(torch.bfloat16).to(DEV)
+    k.attn_decode(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, c.T, H,
+                  c.scale, window, n_splits, part_o, part_ml)
+    err = (out.double().cpu() - c.reference()).abs().max().item()
+    assert err < _attn_tol(torch.bfloat16), err
+
+
+def test_attn_decode_far_key_stands_out():
+    """bfloat16, keys streamed into registers: one key among hundreds carries the answer."""
+    k = _k()
+    H, hd, ps = 2, 64, 16
+    for far in (0, 7, 8, 15, 16, 63, 64, 255, 256, 399, 400):
+        c = PagedCase(torch.bfloat16, H, H, hd, ps, [401], [1], seed=far)
+        kf = c.k_full[0][far, 1].float()
+        c.q[0, hd:] = (kf * (30.0 / (c.scale * float(kf.norm() ** 2)))).to(torch.bfloat16)
+        k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
+        rows = torch.zeros(1, dtype=torch.int32, device=DEV)
+        for n_splits in (1, 4):
+            out = torch.empty(1, H * hd, dtype=torch.bfloat16, device=DEV)
+            po = torch.empty(H * n_splits * hd, dtype=torch.float32, device=DEV)
+            pm = torch.empty(H * n_splits * 2, dtype=torch.float32, device=DEV)
+            k.attn_decode(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, 1,
+                          H, c.scale, 0, n_splits, po, pm)
+            v_far = c.v_full[0][far, 1].double()
+            assert (out[0, hd:].double().cpu() - v_far).abs().max().item() < 0.1, (far, n_splits)
+            assert (out.double().cpu() - c.reference()).abs().max().item() < _attn_tol(torch.bfloat16)
+
+
 def test_attn_far_key_stands_out():
     """One key among hundreds carries the answer: a dropped tile or page shows."""
     k = _k()
@@ -466,3 +508,80 @@ def test_logit_bias_and_penalties():
         if freq[r]:
             want = plain.frequency_penalty(want, hist_rows[r], freq[r], freq_ctx[r])
         assert torch.allclose(x[r].double().cpu(), want, atol=1e-5), r
+
+
+# ---------------------------------------------------------------------------
+# the decode projection: norm fused in front, cache scatter fused behind
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 48, 64), (7, 1000, 96), (16, 80, 200), (8, 4800, 1600),
+                                   (9, 1600, 6400), (13, 333, 1608), (16, 257, 3200)])
+@pytest.mark.parametrize("mode", ["plain", "gelu", "accumulate", "f32out"])
+@pytest.mark.parametrize("normed", [False, True])
+def test_gemm_bf16_decode(M, N, K, mode, normed):
+    k = _k()
+    from mlx_lm_amd.ops import build
+
+    lib = build.load("gemm_bf16_decode")
+    if not lib.gemm_bf16_decode_takes(M, K, int(normed)):
+        assert K > 4096 and normed  # the only sizes of this list it leaves to the general kernels
+    w = _rand((N, K), torch.bfloat16, 11, 0.1)
+    bias = _rand((N,), torch.float32, 12)
+    if normed:
+        x = _rand((M, K), torch.float32, 10, 2.0) + 0.3
+        gamma, beta = 1 + _rand((K,), torch.float32, 14, 0.1), _rand((K,), torch.float32, 15, 0.1)
+        a = k.NormedInput(lambda shape, dtype: torch.empty(shape, dtype=dtype, device=DEV), x, gamma, beta,
+                          1e-5, torch.bfloat16)
+        a_ref = plain.layer_norm(x.double().cpu(), gamma.double().cpu(), beta.double().cpu(), 1e-5)
+        a_ref = a_ref.to(torch.bfloat16).double()  # the kernel rounds the normed rows to bfloat16 too
+    else:
+        a = _rand((M, K), torch.bfloat16, 10)
+        a_ref = a.double().cpu()
+    ref = plain.linear(a_ref, w.double().cpu(), bias.double().cpu())
+    slack = 3e-2 * math.sqrt(K) * 0.1 if normed else 0.0  # a normed value may round the other way
+    if mode == "accumulate":
+        out = _rand((M, N), torch.float32, 13)
+        want = out.double().cpu() + ref
+        k.linear(out, a, w, bias, accumulate=True)
+        tol = 1e-4 * math.sqrt(K) + slack
+    elif mode == "f32out":
+        out = torch.empty(M, N, dtype=torch.float32, device=DEV)
+        k.linear(out, a, w, bias)
+        want, tol = ref, 1e-4 * math.sqrt(K) + slack
+    else:
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        k.linear(out, a, w, bias, gelu=(mode == "gelu"))
+        want = plain.gelu_tanh(ref) if mode == "gelu" else ref
+        tol = None
+    got = out.double().cpu()
+    if tol is None:
+        assert torch.allclose(got, want, rtol=2**-7, atol=1e-3 + slack), (got - want).abs().max()
+    else:
+        assert (got - want).abs().max().item() < tol, (got - want).abs().max()
+
+
+@pytest.mark.parametrize("M", [1, 5, 16, 40])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_projection_scatters_keys_and_values(M, dtype):
+    """Fused (decode kernel) and composed (general kernels) give the same pages and queries."""
+    k = _k()
+    H, Hkv, hd, ps, D = 6, 2, 32, 16, 96
+    c = PagedCase(dtype, H, Hkv, hd, ps, [30] * M, [1] * M, seed=M)
+    qw, kw = H * hd, Hkv * hd
+    w = _rand((qw + 2 * kw, D), dtype, 3, 0.2)
+    bias = _rand((qw + 2 * kw,), torch.float32, 4, 0.1)
+    a = _rand((M, D), dtype, 5)
+    ref = plain.linear(a.double().cpu(), w.double().cpu(), bias.double().cpu())
+    out = torch.full((M, qw + 2 * kw), float("nan")).to(dtype).to(DEV)
+    sc = k.KVScatter(c.kv, c.block_table_dev, c.token_req, c.positions, qw)
+    k.linear(out, a, w, bias, scatter=sc)
+    torch.cuda.synchronize()
+    tol = dict(rtol=2**-7, atol=1e-3) if dtype == torch.bfloat16 else dict(rtol=1e-5, atol=1e-5)
+    assert torch.allclose(out[:, :qw].double().cpu(), ref[:, :qw], **tol)
+    pool = c.pool.cpu()
+    for m in range(M):
+        page, row = c.block_table[m, 30 // ps], 30 % ps
+        assert torch.allclose(pool[page, 0, :, row].reshape(-1).double(), ref[m, qw : qw + kw], **tol)
+        assert torch.allclose(pool[page, 1, :, row].reshape(-1).double(), ref[m, qw + kw :], **tol)
+        # and nothing else in the page was touched
+        assert torch.isnan(pool[page, 0, :, row + 1 :].float()).all()
