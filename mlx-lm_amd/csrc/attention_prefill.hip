@@ -1,0 +1,292 @@
+// Prefill attention for bfloat16 caches on the matrix cores: portions of
+// prompts, 128 consecutive queries of one request per block, keys and values
+// read from the pages in tiles of 64.  Same contract as attn_tile in
+// attention.hip (same tile list, with up to 128 rows a tile); this is the
+// kernel that serving uses for head sizes 32, 64 and 128, attn_tile stays as
+// the general one (any head size, float caches).
+//
+// Replaces scaled_dot_product_attention with the "causal" mask and a cache
+// offset (mlx_lm/models/base.py:24-35,132-139, mlx_lm/models/gpt2.py:60-65).
+//
+// Data flow, chosen so that a lane only ever deals with one query:
+//  * Each of the four waves owns 32 queries.  Scores are computed transposed,
+//    S^T = K Q^T, with v_mfma_f32_32x32x16_bf16: keys are the rows (A-operand,
+//    from LDS), the wave's queries the columns (B-operand, kept in registers).
+//    A lane then holds 16 scores of query (lane % 32) per 32-key subtile, so
+//    the row maximum and sum need a single cross-lane step.
+//  * The rows of a subtile are fed in a permuted key order such that the 8
+//    scores a lane holds per 16-key chunk are 8 *consecutive* keys.  They are
+//    exactly the B-operand fragment of O^T = V^T P^T; no shuffle, no LDS.
+//  * V^T is needed with keys contiguous.  Values sit in the pages with head
+//    columns contiguous, so the value tile is transposed on its way into LDS:
+//    a thread reads the same 8 columns of two neighbouring keys and writes
+//    eight 32-bit words (two keys each).
+//  * Online softmax in 32-bit per lane; outputs leave as O^T accumulators.
+#include "common.h"
+
+struct PrefillArgs {
+  uint16_t* out;
+  const uint16_t* q;
+  const uint16_t* k_pages;
+  const uint16_t* v_pages;
+  const int* block_table;
+  const int* token_req;
+  const int* positions;
+  const int* tiles;  // (first row, n rows <= 128) pairs
+  size_t page_stride;
+  int ldq, ldo, max_blocks;
+  int n_heads, n_kv_heads, page_size, window;
+  float scale;
+};
+
+#define BQ 128  // queries per block
+#define KT 64   // keys per tile
+#define VT_STRIDE (KT + 8)  // 144 bytes a row: 16-byte reads of 32 rows fall on distinct banks
+
+union Frag8 {
+  uint4 u;
+  bf16x8_t v;
+};
+
+// S^T row rho of a 32-key subtile holds this key of the subtile (see above)
+__device__ __forceinline__ int key_of_row(int rho) {
+  const int j = rho >> 3, g = (rho >> 2) & 1, i = rho & 3;
+  return 16 * (j >> 1) + 8 * g + 4 * (j & 1) + i;
+}
+
+template <int HD>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(PrefillArgs p) {
+  constexpr int KS_STRIDE = HD + 8;
+  constexpr int DC = HD / 16;           // 16-column chunks of a head (QK contraction steps)
+  constexpr int DT = HD / 32;           // 32-row tiles of O^T
+  constexpr int K_CHUNKS = KT * HD / 8; // 16-byte pieces of a key tile
+  constexpr int K_PER_T = (K_CHUNKS + 255) / 256;
+  constexpr int V_ITEMS = (KT / 2) * (HD / 8);  // (key pair, 8-column chunk) items of a value tile
+  constexpr int V_PER_T = (V_ITEMS + 255) / 256;
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[KT * KS_STRIDE];
+  __shared__ __attribute__((aligned(16))) uint16_t Vt[HD * VT_STRIDE];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int row0 = p.tiles[2 * blockIdx.x];
+  const int nq = p.tiles[2 * blockIdx.x + 1];
+  const int h = blockIdx.y;
+  const int kv_head = h / (p.n_heads / p.n_kv_heads);
+  const int pos0 = p.positions[row0];
+  const int* table = p.block_table + (size_t)p.token_req[row0] * p.max_blocks;
+  const size_t head_off = (size_t)kv_head * p.page_size * HD;
+
+  const int ql = lane & 31, g = lane >> 5;
+  const int qi = wave * 32 + ql;         // this lane's query within the tile
+  const bool q_live = qi < nq;
+  const int qpos = pos0 + qi;
+  const int q_lo = p.window > 0 ? max(0, qpos - p.window + 1) : 0;
+
+  // the wave's queries as B-operand fragments: column = query, k = head columns
+  Frag8 qf[DC];
+  {
+    const uint16_t* qrow = p.q + (size_t)(row0 + min(qi, nq - 1)) * p.ldq + h * HD + 8 * g;
+#pragma unroll
+    for (int dc = 0; dc < DC; ++dc) {
+      const uint4 t = *(const uint4*)(qrow + dc * 16);
+      qf[dc].u = q_live ? t : make_uint4(0u, 0u, 0u, 0u);
+    }
+  }
+
+  const int k_hi = pos0 + nq;  // one past the last key any query of the tile sees
+  const int k_lo = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
+  const int kt0 = (k_lo / KT) * KT;
+  // keys this wave's queries can see end here; later tiles it only helps to load
+  const int wave_hi = min(k_hi, pos0 + wave * 32 + 32);
+
+  float m = -INFINITY, l = 0.f;
+  f32x16_t ot[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) ot[dt][r] = 0.f;
+
+  uint4 kreg[K_PER_T], vreg[V_PER_T][2];
+
+  auto address = [&](int key, int col) -> size_t {
+    const int kk = min(max(key, k_lo), k_hi - 1);  // pulled into range; zeroed by the caller
+    const int page = table[kk / p.page_size];
+    return (size_t)page * p.page_stride + head_off + (size_t)(kk % p.page_size) * HD + col;
+  };
+  auto fetch = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < K_PER_T; ++i) {
+      const int c = min(tid + 256 * i, K_CHUNKS - 1);  // surplus threads repeat the last piece
+      const int key = kt + c / (HD / 8), col = (c % (HD / 8)) * 8;
+      const uint4 t = *(const uint4*)(p.k_pages + address(key, col));
+      kreg[i] = (key >= k_lo && key < k_hi) ? t : make_uint4(0u, 0u, 0u, 0u);
+    }
+#pragma unroll
+    for (int i = 0; i < V_PER_T; ++i) {
+      const int it = min(tid + 256 * i, V_ITEMS - 1);
+      const int jp = it % (KT / 2), col = (it / (KT / 2)) * 8;
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int key = kt + 2 * jp + e;
+        const uint4 t = *(const uint4*)(p.v_pages + address(key, col));
+        vreg[i][e] = (key >= k_lo && key < k_hi) ? t : make_uint4(0u, 0u, 0u, 0u);
+      }
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int i = 0; i < K_PER_T; ++i) {
+      const int c = tid + 256 * i;
+      if (K_CHUNKS % 256 == 0 || c < K_CHUNKS)
+        *(uint4*)(Ks + (c / (HD / 8)) * KS_STRIDE + (c % (HD / 8)) * 8) = kreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < V_PER_T; ++i) {
+      const int it = tid + 256 * i;
+      if (V_ITEMS % 256 != 0 && it >= V_ITEMS) continue;
+      const int jp = it % (KT / 2), col = (it / (KT / 2)) * 8;
+      const uint32_t a[4] = {vreg[i][0].x, vreg[i][0].y, vreg[i][0].z, vreg[i][0].w};
+      const uint32_t b[4] = {vreg[i][1].x, vreg[i][1].y, vreg[i][1].z, vreg[i][1].w};
+      uint32_t* dst = (uint32_t*)(Vt + col * VT_STRIDE + 2 * jp);
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        // columns col+2w and col+2w+1 of keys 2jp (low half) and 2jp+1 (high half)
+        dst[(2 * w) * (VT_STRIDE / 2)] = (a[w] & 0xffffu) | (b[w] << 16);
+        dst[(2 * w + 1) * (VT_STRIDE / 2)] = (a[w] >> 16) | (b[w] & 0xffff0000u);
+      }
+    }
+  };
+
+  fetch(kt0);
+  for (int kt = kt0; kt < k_hi; kt += KT) {
+    __syncthreads();  // the previous tile is no longer read
+    stage();
+    __syncthreads();
+    if (kt + KT < k_hi) fetch(kt + KT);  // in flight during the arithmetic below
+    if (kt >= wave_hi || wave * 32 >= nq) continue;  // nothing here for this wave (uniform)
+
+    // ---- S^T = K Q^T for the two 32-key subtiles --------------------------------
+    f32x16_t st[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) st[s][r] = 0.f;
+      const uint16_t* krow = Ks + (32 * s + key_of_row(ql)) * KS_STRIDE + 8 * g;
+#pragma unroll
+      for (int dc = 0; dc < DC; ++dc) {
+        Frag8 a;
+        a.u = *(const uint4*)(krow + dc * 16);
+        st[s] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, qf[dc].v, st[s], 0, 0, 0);
+      }
+    }
+    // element r of subtile s: key kt + 32 s + 16 (r / 8) + 8 g + r % 8
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = kt + 32 * s + 16 * (r >> 3) + 8 * g + (r & 7);
+        const bool ok = q_live && key <= qpos && key >= q_lo;
+        st[s][r] = ok ? st[s][r] * p.scale : -INFINITY;
+        tmax = fmaxf(tmax, st[s][r]);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+    const float m_new = fmaxf(m, tmax);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a row with no key yet
+    const float alpha = __expf(m - m_use);
+    float lsum = 0.f;
+    Frag8 pf[2][2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        float e[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          e[i] = __expf(st[s][8 * c + i] - m_use);
+          lsum += e[i];
+        }
+        pf[s][c].u.x = (uint32_t)f32_to_bf16_bits(e[0]) | ((uint32_t)f32_to_bf16_bits(e[1]) << 16);
+        pf[s][c].u.y = (uint32_t)f32_to_bf16_bits(e[2]) | ((uint32_t)f32_to_bf16_bits(e[3]) << 16);
+        pf[s][c].u.z = (uint32_t)f32_to_bf16_bits(e[4]) | ((uint32_t)f32_to_bf16_bits(e[5]) << 16);
+        pf[s][c].u.w = (uint32_t)f32_to_bf16_bits(e[6]) | ((uint32_t)f32_to_bf16_bits(e[7]) << 16);
+      }
+    l = l * alpha + lsum;
+    m = m_new;
+    // ---- O^T = O^T * alpha + V^T P^T ---------------------------------------------
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) ot[dt][r] *= alpha;
+      const uint16_t* vrow = Vt + (dt * 32 + ql) * VT_STRIDE + 8 * g;
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          Frag8 a;
+          a.u = *(const uint4*)(vrow + 32 * s + 16 * c);
+          ot[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pf[s][c].v, ot[dt], 0, 0, 0);
+        }
+    }
+  }
+
+  // the two halves of the wave hold different keys of the same query
+  l += __shfl_xor(l, 32, WAVE);
+  if (q_live) {
+    const float inv = 1.0f / l;
+    uint16_t* orow = p.out + (size_t)(row0 + qi) * p.ldo + h * HD;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        // accumulators 4j .. 4j+3: head columns dt*32 + 8j + 4g + (0..3)
+        uint2 o;
+        o.x = (uint32_t)f32_to_bf16_bits(ot[dt][4 * j] * inv) |
+              ((uint32_t)f32_to_bf16_bits(ot[dt][4 * j + 1] * inv) << 16);
+        o.y = (uint32_t)f32_to_bf16_bits(ot[dt][4 * j + 2] * inv) |
+              ((uint32_t)f32_to_bf16_bits(ot[dt][4 * j + 3] * inv) << 16);
+        *(uint2*)(orow + dt * 32 + 8 * j + 4 * g) = o;
+      }
+  }
+}
+
+DEFINE_LAST_ERROR(mlxlm_last_error)
+
+// tiles: n_tiles pairs (first flat row, number of rows 1..128); the rows of a
+// tile are consecutive tokens of one request at consecutive positions.
+// bfloat16 only, head_dim 32, 64 or 128.
+extern "C" int attn_prefill(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                            const void* v_pages, size_t page_stride, const int* block_table,
+                            int max_blocks, const int* token_req, const int* positions,
+                            const int* tiles, int n_tiles, int n_heads, int n_kv_heads,
+                            int head_dim, int page_size, int window, float scale,
+                            hipStream_t stream) {
+  if (n_tiles <= 0) return 0;
+  if (head_dim != 32 && head_dim != 64 && head_dim != 128)
+    FAIL("attn_prefill: head_dim %d is not 32, 64 or 128 (attn_tile takes the others)", head_dim);
+  if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads != 0)
+    FAIL("attn_prefill: %d query heads cannot be grouped over %d key heads", n_heads, n_kv_heads);
+  if (page_size <= 0) FAIL("attn_prefill: page_size %d must be positive", page_size);
+  if (!out || !q || !k_pages || !v_pages || !block_table || !token_req || !positions || !tiles)
+    FAIL("attn_prefill: null pointer");
+  if (ldq % 8 != 0 || ((uintptr_t)q & 15)) FAIL("attn_prefill: query rows must be 16-byte aligned");
+  if (ldo % 4 != 0 || ((uintptr_t)out & 7)) FAIL("attn_prefill: output rows must be 8-byte aligned");
+  if (page_stride % 8 != 0 || (((uintptr_t)k_pages | (uintptr_t)v_pages) & 15))
+    FAIL("attn_prefill: pages must be 16-byte aligned");
+  if (window < 0) FAIL("attn_prefill: window %d must not be negative", window);
+  PrefillArgs p;
+  p.out = (uint16_t*)out, p.q = (const uint16_t*)q;
+  p.k_pages = (const uint16_t*)k_pages, p.v_pages = (const uint16_t*)v_pages;
+  p.block_table = block_table, p.token_req = token_req, p.positions = positions, p.tiles = tiles;
+  p.page_stride = page_stride, p.ldq = ldq, p.ldo = ldo, p.max_blocks = max_blocks;
+  p.n_heads = n_heads, p.n_kv_heads = n_kv_heads, p.page_size = page_size, p.window = window;
+  p.scale = scale;
+  dim3 grid(n_tiles, n_heads), block(256);
+  if (head_dim == 32)
+    hipLaunchKernelGGL(attn_prefill_kernel<32>, grid, block, 0, stream, p);
+  else if (head_dim == 64)
+    hipLaunchKernelGGL(attn_prefill_kernel<64>, grid, block, 0, stream, p);
+  else
+    hipLaunchKernelGGL(attn_prefill_kernel<128>, grid, block, 0, stream, p);
+  CHECK_LAUNCH("attn_prefill");
+  return 0;
+}

@@ -65,9 +65,12 @@ union Frag {
   bf16x8_t v;
 };
 
-// LV: float4 per lane that a normed row takes (8: K <= 2048, 16: K <= 4096); 0: no norm
-template <int LV>
-__global__ __launch_bounds__(NW * 64, (LV <= 8 ? 2 : 1)) void gemm_bf16_decode_kernel(DecodeGemmArgs p) {
+// LV: float4 per lane that a normed row takes (8: K <= 2048, 16: K <= 4096); 0: no norm.
+// MULTI: K is longer than one pass of NW * U k-blocks (2048); only then is the
+// second set of weight registers needed.
+template <int LV, bool MULTI>
+// (the second bound is waves per SIMD: four keeps two blocks on a CU, except for the long norm)
+__global__ __launch_bounds__(NW * 64, (LV > 8 ? 2 : 4)) void gemm_bf16_decode_kernel(DecodeGemmArgs p) {
   constexpr bool LN = LV > 0;
   constexpr int NV = LN ? LV : 1;
   extern __shared__ __attribute__((aligned(16))) uint16_t As[];  // [M][a_stride]
@@ -98,7 +101,7 @@ __global__ __launch_bounds__(NW * 64, (LV <= 8 ? 2 : 1)) void gemm_bf16_decode_k
     }
   };
 
-  Frag w0[U][2], w1[U][2];
+  Frag w0[U][2], w1[MULTI ? U : 1][2];
   load_pass(w0, 0);  // in flight while the activations are prepared
 
   // ---- activations into LDS ------------------------------------------------
@@ -169,12 +172,16 @@ __global__ __launch_bounds__(NW * 64, (LV <= 8 ? 2 : 1)) void gemm_bf16_decode_k
     }
   };
 
-  const int n_pass = (n_chunks + NW * U - 1) / (NW * U);
-  for (int pass = 0; pass < n_pass; pass += 2) {
-    load_pass(w1, pass + 1);
-    compute_pass(w0, pass);
-    load_pass(w0, pass + 2);
-    compute_pass(w1, pass + 1);
+  if constexpr (MULTI) {
+    const int n_pass = (n_chunks + NW * U - 1) / (NW * U);
+    for (int pass = 0; pass < n_pass; pass += 2) {
+      load_pass(w1, pass + 1);
+      compute_pass(w0, pass);
+      load_pass(w0, pass + 2);
+      compute_pass(w1, pass + 1);
+    }
+  } else {
+    compute_pass(w0, 0);
   }
 
   // ---- sum the waves' tiles in a fixed order, then the epilogue ---------------
@@ -271,10 +278,12 @@ extern "C" int gemm_bf16_decode(
   p.max_blocks = max_blocks, p.q_width = q_width, p.kv_width = kv_width;
   p.head_dim = head_dim, p.page_size = page_size;
   const size_t lds = (size_t)M * p.a_stride * 2;
-  const int which = !ln ? 0 : (K <= 2048 ? 1 : 2);
-  void (*kernels[3])(DecodeGemmArgs) = {gemm_bf16_decode_kernel<0>, gemm_bf16_decode_kernel<8>,
-                                        gemm_bf16_decode_kernel<LN_MAX_V>};
-  static size_t granted[3] = {0, 0, 0};
+  const bool multi = K > NW * U * 64;
+  const int which = (!ln ? 0 : 2) + (multi ? 1 : 0);
+  void (*kernels[4])(DecodeGemmArgs) = {
+      gemm_bf16_decode_kernel<0, false>, gemm_bf16_decode_kernel<0, true>,
+      gemm_bf16_decode_kernel<8, false>, gemm_bf16_decode_kernel<LN_MAX_V, true>};
+  static size_t granted[4] = {0, 0, 0, 0};
   if (lds + sizeof(float) * NW * 256 > 64 * 1024 && granted[which] < lds) {
     hipError_t e = hipFuncSetAttribute((const void*)kernels[which],
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

@@ -5,7 +5,8 @@ import torch
 _TORCH_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
 
 ROW_KERNEL_MAX_Q = 4  # requests with at most this many tokens in a step take the row kernel
-TILE_Q = 16  # queries per tile of the tile kernel
+TILE_Q = 16  # queries per tile of the general tile kernel
+BIG_TILE_Q = 128  # queries per tile of the matrix-core prefill kernel
 
 
 class Scratch:
@@ -64,13 +65,15 @@ class AttentionPlan:
 
     Requests that bring at most ``ROW_KERNEL_MAX_Q`` tokens are handled row by
     row (keys split over blocks); longer portions in tiles of ``TILE_Q``
-    consecutive queries.  ``all_tiles`` covers every row with tiles, for
-    mixers whose head size the row kernel does not take.
+    consecutive queries (``big_tiles``: the same portions in tiles of
+    ``BIG_TILE_Q``, longest context first, for the matrix-core kernel).
+    ``all_tiles`` covers every row with tiles, for mixers whose head size the
+    row kernel does not take.
     """
 
     def __init__(self):
-        self.tiles = self.rows = self.all_tiles = None
-        self.n_tiles = self.n_rows = self.n_all_tiles = 0
+        self.tiles = self.rows = self.all_tiles = self.big_tiles = None
+        self.n_tiles = self.n_rows = self.n_all_tiles = self.n_big_tiles = 0
         self.max_row_context = 0
         self.n_compute_units = 256
 

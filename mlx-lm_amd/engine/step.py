@@ -7,7 +7,7 @@ import torch
 
 from ..cache import CacheManager
 from ..weights.loader import resolve_dtype
-from .context import ROW_KERNEL_MAX_Q, TILE_Q, AttentionPlan, Scratch, StepContext
+from .context import BIG_TILE_Q, ROW_KERNEL_MAX_Q, TILE_Q, AttentionPlan, Scratch, StepContext
 
 
 @dataclass
@@ -174,7 +174,7 @@ class Engine:
         ctx = StepContext(self)
         q_start = 0
         token_ids, positions, token_req, wanted, slot_ids = [], [], [], [], []
-        tiles, rows, all_tiles = [], [], []
+        tiles, rows, all_tiles, big = [], [], [], []
         plan = AttentionPlan()
         for r, e in enumerate(entries):
             rc = cm.requests[e.request_id]
@@ -196,8 +196,13 @@ class Engine:
             else:
                 for s in range(0, n, TILE_Q):
                     tiles.extend((q_start + s, min(TILE_Q, n - s)))
+                for s in range(0, n, BIG_TILE_Q):
+                    big.append((rc.length + s + min(BIG_TILE_Q, n - s), q_start + s, min(BIG_TILE_Q, n - s)))
             q_start += n
         plan.n_tiles, plan.n_rows, plan.n_all_tiles = len(tiles) // 2, len(rows), len(all_tiles) // 2
+        big.sort(reverse=True)  # tiles with the most keys start first
+        big_tiles = [v for _, r0, nr in big for v in (r0, nr)]
+        plan.n_big_tiles = len(big)
 
         # block tables, one per group, padded to the longest of the step
         tables = []
@@ -211,7 +216,7 @@ class Engine:
             tables.append((width, flat))
 
         # everything in one pinned buffer and one copy; pieces start on 4-int boundaries
-        pieces = [token_ids, positions, token_req, wanted, slot_ids, tiles, rows, all_tiles]
+        pieces = [token_ids, positions, token_req, wanted, slot_ids, tiles, rows, all_tiles, big_tiles]
         pieces += [flat for _, flat in tables]
         offsets, total = [], 0
         for p in pieces:
@@ -234,7 +239,8 @@ class Engine:
         ctx.token_ids, ctx.positions, ctx.token_req = piece(0, T), piece(1, T), piece(2, T)
         ctx.wanted_rows, ctx.slot_ids = piece(3, len(wanted)), piece(4, R)
         plan.tiles, plan.rows, plan.all_tiles = piece(5, len(tiles)), piece(6, len(rows)), piece(7, len(all_tiles))
+        plan.big_tiles = piece(8, len(big_tiles))
         ctx.attention_plan = plan
         for gi, (width, flat) in enumerate(tables):
-            ctx.block_tables.append(piece(8 + gi, len(flat)).view(R, width))
+            ctx.block_tables.append(piece(9 + gi, len(flat)).view(R, width))
         return ctx

@@ -316,6 +316,35 @@ def attn_row(out, q, kv, block_table, token_req, positions, rows, n_rows, n_head
     return out
 
 
+ATTN_PREFILL_TILE = 128  # queries per tile of attn_prefill
+
+
+def attn_prefill_takes(q_dtype, kv):
+    """Whether the matrix-core prefill kernel takes this cache geometry."""
+    return q_dtype == torch.bfloat16 and kv.head_dim in (32, 64, 128)
+
+
+def attn_prefill(out, q, kv, block_table, token_req, positions, tiles, n_tiles, n_heads, scale, window=0):
+    """``attn_tile`` on the matrix cores: bfloat16, head_dim 32/64/128, tiles of up to 128 queries."""
+    lib = build.load("attention_prefill")
+    ldq, ldo = _rows2d(q, "q"), _rows2d(out, "out")
+    _need(q.dtype == torch.bfloat16, "attn_prefill: bfloat16 only")
+    _need(q.shape[1] == n_heads * kv.head_dim, "attn_prefill: q width must be n_heads*head_dim")
+    _need(out.shape[1] == n_heads * kv.head_dim and out.dtype == q.dtype, "attn_prefill: out shape/dtype")
+    _attn_common(q, kv, block_table, token_req, positions)
+    _dev(tiles, "tiles", torch.int32)
+    _need(tiles.numel() >= 2 * n_tiles, "attn_prefill: tile list too short")
+    rc = lib.attn_prefill(
+        _ptr(out), _ptr(q), _c_int(ldq), _c_int(ldo), _ptr(kv.k), _ptr(kv.v),
+        _c_size_t(kv.page_stride), _ptr(block_table), _c_int(block_table.shape[1]),
+        _ptr(token_req), _ptr(positions), _ptr(tiles), _c_int(n_tiles), _c_int(n_heads),
+        _c_int(kv.n_kv_heads), _c_int(kv.head_dim), _c_int(kv.page_size), _c_int(window),
+        _c_float(scale), _stream(),
+    )
+    build.check(lib, rc, "attn_prefill")
+    return out
+
+
 def attn_decode_takes(q_dtype, kv):
     """Whether the register-streaming decode kernel takes this cache geometry."""
     return (q_dtype == torch.bfloat16 and kv.head_dim in (32, 64, 128)

@@ -101,8 +101,12 @@ class CausalSelfAttention(Mixer):
                               self.scale, self.window)
             return
         if plan.n_tiles:
-            kernels.attn_tile(out, q, *args, plan.tiles, plan.n_tiles, self.n_heads, self.scale,
-                              self.window)
+            if kernels.attn_prefill_takes(q.dtype, cache.kv):
+                kernels.attn_prefill(out, q, *args, plan.big_tiles, plan.n_big_tiles, self.n_heads,
+                                     self.scale, self.window)
+            else:
+                kernels.attn_tile(out, q, *args, plan.tiles, plan.n_tiles, self.n_heads, self.scale,
+                                  self.window)
         if plan.n_rows:
             n_splits = plan.row_splits(self.n_heads, self.window)
             part_o = part_ml = None

@@ -298,6 +298,51 @@ def test_attn_decode(case, n_splits):
     assert err < _attn_tol(torch.bfloat16), err
 
 
+PREFILL_CASES = [c for c in ATTN_CASES if c[2] in (32, 64, 128)] + [
+    (3, 3, 64, 16, [0, 100, 700], [300, 129, 5], 0),
+    (4, 2, 32, 16, [5, 0], [260, 64], 0),
+    (2, 1, 128, 32, [190, 0], [70, 200], 0),
+    (5, 5, 64, 16, [0, 400], [333, 128], 90),
+]
+
+
+@pytest.mark.parametrize("case", PREFILL_CASES)
+def test_attn_prefill(case):
+    k = _k()
+    H, Hkv, hd, ps, ctx, ql, window = case
+    c = PagedCase(torch.bfloat16, H, Hkv, hd, ps, ctx, ql, seed=hd + H + 3, window=window)
+    assert k.attn_prefill_takes(torch.bfloat16, c.kv)
+    k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
+    tiles = c.tiles(k.ATTN_PREFILL_TILE)
+    out = torch.full((c.T, H * hd), float("nan")).to(torch.bfloat16).to(DEV)
+    k.attn_prefill(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, tiles,
+                   tiles.shape[0], H, c.scale, window)
+    err = (out.double().cpu() - c.reference()).abs().max().item()
+    # the weights P are rounded to bfloat16 before they meet the values
+    assert err < 2.5e-2, err
+
+
+def test_attn_prefill_far_key_stands_out():
+    """Every query of a long portion points at one far key of its own."""
+    k = _k()
+    H, hd, ps, n = 2, 64, 16, 320
+    c = PagedCase(torch.bfloat16, H, H, hd, ps, [70], [n], seed=1)
+    g = torch.Generator().manual_seed(2)
+    far = [int(torch.randint(0, 70 + i + 1, (), generator=g)) for i in range(n)]
+    for i in range(n):
+        kf = c.k_full[0][far[i], 0].float()
+        c.q[i, :hd] = (kf * (30.0 / (c.scale * float(kf.norm() ** 2)))).to(torch.bfloat16)
+    k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
+    tiles = c.tiles(k.ATTN_PREFILL_TILE)
+    out = torch.empty(n, H * hd, dtype=torch.bfloat16, device=DEV)
+    k.attn_prefill(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, tiles,
+                   tiles.shape[0], H, c.scale, 0)
+    got = out[:, :hd].double().cpu()
+    want = torch.stack([c.v_full[0][f, 0] for f in far]).double()
+    assert (got - want).abs().max().item() < 0.1
+    assert (out.double().cpu() - c.reference()).abs().max().item() < 2.5e-2
+
+
 def test_attn_decode_far_key_stands_out():
     """bfloat16, keys streamed into registers: one key among hundreds carries the answer."""
     k = _k()
