@@ -26,7 +26,7 @@
 
 #define NW 8        // waves per block
 #define U 4         // k-blocks per pass and wave
-#define LN_MAX_V 16 // float4 per lane a normed row may take (K <= 4096)
+#define LN_MAX_V 8  // float4 per lane a normed row may take (K <= 2048)
 #define ZERO4 make_uint4(0u, 0u, 0u, 0u)  // a constant, not a variable: see load_pass
 
 struct DecodeGemmArgs {
@@ -65,16 +65,15 @@ union Frag {
   bf16x8_t v;
 };
 
-// LV: float4 per lane that a normed row takes (8: K <= 2048, 16: K <= 4096); 0: no norm.
-// MULTI: K is longer than one pass of NW * U k-blocks (2048); only then is the
-// second set of weight registers needed.
-template <int LV, bool MULTI>
-// (the second bound is waves per SIMD: four keeps two blocks on a CU, except for the long norm)
-__global__ __launch_bounds__(NW * 64, (LV > 8 ? 2 : 4)) void gemm_bf16_decode_kernel(DecodeGemmArgs p) {
-  constexpr bool LN = LV > 0;
-  constexpr int NV = LN ? LV : 1;
+// LN: norm the rows of X in the prologue (K <= 2048: a lane holds its share of
+// a row in NV float4).  MULTI: K is longer than one pass of NW * U k-blocks
+// (2048); only then is the second set of weight registers needed.
+template <bool LN, bool MULTI>
+__global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArgs p) {
+  constexpr int NV = LN_MAX_V;
   extern __shared__ __attribute__((aligned(16))) uint16_t As[];  // [M][a_stride]
   __shared__ float red[NW][256];
+  __shared__ __attribute__((aligned(16))) float gb[LN ? 2 * LN_MAX_V * 256 : 4];  // norm scale, shift
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n0 = blockIdx.x * 16;
@@ -84,56 +83,70 @@ __global__ __launch_bounds__(NW * 64, (LV > 8 ? 2 : 4)) void gemm_bf16_decode_ke
   const int n_chunks = (p.K + 63) / 64;
 
   // Loads are never predicated on their address (a select between an address
-  // and a dummy makes them flat loads, which also count as LDS traffic): every
-  // address is pulled into range and the value is zeroed afterwards, with a
-  // constant (a zero that lives in a variable is a second address to select).
+  // and a dummy makes them flat loads, which also count as LDS traffic) and
+  // weight fragments are not even zeroed when they lie outside the matrix:
+  // every address is pulled into range, and what such a fragment meets is a
+  // zero activation (k >= K) or an output that is never stored (n >= N).  So
+  // nothing has to wait for a weight before the MFMA that uses it.
   auto load_pass = [&](Frag (&w)[U][2], int pass) {
     if (wave + NW * pass * U >= n_chunks) return;  // the whole pass lies beyond K (uniform)
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int c = wave + NW * (pass * U + u);
-      const int k = min(c, n_chunks - 1) * 64 + koff;
-      const uint4 t0 = *(const uint4*)(wrow + min(k, p.K - 8));
-      const uint4 t1 = *(const uint4*)(wrow + min(k + 8, p.K - 8));
-      const bool live = wvalid && c < n_chunks;
-      w[u][0].u = (live && k < p.K) ? t0 : ZERO4;
-      w[u][1].u = (live && k + 8 < p.K) ? t1 : ZERO4;
+      const int c = min(wave + NW * (pass * U + u), n_chunks - 1);
+      const int k = c * 64 + koff;
+      w[u][0].u = *(const uint4*)(wrow + min(k, p.K - 8));
+      w[u][1].u = *(const uint4*)(wrow + min(k + 8, p.K - 8));
     }
   };
 
   Frag w0[U][2], w1[MULTI ? U : 1][2];
-  load_pass(w0, 0);  // in flight while the activations are prepared
 
   // ---- activations into LDS ------------------------------------------------
-  if (LN) {
-    for (int r = wave; r < p.M; r += NW) {
-      const float* x = p.X + (size_t)r * p.ldx;
+  if constexpr (LN) {
+    // Wave w norms rows w and w + 8.  Order of the loads: the first row and
+    // this thread's share of scale and shift, then the weights, so that
+    // waiting for the former leaves the weights in flight.
+    float* gs = gb;
+    float* bs = gb + LN_MAX_V * 256;
+    for (int r = wave, first = 1; first || r < p.M; r += NW, first = 0) {
+      const bool row_live = r < p.M;
+      const float* x = p.X + (size_t)min(r, p.M - 1) * p.ldx;
       float4 v[NV];
+#pragma unroll
+      for (int i = 0; i < NV; ++i) v[i] = *(const float4*)(x + min((lane + 64 * i) * 4, p.K - 4));
+      float4 g4, b4;
+      const int gk = min(tid * 4, p.K - 4);  // K / 4 <= 512 pieces: one a thread, surplus threads repeat the last
+      if (first) {
+        g4 = *(const float4*)(p.gamma + gk);
+        b4 = *(const float4*)(p.beta + gk);
+        asm volatile("" ::: "memory");  // keep the weights' loads behind these
+        __builtin_amdgcn_sched_barrier(0);
+        load_pass(w0, 0);
+      }
       float s = 0.f;
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
-        const int k = (lane + 64 * i) * 4;
-        const float4 t = *(const float4*)(x + min(k, p.K - 4));
-        v[i] = k < p.K ? t : make_float4(0.f, 0.f, 0.f, 0.f);
-        s += v[i].x + v[i].y + v[i].z + v[i].w;
+        if ((lane + 64 * i) * 4 >= p.K) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
       }
       const float mean = wave_sum(s) / (float)p.K;
       float q = 0.f;
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
-        const int k = (lane + 64 * i) * 4;
-        if (k < p.K) {
-          const float a = v[i].x - mean, b = v[i].y - mean, c = v[i].z - mean, d = v[i].w - mean;
-          q += a * a + b * b + c * c + d * d;
-        }
+        const bool in = (lane + 64 * i) * 4 < p.K;
+        const float a = v[i].x - mean, b = v[i].y - mean, c = v[i].z - mean, d = v[i].w - mean;
+        q += in ? (a * a + b * b) + (c * c + d * d) : 0.f;
       }
       const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)p.K + p.eps);
+      if (first) {  // every wave runs the first round
+        *(float4*)(gs + gk) = g4, *(float4*)(bs + gk) = b4;
+        __syncthreads();
+      }
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
         const int k = (lane + 64 * i) * 4;
-        if (k < p.K) {
-          const float4 g = *(const float4*)(p.gamma + k);
-          const float4 b = *(const float4*)(p.beta + k);
+        if (row_live && k < p.K) {
+          const float4 g = *(const float4*)(gs + k), b = *(const float4*)(bs + k);
           uint2 o;
           o.x = pack2((v[i].x - mean) * rstd * g.x + b.x, (v[i].y - mean) * rstd * g.y + b.y);
           o.y = pack2((v[i].z - mean) * rstd * g.z + b.z, (v[i].w - mean) * rstd * g.w + b.w);
@@ -142,6 +155,7 @@ __global__ __launch_bounds__(NW * 64, (LV > 8 ? 2 : 4)) void gemm_bf16_decode_ke
       }
     }
   } else {
+    load_pass(w0, 0);  // in flight while the activations are copied
     const int per_row = p.K / 8;
     for (int c = tid; c < p.M * per_row; c += NW * 64) {
       const int r = c / per_row, k = (c - r * per_row) * 8;
@@ -233,7 +247,7 @@ static int a_stride_for(int K) { return K + ((8 - K % 64) + 64) % 64; }
 // 1 if gemm_bf16_decode takes these sizes (the caller falls back otherwise)
 extern "C" int gemm_bf16_decode_takes(int M, int K, int with_norm) {
   if (M < 1 || M > 16 || K % 8 != 0) return 0;
-  if (with_norm && (K > LN_MAX_V * 256 || K % 4 != 0)) return 0;
+  if (with_norm && (K > LN_MAX_V * 256 || K > NW * U * 64 || K % 4 != 0)) return 0;
   return (size_t)M * a_stride_for(K) * 2 <= MAX_LDS_BYTES;
 }
 
@@ -279,12 +293,13 @@ extern "C" int gemm_bf16_decode(
   p.head_dim = head_dim, p.page_size = page_size;
   const size_t lds = (size_t)M * p.a_stride * 2;
   const bool multi = K > NW * U * 64;
-  const int which = (!ln ? 0 : 2) + (multi ? 1 : 0);
-  void (*kernels[4])(DecodeGemmArgs) = {
-      gemm_bf16_decode_kernel<0, false>, gemm_bf16_decode_kernel<0, true>,
-      gemm_bf16_decode_kernel<8, false>, gemm_bf16_decode_kernel<LN_MAX_V, true>};
-  static size_t granted[4] = {0, 0, 0, 0};
-  if (lds + sizeof(float) * NW * 256 > 64 * 1024 && granted[which] < lds) {
+  const int which = ln ? 2 : (multi ? 1 : 0);
+  void (*kernels[3])(DecodeGemmArgs) = {gemm_bf16_decode_kernel<false, false>,
+                                        gemm_bf16_decode_kernel<false, true>,
+                                        gemm_bf16_decode_kernel<true, false>};
+  static size_t granted[3] = {0, 0, 0};
+  const size_t fixed = sizeof(float) * (NW * 256 + (ln ? 2 * LN_MAX_V * 256 : 4));
+  if (lds + fixed > 64 * 1024 && granted[which] < lds) {
     hipError_t e = hipFuncSetAttribute((const void*)kernels[which],
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) FAIL("gemm_bf16_decode: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(e));

@@ -569,7 +569,7 @@ def test_gemm_bf16_decode(M, N, K, mode, normed):
 
     lib = build.load("gemm_bf16_decode")
     if not lib.gemm_bf16_decode_takes(M, K, int(normed)):
-        assert K > 4096 and normed  # the only sizes of this list it leaves to the general kernels
+        assert K > 2048 and normed  # the only sizes of this list it leaves to the general kernels
     w = _rand((N, K), torch.bfloat16, 11, 0.1)
     bias = _rand((N,), torch.float32, 12)
     if normed:
