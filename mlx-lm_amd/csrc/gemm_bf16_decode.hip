@@ -11,12 +11,27 @@
 // Otherwise the epilogues of gemm_bf16.hip: plain, tanh-GELU, accumulate into
 // the float32 residual stream, float32 out.
 //
-// A block of eight waves owns 16 output features.  The activations (normed or
+// Weights come row-major [N, K] or packed (ldw == 0): tiles of 16 features x
+// 64 k stored in the order the lanes read them, so that a wave's load is 1 KB
+// of consecutive bytes; packed weights stream about twice as fast, because a
+// row-major tile is sixteen 64-byte pieces per load.
+//
+// A block of eight waves owns 16 output features (8 or 4 where N is narrow:
+// a CU can only keep so many loads in flight, so a launch that does not
+// occupy every CU cannot reach the memory's bandwidth).  The activations (normed or
 // copied) sit in LDS as the MFMA B-operand; each wave takes every eighth
 // 64-wide k-block of the 16 weight rows as the A-operand of two
 // v_mfma_f32_16x16x32_bf16 (lane l reads 32 contiguous bytes of row l % 16 at
 // k offset (l / 16) * 16).  Weight loads run two passes of four k-blocks ahead
 // of the MFMAs; the eight partial tiles are summed in a fixed order.
+//
+// Where 16-feature blocks alone are too few to fill the GPU (N = 1600), K is
+// also split over blockIdx.y.  Each split writes its partial tile to a
+// workspace and bumps a counter; the block that arrives last adds the partial
+// tiles in the order of the splits (so the sum does not depend on who was
+// last), runs the epilogue and sets the counter back to zero.  The workspace
+// and the counters belong to the caller; launches that share them must not
+// overlap.
 #include "common.h"
 
 #define FLAG_GELU 1
@@ -48,6 +63,11 @@ struct DecodeGemmArgs {
   const int* token_req;
   const int* positions;
   int max_blocks, q_width, kv_width, head_dim, page_size;
+  // split of K over blockIdx.y: partial tiles and one arrival counter per 16 features
+  int n_splits, chunks_per_split;
+  int rows;            // output features a block owns: 16, 8 or 4 (fewer = more blocks for a narrow N)
+  float* ws;           // [n_blocks][n_splits][256]
+  unsigned int* counters;  // [n_blocks], zero between launches
 };
 
 __device__ __forceinline__ float gelu_tanh(float x) {
@@ -71,16 +91,24 @@ union Frag {
 template <bool LN, bool MULTI>
 __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArgs p) {
   constexpr int NV = LN_MAX_V;
+  constexpr int UU = MULTI ? 2 * U : U;  // k-blocks per pass and wave: long rows keep more in flight
   extern __shared__ __attribute__((aligned(16))) uint16_t As[];  // [M][a_stride]
   __shared__ float red[NW][256];
   __shared__ __attribute__((aligned(16))) float gb[LN ? 2 * LN_MAX_V * 256 : 4];  // norm scale, shift
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * p.rows;
   const int koff = (lane >> 4) * 16;
-  const bool wvalid = n0 + (lane & 15) < p.N;
-  const uint16_t* wrow = p.W + (size_t)(wvalid ? n0 + (lane & 15) : 0) * p.ldw;
-  const int n_chunks = (p.K + 63) / 64;
+  // lanes beyond the block's features (or the matrix) repeat its last row; their results are dropped
+  const uint16_t* wrow = p.W + (size_t)min(n0 + min(lane & 15, p.rows - 1), p.N - 1) * p.ldw;
+  // packed weights (ldw == 0): the 16 x 64 tile of block b and k-block c lies at
+  // (b * n_chunks_all + c) * 1024 elements, first halves of the lanes' 16 values, then second halves
+  const bool packed = p.ldw == 0;
+  const uint16_t* wtile = p.W + (size_t)blockIdx.x * ((p.K + 63) / 64) * 1024 + lane * 8;
+  const int n_chunks_all = (p.K + 63) / 64;
+  const int c_begin = blockIdx.y * p.chunks_per_split;  // this split's k-blocks
+  const int n_chunks = min(n_chunks_all, c_begin + p.chunks_per_split) - c_begin;
+  const int kb = c_begin * 64;  // LDS holds the activations' columns from here on
 
   // Loads are never predicated on their address (a select between an address
   // and a dummy makes them flat loads, which also count as LDS traffic) and
@@ -88,18 +116,23 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArg
   // every address is pulled into range, and what such a fragment meets is a
   // zero activation (k >= K) or an output that is never stored (n >= N).  So
   // nothing has to wait for a weight before the MFMA that uses it.
-  auto load_pass = [&](Frag (&w)[U][2], int pass) {
-    if (wave + NW * pass * U >= n_chunks) return;  // the whole pass lies beyond K (uniform)
+  auto load_pass = [&](Frag (&w)[UU][2], int pass) {
+    if (wave + NW * pass * UU >= n_chunks) return;  // the whole pass lies beyond K (uniform)
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int c = min(wave + NW * (pass * U + u), n_chunks - 1);
+    for (int u = 0; u < UU; ++u) {
+      const int c = c_begin + min(wave + NW * (pass * UU + u), n_chunks - 1);
       const int k = c * 64 + koff;
-      w[u][0].u = *(const uint4*)(wrow + min(k, p.K - 8));
-      w[u][1].u = *(const uint4*)(wrow + min(k + 8, p.K - 8));
+      if (packed) {
+        w[u][0].u = *(const uint4*)(wtile + (size_t)c * 1024);
+        w[u][1].u = *(const uint4*)(wtile + (size_t)c * 1024 + 512);
+      } else {
+        w[u][0].u = *(const uint4*)(wrow + min(k, p.K - 8));
+        w[u][1].u = *(const uint4*)(wrow + min(k + 8, p.K - 8));
+      }
     }
   };
 
-  Frag w0[U][2], w1[MULTI ? U : 1][2];
+  Frag w0[UU][2], w1[MULTI ? UU : 1][2];
 
   // ---- activations into LDS ------------------------------------------------
   if constexpr (LN) {
@@ -156,10 +189,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArg
     }
   } else {
     load_pass(w0, 0);  // in flight while the activations are copied
-    const int per_row = p.K / 8;
+    const int per_row = (min(p.K, kb + n_chunks * 64) - kb) / 8;
     for (int c = tid; c < p.M * per_row; c += NW * 64) {
       const int r = c / per_row, k = (c - r * per_row) * 8;
-      *(uint4*)(As + r * p.a_stride + k) = *(const uint4*)(p.A + (size_t)r * p.lda + k);
+      *(uint4*)(As + r * p.a_stride + k) = *(const uint4*)(p.A + (size_t)r * p.lda + kb + k);
     }
   }
   __syncthreads();
@@ -169,15 +202,15 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArg
   const bool avalid = (lane & 15) < p.M;
   const uint16_t* arow = As + min(lane & 15, p.M - 1) * p.a_stride;
 
-  auto compute_pass = [&](Frag (&w)[U][2], int pass) {
+  auto compute_pass = [&](Frag (&w)[UU][2], int pass) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int c = wave + NW * (pass * U + u);
+    for (int u = 0; u < UU; ++u) {
+      const int c = wave + NW * (pass * UU + u);
       if (c < n_chunks) {  // uniform over the wave
-        const int k = c * 64 + koff;
+        const int k = kb + c * 64 + koff;
         Frag a0, a1;
-        const uint4 t0 = *(const uint4*)(arow + min(k, p.K - 8));
-        const uint4 t1 = *(const uint4*)(arow + min(k + 8, p.K - 8));
+        const uint4 t0 = *(const uint4*)(arow + min(k, p.K - 8) - kb);
+        const uint4 t1 = *(const uint4*)(arow + min(k + 8, p.K - 8) - kb);
         a0.u = (avalid && k < p.K) ? t0 : ZERO4;
         a1.u = (avalid && k + 8 < p.K) ? t1 : ZERO4;
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][0].v, a0.v, acc, 0, 0, 0);
@@ -187,7 +220,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArg
   };
 
   if constexpr (MULTI) {
-    const int n_pass = (n_chunks + NW * U - 1) / (NW * U);
+    const int n_pass = (n_chunks + NW * UU - 1) / (NW * UU);
     for (int pass = 0; pass < n_pass; pass += 2) {
       load_pass(w1, pass + 1);
       compute_pass(w0, pass);
@@ -202,15 +235,38 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArg
 #pragma unroll
   for (int r = 0; r < 4; ++r) red[wave][lane * 4 + r] = acc[r];
   __syncthreads();
+  float v = 0.f;
   if (tid < 256) {
-    float v = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) v += red[w][tid];
+  }
+  if (p.n_splits > 1) {
+    // leave the partial tile, count the arrival; the last block goes on alone
+    __shared__ unsigned int arrived;
+    float* mine = p.ws + ((size_t)blockIdx.x * p.n_splits + blockIdx.y) * 256;
+    if (tid < 256) mine[tid] = v;
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) arrived = atomicAdd(p.counters + blockIdx.x, 1u);
+    __syncthreads();
+    if (arrived != (unsigned int)(p.n_splits - 1)) return;
+    __threadfence();
+    if (tid == 0) p.counters[blockIdx.x] = 0u;  // ready for the next launch
+    if (tid < 256) {
+      const float* all = p.ws + (size_t)blockIdx.x * p.n_splits * 256;
+      v = 0.f;
+      for (int sp = 0; sp < p.n_splits; ++sp)
+        v += __uint_as_float(__hip_atomic_load((const unsigned int*)(all + sp * 256 + tid), __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT));  // from L2, where the others wrote
+    }
+  }
+  if (tid < 256) {
     // element tid = 4 * L + r of the MFMA tile: feature 4 * (L / 16) + r, row L % 16
     const int L = tid >> 2, r = tid & 3;
-    const int n = n0 + 4 * (L >> 4) + r;
+    const int f = 4 * (L >> 4) + r;
+    const int n = n0 + f;
     const int m = L & 15;
-    if (m < p.M && n < p.N) {
+    if (m < p.M && f < p.rows && n < p.N) {
       if (p.bias) v += p.bias[n];
       if (p.flags & FLAG_GELU) v = gelu_tanh(v);
       if ((p.flags & FLAG_KV) && n >= p.q_width) {
@@ -244,11 +300,31 @@ DEFINE_LAST_ERROR(mlxlm_last_error)
 // banks, which holds when the stride in 32-bit words is 4 mod 32.
 static int a_stride_for(int K) { return K + ((8 - K % 64) + 64) % 64; }
 
+// Features per block.
+static int rows_per_block(int N) {
+  // 16 always, for now: with fewer, the lanes of the unused rows repeat a load, which costs the
+  // same address and cache bandwidth as a useful one (measured: no gain at N = 1600, K = 6400)
+  (void)N;
+  return 16;
+}
+
+static int chunks_per_split(int K, int n_splits) { return ((K + 63) / 64 + n_splits - 1) / n_splits; }
+
 // 1 if gemm_bf16_decode takes these sizes (the caller falls back otherwise)
-extern "C" int gemm_bf16_decode_takes(int M, int K, int with_norm) {
-  if (M < 1 || M > 16 || K % 8 != 0) return 0;
-  if (with_norm && (K > LN_MAX_V * 256 || K > NW * U * 64 || K % 4 != 0)) return 0;
-  return (size_t)M * a_stride_for(K) * 2 <= MAX_LDS_BYTES;
+extern "C" int gemm_bf16_decode_takes(int M, int K, int with_norm, int n_splits) {
+  if (M < 1 || M > 16 || K % 8 != 0 || n_splits < 1 || n_splits > (K + 63) / 64) return 0;
+  if (with_norm && (n_splits != 1 || K > LN_MAX_V * 256 || K > NW * U * 64 || K % 4 != 0)) return 0;
+  const int range = K < chunks_per_split(K, n_splits) * 64 ? K : chunks_per_split(K, n_splits) * 64;
+  return (size_t)M * a_stride_for(range) * 2 <= MAX_LDS_BYTES;
+}
+
+// How many ways to split K by default.
+extern "C" int gemm_bf16_decode_splits(int N, int K, int with_norm) {
+  // One, for now: the release/acquire pair that the hand-over between blocks
+  // needs writes back and invalidates an L2 per block on this multi-die GPU,
+  // which costs far more than the parallelism gains (measured: 8 us -> 120 us).
+  (void)N, (void)K, (void)with_norm;
+  return 1;
 }
 
 extern "C" int gemm_bf16_decode(
@@ -256,15 +332,18 @@ extern "C" int gemm_bf16_decode(
     const float* beta, float eps, const void* W, const float* bias, int M, int N, int K, int ldw,
     int ldo, int flags, void* k_pages, void* v_pages, size_t page_stride, const int* block_table,
     int max_blocks, const int* token_req, const int* positions, int q_width, int kv_width,
-    int head_dim, int page_size, hipStream_t stream) {
+    int head_dim, int page_size, int n_splits, float* ws, size_t ws_floats, unsigned int* counters,
+    size_t n_counters, hipStream_t stream) {
   if (M == 0) return 0;
   const bool ln = X != nullptr;
-  if (!gemm_bf16_decode_takes(M, K, ln))
+  if (!gemm_bf16_decode_takes(M, K, ln, n_splits))
     FAIL("gemm_bf16_decode: M=%d K=%d%s is outside what this kernel takes", M, K, ln ? " with norm" : "");
   if (N <= 0) FAIL("gemm_bf16_decode: bad N=%d", N);
   if ((A == nullptr) == (X == nullptr)) FAIL("gemm_bf16_decode: give activations or a residual stream to norm");
   if (!W || !out) FAIL("gemm_bf16_decode: null pointer");
-  if (ldw % 8 != 0 || ldw < K || ((uintptr_t)W & 15)) FAIL("gemm_bf16_decode: W rows must be 16-byte aligned");
+  // ldw == 0: W is packed by pack_weight_for_decode (tiles of 16 features x 64 k, zero padded)
+  if (ldw != 0 && (ldw % 8 != 0 || ldw < K)) FAIL("gemm_bf16_decode: W rows must be 16-byte aligned");
+  if ((uintptr_t)W & 15) FAIL("gemm_bf16_decode: W must be 16-byte aligned");
   if (A && (lda % 8 != 0 || lda < K || ((uintptr_t)A & 15))) FAIL("gemm_bf16_decode: A rows must be 16-byte aligned");
   if (X && (ldx % 4 != 0 || ldx < K || ((uintptr_t)X & 15))) FAIL("gemm_bf16_decode: X rows must be 16-byte aligned");
   if (X && (!gamma || !beta || ((uintptr_t)gamma & 15) || ((uintptr_t)beta & 15)))
@@ -286,13 +365,24 @@ extern "C" int gemm_bf16_decode(
   p.W = (const uint16_t*)W, p.bias = bias, p.out = out, p.A = (const uint16_t*)A, p.X = X;
   p.gamma = gamma, p.beta = beta, p.eps = eps;
   p.M = M, p.N = N, p.K = K, p.lda = lda, p.ldx = ldx, p.ldw = ldw, p.ldo = ldo, p.flags = flags;
-  p.a_stride = a_stride_for(K);
   p.k_pages = (uint16_t*)k_pages, p.v_pages = (uint16_t*)v_pages, p.page_stride = page_stride;
   p.block_table = block_table, p.token_req = token_req, p.positions = positions;
   p.max_blocks = max_blocks, p.q_width = q_width, p.kv_width = kv_width;
   p.head_dim = head_dim, p.page_size = page_size;
+  p.rows = rows_per_block(N);
+  const int n_blocks = (N + p.rows - 1) / p.rows;
+  p.n_splits = n_splits, p.chunks_per_split = chunks_per_split(K, n_splits);
+  p.ws = ws, p.counters = counters;
+  if (n_splits > 1) {
+    if (!ws || !counters) FAIL("gemm_bf16_decode: a split of K needs the workspace and the counters");
+    if (ws_floats < (size_t)n_blocks * n_splits * 256 || n_counters < (size_t)n_blocks)
+      FAIL("gemm_bf16_decode: workspace of %zu floats / %zu counters is too small for %d blocks x %d splits",
+           ws_floats, n_counters, n_blocks, n_splits);
+  }
+  const int range = K < p.chunks_per_split * 64 ? K : p.chunks_per_split * 64;
+  p.a_stride = a_stride_for(range);
   const size_t lds = (size_t)M * p.a_stride * 2;
-  const bool multi = K > NW * U * 64;
+  const bool multi = p.chunks_per_split > NW * U;
   const int which = ln ? 2 : (multi ? 1 : 0);
   void (*kernels[3])(DecodeGemmArgs) = {gemm_bf16_decode_kernel<false, false>,
                                         gemm_bf16_decode_kernel<false, true>,
@@ -305,7 +395,7 @@ extern "C" int gemm_bf16_decode(
     if (e != hipSuccess) FAIL("gemm_bf16_decode: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(e));
     granted[which] = lds;
   }
-  hipLaunchKernelGGL(kernels[which], dim3((N + 15) / 16), dim3(NW * 64), lds, stream, p);
+  hipLaunchKernelGGL(kernels[which], dim3(n_blocks, n_splits), dim3(NW * 64), lds, stream, p);
   CHECK_LAUNCH("gemm_bf16_decode");
   return 0;
 }

@@ -131,18 +131,72 @@ class KVScatter:
         self.kv_width = kv.n_kv_heads * kv.head_dim
 
 
-def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatter=None):
+class PackedWeight:
+    """A bfloat16 weight matrix ``[N, K]`` in the order the decode kernel's lanes read it.
+
+    Tiles of 16 features by 64 k, zero padded; tile ``(b, c)`` holds, for lane
+    ``l`` (feature ``l % 16``, k group ``l // 16``), first the 8 values
+    ``k = 64 c + 16 (l // 16) + 0..7`` of all lanes, then the 8 values ``+ 8..15``.
+    A wave's load is then 1 KB of consecutive bytes.  The matrix is kept
+    row-major as well (``w``) for the kernels that take many rows.
+    """
+
+    def __init__(self, w):
+        _need(w.dtype == torch.bfloat16 and w.dim() == 2, "PackedWeight: a 2-D bfloat16 matrix")
+        self.w = w
+        self.shape, self.dtype, self.device = tuple(w.shape), w.dtype, w.device
+        N, K = w.shape
+        Np, Kp = (N + 15) // 16 * 16, (K + 63) // 64 * 64
+        padded = torch.zeros((Np, Kp), dtype=w.dtype, device=w.device)
+        padded[:N, :K] = w
+        # (block, feature, k-block, k group, half, 8) -> (block, k-block, half, k group, feature, 8)
+        t = padded.view(Np // 16, 16, Kp // 64, 4, 2, 8).permute(0, 2, 4, 3, 1, 5)
+        self.packed = t.contiguous().view(-1)
+
+
+def for_decode(w):
+    """``w`` with a packed copy beside it where the decode kernel can use one
+    (bfloat16 on the GPU); anything else is returned as it is."""
+    if isinstance(w, torch.Tensor) and w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2:
+        return PackedWeight(w)
+    return w
+
+
+_SPLIT_WS = {}
+
+
+def _split_workspace(device):
+    """Partial tiles and arrival counters for projections that split K over blocks.
+
+    One pair per device, made at first use and kept: the kernels leave the
+    counters at zero, and launches on one stream follow each other.
+    """
+    key = (device.type, device.index)
+    pair = _SPLIT_WS.get(key)
+    if pair is None:
+        pair = (torch.empty(4096 * 8 * 256, dtype=torch.float32, device=device),
+                torch.zeros(4096, dtype=torch.int32, device=device))
+        _SPLIT_WS[key] = pair
+    return pair
+
+
+def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatter=None, splits=None):
     """``out = epilogue(a @ w.T + bias)``.
 
-    ``a`` is ``[M, K]`` (or a ``NormedInput``), ``w`` is ``[N, K]``, both
+    ``a`` is ``[M, K]`` (or a ``NormedInput``), ``w`` is ``[N, K]`` (or a
+    ``PackedWeight``, whose packed copy the decode kernel reads), both
     float32 or both bfloat16; ``bias`` float32.  ``accumulate`` adds into a
     float32 ``out`` (the residual stream); otherwise ``out`` is float32 or the
     operands' dtype.  With ``scatter`` (a ``KVScatter``) the columns from
     ``scatter.q_width`` on are also written to the key/value pages.  Up to 16
     bfloat16 rows go to the decode kernel, which fuses the norm and the
-    scatter; everything else is composed from the general kernels.
+    scatter (and splits K over ``splits`` blocks: by default as many as fill
+    the GPU); everything else is composed from the general kernels.
     """
     lazy = a if isinstance(a, NormedInput) else None
+    packed = w if isinstance(w, PackedWeight) else None
+    if packed is not None:
+        w = packed.w
     M, K = a.shape
     N = w.shape[0]
     ldw, ldo = _rows2d(w, "w"), _rows2d(out, "out")
@@ -171,7 +225,9 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
 
     if w.dtype == torch.bfloat16 and variant == 0 and 0 < M <= 16:
         lib = build.load("gemm_bf16_decode")
-        if lib.gemm_bf16_decode_takes(_c_int(M), _c_int(K), _c_int(1 if lazy else 0)):
+        n_splits = lib.gemm_bf16_decode_splits(_c_int(N), _c_int(K), _c_int(1 if lazy else 0)) if splits is None else splits
+        if lib.gemm_bf16_decode_takes(_c_int(M), _c_int(K), _c_int(1 if lazy else 0), _c_int(n_splits)):
+            ws, counters = _split_workspace(w.device) if n_splits > 1 else (None, None)
             if lazy:
                 _dev(lazy.x, "x", torch.float32)
                 A, lda, X, ldx = None, 0, lazy.x, lazy.x.stride(0)
@@ -181,14 +237,17 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
             sc = scatter
             rc = lib.gemm_bf16_decode(
                 _ptr(out), _ptr(A), _c_int(lda), _ptr(X), _c_int(ldx), _ptr(gamma), _ptr(beta),
-                _c_float(eps), _ptr(w), _ptr(bias), _c_int(M), _c_int(N), _c_int(K), _c_int(ldw),
+                _c_float(eps), _ptr(packed.packed if packed else w), _ptr(bias), _c_int(M), _c_int(N),
+                _c_int(K), _c_int(0 if packed else ldw),
                 _c_int(ldo), _c_int(flags | (GEMM_KV if sc else 0)),
                 _ptr(sc.kv.k if sc else None), _ptr(sc.kv.v if sc else None),
                 _c_size_t(sc.kv.page_stride if sc else 0), _ptr(sc.block_table if sc else None),
                 _c_int(sc.block_table.shape[1] if sc else 0), _ptr(sc.token_req if sc else None),
                 _ptr(sc.positions if sc else None), _c_int(sc.q_width if sc else 0),
                 _c_int(sc.kv_width if sc else 0), _c_int(sc.kv.head_dim if sc else 0),
-                _c_int(sc.kv.page_size if sc else 0), _stream(),
+                _c_int(sc.kv.page_size if sc else 0), _c_int(n_splits), _ptr(ws),
+                _c_size_t(ws.numel() if ws is not None else 0), _ptr(counters),
+                _c_size_t(counters.numel() if counters is not None else 0), _stream(),
             )
             build.check(lib, rc, "linear")
             return out

@@ -70,6 +70,7 @@ class CausalSelfAttention(Mixer):
         if self.has_bias:
             self.qkv_b = tensors[n(self.qkv_name + ".bias")]
             self.out_b = tensors[n(self.out_name + ".bias")]
+        self.qkv_w, self.out_w = kernels.for_decode(self.qkv_w), kernels.for_decode(self.out_w)
         if self.position is not None:
             self.position.load(tensors)
 

@@ -40,6 +40,7 @@ class GeluMLP(FeedForward):
         n = self._name
         self.fc_w, self.fc_b = tensors[n("c_fc.weight")], tensors[n("c_fc.bias")]
         self.proj_w, self.proj_b = tensors[n("c_proj.weight")], tensors[n("c_proj.bias")]
+        self.fc_w, self.proj_w = kernels.for_decode(self.fc_w), kernels.for_decode(self.proj_w)
 
     def forward(self, ctx, x, residual):
         act = ctx.scratch((x.shape[0], self.inner), ctx.dtype)

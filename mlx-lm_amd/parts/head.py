@@ -24,7 +24,7 @@ class LinearHead(Part):
         return {self.weight_name: TensorSpec((self.vocab_size, self.width), "matrix")}
 
     def load(self, tensors):
-        self.weight = tensors[self.weight_name]
+        self.weight = kernels.for_decode(tensors[self.weight_name])
 
     def forward(self, ctx, x, out):
         kernels.linear(out, x, self.weight)

@@ -563,12 +563,13 @@ def test_logit_bias_and_penalties():
                                    (9, 1600, 6400), (13, 333, 1608), (16, 257, 3200)])
 @pytest.mark.parametrize("mode", ["plain", "gelu", "accumulate", "f32out"])
 @pytest.mark.parametrize("normed", [False, True])
-def test_gemm_bf16_decode(M, N, K, mode, normed):
+@pytest.mark.parametrize("packed", [False, True])
+def test_gemm_bf16_decode(M, N, K, mode, normed, packed):
     k = _k()
     from mlx_lm_amd.ops import build
 
     lib = build.load("gemm_bf16_decode")
-    if not lib.gemm_bf16_decode_takes(M, K, int(normed)):
+    if not lib.gemm_bf16_decode_takes(M, K, int(normed), 1):
         assert K > 2048 and normed  # the only sizes of this list it leaves to the general kernels
     w = _rand((N, K), torch.bfloat16, 11, 0.1)
     bias = _rand((N,), torch.float32, 12)
@@ -583,6 +584,8 @@ def test_gemm_bf16_decode(M, N, K, mode, normed):
         a = _rand((M, K), torch.bfloat16, 10)
         a_ref = a.double().cpu()
     ref = plain.linear(a_ref, w.double().cpu(), bias.double().cpu())
+    if packed:
+        w = k.PackedWeight(w)  # tiles in the lanes' order, with a row-major copy beside
     slack = 3e-2 * math.sqrt(K) * 0.1 if normed else 0.0  # a normed value may round the other way
     if mode == "accumulate":
         out = _rand((M, N), torch.float32, 13)
@@ -603,6 +606,36 @@ def test_gemm_bf16_decode(M, N, K, mode, normed):
         assert torch.allclose(got, want, rtol=2**-7, atol=1e-3 + slack), (got - want).abs().max()
     else:
         assert (got - want).abs().max().item() < tol, (got - want).abs().max()
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 48, 1024), (8, 1600, 6400), (16, 80, 200), (16, 1600, 6400), (11, 333, 1608)])
+@pytest.mark.parametrize("mode", ["plain", "accumulate"])
+def test_gemm_bf16_decode_split_k(M, N, K, mode):
+    """K split over blocks: the last block to arrive adds the partial tiles in a fixed order,
+    so every number of splits gives the same bits run after run, and counters return to zero."""
+    k = _k()
+    a = _rand((M, K), torch.bfloat16, 10)
+    w = _rand((N, K), torch.bfloat16, 11, 0.1)
+    bias = _rand((N,), torch.float32, 12)
+    ref = plain.linear(a.double().cpu(), w.double().cpu(), bias.double().cpu())
+    for splits in (2, 3, 8):
+        if splits > (K + 63) // 64:
+            continue
+        outs = []
+        for _ in range(3):
+            if mode == "accumulate":
+                out = _rand((M, N), torch.float32, 13)
+                k.linear(out, a, w, bias, accumulate=True, splits=splits)
+                want = _rand((M, N), torch.float32, 13).double().cpu() + ref
+            else:
+                out = torch.empty(M, N, dtype=torch.float32, device=DEV)
+                k.linear(out, a, w, bias, splits=splits)
+                want = ref
+            outs.append(out.clone())
+        assert (outs[0].double().cpu() - want).abs().max().item() < 1e-4 * math.sqrt(K), splits
+        assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2]), splits
+    _, counters = k._split_workspace(a.device)
+    assert int(counters.abs().sum()) == 0
 
 
 @pytest.mark.parametrize("M", [1, 5, 16, 40])
