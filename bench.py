@@ -98,7 +98,7 @@ def run_decode(engine, sample, batch, prompt_len, steps, warmup, vocab, seed):
 
     def one(logits, n):
         tokens, _ = sample(logits, greedy, seeds, [n] * batch)
-        toks = tokens.tolist()  # the host reads every token, as generation does
+        toks = tokens.tolist()  # the host reads every token, as generation does (the step's only wait)
         return engine.step([StepEntry(r, [t], [0]) for r, t in zip(rids, toks)])
 
     n = 0

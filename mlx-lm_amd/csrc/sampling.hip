@@ -107,14 +107,25 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(SampleArgs 
   const float* x = a.logits + (size_t)r * a.ld;
   const int tid = threadIdx.x, nt = blockDim.x;
 
-  // log-sum-exp
-  float mx = -INFINITY;
-  for (int i = tid; i < V; i += nt) mx = fmaxf(mx, x[i]);
-  mx = block_max(mx, red);
-  float se = 0.f;
-  for (int i = tid; i < V; i += nt) se += expf(x[i] - mx);
-  se = block_sum(se, red);
-  const float lse = mx + logf(se);
+  // One pass over the row: running maximum, sum of exponentials relative to it
+  // (rescaled whenever the maximum moves) and the first index of the maximum.
+  float mx = -INFINITY, se = 0.f;
+  int bi = 0x7fffffff;
+  for (int i = tid; i < V; i += nt) {
+    const float v = x[i];
+    if (v > mx) {
+      se = se * expf(mx - v) + 1.f;
+      mx = v, bi = i;
+    } else {
+      se += expf(v - mx);
+    }
+  }
+  const float row_max = block_max(mx, red);
+  se = block_sum(mx == -INFINITY ? 0.f : se * expf(mx - row_max), red);
+  const float lse = row_max + logf(se);
+  float bv = mx;
+  block_argmax(bv, bi, red, redi);  // ties go to the lowest index
+  mx = row_max;
 
   if (a.logprobs) {
     float* lp = a.logprobs + (size_t)r * a.ld_logprobs;
@@ -123,13 +134,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(SampleArgs 
 
   const float temp = a.temp[r];
   if (temp == 0.f) {
-    float bv = -INFINITY;
-    int bi = 0x7fffffff;
-    for (int i = tid; i < V; i += nt) {
-      const float v = x[i];
-      if (v > bv) bv = v, bi = i;
-    }
-    block_argmax(bv, bi, red, redi);
     if (tid == 0) a.tokens[r] = bi, a.token_logprob[r] = bv - lse;
     return;
   }
@@ -227,8 +231,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(SampleArgs 
   const float inv_temp = 1.f / temp;
   const unsigned long long seed = a.seed[r];
   const unsigned int counter = (unsigned int)a.counter[r];
-  float bv = -INFINITY;
-  int bi = 0x7fffffff;
+  bv = -INFINITY, bi = 0x7fffffff;
   for (int i = tid; i < V; i += nt) {
     const float lp = x[i] - lse;
     if (!kept(i, lp)) continue;

@@ -20,7 +20,7 @@ from . import sample_utils
 from .engine.scheduler import Request, Scheduler
 from .engine.step import Engine
 from .sample_utils import Sampler, make_logits_processors, make_sampler
-from .sampling import apply_processors, sample_batch
+from .sampling import apply_processors, read_sampled, sample_batch
 
 DEFAULT_PROMPT = "hello"
 DEFAULT_MAX_TOKENS = 100
@@ -82,7 +82,7 @@ def make_sample_fn():
         want = bool(custom) or any(r.want_logprobs for r in requests)
         out = sample_batch(logits, samplers, [r.seed for r in requests],
                            [len(r.generated) for r in requests], want_logprobs=want)
-        tokens, token_lp = out[0].tolist(), out[1].tolist()
+        tokens, token_lp = read_sampled(out[0], out[1])
         logprobs = out[2] if want else None
         results = []
         for i, r in enumerate(requests):

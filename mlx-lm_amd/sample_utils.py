@@ -75,7 +75,7 @@ class Sampler:
         tokens, _ = sample_batch(logprobs, [self] * n, seeds=[seed + i for i in range(n)],
                                  counters=[self._calls] * n)
         self._calls += 1
-        return tokens
+        return tokens.clone()  # the batch sampler's buffers are reused
 
 
 def make_sampler(temp=0.0, top_p=0.0, min_p=0.0, min_tokens_to_keep=1, top_k=0, xtc_probability=0.0,

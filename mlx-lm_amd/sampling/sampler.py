@@ -73,6 +73,36 @@ def apply_processors(logits, processors, histories):
     return logits[0] if single else logits
 
 
+class _ParamRing:
+    """Pinned host arrays for the sampling kernel's per-row options, reused in turn.
+
+    One asynchronous copy a call brings all of them to the device, so nothing
+    here waits for the GPU; an array is written again only after the copy
+    that read it has finished.
+    """
+
+    FIELDS = 12  # 32-bit words per row: ten options, and the seed's two halves
+
+    def __init__(self, n=4):
+        self.slots = [None] * n
+        self.i = 0
+
+    def get(self, rows, device):
+        self.i = (self.i + 1) % len(self.slots)
+        slot = self.slots[self.i]
+        if slot is None or slot[0].numel() < rows * self.FIELDS or slot[1].device != device:
+            n = max(rows, 64) * self.FIELDS
+            host = torch.empty(n, dtype=torch.int32, pin_memory=True)
+            slot = [host, torch.empty(n, dtype=torch.int32, device=device), None]
+            self.slots[self.i] = slot
+        if slot[2] is not None:
+            slot[2].synchronize()
+        return slot
+
+
+_RING = _ParamRing()
+
+
 def sample_batch(logits, samplers, seeds, counters, want_logprobs=False):
     """One token for each row of float32 ``logits [R, V]``.
 
@@ -81,8 +111,10 @@ def sample_batch(logits, samplers, seeds, counters, want_logprobs=False):
     it.  Returns ``(tokens, token_logprobs)`` as device tensors and, with
     ``want_logprobs``, the normalised log-probabilities ``[R, V]`` as a third.
     ``logits - logsumexp(logits)`` then the sampler, as in
-    mlx_lm/generate.py:411-412.
+    mlx_lm/generate.py:411-412.  Nothing here waits for the GPU.
     """
+    import numpy as np
+
     R, V = logits.shape
     dev = logits.device
     special = []
@@ -92,17 +124,59 @@ def sample_batch(logits, samplers, seeds, counters, want_logprobs=False):
             if special and special != list(s.xtc_special_tokens):
                 raise ValueError("rows of one batch must share their xtc_special_tokens")
             special = list(s.xtc_special_tokens)
-    tokens = torch.empty(R, dtype=torch.int32, device=dev)
-    token_logprob = torch.empty(R, dtype=torch.float32, device=dev)
+    slot = _RING.get(R, dev)
+    host, device_buf = slot[0], slot[1]
+    h = host.numpy()
+    n = R * _ParamRing.FIELDS
+    hf = h[:n].view(np.float32)
+    # rows of R words each: 0 temp, 1 top_p, 2 min_p, 3 xtc_prob, 4 xtc_thr (floats);
+    # 5 min_keep, 6 top_k, 7 counter (ints); 8..9 the seeds (R 64-bit words); 10 tokens, 11 logprob (out)
+    hf[0 * R : 1 * R] = [s.temp for s in samplers]
+    hf[1 * R : 2 * R] = [s.top_p for s in samplers]
+    hf[2 * R : 3 * R] = [s.min_p for s in samplers]
+    hf[3 * R : 4 * R] = [s.xtc_probability for s in samplers]
+    hf[4 * R : 5 * R] = [s.xtc_threshold for s in samplers]
+    h[5 * R : 6 * R] = [s.min_tokens_to_keep for s in samplers]
+    h[6 * R : 7 * R] = [s.top_k for s in samplers]
+    h[7 * R : 8 * R] = counters
+    h[8 * R : 10 * R].view(np.int64)[:] = [int(x) & 0x7FFFFFFFFFFFFFFF for x in seeds]
+    d = device_buf[:n]
+    d[: 10 * R].copy_(host[: 10 * R], non_blocking=True)
+    ev = slot[2] or torch.cuda.Event()
+    ev.record()
+    slot[2] = ev
+    f = d.view(torch.float32)
+    tokens = d[10 * R : 11 * R]
+    token_logprob = f[11 * R : 12 * R]
     logprobs = torch.empty((R, V), dtype=torch.float32, device=dev) if want_logprobs else None
-    f32 = lambda name: _col([float(getattr(s, name)) for s in samplers], torch.float32, dev)
-    i32 = lambda name: _col([int(getattr(s, name)) for s in samplers], torch.int32, dev)
     kernels.sample_rows(
-        tokens, token_logprob, logits, f32("temp"), f32("top_p"), f32("min_p"),
-        i32("min_tokens_to_keep"), i32("top_k"), f32("xtc_probability"), f32("xtc_threshold"),
-        _col([int(x) & 0x7FFFFFFFFFFFFFFF for x in seeds], torch.int64, dev),
-        _col([int(c) for c in counters], torch.int32, dev),
-        _col(special, torch.int32, dev) if special else None, logprobs)
+        tokens, token_logprob, logits, f[0:R], f[R : 2 * R], f[2 * R : 3 * R], d[5 * R : 6 * R],
+        d[6 * R : 7 * R], f[3 * R : 4 * R], f[4 * R : 5 * R], d[8 * R : 10 * R].view(torch.int64),
+        d[7 * R : 8 * R], _col(special, torch.int32, dev) if special else None, logprobs)
+    # tokens and their log-probabilities lie side by side: one copy brings both to the host
+    out = SampledRows(d[10 * R : 12 * R], R)
     if want_logprobs:
-        return tokens, token_logprob, logprobs
-    return tokens, token_logprob
+        return out.tokens, out.token_logprob, logprobs
+    return out.tokens, out.token_logprob
+
+
+class SampledRows:
+    """Tokens and their log-probabilities as one device array (tokens first)."""
+
+    def __init__(self, both, rows):
+        self.both, self.rows = both, rows
+        self.tokens = both[:rows]
+        self.token_logprob = both[rows:].view(torch.float32)
+
+
+def read_sampled(tokens, token_logprob):
+    """``(tokens, logprobs)`` as Python lists with a single device-to-host copy
+    when the two came from one ``sample_batch`` call."""
+    import numpy as np
+
+    R = tokens.numel()
+    if (token_logprob.data_ptr() == tokens.data_ptr() + 4 * R and tokens.dtype == torch.int32
+            and tokens.is_contiguous() and token_logprob.is_contiguous()):
+        both = torch.as_strided(tokens, (2 * R,), (1,)).cpu().numpy()
+        return both[:R].tolist(), both[R:].view(np.float32).tolist()
+    return tokens.tolist(), token_logprob.tolist()
