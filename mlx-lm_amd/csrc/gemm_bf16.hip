@@ -8,7 +8,9 @@
 //
 // Two kernels:
 //  * gemm_bf16_tile: 128x128x64 block tile, 4 waves in 2x2, each wave a 64x64
-//    tile of four v_mfma_f32_32x32x16_bf16 accumulators.  Any M, N; K % 8 == 0.
+//    tile of four v_mfma_f32_32x32x16_bf16 accumulators; two k-blocks in LDS,
+//    two more in registers; tiles dealt to the dies in super-tiles that share
+//    their operands in a die's L2.  Any M, N; K % 8 == 0.
 //  * gemm_bf16_skinny: M <= 64 rows (decode).  A block of four waves owns 16
 //    output features and splits K among its waves; W streams from HBM once
 //    as the MFMA A-operand, the activations are the B-operand.
@@ -59,17 +61,41 @@ __device__ __forceinline__ void store_out(const GemmArgs& p, int m, int n, float
 #define BN 128
 #define BK 64
 #define LDS_STRIDE (BK + 8)  // 144 bytes a row: 16-byte reads of 16 rows hit distinct banks
+#define SUPER_M 8            // tiles of a super-tile along m
+#define SUPER_N 4            // and along n: 32 tiles, one per CU of a die
 
-__global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(GemmArgs p) {
-  __shared__ __attribute__((aligned(16))) uint16_t As[BM * LDS_STRIDE];
-  __shared__ __attribute__((aligned(16))) uint16_t Bs[BN * LDS_STRIDE];
+// Which tile a block works on.  Blocks go to the eight dies (each with an L2 of
+// its own) in turn, so block b runs on die b % 8.  Tiles are grouped in
+// super-tiles of 8 x 4 that share their rows of A and of W; a die works
+// through whole super-tiles, so what one of its blocks brings into the L2 the
+// others find there.  Returns false for the padding blocks of the grid.
+__device__ __forceinline__ bool tile_of_block(int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int super_m = (tiles_m + SUPER_M - 1) / SUPER_M, super_n = (tiles_n + SUPER_N - 1) / SUPER_N;
+  const int die = blockIdx.x & 7, local = blockIdx.x >> 3;
+  const int st = (local / (SUPER_M * SUPER_N)) * 8 + die;
+  const int pos = local % (SUPER_M * SUPER_N);
+  if (st >= super_m * super_n) return false;
+  tm = (st % super_m) * SUPER_M + pos % SUPER_M;
+  tn = (st / super_m) * SUPER_N + pos / SUPER_M;
+  return tm < tiles_m && tn < tiles_n;
+}
 
+// Pipeline: LDS holds two k-blocks; registers hold two more on their way.  In
+// iteration i the loads of k-block i+2 are issued, k-block i is multiplied
+// out of LDS, then k-block i+1 (loaded an iteration ago) goes from registers
+// to the other half of LDS; one barrier an iteration.
+__global__ __launch_bounds__(256, 2) void gemm_bf16_tile_kernel(GemmArgs p) {
+  __shared__ __attribute__((aligned(16))) uint16_t As[2][BM * LDS_STRIDE];
+  __shared__ __attribute__((aligned(16))) uint16_t Bs[2][BN * LDS_STRIDE];
+
+  int tm, tn;
+  if (!tile_of_block((p.M + BM - 1) / BM, (p.N + BN - 1) / BN, tm, tn)) return;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int m0 = blockIdx.y * BM;
-  const int n0 = blockIdx.x * BN;
+  const int m0 = tm * BM;
+  const int n0 = tn * BN;
 
   f32x16_t acc[2][2];
 #pragma unroll
@@ -79,80 +105,157 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile_kernel(GemmArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // each thread moves four 16-byte pieces of A and of W per k-block
-  uint4 ra[4], rb[4];
+  // each thread moves four 16-byte pieces of A and of W per k-block: piece c
+  // is row c / 8, columns (c % 8) * 8 ..; rows beyond the matrix repeat its
+  // last row (their products land in rows or columns that are never stored)
+  // (32-bit element offsets and one LDS offset: registers are scarce here)
+  int a_off[4], b_off[4];
+  const int lds_off0 = (tid >> 3) * LDS_STRIDE + (tid & 7) * 8;  // piece i lies 32 rows further down
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = (tid >> 3) + 32 * i, kc = (tid & 7) * 8;
+    a_off[i] = min(m0 + row, p.M - 1) * p.lda + kc;
+    b_off[i] = min(n0 + row, p.N - 1) * p.ldw + kc;
+  }
+  const int kc_mine = (tid & 7) * 8;
 
-  auto load_global = [&](int k0) {
+  uint4 ra[2][4], rb[2][4];
+  auto load_global = [&](uint4 (&xa)[4], uint4 (&xb)[4], int k0) {
+    // a piece beyond K is read from where it still fits and zeroed when it goes to LDS
+    // (zeroing it here would make the loads wait at once)
+    const int kk = (k0 + kc_mine < p.K) ? k0 : 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int c = tid + 256 * i;
-      const int row = c >> 3;
-      const int kc = (c & 7) * 8;
-      const int gk = k0 + kc;
-      const int gm = m0 + row, gn = n0 + row;
-      const int ck = min(gk, p.K - 8);
-      const uint4 ta = *(const uint4*)(p.A + (size_t)min(gm, p.M - 1) * p.lda + ck);
-      const uint4 tb = *(const uint4*)(p.W + (size_t)min(gn, p.N - 1) * p.ldw + ck);
-      ra[i] = (gm < p.M && gk < p.K) ? ta : ZERO4;
-      rb[i] = (gn < p.N && gk < p.K) ? tb : ZERO4;
+      xa[i] = *(const uint4*)(p.A + a_off[i] + kk);
+      xb[i] = *(const uint4*)(p.W + b_off[i] + kk);
     }
   };
-  auto store_lds = [&]() {
+  auto store_lds = [&](int stage, const uint4 (&xa)[4], const uint4 (&xb)[4], int k0) {
+    const bool in = k0 + kc_mine < p.K;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int c = tid + 256 * i;
-      const int row = c >> 3;
-      const int kc = (c & 7) * 8;
-      *(uint4*)(As + row * LDS_STRIDE + kc) = ra[i];
-      *(uint4*)(Bs + row * LDS_STRIDE + kc) = rb[i];
+      *(uint4*)(As[stage] + lds_off0 + i * 32 * LDS_STRIDE) = in ? xa[i] : ZERO4;
+      *(uint4*)(Bs[stage] + lds_off0 + i * 32 * LDS_STRIDE) = in ? xb[i] : ZERO4;
     }
   };
 
-  load_global(0);
-  store_lds();
+  const int n_blocks = (p.K + BK - 1) / BK;
+  load_global(ra[0], rb[0], 0);
+  if (n_blocks > 1) load_global(ra[1], rb[1], BK);
+  store_lds(0, ra[0], rb[0], 0);
   __syncthreads();
 
   const int frag_row = lane & 31;
   const int frag_k = (lane >> 5) * 8;
+  const uint16_t* a_frag = As[0] + (wm * 64 + frag_row) * LDS_STRIDE + frag_k;
+  const uint16_t* b_frag = Bs[0] + (wn * 64 + frag_row) * LDS_STRIDE + frag_k;
 
-  for (int k0 = 0; k0 < p.K; k0 += BK) {
-    const bool more = (k0 + BK) < p.K;
-    if (more) load_global(k0 + BK);
+  auto multiply = [&](int stage) {
+    const uint16_t* af = a_frag + stage * (BM * LDS_STRIDE);
+    const uint16_t* bf = b_frag + stage * (BN * LDS_STRIDE);
 #pragma unroll
     for (int ks = 0; ks < BK; ks += 16) {
       bf16x8_t a[2], b[2];
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
-        a[i] = *(const bf16x8_t*)(As + (wm * 64 + i * 32 + frag_row) * LDS_STRIDE + ks + frag_k);
+      for (int i = 0; i < 2; ++i) a[i] = *(const bf16x8_t*)(af + i * 32 * LDS_STRIDE + ks);
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
-        b[j] = *(const bf16x8_t*)(Bs + (wn * 64 + j * 32 + frag_row) * LDS_STRIDE + ks + frag_k);
+      for (int j = 0; j < 2; ++j) b[j] = *(const bf16x8_t*)(bf + j * 32 * LDS_STRIDE + ks);
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
     }
-    __syncthreads();
-    if (more) {
-      store_lds();
-      __syncthreads();
+  };
+
+  // Two k-blocks an iteration, so that the register sets are named statically.
+  // The steady part has no branch and no select inside: only then does the
+  // compiler count exactly how many loads may stay in flight at each wait
+  // (a conditional load makes it wait for all of them).
+  auto load_whole = [&](uint4 (&xa)[4], uint4 (&xb)[4], int k0) {  // a k-block that lies inside K
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      xa[i] = *(const uint4*)(p.A + a_off[i] + k0);
+      xb[i] = *(const uint4*)(p.W + b_off[i] + k0);
     }
+  };
+  auto store_whole = [&](int stage, const uint4 (&xa)[4], const uint4 (&xb)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      *(uint4*)(As[stage] + lds_off0 + i * 32 * LDS_STRIDE) = xa[i];
+      *(uint4*)(Bs[stage] + lds_off0 + i * 32 * LDS_STRIDE) = xb[i];
+    }
+  };
+  int kb = 0;
+  const int whole_blocks = p.K / BK;  // k-blocks that need no masking
+  for (; kb + 4 <= whole_blocks; kb += 2) {
+    load_whole(ra[0], rb[0], (kb + 2) * BK);
+    __builtin_amdgcn_sched_barrier(0);  // the loads go out before the arithmetic, not after it
+    multiply(0);
+    store_whole(1, ra[1], rb[1]);
+    __syncthreads();
+    load_whole(ra[1], rb[1], (kb + 3) * BK);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(1);
+    store_whole(0, ra[0], rb[0]);
+    __syncthreads();
+  }
+  // the last few k-blocks, with every guard
+  for (; kb < n_blocks; kb += 2) {
+    if (kb + 2 < n_blocks) load_global(ra[0], rb[0], (kb + 2) * BK);
+    multiply(0);
+    if (kb + 1 < n_blocks) store_lds(1, ra[1], rb[1], (kb + 1) * BK);
+    __syncthreads();
+    if (kb + 1 >= n_blocks) break;
+    if (kb + 3 < n_blocks) load_global(ra[1], rb[1], (kb + 3) * BK);
+    multiply(1);
+    if (kb + 2 < n_blocks) store_lds(0, ra[0], rb[0], (kb + 2) * BK);
+    __syncthreads();
   }
 
-  // accumulator r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
+  // Epilogue.  Accumulator r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4,
+  // column lane%32, so a store covers 32 neighbouring columns of two rows.
+  // (With the operands swapped a lane would hold four neighbouring columns and
+  // store them as one piece, but every lane in another row: measured slower.)
+  // What is read (bias, the residual stream to add to) is read for a whole
+  // 32x32 tile before anything is stored: a load that comes after a store to
+  // memory it might alias waits for it, sixteen times over.
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int j = 0; j < 2; ++j) {
+    const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+    const int nc = min(n, p.N - 1);
+    const float bias = p.bias ? p.bias[nc] : 0.f;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+    for (int i = 0; i < 2; ++i) {
+      const int mb = m0 + wm * 64 + i * 32 + 4 * (lane >> 5);
+      float v[16];
+      if (p.flags & FLAG_ACCUMULATE) {
+        const float* o = (const float*)p.out;
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          v[r] = o[(size_t)min(mb + 8 * (r >> 2) + (r & 3), p.M - 1) * p.ldo + nc];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) v[r] += acc[i][j][r] + bias;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          v[r] = acc[i][j][r] + bias;
+          if (p.flags & FLAG_GELU) v[r] = gelu_tanh(v[r]);
+        }
+      }
       if (n >= p.N) continue;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (m < p.M) store_out(p, m, n, acc[i][j][r]);
+        const int m = mb + 8 * (r >> 2) + (r & 3);
+        if (m >= p.M) continue;
+        const size_t idx = (size_t)m * p.ldo + n;
+        if (p.flags & (FLAG_ACCUMULATE | FLAG_OUT_F32))
+          ((float*)p.out)[idx] = v[r];
+        else
+          ((uint16_t*)p.out)[idx] = f32_to_bf16_bits(v[r]);
       }
     }
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -244,6 +347,8 @@ static int check_args(const GemmArgs& p) {
     FAIL("gemm_bf16: row strides smaller than the rows (lda=%d ldw=%d ldo=%d)", p.lda, p.ldw, p.ldo);
   if (!p.A || !p.W || !p.out) FAIL("gemm_bf16: null pointer");
   if (((uintptr_t)p.A | (uintptr_t)p.W) & 15) FAIL("gemm_bf16: A and W must be 16-byte aligned");
+  if ((size_t)p.M * p.lda >= (1u << 31) || (size_t)p.N * p.ldw >= (1u << 31))
+    FAIL("gemm_bf16: operands of 2^31 elements or more are not supported");
   if ((p.flags & FLAG_ACCUMULATE) && (p.flags & FLAG_GELU))
     FAIL("gemm_bf16: GELU and accumulate cannot be combined");
   return 0;
@@ -277,7 +382,10 @@ extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* b
     else
       hipLaunchKernelGGL(gemm_bf16_skinny_kernel<4>, grid, block, 0, stream, p);
   } else if (variant == 1) {
-    dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM), block(256);
+    const int super_m = ((M + BM - 1) / BM + SUPER_M - 1) / SUPER_M;
+    const int super_n = ((N + BN - 1) / BN + SUPER_N - 1) / SUPER_N;
+    const int per_die = (super_m * super_n + 7) / 8;  // super-tiles a die works through
+    dim3 grid(per_die * 8 * SUPER_M * SUPER_N), block(256);
     hipLaunchKernelGGL(gemm_bf16_tile_kernel, grid, block, 0, stream, p);
   } else {
     FAIL("gemm_bf16: unknown variant %d", variant);

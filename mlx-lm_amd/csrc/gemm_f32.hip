@@ -125,27 +125,40 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs p) {
     }
   }
 
-  // accumulator r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
+  // Epilogue.  Accumulator r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4,
+  // column lane%32.  What is read (bias, the residual stream to add to) is
+  // read for a whole 32x32 tile before anything is stored: a load that comes
+  // after a store to memory it might alias waits for it, sixteen times over.
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+  for (int j = 0; j < TN; ++j) {
+    const int n = n0 + wn * TN * 32 + j * 32 + (lane & 31);
+    const int nc = min(n, p.N - 1);
+    const float bias = p.bias ? p.bias[nc] : 0.f;
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int n = n0 + wn * TN * 32 + j * 32 + (lane & 31);
+    for (int i = 0; i < TM; ++i) {
+      const int mb = m0 + wm * TM * 32 + i * 32 + 4 * (lane >> 5);
+      float v[16];
+      if (p.flags & FLAG_ACCUMULATE) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          v[r] = p.out[(size_t)min(mb + 8 * (r >> 2) + (r & 3), p.M - 1) * p.ldo + nc];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) v[r] += acc[i][j][r] + bias;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          v[r] = acc[i][j][r] + bias;
+          if (p.flags & FLAG_GELU) v[r] = gelu_tanh(v[r]);
+        }
+      }
       if (n >= p.N) continue;
-      const float bias = p.bias ? p.bias[n] : 0.f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm * TM * 32 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (m >= p.M) continue;
-        float v = acc[i][j][r] + bias;
-        if (p.flags & FLAG_GELU) v = gelu_tanh(v);
-        float* o = p.out + (size_t)m * p.ldo + n;
-        if (p.flags & FLAG_ACCUMULATE)
-          *o += v;
-        else
-          *o = v;
+        const int m = mb + 8 * (r >> 2) + (r & 3);
+        if (m < p.M) p.out[(size_t)m * p.ldo + n] = v[r];
       }
     }
+  }
 }
 
 DEFINE_LAST_ERROR(mlxlm_last_error)
