@@ -1,5 +1,6 @@
-// Linear layer for decode steps: at most 16 rows of activations against a
-// bfloat16 weight matrix that streams from HBM exactly once.
+// Linear layer for decode steps: at most 64 rows of activations (the main
+// kernel: up to 16; a wide variant: 17 to 64) against a bfloat16 weight matrix
+// that streams from HBM exactly once.
 //   out[m, n] = epilogue( sum_k A[m, k] * W[n, k] + bias[n] )
 // with two fusions that save a launch and a round trip through memory each:
 //  * prologue: A may be given as the float32 residual stream plus LayerNorm
@@ -84,6 +85,31 @@ union Frag {
   uint4 u;
   bf16x8_t v;
 };
+
+// bias, activation and where one output goes: the matrix, the residual stream or a cache page
+__device__ __forceinline__ void finish(const DecodeGemmArgs& p, int m, int n, float v) {
+  if (p.bias) v += p.bias[n];
+  if (p.flags & FLAG_GELU) v = gelu_tanh(v);
+  if ((p.flags & FLAG_KV) && n >= p.q_width) {
+    const int c = n - p.q_width;
+    const bool is_v = c >= p.kv_width;
+    const int cc = is_v ? c - p.kv_width : c;
+    const int head = cc / p.head_dim, d = cc - head * p.head_dim;
+    const int pos = p.positions[m];
+    const int page = p.block_table[(size_t)p.token_req[m] * p.max_blocks + pos / p.page_size];
+    const size_t dst = (size_t)page * p.page_stride +
+                       ((size_t)head * p.page_size + pos % p.page_size) * p.head_dim + d;
+    (is_v ? p.v_pages : p.k_pages)[dst] = f32_to_bf16_bits(v);
+  } else {
+    const size_t idx = (size_t)m * p.ldo + n;
+    if (p.flags & FLAG_ACCUMULATE)
+      ((float*)p.out)[idx] += v;
+    else if (p.flags & FLAG_OUT_F32)
+      ((float*)p.out)[idx] = v;
+    else
+      ((uint16_t*)p.out)[idx] = f32_to_bf16_bits(v);
+  }
+}
 
 // LN: norm the rows of X in the prologue (K <= 2048: a lane holds its share of
 // a row in NV float4).  MULTI: K is longer than one pass of NW * U k-blocks
@@ -266,29 +292,105 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArg
     const int f = 4 * (L >> 4) + r;
     const int n = n0 + f;
     const int m = L & 15;
-    if (m < p.M && f < p.rows && n < p.N) {
-      if (p.bias) v += p.bias[n];
-      if (p.flags & FLAG_GELU) v = gelu_tanh(v);
-      if ((p.flags & FLAG_KV) && n >= p.q_width) {
-        const int c = n - p.q_width;
-        const bool is_v = c >= p.kv_width;
-        const int cc = is_v ? c - p.kv_width : c;
-        const int head = cc / p.head_dim, d = cc - head * p.head_dim;
-        const int pos = p.positions[m];
-        const int page = p.block_table[(size_t)p.token_req[m] * p.max_blocks + pos / p.page_size];
-        const size_t dst = (size_t)page * p.page_stride +
-                           ((size_t)head * p.page_size + pos % p.page_size) * p.head_dim + d;
-        (is_v ? p.v_pages : p.k_pages)[dst] = f32_to_bf16_bits(v);
-      } else {
-        const size_t idx = (size_t)m * p.ldo + n;
-        if (p.flags & FLAG_ACCUMULATE)
-          ((float*)p.out)[idx] += v;
-        else if (p.flags & FLAG_OUT_F32)
-          ((float*)p.out)[idx] = v;
-        else
-          ((uint16_t*)p.out)[idx] = f32_to_bf16_bits(v);
+    if (m < p.M && f < p.rows && n < p.N) finish(p, m, n, v);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// 17 to 64 rows of activations (MT groups of 16): they no longer fit in LDS
+// whole, so they pass through it in chunks of 512 columns, one k-block a wave.
+// Weights: packed or row-major as above, two chunks ahead in registers.
+#define WIDE_CHUNK (NW * 64)          // columns staged at a time
+#define WIDE_STRIDE (WIDE_CHUNK + 8)  // LDS row stride: 16-byte reads of 16 rows on distinct banks
+
+template <int MT>
+__global__ __launch_bounds__(NW * 64, 2) void gemm_bf16_decode_wide_kernel(DecodeGemmArgs p) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t As[];  // [MT * 16][WIDE_STRIDE]
+  __shared__ float red[NW][MT][256];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n0 = blockIdx.x * 16;
+  const int koff = (lane >> 4) * 16;
+  const int n_chunks = (p.K + 63) / 64;               // k-blocks
+  const int n_stages = (n_chunks + NW - 1) / NW;      // chunks of NW k-blocks
+  const bool packed = p.ldw == 0;
+  const uint16_t* wrow = p.W + (size_t)min(n0 + (lane & 15), p.N - 1) * p.ldw;
+  const uint16_t* wtile = p.W + (size_t)blockIdx.x * n_chunks * 1024 + lane * 8;
+
+  auto load_w = [&](Frag (&w)[2], int stage) {
+    const int c = min(stage * NW + wave, n_chunks - 1);
+    if (packed) {
+      w[0].u = *(const uint4*)(wtile + (size_t)c * 1024);
+      w[1].u = *(const uint4*)(wtile + (size_t)c * 1024 + 512);
+    } else {
+      const int k = c * 64 + koff;
+      w[0].u = *(const uint4*)(wrow + min(k, p.K - 8));
+      w[1].u = *(const uint4*)(wrow + min(k + 8, p.K - 8));
+    }
+  };
+
+  f32x4_t acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+  Frag w[3][2];  // this stage's fragments and the next two
+  load_w(w[0], 0);
+  load_w(w[1], 1);
+
+  const int rows = min(p.M, MT * 16);
+  const uint16_t* arow[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) arow[t] = As + min(t * 16 + (lane & 15), rows - 1) * WIDE_STRIDE + koff;
+
+  // three stages an iteration, so that the register sets are named statically
+  auto one_stage = [&](int stage, Frag (&cur)[2], Frag (&next2)[2]) {
+    if (stage >= n_stages) return;
+    load_w(next2, stage + 2);
+    __syncthreads();  // the previous chunk is no longer read
+    const int k0 = stage * WIDE_CHUNK;
+    const int width = min(WIDE_CHUNK, p.K - k0);  // a multiple of 8
+    const int per_row = width / 8;
+    for (int c = tid; c < rows * per_row; c += NW * 64) {
+      const int r = c / per_row, k = (c - r * per_row) * 8;
+      *(uint4*)(As + r * WIDE_STRIDE + k) = *(const uint4*)(p.A + (size_t)r * p.lda + k0 + k);
+    }
+    __syncthreads();
+    if (stage * NW + wave < n_chunks) {  // uniform over the wave
+      const int kl = wave * 64 + koff;   // this lane's columns within the chunk
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const bool live = t * 16 + (lane & 15) < p.M;
+        Frag a0, a1;
+        // (columns beyond `width` are stale LDS of an earlier chunk: read, then dropped)
+        const uint4 t0 = *(const uint4*)(arow[t] + wave * 64);
+        const uint4 t1 = *(const uint4*)(arow[t] + wave * 64 + 8);
+        a0.u = (live && kl < width) ? t0 : ZERO4;
+        a1.u = (live && kl + 8 < width) ? t1 : ZERO4;
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[0].v, a0.v, acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[1].v, a1.v, acc[t], 0, 0, 0);
       }
     }
+  };
+  for (int stage = 0; stage < n_stages; stage += 3) {
+    one_stage(stage, w[0], w[2]);
+    one_stage(stage + 1, w[1], w[0]);
+    one_stage(stage + 2, w[2], w[1]);
+  }
+
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][t][lane * 4 + r] = acc[t][r];
+  __syncthreads();
+  for (int e = tid; e < MT * 256; e += NW * 64) {
+    const int t = e >> 8, i = e & 255;
+    float v = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < NW; ++wv) v += red[wv][t][i];
+    const int L = i >> 2, r = i & 3;
+    const int n = n0 + 4 * (L >> 4) + r;
+    const int m = t * 16 + (L & 15);
+    if (m < p.M && n < p.N) finish(p, m, n, v);
   }
 }
 
@@ -312,6 +414,7 @@ static int chunks_per_split(int K, int n_splits) { return ((K + 63) / 64 + n_spl
 
 // 1 if gemm_bf16_decode takes these sizes (the caller falls back otherwise)
 extern "C" int gemm_bf16_decode_takes(int M, int K, int with_norm, int n_splits) {
+  if (M > 16 && M <= 64) return !with_norm && n_splits == 1 && K % 8 == 0;  // the wide kernel
   if (M < 1 || M > 16 || K % 8 != 0 || n_splits < 1 || n_splits > (K + 63) / 64) return 0;
   if (with_norm && (n_splits != 1 || K > LN_MAX_V * 256 || K > NW * U * 64 || K % 4 != 0)) return 0;
   const int range = K < chunks_per_split(K, n_splits) * 64 ? K : chunks_per_split(K, n_splits) * 64;
@@ -369,6 +472,24 @@ extern "C" int gemm_bf16_decode(
   p.block_table = block_table, p.token_req = token_req, p.positions = positions;
   p.max_blocks = max_blocks, p.q_width = q_width, p.kv_width = kv_width;
   p.head_dim = head_dim, p.page_size = page_size;
+  if (M > 16) {
+    p.rows = 16, p.n_splits = 1, p.chunks_per_split = 0, p.ws = nullptr, p.counters = nullptr, p.a_stride = 0;
+    const int mt = (M + 15) / 16;
+    const size_t lds = (size_t)mt * 16 * WIDE_STRIDE * 2;
+    void (*wide[3])(DecodeGemmArgs) = {gemm_bf16_decode_wide_kernel<2>, gemm_bf16_decode_wide_kernel<3>,
+                                       gemm_bf16_decode_wide_kernel<4>};
+    static size_t granted_wide[3] = {0, 0, 0};
+    const size_t fixed = sizeof(float) * NW * mt * 256;
+    if (lds + fixed > 64 * 1024 && granted_wide[mt - 2] < lds) {
+      hipError_t e = hipFuncSetAttribute((const void*)wide[mt - 2], hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)lds);
+      if (e != hipSuccess) FAIL("gemm_bf16_decode: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+      granted_wide[mt - 2] = lds;
+    }
+    hipLaunchKernelGGL(wide[mt - 2], dim3((N + 15) / 16), dim3(NW * 64), lds, stream, p);
+    CHECK_LAUNCH("gemm_bf16_decode");
+    return 0;
+  }
   p.rows = rows_per_block(N);
   const int n_blocks = (N + p.rows - 1) / p.rows;
   p.n_splits = n_splits, p.chunks_per_split = chunks_per_split(K, n_splits);

@@ -223,8 +223,11 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
     else:
         _need(out.dtype == torch.bfloat16, "linear: out must be float32 or bfloat16")
 
-    if w.dtype == torch.bfloat16 and variant == 0 and 0 < M <= 16:
+    # (for very wide outputs the general skinny kernel does better than the decode kernel's wide variant)
+    if w.dtype == torch.bfloat16 and variant == 0 and (0 < M <= 16 or (M <= 64 and N <= 8192)):
         lib = build.load("gemm_bf16_decode")
+        if M > 16 and lazy:
+            a, lazy = lazy.materialize(), None  # the wide kernel takes its rows normed
         n_splits = lib.gemm_bf16_decode_splits(_c_int(N), _c_int(K), _c_int(1 if lazy else 0)) if splits is None else splits
         if lib.gemm_bf16_decode_takes(_c_int(M), _c_int(K), _c_int(1 if lazy else 0), _c_int(n_splits)):
             ws, counters = _split_workspace(w.device) if n_splits > 1 else (None, None)

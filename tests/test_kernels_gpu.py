@@ -608,6 +608,39 @@ def test_gemm_bf16_decode(M, N, K, mode, normed, packed):
         assert (got - want).abs().max().item() < tol, (got - want).abs().max()
 
 
+@pytest.mark.parametrize("M,N,K", [(17, 48, 64), (33, 257, 384), (64, 4800, 1600), (40, 1600, 6400), (64, 333, 1608),
+                                   (48, 80, 200), (20, 100, 520)])
+@pytest.mark.parametrize("mode", ["plain", "gelu", "accumulate", "f32out"])
+@pytest.mark.parametrize("packed", [False, True])
+def test_gemm_bf16_decode_wide(M, N, K, mode, packed):
+    """17 to 64 rows: the activations pass through LDS in chunks of 512 columns."""
+    k = _k()
+    a = _rand((M, K), torch.bfloat16, 10)
+    w = _rand((N, K), torch.bfloat16, 11, 0.1)
+    bias = _rand((N,), torch.float32, 12)
+    ref = plain.linear(a.double().cpu(), w.double().cpu(), bias.double().cpu())
+    if packed:
+        w = k.PackedWeight(w)
+    if mode == "accumulate":
+        out = _rand((M, N), torch.float32, 13)
+        want = out.double().cpu() + ref
+        k.linear(out, a, w, bias, accumulate=True)
+        tol = 1e-4 * math.sqrt(K)
+    elif mode == "f32out":
+        out = torch.empty(M, N, dtype=torch.float32, device=DEV)
+        k.linear(out, a, w, bias)
+        want, tol = ref, 1e-4 * math.sqrt(K)
+    else:
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        k.linear(out, a, w, bias, gelu=(mode == "gelu"))
+        want, tol = (plain.gelu_tanh(ref) if mode == "gelu" else ref), None
+    got = out.double().cpu()
+    if tol is None:
+        assert torch.allclose(got, want, rtol=2**-7, atol=1e-3), (got - want).abs().max()
+    else:
+        assert (got - want).abs().max().item() < tol, (got - want).abs().max()
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 48, 1024), (8, 1600, 6400), (16, 80, 200), (16, 1600, 6400), (11, 333, 1608)])
 @pytest.mark.parametrize("mode", ["plain", "accumulate"])
 def test_gemm_bf16_decode_split_k(M, N, K, mode):
