@@ -1,8 +1,7 @@
-// Linear layer for decode steps: at most 64 rows of activations (the main
-// kernel: up to 16; a wide variant: 17 to 64) against a bfloat16 weight matrix
-// that streams from HBM exactly once.
+// Linear layer for decode steps: at most 64 rows of activations against a
+// bfloat16 weight matrix that streams from HBM exactly once.
 //   out[m, n] = epilogue( sum_k A[m, k] * W[n, k] + bias[n] )
-// with two fusions that save a launch and a round trip through memory each:
+// with fusions that save launches and round trips through memory:
 //  * prologue: A may be given as the float32 residual stream plus LayerNorm
 //    parameters; every block then norms the (few) rows itself into LDS
 //    (mlx_lm/models/gpt2.py:104,106: ln_1 / ln_2 before c_attn / c_fc);
@@ -17,22 +16,29 @@
 // of consecutive bytes; packed weights stream about twice as fast, because a
 // row-major tile is sixteen 64-byte pieces per load.
 //
-// A block of eight waves owns 16 output features (8 or 4 where N is narrow:
-// a CU can only keep so many loads in flight, so a launch that does not
-// occupy every CU cannot reach the memory's bandwidth).  The activations (normed or
-// copied) sit in LDS as the MFMA B-operand; each wave takes every eighth
-// 64-wide k-block of the 16 weight rows as the A-operand of two
-// v_mfma_f32_16x16x32_bf16 (lane l reads 32 contiguous bytes of row l % 16 at
-// k offset (l / 16) * 16).  Weight loads run two passes of four k-blocks ahead
+// Up to 16 rows: a block of eight waves owns 16 output features.  The
+// activations (normed or copied) sit in LDS whole as the MFMA B-operand; each
+// wave takes every eighth 64-wide k-block of the 16 weight rows as the
+// A-operand of two v_mfma_f32_16x16x32_bf16 (lane l reads 32 contiguous bytes
+// of row l % 16 at k offset (l / 16) * 16).  Weight loads run two passes ahead
 // of the MFMAs; the eight partial tiles are summed in a fixed order.
 //
-// Where 16-feature blocks alone are too few to fill the GPU (N = 1600), K is
-// also split over blockIdx.y.  Each split writes its partial tile to a
-// workspace and bumps a counter; the block that arrives last adds the partial
-// tiles in the order of the splits (so the sum does not depend on who was
-// last), runs the epilogue and sets the counter back to zero.  The workspace
-// and the counters belong to the caller; launches that share them must not
-// overlap.
+// 17 to 64 rows: every block re-reading all activations would cost more than
+// the weights, so a block takes 64 or 128 features (16 a wave) and a slice of
+// K; the slice of the activations passes through LDS once for all its waves.
+//
+// A CU keeps only so many loads in flight, so a launch that does not occupy
+// every CU cannot reach the memory's bandwidth.  Where the feature blocks alone
+// are too few, K is split over blockIdx.y: each split then writes its partial
+// sums [split][m][n] in float32 to a workspace instead of running the
+// epilogue, and a second, small kernel adds them in the order of the splits
+// and runs the epilogue (sum_partials), or, for the residual stream, adds them
+// to it and norms the new rows in the same pass (sum_partials_norm): the
+// LayerNorm that follows a block's last projection costs no launch of its own
+// and the next projection needs no norm prologue.  (A hand-over inside one
+// kernel, last block to arrive sums, was tried: the release/acquire pair it
+// needs writes back and invalidates an L2 per block on this multi-die GPU and
+// took 120 us where the whole product takes 8.)
 #include "common.h"
 
 #define FLAG_GELU 1
@@ -64,11 +70,11 @@ struct DecodeGemmArgs {
   const int* token_req;
   const int* positions;
   int max_blocks, q_width, kv_width, head_dim, page_size;
-  // split of K over blockIdx.y: partial tiles and one arrival counter per 16 features
+  // split of K over blockIdx.y
   int n_splits, chunks_per_split;
-  int rows;            // output features a block owns: 16, 8 or 4 (fewer = more blocks for a narrow N)
-  float* ws;           // [n_blocks][n_splits][256]
-  unsigned int* counters;  // [n_blocks], zero between launches
+  int rows;            // output features a block of the 16-row kernel owns (16)
+  float* ws;           // [n_splits][M][N] partial sums, when n_splits > 1
+  int vec4;            // four outputs at a time: N, ldo and the scatter widths are multiples of 4, pointers aligned
 };
 
 __device__ __forceinline__ float gelu_tanh(float x) {
@@ -108,6 +114,62 @@ __device__ __forceinline__ void finish(const DecodeGemmArgs& p, int m, int n, fl
       ((float*)p.out)[idx] = v;
     else
       ((uint16_t*)p.out)[idx] = f32_to_bf16_bits(v);
+  }
+}
+
+// The same for outputs n .. n + 3 of row m (n % 4 == 0, p.vec4 holds).
+__device__ __forceinline__ void finish4(const DecodeGemmArgs& p, int m, int n, float4 v) {
+  if (p.bias) {
+    const float4 b = *(const float4*)(p.bias + n);
+    v.x += b.x, v.y += b.y, v.z += b.z, v.w += b.w;
+  }
+  if (p.flags & FLAG_GELU) v.x = gelu_tanh(v.x), v.y = gelu_tanh(v.y), v.z = gelu_tanh(v.z), v.w = gelu_tanh(v.w);
+  uint2 packed;
+  packed.x = pack2(v.x, v.y), packed.y = pack2(v.z, v.w);
+  if ((p.flags & FLAG_KV) && n >= p.q_width) {
+    const int c = n - p.q_width;
+    const bool is_v = c >= p.kv_width;
+    const int cc = is_v ? c - p.kv_width : c;
+    const int head = cc / p.head_dim, d = cc - head * p.head_dim;
+    const int pos = p.positions[m];
+    const int page = p.block_table[(size_t)p.token_req[m] * p.max_blocks + pos / p.page_size];
+    const size_t dst = (size_t)page * p.page_stride +
+                       ((size_t)head * p.page_size + pos % p.page_size) * p.head_dim + d;
+    *(uint2*)((is_v ? p.v_pages : p.k_pages) + dst) = packed;
+  } else {
+    const size_t idx = (size_t)m * p.ldo + n;
+    if (p.flags & FLAG_ACCUMULATE) {
+      float4* o = (float4*)((float*)p.out + idx);
+      const float4 h = *o;
+      *o = make_float4(h.x + v.x, h.y + v.y, h.z + v.z, h.w + v.w);
+    } else if (p.flags & FLAG_OUT_F32) {
+      *(float4*)((float*)p.out + idx) = v;
+    } else {
+      *(uint2*)((uint16_t*)p.out + idx) = packed;
+    }
+  }
+}
+
+// Four outputs of a row from an MFMA tile: to the workspace when K is split, else through the epilogue.
+__device__ __forceinline__ void emit4(const DecodeGemmArgs& p, int split, int m, int n, float4 v) {
+  if (m >= p.M || n >= p.N) return;
+  if (p.n_splits > 1) {
+    float* dst = p.ws + ((size_t)split * p.M + m) * p.N + n;
+    if (p.vec4) {
+      *(float4*)dst = v;
+    } else {
+      dst[0] = v.x;
+      if (n + 1 < p.N) dst[1] = v.y;
+      if (n + 2 < p.N) dst[2] = v.z;
+      if (n + 3 < p.N) dst[3] = v.w;
+    }
+  } else if (p.vec4) {
+    finish4(p, m, n, v);
+  } else {
+    finish(p, m, n, v.x);
+    if (n + 1 < p.N) finish(p, m, n + 1, v.y);
+    if (n + 2 < p.N) finish(p, m, n + 2, v.z);
+    if (n + 3 < p.N) finish(p, m, n + 3, v.w);
   }
 }
 
@@ -215,10 +277,23 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArg
     }
   } else {
     load_pass(w0, 0);  // in flight while the activations are copied
+    // four independent loads a thread and round: one trip to L2 instead of four in a row
     const int per_row = (min(p.K, kb + n_chunks * 64) - kb) / 8;
-    for (int c = tid; c < p.M * per_row; c += NW * 64) {
-      const int r = c / per_row, k = (c - r * per_row) * 8;
-      *(uint4*)(As + r * p.a_stride + k) = *(const uint4*)(p.A + (size_t)r * p.lda + kb + k);
+    const int total = p.M * per_row;
+    for (int c0 = tid; c0 < total; c0 += 4 * NW * 64) {
+      uint4 t[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int c = min(c0 + j * NW * 64, total - 1);
+        const int r = c / per_row, k = (c - r * per_row) * 8;
+        t[j] = *(const uint4*)(p.A + (size_t)r * p.lda + kb + k);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int c = c0 + j * NW * 64;
+        const int r = c / per_row, k = (c - r * per_row) * 8;
+        if (c < total) *(uint4*)(As + r * p.a_stride + k) = t[j];
+      }
     }
   }
   __syncthreads();
@@ -266,240 +341,373 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArg
 #pragma unroll
     for (int w = 0; w < NW; ++w) v += red[w][tid];
   }
-  if (p.n_splits > 1) {
-    // leave the partial tile, count the arrival; the last block goes on alone
-    __shared__ unsigned int arrived;
-    float* mine = p.ws + ((size_t)blockIdx.x * p.n_splits + blockIdx.y) * 256;
-    if (tid < 256) mine[tid] = v;
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) arrived = atomicAdd(p.counters + blockIdx.x, 1u);
-    __syncthreads();
-    if (arrived != (unsigned int)(p.n_splits - 1)) return;
-    __threadfence();
-    if (tid == 0) p.counters[blockIdx.x] = 0u;  // ready for the next launch
-    if (tid < 256) {
-      const float* all = p.ws + (size_t)blockIdx.x * p.n_splits * 256;
-      v = 0.f;
-      for (int sp = 0; sp < p.n_splits; ++sp)
-        v += __uint_as_float(__hip_atomic_load((const unsigned int*)(all + sp * 256 + tid), __ATOMIC_RELAXED,
-                                               __HIP_MEMORY_SCOPE_AGENT));  // from L2, where the others wrote
-    }
-  }
   if (tid < 256) {
     // element tid = 4 * L + r of the MFMA tile: feature 4 * (L / 16) + r, row L % 16
     const int L = tid >> 2, r = tid & 3;
     const int f = 4 * (L >> 4) + r;
     const int n = n0 + f;
     const int m = L & 15;
-    if (m < p.M && f < p.rows && n < p.N) finish(p, m, n, v);
+    if (m < p.M && f < p.rows && n < p.N) {
+      if (p.n_splits > 1)
+        p.ws[((size_t)blockIdx.y * p.M + m) * p.N + n] = v;  // summed, and finished, by sum_partials
+      else
+        finish(p, m, n, v);
+    }
   }
 }
 
 // ---------------------------------------------------------------------------
-// 17 to 64 rows of activations (MT groups of 16): they no longer fit in LDS
-// whole, so they pass through it in chunks of 512 columns, one k-block a wave.
-// Weights: packed or row-major as above, two chunks ahead in registers.
-#define WIDE_CHUNK (NW * 64)          // columns staged at a time
-#define WIDE_STRIDE (WIDE_CHUNK + 8)  // LDS row stride: 16-byte reads of 16 rows on distinct banks
+// 17 to 64 rows of activations (MT groups of 16).  Wave w of block (x, y) owns
+// features 16 * (NWV * x + w) .. + 15 and the k-blocks of split y; the rows'
+// columns of that split pass through LDS in stretches of MID_KB k-blocks, read
+// by all waves.  Weights: packed or row-major as above, a stretch at a time in
+// registers.
+#define MID_KB 8
+#define MID_COLS (MID_KB * 64)
+#define MID_STRIDE (MID_COLS + 8)  // LDS row stride: 16-byte reads of 16 rows on distinct banks
 
-template <int MT>
-__global__ __launch_bounds__(NW * 64, 2) void gemm_bf16_decode_wide_kernel(DecodeGemmArgs p) {
-  extern __shared__ __attribute__((aligned(16))) uint16_t As[];  // [MT * 16][WIDE_STRIDE]
-  __shared__ float red[NW][MT][256];
+template <int MT, int NWV>
+__global__ __launch_bounds__(NWV * 64) void gemm_bf16_mid_kernel(DecodeGemmArgs p) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t As[];  // [MT * 16][MID_STRIDE]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n0 = blockIdx.x * 16;
   const int koff = (lane >> 4) * 16;
-  const int n_chunks = (p.K + 63) / 64;               // k-blocks
-  const int n_stages = (n_chunks + NW - 1) / NW;      // chunks of NW k-blocks
+  const int n_chunks_all = (p.K + 63) / 64;
+  const int c_begin = blockIdx.y * p.chunks_per_split;
+  const int n_chunks = min(n_chunks_all, c_begin + p.chunks_per_split) - c_begin;
+  const int k_end = min(p.K, (c_begin + n_chunks) * 64);
   const bool packed = p.ldw == 0;
-  const uint16_t* wrow = p.W + (size_t)min(n0 + (lane & 15), p.N - 1) * p.ldw;
-  const uint16_t* wtile = p.W + (size_t)blockIdx.x * n_chunks * 1024 + lane * 8;
-
-  auto load_w = [&](Frag (&w)[2], int stage) {
-    const int c = min(stage * NW + wave, n_chunks - 1);
-    if (packed) {
-      w[0].u = *(const uint4*)(wtile + (size_t)c * 1024);
-      w[1].u = *(const uint4*)(wtile + (size_t)c * 1024 + 512);
-    } else {
-      const int k = c * 64 + koff;
-      w[0].u = *(const uint4*)(wrow + min(k, p.K - 8));
-      w[1].u = *(const uint4*)(wrow + min(k + 8, p.K - 8));
-    }
-  };
+  // a wave beyond the matrix repeats the last tile; its results are dropped
+  const int tile = min((int)blockIdx.x * NWV + wave, (p.N + 15) / 16 - 1);
+  const int n0 = ((int)blockIdx.x * NWV + wave) * 16;
+  const uint16_t* wrow = p.W + (size_t)min(tile * 16 + (lane & 15), p.N - 1) * p.ldw;
+  const uint16_t* wtile = p.W + (size_t)tile * n_chunks_all * 1024 + lane * 8;
 
   f32x4_t acc[MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  for (int g = 0; g < MT; ++g) acc[g] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
-  Frag w[3][2];  // this stage's fragments and the next two
-  load_w(w[0], 0);
-  load_w(w[1], 1);
-
-  const int rows = min(p.M, MT * 16);
   const uint16_t* arow[MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) arow[t] = As + min(t * 16 + (lane & 15), rows - 1) * WIDE_STRIDE + koff;
+  for (int g = 0; g < MT; ++g) arow[g] = As + min(g * 16 + (lane & 15), p.M - 1) * MID_STRIDE + koff;
 
-  // three stages an iteration, so that the register sets are named statically
-  auto one_stage = [&](int stage, Frag (&cur)[2], Frag (&next2)[2]) {
-    if (stage >= n_stages) return;
-    load_w(next2, stage + 2);
-    __syncthreads();  // the previous chunk is no longer read
-    const int k0 = stage * WIDE_CHUNK;
-    const int width = min(WIDE_CHUNK, p.K - k0);  // a multiple of 8
-    const int per_row = width / 8;
-    for (int c = tid; c < rows * per_row; c += NW * 64) {
-      const int r = c / per_row, k = (c - r * per_row) * 8;
-      *(uint4*)(As + r * WIDE_STRIDE + k) = *(const uint4*)(p.A + (size_t)r * p.lda + k0 + k);
-    }
-    __syncthreads();
-    if (stage * NW + wave < n_chunks) {  // uniform over the wave
-      const int kl = wave * 64 + koff;   // this lane's columns within the chunk
+  for (int c0 = 0; c0 < n_chunks; c0 += MID_KB) {  // uniform over the block
+    Frag w[MID_KB][2];
 #pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        const bool live = t * 16 + (lane & 15) < p.M;
-        Frag a0, a1;
-        // (columns beyond `width` are stale LDS of an earlier chunk: read, then dropped)
-        const uint4 t0 = *(const uint4*)(arow[t] + wave * 64);
-        const uint4 t1 = *(const uint4*)(arow[t] + wave * 64 + 8);
-        a0.u = (live && kl < width) ? t0 : ZERO4;
-        a1.u = (live && kl + 8 < width) ? t1 : ZERO4;
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[0].v, a0.v, acc[t], 0, 0, 0);
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[1].v, a1.v, acc[t], 0, 0, 0);
+    for (int u = 0; u < MID_KB; ++u) {
+      const int c = c_begin + min(c0 + u, n_chunks - 1);
+      if (packed) {
+        w[u][0].u = *(const uint4*)(wtile + (size_t)c * 1024);
+        w[u][1].u = *(const uint4*)(wtile + (size_t)c * 1024 + 512);
+      } else {
+        const int k = c * 64 + koff;
+        w[u][0].u = *(const uint4*)(wrow + min(k, p.K - 8));
+        w[u][1].u = *(const uint4*)(wrow + min(k + 8, p.K - 8));
       }
     }
-  };
-  for (int stage = 0; stage < n_stages; stage += 3) {
-    one_stage(stage, w[0], w[2]);
-    one_stage(stage + 1, w[1], w[0]);
-    one_stage(stage + 2, w[2], w[1]);
+    __syncthreads();  // the stretch before is no longer read
+    const int k0 = (c_begin + c0) * 64;
+    const int width = min(MID_COLS, k_end - k0);  // a multiple of 8
+    const int per_row = width / 8, total = p.M * per_row;
+    for (int i0 = tid; i0 < total; i0 += 4 * NWV * 64) {
+      uint4 t[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = min(i0 + j * NWV * 64, total - 1);
+        const int r = i / per_row, k = (i - r * per_row) * 8;
+        t[j] = *(const uint4*)(p.A + (size_t)r * p.lda + k0 + k);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int i = i0 + j * NWV * 64;
+        const int r = i / per_row, k = (i - r * per_row) * 8;
+        if (i < total) *(uint4*)(As + r * MID_STRIDE + k) = t[j];
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < MID_KB; ++u) {
+      if (c0 + u < n_chunks) {  // uniform
+        const int kl = u * 64 + koff;  // this lane's columns within the stretch
+#pragma unroll
+        for (int g = 0; g < MT; ++g) {
+          const bool live = g * 16 + (lane & 15) < p.M;
+          Frag a0, a1;
+          // (columns from `width` on are stale LDS: read, then dropped)
+          const uint4 t0 = *(const uint4*)(arow[g] + u * 64);
+          const uint4 t1 = *(const uint4*)(arow[g] + u * 64 + 8);
+          a0.u = (live && kl < width) ? t0 : ZERO4;
+          a1.u = (live && kl + 8 < width) ? t1 : ZERO4;
+          acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][0].v, a0.v, acc[g], 0, 0, 0);
+          acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][1].v, a1.v, acc[g], 0, 0, 0);
+        }
+      }
+    }
   }
+  // accumulator r of tile g: feature 4 * (lane / 16) + r, row 16 g + lane % 16
+#pragma unroll
+  for (int g = 0; g < MT; ++g)
+    emit4(p, blockIdx.y, g * 16 + (lane & 15), n0 + 4 * (lane >> 4),
+          make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]));
+}
 
+// ---------------------------------------------------------------------------
+// The second step of a split product: out = epilogue(sum over splits, in their order).
+__global__ __launch_bounds__(256) void sum_partials_kernel(DecodeGemmArgs p) {
+  const int n4 = (p.N + 3) / 4;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= p.M * n4) return;
+  const int m = i / n4, n = (i - m * n4) * 4;
+  const float* src = p.ws + (size_t)m * p.N + n;
+  const size_t step = (size_t)p.M * p.N;
+  if (p.vec4) {
+    // four splits' loads at a time, none waiting for another (surplus ones repeat the last and are dropped)
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int s0 = 0; s0 < p.n_splits; s0 += 4) {
+      float4 t[4];
 #pragma unroll
-  for (int t = 0; t < MT; ++t)
+      for (int j = 0; j < 4; ++j) t[j] = *(const float4*)(src + min(s0 + j, p.n_splits - 1) * step);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[wave][t][lane * 4 + r] = acc[t][r];
-  __syncthreads();
-  for (int e = tid; e < MT * 256; e += NW * 64) {
-    const int t = e >> 8, i = e & 255;
-    float v = 0.f;
+      for (int j = 0; j < 4; ++j)
+        if (s0 + j < p.n_splits) v.x += t[j].x, v.y += t[j].y, v.z += t[j].z, v.w += t[j].w;
+    }
+    finish4(p, m, n, v);
+  } else {
+    for (int j = 0; j < 4 && n + j < p.N; ++j) {
+      float v = src[j];
+      for (int s = 1; s < p.n_splits; ++s) v += src[s * step + j];
+      finish(p, m, n + j, v);
+    }
+  }
+}
+
+// The second step for the residual stream, with the norm that follows it:
+//   h[m] += bias + sum over splits;  out[m] = LayerNorm(h[m]) * gamma + beta
+// One block a row, the row in registers (NV4 float4 a thread); N % 4 == 0.
+struct SumNormArgs {
+  float* h;
+  const float* ws;
+  const float* bias;
+  const float* gamma;
+  const float* beta;
+  void* out;
+  float eps;
+  int M, N, ldh, n_splits, out_dtype;
+};
+
+template <int NV4>
+__global__ __launch_bounds__(256) void sum_partials_norm_kernel(SumNormArgs q) {
+  __shared__ float red[32];
+  const int m = blockIdx.x, tid = threadIdx.x;
+  float* hrow = q.h + (size_t)m * q.ldh;
+  const size_t step = (size_t)q.M * q.N;
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f), one = make_float4(1.f, 1.f, 1.f, 1.f);
+  // Few blocks, little data: what counts is how many trips to memory follow
+  // one another.  Everything the row needs is asked for at once.
+  float4 v[NV4], bias[NV4], g[NV4], b[NV4];
 #pragma unroll
-    for (int wv = 0; wv < NW; ++wv) v += red[wv][t][i];
-    const int L = i >> 2, r = i & 3;
-    const int n = n0 + 4 * (L >> 4) + r;
-    const int m = t * 16 + (L & 15);
-    if (m < p.M && n < p.N) finish(p, m, n, v);
+  for (int i = 0; i < NV4; ++i) {
+    const int k = min((tid + 256 * i) * 4, q.N - 4);
+    v[i] = *(const float4*)(hrow + k);
+    bias[i] = q.bias ? *(const float4*)(q.bias + k) : zero;
+    g[i] = q.gamma ? *(const float4*)(q.gamma + k) : one;
+    b[i] = q.beta ? *(const float4*)(q.beta + k) : zero;
+  }
+  float4 part[NV4];
+#pragma unroll
+  for (int i = 0; i < NV4; ++i) part[i] = zero;
+  for (int s0 = 0; s0 < q.n_splits; s0 += 4) {
+    float4 t[NV4][4];
+#pragma unroll
+    for (int i = 0; i < NV4; ++i) {
+      const float* src = q.ws + (size_t)m * q.N + min((tid + 256 * i) * 4, q.N - 4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) t[i][j] = *(const float4*)(src + min(s0 + j, q.n_splits - 1) * step);
+    }
+#pragma unroll
+    for (int i = 0; i < NV4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (s0 + j < q.n_splits)
+          part[i].x += t[i][j].x, part[i].y += t[i][j].y, part[i].z += t[i][j].z, part[i].w += t[i][j].w;
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV4; ++i) {
+    const int k = (tid + 256 * i) * 4;
+    v[i].x += bias[i].x + part[i].x, v[i].y += bias[i].y + part[i].y;
+    v[i].z += bias[i].z + part[i].z, v[i].w += bias[i].w + part[i].w;
+    if (k < q.N) {
+      *(float4*)(hrow + k) = v[i];
+      s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+    }
+  }
+  const float mean = block_sum(s, red) / (float)q.N;
+  float qq = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV4; ++i) {
+    if ((tid + 256 * i) * 4 < q.N) {
+      const float a = v[i].x - mean, bb = v[i].y - mean, c = v[i].z - mean, d = v[i].w - mean;
+      qq += (a * a + bb * bb) + (c * c + d * d);
+    }
+  }
+  const float rstd = 1.0f / sqrtf(block_sum(qq, red) / (float)q.N + q.eps);
+#pragma unroll
+  for (int i = 0; i < NV4; ++i) {
+    const int k = (tid + 256 * i) * 4;
+    if (k >= q.N) continue;
+    const float y0 = (v[i].x - mean) * rstd * g[i].x + b[i].x, y1 = (v[i].y - mean) * rstd * g[i].y + b[i].y;
+    const float y2 = (v[i].z - mean) * rstd * g[i].z + b[i].z, y3 = (v[i].w - mean) * rstd * g[i].w + b[i].w;
+    if (q.out_dtype == DT_F32) {
+      *(float4*)((float*)q.out + (size_t)m * q.N + k) = make_float4(y0, y1, y2, y3);
+    } else {
+      uint2 o;
+      o.x = pack2(y0, y1), o.y = pack2(y2, y3);
+      *(uint2*)((uint16_t*)q.out + (size_t)m * q.N + k) = o;
+    }
   }
 }
 
 DEFINE_LAST_ERROR(mlxlm_last_error)
 
 #define MAX_LDS_BYTES (120 * 1024)
+#define MID_WAVES 4
 
 // LDS row stride: rows of 16-byte reads from 16 lanes must fall on distinct
 // banks, which holds when the stride in 32-bit words is 4 mod 32.
 static int a_stride_for(int K) { return K + ((8 - K % 64) + 64) % 64; }
 
-// Features per block.
-static int rows_per_block(int N) {
-  // 16 always, for now: with fewer, the lanes of the unused rows repeat a load, which costs the
-  // same address and cache bandwidth as a useful one (measured: no gain at N = 1600, K = 6400)
-  (void)N;
-  return 16;
-}
-
 static int chunks_per_split(int K, int n_splits) { return ((K + 63) / 64 + n_splits - 1) / n_splits; }
 
 // 1 if gemm_bf16_decode takes these sizes (the caller falls back otherwise)
 extern "C" int gemm_bf16_decode_takes(int M, int K, int with_norm, int n_splits) {
-  if (M > 16 && M <= 64) return !with_norm && n_splits == 1 && K % 8 == 0;  // the wide kernel
-  if (M < 1 || M > 16 || K % 8 != 0 || n_splits < 1 || n_splits > (K + 63) / 64) return 0;
+  if (M < 1 || M > 64 || K < 8 || K % 8 != 0 || n_splits < 1 || n_splits > (K + 63) / 64) return 0;
+  if (M > 16) return !with_norm;
   if (with_norm && (n_splits != 1 || K > LN_MAX_V * 256 || K > NW * U * 64 || K % 4 != 0)) return 0;
   const int range = K < chunks_per_split(K, n_splits) * 64 ? K : chunks_per_split(K, n_splits) * 64;
   return (size_t)M * a_stride_for(range) * 2 <= MAX_LDS_BYTES;
 }
 
-// How many ways to split K by default.
-extern "C" int gemm_bf16_decode_splits(int N, int K, int with_norm) {
-  // One, for now: the release/acquire pair that the hand-over between blocks
-  // needs writes back and invalidates an L2 per block on this multi-die GPU,
-  // which costs far more than the parallelism gains (measured: 8 us -> 120 us).
-  (void)N, (void)K, (void)with_norm;
-  return 1;
+// Into how many parts to split K so that the launch fills the GPU (1: no
+// split, the product's kernel runs the epilogue itself).  `force` > 0 asks for
+// that many wherever a split is possible at all (for tests of small sizes).
+extern "C" int gemm_bf16_decode_splits(int M, int N, int K, int with_norm, int force) {
+  const int n_chunks = (K + 63) / 64;
+  if (with_norm || M < 1 || M > 64) return 1;
+  int want;
+  if (force > 0) {
+    want = force;
+  } else if (M <= 16) {
+    const int n_blocks = (N + 15) / 16;
+    if (n_blocks >= 200) return 1;
+    want = (512 + n_blocks - 1) / n_blocks;  // two blocks a CU (measured at N = 1600: K = 6400 is best in 5, K = 1600 in 2 to 6)
+    if (want > n_chunks / 4) want = n_chunks / 4;  // at least four k-blocks a split
+  } else {
+    const int n_blocks = (N + 16 * MID_WAVES - 1) / (16 * MID_WAVES);
+    want = (512 + n_blocks - 1) / n_blocks;
+    if (want > n_chunks / 2) want = n_chunks / 2;
+    if (want > 16) want = 16;
+  }
+  if (want < 1) want = 1;
+  if (want > n_chunks) want = n_chunks;
+  const int cps = (n_chunks + want - 1) / want;
+  return (n_chunks + cps - 1) / cps;  // no empty split
 }
 
+static bool aligned16(const void* q) { return ((uintptr_t)q & 15) == 0; }
+
+// Checks and fields that the product and sum_partials share.  Returns 0 or -1.
+static int fill_epilogue(DecodeGemmArgs& p, const char* who, void* out, const float* bias, int M, int N,
+                         int ldo, int flags, void* k_pages, void* v_pages, size_t page_stride,
+                         const int* block_table, int max_blocks, const int* token_req,
+                         const int* positions, int q_width, int kv_width, int head_dim, int page_size) {
+  if (N <= 0) FAIL("%s: bad N=%d", who, N);
+  if (!out) FAIL("%s: null pointer", who);
+  if ((flags & FLAG_ACCUMULATE) && (flags & (FLAG_GELU | FLAG_KV)))
+    FAIL("%s: accumulate cannot be combined with GELU or the cache scatter", who);
+  if (flags & FLAG_KV) {
+    if (!k_pages || !v_pages || !block_table || !token_req || !positions)
+      FAIL("%s: the cache scatter needs pages, block table, token_req and positions", who);
+    if (head_dim <= 0 || page_size <= 0 || kv_width % head_dim != 0 || q_width + 2 * kv_width != N)
+      FAIL("%s: q_width %d + 2 * kv_width %d must be N=%d, kv_width a multiple of head_dim %d", who,
+           q_width, kv_width, N, head_dim);
+    if (flags & (FLAG_OUT_F32 | FLAG_GELU)) FAIL("%s: the cache scatter writes bfloat16, no GELU", who);
+    if (ldo < q_width) FAIL("%s: ldo=%d smaller than q_width=%d", who, ldo, q_width);
+  } else if (ldo < N) {
+    FAIL("%s: ldo=%d smaller than N=%d", who, ldo, N);
+  }
+  p.bias = bias, p.out = out, p.M = M, p.N = N, p.ldo = ldo, p.flags = flags;
+  p.k_pages = (uint16_t*)k_pages, p.v_pages = (uint16_t*)v_pages, p.page_stride = page_stride;
+  p.block_table = block_table, p.token_req = token_req, p.positions = positions;
+  p.max_blocks = max_blocks, p.q_width = q_width, p.kv_width = kv_width;
+  p.head_dim = head_dim, p.page_size = page_size;
+  p.vec4 = N % 4 == 0 && ldo % 4 == 0 && aligned16(out) && aligned16(bias);
+  if (flags & FLAG_KV)
+    p.vec4 = p.vec4 && q_width % 4 == 0 && kv_width % 4 == 0 && head_dim % 4 == 0 && page_stride % 4 == 0 &&
+             aligned16(k_pages) && aligned16(v_pages);
+  return 0;
+}
+
+// With n_splits > 1 the epilogue does not run: the partial sums go to `ws`
+// ([n_splits][M][N] floats) and sum_partials or sum_partials_norm finishes.
 extern "C" int gemm_bf16_decode(
     void* out, const void* A, int lda, const float* X, int ldx, const float* gamma,
     const float* beta, float eps, const void* W, const float* bias, int M, int N, int K, int ldw,
     int ldo, int flags, void* k_pages, void* v_pages, size_t page_stride, const int* block_table,
     int max_blocks, const int* token_req, const int* positions, int q_width, int kv_width,
-    int head_dim, int page_size, int n_splits, float* ws, size_t ws_floats, unsigned int* counters,
-    size_t n_counters, hipStream_t stream) {
+    int head_dim, int page_size, int n_splits, float* ws, size_t ws_floats, hipStream_t stream) {
   if (M == 0) return 0;
   const bool ln = X != nullptr;
   if (!gemm_bf16_decode_takes(M, K, ln, n_splits))
-    FAIL("gemm_bf16_decode: M=%d K=%d%s is outside what this kernel takes", M, K, ln ? " with norm" : "");
-  if (N <= 0) FAIL("gemm_bf16_decode: bad N=%d", N);
+    FAIL("gemm_bf16_decode: M=%d K=%d%s in %d splits is outside what this kernel takes", M, K,
+         ln ? " with norm" : "", n_splits);
   if ((A == nullptr) == (X == nullptr)) FAIL("gemm_bf16_decode: give activations or a residual stream to norm");
-  if (!W || !out) FAIL("gemm_bf16_decode: null pointer");
-  // ldw == 0: W is packed by pack_weight_for_decode (tiles of 16 features x 64 k, zero padded)
+  if (!W) FAIL("gemm_bf16_decode: null pointer");
+  // ldw == 0: W is packed (tiles of 16 features x 64 k, zero padded)
   if (ldw != 0 && (ldw % 8 != 0 || ldw < K)) FAIL("gemm_bf16_decode: W rows must be 16-byte aligned");
-  if ((uintptr_t)W & 15) FAIL("gemm_bf16_decode: W must be 16-byte aligned");
-  if (A && (lda % 8 != 0 || lda < K || ((uintptr_t)A & 15))) FAIL("gemm_bf16_decode: A rows must be 16-byte aligned");
-  if (X && (ldx % 4 != 0 || ldx < K || ((uintptr_t)X & 15))) FAIL("gemm_bf16_decode: X rows must be 16-byte aligned");
-  if (X && (!gamma || !beta || ((uintptr_t)gamma & 15) || ((uintptr_t)beta & 15)))
+  if (!aligned16(W)) FAIL("gemm_bf16_decode: W must be 16-byte aligned");
+  if (A && (lda % 8 != 0 || lda < K || !aligned16(A))) FAIL("gemm_bf16_decode: A rows must be 16-byte aligned");
+  if (X && (ldx % 4 != 0 || ldx < K || !aligned16(X))) FAIL("gemm_bf16_decode: X rows must be 16-byte aligned");
+  if (X && (!gamma || !beta || !aligned16(gamma) || !aligned16(beta)))
     FAIL("gemm_bf16_decode: the norm needs scale and shift, 16-byte aligned");
-  if ((flags & FLAG_ACCUMULATE) && (flags & (FLAG_GELU | FLAG_KV)))
-    FAIL("gemm_bf16_decode: accumulate cannot be combined with GELU or the cache scatter");
-  if (flags & FLAG_KV) {
-    if (!k_pages || !v_pages || !block_table || !token_req || !positions)
-      FAIL("gemm_bf16_decode: the cache scatter needs pages, block table, token_req and positions");
-    if (head_dim <= 0 || page_size <= 0 || kv_width % head_dim != 0 || q_width + 2 * kv_width != N)
-      FAIL("gemm_bf16_decode: q_width %d + 2 * kv_width %d must be N=%d, kv_width a multiple of head_dim %d",
-           q_width, kv_width, N, head_dim);
-    if (flags & (FLAG_OUT_F32 | FLAG_GELU)) FAIL("gemm_bf16_decode: the cache scatter writes bfloat16, no GELU");
-    if (ldo < q_width) FAIL("gemm_bf16_decode: ldo=%d smaller than q_width=%d", ldo, q_width);
-  } else if (ldo < N) {
-    FAIL("gemm_bf16_decode: ldo=%d smaller than N=%d", ldo, N);
-  }
   DecodeGemmArgs p;
-  p.W = (const uint16_t*)W, p.bias = bias, p.out = out, p.A = (const uint16_t*)A, p.X = X;
+  if (fill_epilogue(p, "gemm_bf16_decode", out, bias, M, N, ldo, flags, k_pages, v_pages, page_stride,
+                    block_table, max_blocks, token_req, positions, q_width, kv_width, head_dim, page_size))
+    return -1;
+  p.W = (const uint16_t*)W, p.A = (const uint16_t*)A, p.X = X;
   p.gamma = gamma, p.beta = beta, p.eps = eps;
-  p.M = M, p.N = N, p.K = K, p.lda = lda, p.ldx = ldx, p.ldw = ldw, p.ldo = ldo, p.flags = flags;
-  p.k_pages = (uint16_t*)k_pages, p.v_pages = (uint16_t*)v_pages, p.page_stride = page_stride;
-  p.block_table = block_table, p.token_req = token_req, p.positions = positions;
-  p.max_blocks = max_blocks, p.q_width = q_width, p.kv_width = kv_width;
-  p.head_dim = head_dim, p.page_size = page_size;
+  p.K = K, p.lda = lda, p.ldx = ldx, p.ldw = ldw;
+  p.rows = 16;
+  p.n_splits = n_splits, p.chunks_per_split = chunks_per_split(K, n_splits);
+  p.ws = ws;
+  if (n_splits > 1) {
+    if (!ws || !aligned16(ws)) FAIL("gemm_bf16_decode: a split of K needs a 16-byte aligned workspace");
+    if (ws_floats < (size_t)n_splits * M * N)
+      FAIL("gemm_bf16_decode: workspace of %zu floats is too small for %d splits of %d x %d", ws_floats,
+           n_splits, M, N);
+    if ((p.chunks_per_split * (n_splits - 1)) >= (K + 63) / 64)
+      FAIL("gemm_bf16_decode: %d splits of K=%d leave one empty", n_splits, K);
+    p.vec4 = N % 4 == 0;  // of the workspace's rows, here
+  }
   if (M > 16) {
-    p.rows = 16, p.n_splits = 1, p.chunks_per_split = 0, p.ws = nullptr, p.counters = nullptr, p.a_stride = 0;
+    p.a_stride = MID_STRIDE;
     const int mt = (M + 15) / 16;
-    const size_t lds = (size_t)mt * 16 * WIDE_STRIDE * 2;
-    void (*wide[3])(DecodeGemmArgs) = {gemm_bf16_decode_wide_kernel<2>, gemm_bf16_decode_wide_kernel<3>,
-                                       gemm_bf16_decode_wide_kernel<4>};
-    static size_t granted_wide[3] = {0, 0, 0};
-    const size_t fixed = sizeof(float) * NW * mt * 256;
-    if (lds + fixed > 64 * 1024 && granted_wide[mt - 2] < lds) {
-      hipError_t e = hipFuncSetAttribute((const void*)wide[mt - 2], hipFuncAttributeMaxDynamicSharedMemorySize,
+    const size_t lds = (size_t)mt * 16 * MID_STRIDE * 2;
+    void (*mid[3])(DecodeGemmArgs) = {gemm_bf16_mid_kernel<2, MID_WAVES>, gemm_bf16_mid_kernel<3, MID_WAVES>,
+                                      gemm_bf16_mid_kernel<4, MID_WAVES>};
+    static size_t granted_mid[3] = {0, 0, 0};
+    if (lds > 64 * 1024 && granted_mid[mt - 2] < lds) {
+      hipError_t e = hipFuncSetAttribute((const void*)mid[mt - 2], hipFuncAttributeMaxDynamicSharedMemorySize,
                                          (int)lds);
       if (e != hipSuccess) FAIL("gemm_bf16_decode: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-      granted_wide[mt - 2] = lds;
+      granted_mid[mt - 2] = lds;
     }
-    hipLaunchKernelGGL(wide[mt - 2], dim3((N + 15) / 16), dim3(NW * 64), lds, stream, p);
+    const int n_blocks = (N + 16 * MID_WAVES - 1) / (16 * MID_WAVES);
+    hipLaunchKernelGGL(mid[mt - 2], dim3(n_blocks, n_splits), dim3(MID_WAVES * 64), lds, stream, p);
     CHECK_LAUNCH("gemm_bf16_decode");
     return 0;
   }
-  p.rows = rows_per_block(N);
   const int n_blocks = (N + p.rows - 1) / p.rows;
-  p.n_splits = n_splits, p.chunks_per_split = chunks_per_split(K, n_splits);
-  p.ws = ws, p.counters = counters;
-  if (n_splits > 1) {
-    if (!ws || !counters) FAIL("gemm_bf16_decode: a split of K needs the workspace and the counters");
-    if (ws_floats < (size_t)n_blocks * n_splits * 256 || n_counters < (size_t)n_blocks)
-      FAIL("gemm_bf16_decode: workspace of %zu floats / %zu counters is too small for %d blocks x %d splits",
-           ws_floats, n_counters, n_blocks, n_splits);
-  }
   const int range = K < p.chunks_per_split * 64 ? K : p.chunks_per_split * 64;
   p.a_stride = a_stride_for(range);
   const size_t lds = (size_t)M * p.a_stride * 2;
@@ -518,5 +726,50 @@ extern "C" int gemm_bf16_decode(
   }
   hipLaunchKernelGGL(kernels[which], dim3(n_blocks, n_splits), dim3(NW * 64), lds, stream, p);
   CHECK_LAUNCH("gemm_bf16_decode");
+  return 0;
+}
+
+// out = epilogue(sum of the n_splits partial products in ws): what gemm_bf16_decode left out.
+extern "C" int sum_partials(void* out, const float* ws, int n_splits, const float* bias, int M, int N,
+                            int ldo, int flags, void* k_pages, void* v_pages, size_t page_stride,
+                            const int* block_table, int max_blocks, const int* token_req,
+                            const int* positions, int q_width, int kv_width, int head_dim,
+                            int page_size, hipStream_t stream) {
+  if (M == 0) return 0;
+  if (M < 0 || n_splits < 1 || !ws) FAIL("sum_partials: bad M=%d, splits=%d or workspace", M, n_splits);
+  DecodeGemmArgs p = {};
+  if (fill_epilogue(p, "sum_partials", out, bias, M, N, ldo, flags, k_pages, v_pages, page_stride,
+                    block_table, max_blocks, token_req, positions, q_width, kv_width, head_dim, page_size))
+    return -1;
+  p.ws = (float*)ws, p.n_splits = n_splits;
+  p.vec4 = p.vec4 && aligned16(ws);
+  const long total = (long)M * ((N + 3) / 4);
+  hipLaunchKernelGGL(sum_partials_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, p);
+  CHECK_LAUNCH("sum_partials");
+  return 0;
+}
+
+// 1 if sum_partials_norm takes this width
+extern "C" int sum_partials_norm_takes(int N, int ldh) { return N > 0 && N % 4 == 0 && N <= 8192 && ldh % 4 == 0; }
+
+// h[m] += bias + sum of the partial products;  out[m] = LayerNorm(h[m]) (float32 or bfloat16, [M][N])
+extern "C" int sum_partials_norm(float* h, int ldh, const float* ws, int n_splits, const float* bias,
+                                 const float* gamma, const float* beta, float eps, void* out,
+                                 int out_dtype, int M, int N, hipStream_t stream) {
+  if (M == 0) return 0;
+  if (M < 0 || n_splits < 1 || !ws || !h || !out) FAIL("sum_partials_norm: bad M=%d, splits=%d or null pointer", M, n_splits);
+  if (!sum_partials_norm_takes(N, ldh) || ldh < N)
+    FAIL("sum_partials_norm: width %d (row stride %d) must be a multiple of 4, at most 8192", N, ldh);
+  if (!aligned16(h) || !aligned16(ws) || !aligned16(bias) || !aligned16(gamma) || !aligned16(beta) || !aligned16(out))
+    FAIL("sum_partials_norm: pointers must be 16-byte aligned");
+  if (out_dtype != DT_F32 && out_dtype != DT_BF16) FAIL("sum_partials_norm: unknown dtype code %d", out_dtype);
+  SumNormArgs q;
+  q.h = h, q.ws = ws, q.bias = bias, q.gamma = gamma, q.beta = beta, q.out = out, q.eps = eps;
+  q.M = M, q.N = N, q.ldh = ldh, q.n_splits = n_splits, q.out_dtype = out_dtype;
+  if (N <= 2048)
+    hipLaunchKernelGGL(sum_partials_norm_kernel<2>, dim3(M), dim3(256), 0, stream, q);
+  else
+    hipLaunchKernelGGL(sum_partials_norm_kernel<8>, dim3(M), dim3(256), 0, stream, q);
+  CHECK_LAUNCH("sum_partials_norm");
   return 0;
 }

@@ -39,6 +39,76 @@ __global__ __launch_bounds__(256) void layernorm_kernel(T* __restrict__ out,
   }
 }
 
+// One wave a row, the row held in registers (NV float4 a lane): the input is
+// read once, the statistics need no barrier.  width % 4 == 0, width <= 256 * NV.
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void layernorm_wave_kernel(T* __restrict__ out,
+                                                             const float* __restrict__ x,
+                                                             const int* __restrict__ rows,
+                                                             const float* __restrict__ gamma,
+                                                             const float* __restrict__ beta,
+                                                             float eps, int n_rows, int width) {
+  const int lane = threadIdx.x & 63;
+  const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= n_rows) return;  // whole waves leave; no barrier follows
+  const float* xr = x + (size_t)(rows ? rows[r] : r) * width;
+  float4 v[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) v[i] = *(const float4*)(xr + min((lane + 64 * i) * 4, width - 4));
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    if ((lane + 64 * i) * 4 >= width) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+  }
+  const float mean = wave_sum(s) / (float)width;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const float a = v[i].x - mean, b = v[i].y - mean, c = v[i].z - mean, d = v[i].w - mean;
+    q += (lane + 64 * i) * 4 < width ? (a * a + b * b) + (c * c + d * d) : 0.f;
+  }
+  const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)width + eps);
+  T* o = out + (size_t)r * width;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int k = (lane + 64 * i) * 4;
+    if (k >= width) continue;
+    float y[4] = {(v[i].x - mean) * rstd, (v[i].y - mean) * rstd, (v[i].z - mean) * rstd,
+                  (v[i].w - mean) * rstd};
+    if (gamma) {
+      const float4 g = *(const float4*)(gamma + k);
+      y[0] *= g.x, y[1] *= g.y, y[2] *= g.z, y[3] *= g.w;
+    }
+    if (beta) {
+      const float4 b = *(const float4*)(beta + k);
+      y[0] += b.x, y[1] += b.y, y[2] += b.z, y[3] += b.w;
+    }
+    if constexpr (sizeof(T) == 4) {
+      *(float4*)((float*)o + k) = make_float4(y[0], y[1], y[2], y[3]);
+    } else {
+      uint2 pk;
+      pk.x = f32_to_bf16_bits(y[0]) | ((uint32_t)f32_to_bf16_bits(y[1]) << 16);
+      pk.y = f32_to_bf16_bits(y[2]) | ((uint32_t)f32_to_bf16_bits(y[3]) << 16);
+      *(uint2*)((uint16_t*)o + k) = pk;
+    }
+  }
+}
+
+template <typename T>
+static void launch_wave(int nv, dim3 grid, hipStream_t stream, T* out, const float* x, const int* rows,
+                        const float* gamma, const float* beta, float eps, int n_rows, int width) {
+  dim3 block(256);
+  if (nv <= 2)
+    hipLaunchKernelGGL((layernorm_wave_kernel<T, 2>), grid, block, 0, stream, out, x, rows, gamma, beta, eps, n_rows, width);
+  else if (nv <= 4)
+    hipLaunchKernelGGL((layernorm_wave_kernel<T, 4>), grid, block, 0, stream, out, x, rows, gamma, beta, eps, n_rows, width);
+  else if (nv <= 8)
+    hipLaunchKernelGGL((layernorm_wave_kernel<T, 8>), grid, block, 0, stream, out, x, rows, gamma, beta, eps, n_rows, width);
+  else
+    hipLaunchKernelGGL((layernorm_wave_kernel<T, 16>), grid, block, 0, stream, out, x, rows, gamma, beta, eps, n_rows, width);
+}
+
 DEFINE_LAST_ERROR(mlxlm_last_error)
 
 extern "C" int layernorm(void* out, const float* x, const int* rows, const float* gamma,
@@ -47,15 +117,24 @@ extern "C" int layernorm(void* out, const float* x, const int* rows, const float
   if (n_rows <= 0) return 0;
   if (width <= 0) FAIL("layernorm: width %d must be positive", width);
   if (!out || !x) FAIL("layernorm: null pointer");
-  dim3 grid(n_rows), block(256);
-  if (out_dtype == DT_F32)
-    hipLaunchKernelGGL(layernorm_kernel<float>, grid, block, 0, stream, (float*)out, x, rows, gamma,
-                       beta, eps, width);
-  else if (out_dtype == DT_BF16)
-    hipLaunchKernelGGL(layernorm_kernel<bf16>, grid, block, 0, stream, (bf16*)out, x, rows, gamma,
-                       beta, eps, width);
-  else
-    FAIL("layernorm: unknown dtype code %d", out_dtype);
+  if (out_dtype != DT_F32 && out_dtype != DT_BF16) FAIL("layernorm: unknown dtype code %d", out_dtype);
+  const bool aligned = !(((uintptr_t)x | (uintptr_t)out | (uintptr_t)gamma | (uintptr_t)beta) & 15);
+  if (width % 4 == 0 && width <= 4096 && aligned) {  // a wave a row
+    const int nv = (width / 4 + 63) / 64;
+    dim3 grid((n_rows + 3) / 4);
+    if (out_dtype == DT_F32)
+      launch_wave<float>(nv, grid, stream, (float*)out, x, rows, gamma, beta, eps, n_rows, width);
+    else
+      launch_wave<bf16>(nv, grid, stream, (bf16*)out, x, rows, gamma, beta, eps, n_rows, width);
+  } else {
+    dim3 grid(n_rows), block(256);
+    if (out_dtype == DT_F32)
+      hipLaunchKernelGGL(layernorm_kernel<float>, grid, block, 0, stream, (float*)out, x, rows, gamma,
+                         beta, eps, width);
+    else
+      hipLaunchKernelGGL(layernorm_kernel<bf16>, grid, block, 0, stream, (bf16*)out, x, rows, gamma,
+                         beta, eps, width);
+  }
   CHECK_LAUNCH("layernorm");
   return 0;
 }

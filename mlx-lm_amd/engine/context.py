@@ -108,6 +108,11 @@ class StepContext:
         self.q_starts, self.q_lens, self.context_lens, self.state_slots = [], [], [], []
         self.attention_plan = AttentionPlan()
         self._views = {}
+        # a projection's sum into the residual stream that the next norm will add
+        from ..ops.kernels import PendingSum
+
+        self.pending = PendingSum()
+        self.wants_every_row = False  # wanted_rows is 0 .. n_tokens - 1
 
     def scratch(self, shape, dtype):
         return self._scratch.take(shape, dtype)

@@ -53,6 +53,7 @@ class DecodeGraph:
         eng, B = self.engine, self.batch
         ctx = StepContext(eng)
         ctx.n_tokens = ctx.n_requests = ctx.n_wanted = B
+        ctx.wants_every_row = True
         ctx.token_ids, ctx.positions, ctx.token_req = self._piece(0, B), self._piece(1, B), self._piece(2, B)
         ctx.wanted_rows, ctx.slot_ids = self._piece(3, B), self._piece(4, B)
         plan = AttentionPlan()

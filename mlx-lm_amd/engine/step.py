@@ -236,6 +236,7 @@ class Engine:
             return dev[offsets[i] : offsets[i] + n]
 
         ctx.n_tokens, ctx.n_requests, ctx.n_wanted = T, R, len(wanted)
+        ctx.wants_every_row = wanted == list(range(T))
         ctx.token_ids, ctx.positions, ctx.token_req = piece(0, T), piece(1, T), piece(2, T)
         ctx.wanted_rows, ctx.slot_ids = piece(3, len(wanted)), piece(4, R)
         plan.tiles, plan.rows, plan.all_tiles = piece(5, len(tiles)), piece(6, len(rows)), piece(7, len(all_tiles))

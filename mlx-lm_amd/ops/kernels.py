@@ -163,24 +163,121 @@ def for_decode(w):
 
 
 _SPLIT_WS = {}
+SPLIT_WS_FLOATS = 8 << 20  # 32 MB: sixteen splits of 64 rows by 8192 features
+
+# Tests set this to split K wherever the kernels can, also at sizes where the
+# launch would fill the GPU without (tiny models): 0 leaves the choice to the library.
+force_splits = 0
 
 
-def _split_workspace(device):
-    """Partial tiles and arrival counters for projections that split K over blocks.
+def split_workspace(device):
+    """Float32 room for the partial sums of projections that split K over blocks.
 
-    One pair per device, made at first use and kept: the kernels leave the
-    counters at zero, and launches on one stream follow each other.
+    One per device, made at first use and kept (before any step is recorded):
+    launches on one stream follow each other, and at most one sum is pending.
     """
-    key = (device.type, device.index)
-    pair = _SPLIT_WS.get(key)
-    if pair is None:
-        pair = (torch.empty(4096 * 8 * 256, dtype=torch.float32, device=device),
-                torch.zeros(4096, dtype=torch.int32, device=device))
-        _SPLIT_WS[key] = pair
-    return pair
+    device = torch.device(device)
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    ws = _SPLIT_WS.get(key)
+    if ws is None:
+        ws = torch.empty(SPLIT_WS_FLOATS, dtype=torch.float32, device=device)
+        _SPLIT_WS[key] = ws
+    return ws
 
 
-def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatter=None, splits=None):
+class PendingSum:
+    """Partial products that still have to be added into the residual stream.
+
+    A projection that splits K leaves ``n_splits`` partial sums in the
+    workspace; with a ``PendingSum`` given, ``linear(accumulate=True)`` may
+    stop there.  Whoever reads the stream next either adds them and norms the
+    rows in one kernel (``settle_normed``) or just adds them (``settle``).
+    ``allowed`` is set by a caller that promises to do so.
+    """
+
+    def __init__(self):
+        self.allowed = False
+        self.target = None
+        self.ws = self.bias = None
+        self.n_splits = 0
+
+    def waits_on(self, x):
+        return self.target is not None and self.target.data_ptr() == x.data_ptr() and self.target.shape == x.shape
+
+    def settle(self):
+        """Add what is pending (if anything) into its target."""
+        if self.target is None:
+            return
+        target, self.target = self.target, None
+        sum_partials(target, self.ws, self.n_splits, self.bias, accumulate=True)
+
+    def settle_normed(self, out, gamma, beta, eps):
+        """Add what is pending into its target and write the LayerNorm of the new rows to ``out``."""
+        target, self.target = self.target, None
+        _need(target is not None, "settle_normed: nothing is pending")
+        sum_partials_norm(target, self.ws, self.n_splits, self.bias, gamma, beta, eps, out)
+
+    def can_norm(self, x):
+        lib = build.load("gemm_bf16_decode")
+        return (self.waits_on(x) and x.stride(1) == 1
+                and bool(lib.sum_partials_norm_takes(_c_int(x.shape[1]), _c_int(x.stride(0)))))
+
+
+def _scatter_args(sc):
+    return (
+        _ptr(sc.kv.k if sc else None), _ptr(sc.kv.v if sc else None),
+        _c_size_t(sc.kv.page_stride if sc else 0), _ptr(sc.block_table if sc else None),
+        _c_int(sc.block_table.shape[1] if sc else 0), _ptr(sc.token_req if sc else None),
+        _ptr(sc.positions if sc else None), _c_int(sc.q_width if sc else 0),
+        _c_int(sc.kv_width if sc else 0), _c_int(sc.kv.head_dim if sc else 0),
+        _c_int(sc.kv.page_size if sc else 0),
+    )
+
+
+def sum_partials(out, ws, n_splits, bias=None, gelu=False, accumulate=False, scatter=None):
+    """``out = epilogue(sum of the partial products ws[:n_splits] + bias)``: the
+    second step of a projection that split K (``linear`` runs it itself unless
+    the sum stays pending)."""
+    lib = build.load("gemm_bf16_decode")
+    M, N = out.shape
+    _dev(out, "out")
+    _dev(ws, "ws", torch.float32)
+    _need(ws.numel() >= n_splits * M * N, "sum_partials: workspace too small")
+    flags = (GEMM_GELU if gelu else 0) | (GEMM_ACCUMULATE if accumulate else 0)
+    if out.dtype == torch.float32:
+        flags |= 0 if accumulate else GEMM_OUT_F32
+    else:
+        _need(out.dtype == torch.bfloat16 and not accumulate, "sum_partials: out must be float32 or bfloat16")
+    if scatter is not None:
+        flags |= GEMM_KV
+    rc = lib.sum_partials(_ptr(out), _ptr(ws), _c_int(n_splits), _ptr(bias), _c_int(M), _c_int(N),
+                          _c_int(_rows2d(out, "out")), _c_int(flags), *_scatter_args(scatter), _stream())
+    build.check(lib, rc, "sum_partials")
+    return out
+
+
+def sum_partials_norm(h, ws, n_splits, bias, gamma, beta, eps, out):
+    """``h += bias + sum of the partial products``; ``out = LayerNorm(h)`` (rows of ``h``, all of them)."""
+    lib = build.load("gemm_bf16_decode")
+    M, N = h.shape
+    _dev(h, "h", torch.float32)
+    _dev(ws, "ws", torch.float32)
+    _dev(out, "out")
+    _need(out.dtype in DT and tuple(out.shape) == (M, N) and out.is_contiguous(), "sum_partials_norm: out")
+    _need(ws.numel() >= n_splits * M * N, "sum_partials_norm: workspace too small")
+    for name, v in (("bias", bias), ("gamma", gamma), ("beta", beta)):
+        if v is not None:
+            _dev(v, name, torch.float32)
+            _need(v.numel() == N, f"sum_partials_norm: {name} has {v.numel()} elements, width is {N}")
+    rc = lib.sum_partials_norm(_ptr(h), _c_int(_rows2d(h, "h")), _ptr(ws), _c_int(n_splits), _ptr(bias),
+                               _ptr(gamma), _ptr(beta), _c_float(eps), _ptr(out), _c_int(DT[out.dtype]),
+                               _c_int(M), _c_int(N), _stream())
+    build.check(lib, rc, "sum_partials_norm")
+    return out
+
+
+def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatter=None, splits=None,
+           pending=None):
     """``out = epilogue(a @ w.T + bias)``.
 
     ``a`` is ``[M, K]`` (or a ``NormedInput``), ``w`` is ``[N, K]`` (or a
@@ -188,10 +285,13 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
     float32 or both bfloat16; ``bias`` float32.  ``accumulate`` adds into a
     float32 ``out`` (the residual stream); otherwise ``out`` is float32 or the
     operands' dtype.  With ``scatter`` (a ``KVScatter``) the columns from
-    ``scatter.q_width`` on are also written to the key/value pages.  Up to 16
-    bfloat16 rows go to the decode kernel, which fuses the norm and the
-    scatter (and splits K over ``splits`` blocks: by default as many as fill
-    the GPU); everything else is composed from the general kernels.
+    ``scatter.q_width`` on are also written to the key/value pages.  Up to 64
+    bfloat16 rows go to the decode kernels, which fuse the norm (up to 16
+    rows) and the scatter and, where the output is too narrow to fill the GPU,
+    split K over ``splits`` blocks and add the partial sums in a second
+    kernel; with ``accumulate`` and a ``pending`` that allows it, that second
+    step is left to the next reader of ``out``.  Everything else is composed
+    from the general kernels.
     """
     lazy = a if isinstance(a, NormedInput) else None
     packed = w if isinstance(w, PackedWeight) else None
@@ -212,6 +312,8 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
     if accumulate:
         _need(out.dtype == torch.float32, "linear: accumulate needs a float32 out")
         flags |= GEMM_ACCUMULATE
+        if pending is not None and pending.waits_on(out):
+            pending.settle()  # an earlier sum into the same rows goes first
     if scatter is not None:
         _need(not accumulate and not gelu and out.dtype == w.dtype, "linear: scatter goes with a plain epilogue")
         _need(scatter.q_width + 2 * scatter.kv_width == N, "linear: scatter widths do not add up to N")
@@ -223,36 +325,44 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
     else:
         _need(out.dtype == torch.bfloat16, "linear: out must be float32 or bfloat16")
 
-    # (for very wide outputs the general skinny kernel does better than the decode kernel's wide variant)
-    if w.dtype == torch.bfloat16 and variant == 0 and (0 < M <= 16 or (M <= 64 and N <= 8192)):
+    if w.dtype == torch.bfloat16 and variant == 0 and 0 < M <= 64:
         lib = build.load("gemm_bf16_decode")
         if M > 16 and lazy:
-            a, lazy = lazy.materialize(), None  # the wide kernel takes its rows normed
-        n_splits = lib.gemm_bf16_decode_splits(_c_int(N), _c_int(K), _c_int(1 if lazy else 0)) if splits is None else splits
-        if lib.gemm_bf16_decode_takes(_c_int(M), _c_int(K), _c_int(1 if lazy else 0), _c_int(n_splits)):
-            ws, counters = _split_workspace(w.device) if n_splits > 1 else (None, None)
+            a, lazy = lazy.materialize(), None  # only the 16-row kernel norms its rows itself
+        with_norm = _c_int(1 if lazy else 0)
+        if splits is None:
+            n_splits = lib.gemm_bf16_decode_splits(_c_int(M), _c_int(N), _c_int(K), with_norm, _c_int(force_splits))
+        else:
+            n_chunks = (K + 63) // 64
+            per_split = -(-n_chunks // max(1, min(splits, n_chunks)))
+            n_splits = -(-n_chunks // per_split)  # no split without k-blocks
+        ws = None
+        if n_splits > 1:
+            ws = split_workspace(w.device)
+            n_splits = max(1, min(n_splits, ws.numel() // (M * N)))
+        if lib.gemm_bf16_decode_takes(_c_int(M), _c_int(K), with_norm, _c_int(n_splits)):
             if lazy:
                 _dev(lazy.x, "x", torch.float32)
                 A, lda, X, ldx = None, 0, lazy.x, lazy.x.stride(0)
                 gamma, beta, eps = lazy.gamma, lazy.beta, lazy.eps
             else:
                 A, lda, X, ldx, gamma, beta, eps = a, _rows2d(a, "a"), None, 0, None, None, 0.0
-            sc = scatter
+            if n_splits > 1 and pending is not None:
+                pending.settle()  # the workspace is about to be written again
             rc = lib.gemm_bf16_decode(
                 _ptr(out), _ptr(A), _c_int(lda), _ptr(X), _c_int(ldx), _ptr(gamma), _ptr(beta),
                 _c_float(eps), _ptr(packed.packed if packed else w), _ptr(bias), _c_int(M), _c_int(N),
                 _c_int(K), _c_int(0 if packed else ldw),
-                _c_int(ldo), _c_int(flags | (GEMM_KV if sc else 0)),
-                _ptr(sc.kv.k if sc else None), _ptr(sc.kv.v if sc else None),
-                _c_size_t(sc.kv.page_stride if sc else 0), _ptr(sc.block_table if sc else None),
-                _c_int(sc.block_table.shape[1] if sc else 0), _ptr(sc.token_req if sc else None),
-                _ptr(sc.positions if sc else None), _c_int(sc.q_width if sc else 0),
-                _c_int(sc.kv_width if sc else 0), _c_int(sc.kv.head_dim if sc else 0),
-                _c_int(sc.kv.page_size if sc else 0), _c_int(n_splits), _ptr(ws),
-                _c_size_t(ws.numel() if ws is not None else 0), _ptr(counters),
-                _c_size_t(counters.numel() if counters is not None else 0), _stream(),
+                _c_int(ldo), _c_int(flags | (GEMM_KV if scatter else 0)), *_scatter_args(scatter),
+                _c_int(n_splits), _ptr(ws if n_splits > 1 else None),
+                _c_size_t(ws.numel() if n_splits > 1 else 0), _stream(),
             )
             build.check(lib, rc, "linear")
+            if n_splits > 1:
+                if accumulate and pending is not None and pending.allowed:
+                    pending.target, pending.ws, pending.n_splits, pending.bias = out, ws, n_splits, bias
+                else:
+                    sum_partials(out, ws, n_splits, bias, gelu=gelu, accumulate=accumulate, scatter=scatter)
             return out
 
     if lazy:

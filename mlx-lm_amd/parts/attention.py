@@ -92,7 +92,7 @@ class CausalSelfAttention(Mixer):
                 kernels.kv_write(k, v, cache.kv, cache.block_table, ctx.token_req, ctx.positions)
         out = ctx.scratch((T, self.q_width), ctx.dtype)
         self.attend(ctx, out, q, cache)
-        kernels.linear(residual, out, self.out_w, self.out_b, accumulate=True)
+        kernels.linear(residual, out, self.out_w, self.out_b, accumulate=True, pending=ctx.pending)
 
     def attend(self, ctx, out, q, cache):
         plan = ctx.attention_plan

@@ -17,12 +17,19 @@ class PreNormBlock(Block):
     def parts(self):
         return (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)
 
+    # A mixer's or feed-forward's last projection may leave its sum into ``h``
+    # pending (``ctx.pending``); the norm that reads ``h`` next adds it.
+    handles_pending = True
+
+    def _normed(self, ctx, norm, h, consumer):
+        if not getattr(norm, "settles_pending", False):
+            ctx.pending.settle()
+        return norm.forward(ctx, h, lazy=getattr(consumer, "accepts_lazy_input", False))
+
     def forward(self, ctx, h, cache, writes_cache=True):
         mark = ctx.scratch_mark()
-        lazy = getattr(self.mixer, "accepts_lazy_input", False)
-        self.mixer.forward(ctx, self.mixer_norm.forward(ctx, h, lazy=lazy), h, cache, writes_cache)
-        lazy = getattr(self.ffn, "accepts_lazy_input", False)
-        self.ffn.forward(ctx, self.ffn_norm.forward(ctx, h, lazy=lazy), h)
+        self.mixer.forward(ctx, self._normed(ctx, self.mixer_norm, h, self.mixer), h, cache, writes_cache)
+        self.ffn.forward(ctx, self._normed(ctx, self.ffn_norm, h, self.ffn), h)
         ctx.scratch_release(mark)
         return h
 

@@ -45,7 +45,7 @@ class GeluMLP(FeedForward):
     def forward(self, ctx, x, residual):
         act = ctx.scratch((x.shape[0], self.inner), ctx.dtype)
         kernels.linear(act, x, self.fc_w, self.fc_b, gelu=True)
-        kernels.linear(residual, act, self.proj_w, self.proj_b, accumulate=True)
+        kernels.linear(residual, act, self.proj_w, self.proj_b, accumulate=True, pending=ctx.pending)
 
 
 register_feed_forward("gelu_mlp", GeluMLP)

@@ -103,11 +103,23 @@ class DecoderModel:
         h = ctx.scratch((ctx.n_tokens, self.width), "float32")
         add = self.embedding_positions.embedding_term(ctx) if self.embedding_positions else None
         self.embedding.forward(ctx, h, add)
+        pending = ctx.pending
         for run in self.schedule:
-            self.layers[run.layer].forward(ctx, h, ctx.cache_view(run.cache), run.writes_cache)
+            block = self.layers[run.layer]
+            # a block that does not know of pending sums gets the stream with everything added
+            pending.allowed = getattr(block, "handles_pending", False)
+            if not pending.allowed:
+                pending.settle()
+            block.forward(ctx, h, ctx.cache_view(run.cache), run.writes_cache)
+        pending.allowed = False
+        if ctx.n_wanted == 0 or not getattr(self.final_norm, "settles_pending", False):
+            pending.settle()
         if ctx.n_wanted == 0:
             return None
-        x = self.final_norm.forward(ctx, h, rows=ctx.wanted_rows, n_rows=ctx.n_wanted)
+        if ctx.wants_every_row:
+            x = self.final_norm.forward(ctx, h)
+        else:
+            x = self.final_norm.forward(ctx, h, rows=ctx.wanted_rows, n_rows=ctx.n_wanted)
         logits = ctx.logits_out(ctx.n_wanted, self.vocab_size)
         self.head.forward(ctx, x, logits)
         return logits

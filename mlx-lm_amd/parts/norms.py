@@ -29,7 +29,17 @@ class LayerNorm(Norm):
         self.weight = tensors[self._name("weight")]
         self.bias = tensors[self._name("bias")] if self.has_bias else None
 
+    settles_pending = True  # adds a sum that is pending on ``x`` before (or while) it norms the rows
+
     def forward(self, ctx, x, rows=None, n_rows=None, lazy=False):
+        pending = ctx.pending
+        if pending.waits_on(x):
+            if rows is None and pending.can_norm(x):
+                # the last projection split its sum: add the parts and norm the new rows in one kernel
+                out = ctx.scratch((x.shape[0], self.width), ctx.dtype)
+                pending.settle_normed(out, self.weight, self.bias, self.eps)
+                return out
+            pending.settle()
         if lazy and rows is None:
             # the consumer's first matrix product may norm the rows itself
             return kernels.NormedInput(ctx.scratch, x, self.weight, self.bias, self.eps, ctx.dtype)

@@ -197,6 +197,64 @@ def test_mixed_batches_with_few_pages(folders, dtype, name, sharp):
         _close(torch.cat(got[rid]), want, dtype, f"mixed, request {rid}")
 
 
+@pytest.mark.parametrize("name,sharp", [("B", 8.0), ("C", 0.0)])
+@pytest.mark.parametrize("use_graphs", [False, True])
+def test_split_sums_in_the_engine(folders, monkeypatch, name, sharp, use_graphs):
+    """Projections that split K (forced here: tiny layers would not) leave their sums into the
+    residual stream pending between the parts; the next norm adds them.  Mixed batches and
+    recorded decode steps, against the plain implementation."""
+    from mlx_lm_amd.engine import Engine, StepEntry
+    from mlx_lm_amd.ops import kernels
+    from mlx_lm_amd.utils import load_model
+
+    calls = {"normed": 0, "plain": 0}
+    settle_normed, settle = kernels.PendingSum.settle_normed, kernels.PendingSum.settle
+
+    def count_normed(self, *a):
+        calls["normed"] += 1
+        return settle_normed(self, *a)
+
+    def count_plain(self):
+        calls["plain"] += self.target is not None
+        return settle(self)
+
+    monkeypatch.setattr(kernels, "force_splits", 2)
+    monkeypatch.setattr(kernels.PendingSum, "settle_normed", count_normed)
+    monkeypatch.setattr(kernels.PendingSum, "settle", count_plain)
+    folder, config, weights = folders[(name, sharp)]
+    P = config["n_positions"]
+    lengths = [min(P, n) for n in (100, 37, 128, 64, 90, 17)]
+    tokens, steps = _mixed_trace(config, seed=5, lengths=lengths)
+    model, _ = load_model(folder, dtype="bfloat16")
+    eng = Engine(model, dtype="bfloat16", page_size=16, n_pages=_held(lengths, 4) // 16, max_requests=8,
+                 use_graphs=use_graphs)
+    got = {rid: [] for rid in tokens}
+    for s in steps:
+        for e in s["entries"]:
+            if not eng.has_request(e["id"]):
+                eng.add_request(e["id"])
+        logits = eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        i = 0
+        for e in s["entries"]:
+            got[e["id"]].append(logits[i : i + len(e["want"])].clone())
+            i += len(e["want"])
+        for rid in s["end"]:
+            eng.end_request(rid)
+    assert calls["normed"] > 2 * len(model.layers)  # the fused kernel ran, in many steps
+    # a few tokens of which only the last is wanted: the last block's sum is added without a norm,
+    # since the final norm gathers its rows
+    extra = helpers.random_tokens(11, config["vocab_size"], seed=77)
+    eng.add_request("extra")
+    before = calls["plain"]
+    got["extra"] = [eng.step([StepEntry("extra", extra, [10])]).clone()]
+    assert calls["plain"] == before + 1
+    want = _plain_logits(weights, config, extra, "bfloat16")[10:]
+    _close(got.pop("extra")[0], want, "bfloat16", "split sums, gathered rows")
+    for rid, toks in tokens.items():
+        want = _plain_logits(weights, config, toks, "bfloat16")
+        _close(torch.cat(got[rid]), want, "bfloat16", f"split sums, request {rid}")
+
+
 @pytest.mark.parametrize("page_size", [16, 32, 64])
 def test_page_sizes_agree(folders, page_size):
     folder, config, weights = folders[("B", 8.0)]
