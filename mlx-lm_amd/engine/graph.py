@@ -1,4 +1,4 @@
-"""Decode steps recorded once as a HIP graph and replayed.
+"""Steps recorded once as a HIP graph and replayed.
 
 A step in which every request brings exactly one token and wants its logits
 has the same launches every time: only the contents of the integer arrays
@@ -7,6 +7,12 @@ once eagerly, then captured with its host-to-device copy into a graph; later
 steps of the same batch size fill the pinned host array and replay.  This
 takes the place of the reference's one-step-ahead ``mx.async_eval`` pipelining
 (mlx_lm/generate.py:446-451,1449-1456) as the cure for launch latency.
+
+Any other step has the same launches as an earlier one of the same shape
+(tokens and wanted places per request): a scheduler that cuts prompts into
+portions of one size brings the same shapes again and again.  ``StepGraph``
+records such a step; its integer arrays are built as for an eager step, but
+into a device buffer of the graph's own.
 """
 
 import numpy as np
@@ -109,4 +115,39 @@ class DecodeGraph:
             self._copied = torch.cuda.Event()
         self.graph.replay()
         self._copied.record()
+        return self.logits
+
+
+class StepGraph:
+    """A recorded step of one shape (tokens per request, number of wanted places)."""
+
+    def __init__(self, engine):
+        self.engine = engine
+        self.dev = None  # the step's integer arrays, at the same offsets every time
+        self.graph = None
+        self.logits = None
+        self.failed = False
+        self._keep = None
+
+    def run(self, entries):
+        eng = self.engine
+        ctx = eng._build_context(entries, static=self)
+        if self.graph is None:
+            # the shape has run eagerly before: libraries are loaded and scratch memory is large enough
+            graph = torch.cuda.CUDAGraph()
+            eng.scratch.frozen = True
+            try:
+                with torch.cuda.graph(graph):
+                    eng.scratch.reset()
+                    self.logits = eng.decoder.forward(ctx)
+            except Exception:
+                self.failed = True  # this shape stays eager (an error of the step itself comes again below)
+            finally:
+                eng.scratch.frozen = False
+            if self.failed:
+                eng.scratch.reset()
+                return eng.decoder.forward(ctx)
+            self.graph = graph
+            self._keep = (eng.scratch.buffer, eng._logits)
+        self.graph.replay()
         return self.logits

@@ -1,5 +1,6 @@
 """The step function: one batch of (request, its next tokens) through the model."""
 
+from collections import OrderedDict
 from dataclasses import dataclass
 from typing import List, Sequence
 
@@ -59,7 +60,7 @@ class Engine:
     """
 
     def __init__(self, model, dtype="bfloat16", device="cuda:0", page_size=16, n_pages=None,
-                 max_tokens=None, max_requests=64, use_graphs=True):
+                 max_tokens=None, max_requests=64, use_graphs=True, record_prompt_steps=False):
         if not torch.cuda.is_available():
             raise RuntimeError("the engine needs a GPU: torch.cuda.is_available() is false")
         self.model = model
@@ -81,6 +82,16 @@ class Engine:
         # decode steps are recorded as graphs where every part launches kernels only
         self.use_graphs = use_graphs and all(getattr(p, "graph_safe", False) for p in self.decoder.parts())
         self._graphs = {}
+        # Other steps whose shape keeps coming back (portions of prompts of the scheduler's size, with
+        # or without decoding requests beside them) could be recorded too.  Switched off: the first
+        # run of it ended in an abort of the process whose message was lost, and no cause has been
+        # shown since; asking for it raises until one has.
+        if record_prompt_steps:
+            raise NotImplementedError("recording steps other than decode steps is switched off: "
+                                      "its first run aborted and the cause is not known")
+        self.record_prompt_steps = False
+        self._step_graphs = OrderedDict()
+        self._shape_seen = {}
 
     # -- buffers ---------------------------------------------------------------
 
@@ -158,6 +169,8 @@ class Engine:
 
                 graph = self._graphs[len(entries)] = DecodeGraph(self, len(entries))
             logits = graph.run(entries)
+        elif self.record_prompt_steps and (graph := self._recorded_step(entries)) is not None:
+            logits = graph.run(entries)
         else:
             ctx = self._build_context(entries)
             self.scratch.reset()
@@ -167,7 +180,36 @@ class Engine:
         self.steps += 1
         return logits
 
-    def _build_context(self, entries):
+    RECORD_AFTER = 2  # sightings of a shape before its step is recorded
+    MAX_RECORDED = 24
+
+    def _recorded_step(self, entries):
+        """The recorded step for this batch's shape, if it has one (or is due one)."""
+        q_lens = tuple(len(e.tokens) for e in entries)
+        n_wanted = sum(len(e.want) for e in entries)
+        every = n_wanted == sum(q_lens) and all(list(e.want) == list(range(len(e.tokens))) for e in entries)
+        key = (q_lens, n_wanted, every)
+        graph = self._step_graphs.get(key)
+        if graph is not None:
+            self._step_graphs.move_to_end(key)
+            return None if graph.failed else graph
+        seen = self._shape_seen.get(key, 0)
+        if seen < self.RECORD_AFTER:
+            if len(self._shape_seen) > 4096:
+                self._shape_seen.clear()
+            self._shape_seen[key] = seen + 1
+            return None
+        from .graph import StepGraph
+
+        graph = self._step_graphs[key] = StepGraph(self)
+        self._shape_seen.pop(key, None)
+        while len(self._step_graphs) > self.MAX_RECORDED:
+            self._step_graphs.popitem(last=False)
+        return graph
+
+    def _build_context(self, entries, static=None):
+        """The step's context.  ``static`` (a ``StepGraph``): the integer arrays go to that graph's own
+        device buffer, at offsets that depend on the step's shape only."""
         cm = self.cache
         R = len(entries)
         T = sum(len(e.tokens) for e in entries)
@@ -200,6 +242,8 @@ class Engine:
                     big.append((rc.length + s + min(BIG_TILE_Q, n - s), q_start + s, min(BIG_TILE_Q, n - s)))
             q_start += n
         plan.n_tiles, plan.n_rows, plan.n_all_tiles = len(tiles) // 2, len(rows), len(all_tiles) // 2
+        if static is not None and rows:
+            plan.max_row_context = self.decoder.max_positions  # how keys are split must not depend on lengths
         big.sort(reverse=True)  # tiles with the most keys start first
         big_tiles = [v for _, r0, nr in big for v in (r0, nr)]
         plan.n_big_tiles = len(big)
@@ -208,6 +252,8 @@ class Engine:
         tables = []
         for gi in range(len(cm.groups)):
             width = max(1, max(len(cm.requests[e.request_id].blocks[gi]) for e in entries))
+            if static is not None:
+                width = cm.blocks_for(self.decoder.max_positions)
             flat = []
             for e in entries:
                 b = cm.requests[e.request_id].blocks[gi]
@@ -226,9 +272,16 @@ class Engine:
         for off, p in zip(offsets, pieces):
             if p:
                 host[off : off + len(p)] = torch.tensor(p, dtype=torch.int32)
-        if self._meta_dev is None or self._meta_dev.numel() < total:
-            self._meta_dev = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
-        dev = self._meta_dev
+        if static is not None:
+            if static.dev is None:
+                static.dev = torch.empty(total, dtype=torch.int32, device=self.device)
+            if static.dev.numel() != total:
+                raise RuntimeError("a recorded step's arrays changed size")
+            dev = static.dev
+        else:
+            if self._meta_dev is None or self._meta_dev.numel() < total:
+                self._meta_dev = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
+            dev = self._meta_dev
         dev[:total].copy_(host[:total], non_blocking=True)
         self._ring.mark()
 
