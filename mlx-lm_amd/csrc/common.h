@@ -61,6 +61,20 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// tanh-GELU: 0.5 x (1 + tanh(u)) with u = sqrt(2/pi) (x + 0.044715 x^3), written
+// as x / (1 + exp(-2u)): one exponential and one division instead of a tanh.
+// `gelu_tanh` keeps float accuracy; `gelu_tanh_fast` uses the hardware's
+// exponential and reciprocal (a few ulp), for results that are rounded to
+// bfloat16 anyway.  Large |x| gives x or -0 without special cases.
+__device__ __forceinline__ float gelu_tanh(float x) {
+  const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  return x / (1.0f + expf(-2.0f * u));
+}
+__device__ __forceinline__ float gelu_tanh_fast(float x) {
+  const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  return __fdividef(x, 1.0f + __expf(-2.0f * u));
+}
+
 // Sum over a block of up to 1024 threads; `red` is LDS of at least 17 floats.
 // Every thread gets the result.  Safe to call repeatedly with the same `red`.
 __device__ __forceinline__ float block_sum(float v, float* red) {

@@ -35,15 +35,9 @@ struct GemmArgs {
   int flags;
 };
 
-__device__ __forceinline__ float gelu_tanh(float x) {
-  const float c = 0.7978845608028654f;  // sqrt(2/pi)
-  const float u = c * (x + 0.044715f * x * x * x);
-  return 0.5f * x * (1.0f + tanhf(u));
-}
-
 __device__ __forceinline__ void store_out(const GemmArgs& p, int m, int n, float v) {
   if (p.bias) v += p.bias[n];
-  if (p.flags & FLAG_GELU) v = gelu_tanh(v);
+  if (p.flags & FLAG_GELU) v = gelu_tanh_fast(v);
   const size_t idx = (size_t)m * p.ldo + n;
   if (p.flags & FLAG_ACCUMULATE) {
     float* o = (float*)p.out;
@@ -57,18 +51,15 @@ __device__ __forceinline__ void store_out(const GemmArgs& p, int m, int n, float
 
 // ---------------------------------------------------------------------------
 
-#define BM 128
-#define BN 128
 #define BK 64
 #define LDS_STRIDE (BK + 8)  // 144 bytes a row: 16-byte reads of 16 rows hit distinct banks
-#define SUPER_M 8            // tiles of a super-tile along m
-#define SUPER_N 4            // and along n: 32 tiles, one per CU of a die
 
 // Which tile a block works on.  Blocks go to the eight dies (each with an L2 of
 // its own) in turn, so block b runs on die b % 8.  Tiles are grouped in
-// super-tiles of 8 x 4 that share their rows of A and of W; a die works
-// through whole super-tiles, so what one of its blocks brings into the L2 the
-// others find there.  Returns false for the padding blocks of the grid.
+// super-tiles of SUPER_M x SUPER_N that share their rows of A and of W; a die
+// works through whole super-tiles, so what one of its blocks brings into the
+// L2 the others find there.  Returns false for the padding blocks of the grid.
+template <int SUPER_M, int SUPER_N>
 __device__ __forceinline__ bool tile_of_block(int tiles_m, int tiles_n, int& tm, int& tn) {
   const int super_m = (tiles_m + SUPER_M - 1) / SUPER_M, super_n = (tiles_n + SUPER_N - 1) / SUPER_N;
   const int die = blockIdx.x & 7, local = blockIdx.x >> 3;
@@ -80,63 +71,79 @@ __device__ __forceinline__ bool tile_of_block(int tiles_m, int tiles_n, int& tm,
   return tm < tiles_m && tn < tiles_n;
 }
 
+// The shape of a block: WAVES_M x WAVES_N waves, each with TM x TN MFMA tiles of
+// 32 x 32.  What bounds this kernel is how fast a CU is fed from the L2s, so
+// the larger the block's tile, the fewer bytes per product: 128 x 128 (two
+// blocks a CU) where the matrix gives few tiles, 256 x 256 (one block a CU,
+// half the bytes) where it gives enough of them.
+template <int WAVES_M_, int WAVES_N_, int TM_, int TN_, int SUPER_M_, int SUPER_N_, int BLOCKS_PER_CU_>
+struct TileShape {
+  static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, TM = TM_, TN = TN_;
+  static constexpr int SUPER_M = SUPER_M_, SUPER_N = SUPER_N_, BLOCKS_PER_CU = BLOCKS_PER_CU_;
+  static constexpr int THREADS = 64 * WAVES_M * WAVES_N;
+  static constexpr int BM = WAVES_M * TM * 32, BN = WAVES_N * TN * 32;
+  static constexpr int PA = BM * 8 / THREADS, PB = BN * 8 / THREADS;  // 16-byte pieces a thread moves per k-block
+  static constexpr int ROW_STEP = THREADS / 8;                          // rows between a thread's pieces
+};
+using Tile128 = TileShape<2, 2, 2, 2, 8, 4, 2>;
+using Tile256 = TileShape<2, 4, 4, 2, 4, 2, 1>;
+
 // Pipeline: LDS holds two k-blocks; registers hold two more on their way.  In
 // iteration i the loads of k-block i+2 are issued, k-block i is multiplied
 // out of LDS, then k-block i+1 (loaded an iteration ago) goes from registers
 // to the other half of LDS; one barrier an iteration.
-__global__ __launch_bounds__(256, 2) void gemm_bf16_tile_kernel(GemmArgs p) {
+template <typename S>
+__global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_kernel(GemmArgs p) {
+  constexpr int BM = S::BM, BN = S::BN, TM = S::TM, TN = S::TN, PA = S::PA, PB = S::PB;
   __shared__ __attribute__((aligned(16))) uint16_t As[2][BM * LDS_STRIDE];
   __shared__ __attribute__((aligned(16))) uint16_t Bs[2][BN * LDS_STRIDE];
 
   int tm, tn;
-  if (!tile_of_block((p.M + BM - 1) / BM, (p.N + BN - 1) / BN, tm, tn)) return;
+  if (!tile_of_block<S::SUPER_M, S::SUPER_N>((p.M + BM - 1) / BM, (p.N + BN - 1) / BN, tm, tn)) return;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / S::WAVES_N, wn = wave % S::WAVES_N;
   const int m0 = tm * BM;
   const int n0 = tn * BN;
 
-  f32x16_t acc[2][2];
+  f32x16_t acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // each thread moves four 16-byte pieces of A and of W per k-block: piece c
+  // each thread moves PA 16-byte pieces of A and PB of W per k-block: piece c
   // is row c / 8, columns (c % 8) * 8 ..; rows beyond the matrix repeat its
   // last row (their products land in rows or columns that are never stored)
   // (32-bit element offsets and one LDS offset: registers are scarce here)
-  int a_off[4], b_off[4];
-  const int lds_off0 = (tid >> 3) * LDS_STRIDE + (tid & 7) * 8;  // piece i lies 32 rows further down
+  constexpr int ROW_STEP = S::ROW_STEP;
+  int a_off[PA], b_off[PB];
+  const int lds_off0 = (tid >> 3) * LDS_STRIDE + (tid & 7) * 8;  // piece i lies ROW_STEP rows further down
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int row = (tid >> 3) + 32 * i, kc = (tid & 7) * 8;
-    a_off[i] = min(m0 + row, p.M - 1) * p.lda + kc;
-    b_off[i] = min(n0 + row, p.N - 1) * p.ldw + kc;
-  }
+  for (int i = 0; i < PA; ++i) a_off[i] = min(m0 + (tid >> 3) + ROW_STEP * i, p.M - 1) * p.lda + (tid & 7) * 8;
+#pragma unroll
+  for (int i = 0; i < PB; ++i) b_off[i] = min(n0 + (tid >> 3) + ROW_STEP * i, p.N - 1) * p.ldw + (tid & 7) * 8;
   const int kc_mine = (tid & 7) * 8;
 
-  uint4 ra[2][4], rb[2][4];
-  auto load_global = [&](uint4 (&xa)[4], uint4 (&xb)[4], int k0) {
+  uint4 ra[2][PA], rb[2][PB];
+  auto load_global = [&](uint4 (&xa)[PA], uint4 (&xb)[PB], int k0) {
     // a piece beyond K is read from where it still fits and zeroed when it goes to LDS
     // (zeroing it here would make the loads wait at once)
     const int kk = (k0 + kc_mine < p.K) ? k0 : 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      xa[i] = *(const uint4*)(p.A + a_off[i] + kk);
-      xb[i] = *(const uint4*)(p.W + b_off[i] + kk);
-    }
+    for (int i = 0; i < PA; ++i) xa[i] = *(const uint4*)(p.A + a_off[i] + kk);
+#pragma unroll
+    for (int i = 0; i < PB; ++i) xb[i] = *(const uint4*)(p.W + b_off[i] + kk);
   };
-  auto store_lds = [&](int stage, const uint4 (&xa)[4], const uint4 (&xb)[4], int k0) {
+  auto store_lds = [&](int stage, const uint4 (&xa)[PA], const uint4 (&xb)[PB], int k0) {
     const bool in = k0 + kc_mine < p.K;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      *(uint4*)(As[stage] + lds_off0 + i * 32 * LDS_STRIDE) = in ? xa[i] : ZERO4;
-      *(uint4*)(Bs[stage] + lds_off0 + i * 32 * LDS_STRIDE) = in ? xb[i] : ZERO4;
-    }
+    for (int i = 0; i < PA; ++i) *(uint4*)(As[stage] + lds_off0 + i * ROW_STEP * LDS_STRIDE) = in ? xa[i] : ZERO4;
+#pragma unroll
+    for (int i = 0; i < PB; ++i) *(uint4*)(Bs[stage] + lds_off0 + i * ROW_STEP * LDS_STRIDE) = in ? xb[i] : ZERO4;
   };
 
   const int n_blocks = (p.K + BK - 1) / BK;
@@ -147,23 +154,23 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_tile_kernel(GemmArgs p) {
 
   const int frag_row = lane & 31;
   const int frag_k = (lane >> 5) * 8;
-  const uint16_t* a_frag = As[0] + (wm * 64 + frag_row) * LDS_STRIDE + frag_k;
-  const uint16_t* b_frag = Bs[0] + (wn * 64 + frag_row) * LDS_STRIDE + frag_k;
+  const uint16_t* a_frag = As[0] + (wm * TM * 32 + frag_row) * LDS_STRIDE + frag_k;
+  const uint16_t* b_frag = Bs[0] + (wn * TN * 32 + frag_row) * LDS_STRIDE + frag_k;
 
   auto multiply = [&](int stage) {
     const uint16_t* af = a_frag + stage * (BM * LDS_STRIDE);
     const uint16_t* bf = b_frag + stage * (BN * LDS_STRIDE);
 #pragma unroll
     for (int ks = 0; ks < BK; ks += 16) {
-      bf16x8_t a[2], b[2];
+      bf16x8_t a[TM], b[TN];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) a[i] = *(const bf16x8_t*)(af + i * 32 * LDS_STRIDE + ks);
+      for (int i = 0; i < TM; ++i) a[i] = *(const bf16x8_t*)(af + i * 32 * LDS_STRIDE + ks);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) b[j] = *(const bf16x8_t*)(bf + j * 32 * LDS_STRIDE + ks);
+      for (int j = 0; j < TN; ++j) b[j] = *(const bf16x8_t*)(bf + j * 32 * LDS_STRIDE + ks);
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
     }
   };
@@ -172,19 +179,17 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_tile_kernel(GemmArgs p) {
   // The steady part has no branch and no select inside: only then does the
   // compiler count exactly how many loads may stay in flight at each wait
   // (a conditional load makes it wait for all of them).
-  auto load_whole = [&](uint4 (&xa)[4], uint4 (&xb)[4], int k0) {  // a k-block that lies inside K
+  auto load_whole = [&](uint4 (&xa)[PA], uint4 (&xb)[PB], int k0) {  // a k-block that lies inside K
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      xa[i] = *(const uint4*)(p.A + a_off[i] + k0);
-      xb[i] = *(const uint4*)(p.W + b_off[i] + k0);
-    }
+    for (int i = 0; i < PA; ++i) xa[i] = *(const uint4*)(p.A + a_off[i] + k0);
+#pragma unroll
+    for (int i = 0; i < PB; ++i) xb[i] = *(const uint4*)(p.W + b_off[i] + k0);
   };
-  auto store_whole = [&](int stage, const uint4 (&xa)[4], const uint4 (&xb)[4]) {
+  auto store_whole = [&](int stage, const uint4 (&xa)[PA], const uint4 (&xb)[PB]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      *(uint4*)(As[stage] + lds_off0 + i * 32 * LDS_STRIDE) = xa[i];
-      *(uint4*)(Bs[stage] + lds_off0 + i * 32 * LDS_STRIDE) = xb[i];
-    }
+    for (int i = 0; i < PA; ++i) *(uint4*)(As[stage] + lds_off0 + i * ROW_STEP * LDS_STRIDE) = xa[i];
+#pragma unroll
+    for (int i = 0; i < PB; ++i) *(uint4*)(Bs[stage] + lds_off0 + i * ROW_STEP * LDS_STRIDE) = xb[i];
   };
   int kb = 0;
   const int whole_blocks = p.K / BK;  // k-blocks that need no masking
@@ -221,13 +226,13 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_tile_kernel(GemmArgs p) {
   // 32x32 tile before anything is stored: a load that comes after a store to
   // memory it might alias waits for it, sixteen times over.
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+  for (int j = 0; j < TN; ++j) {
+    const int n = n0 + wn * TN * 32 + j * 32 + (lane & 31);
     const int nc = min(n, p.N - 1);
     const float bias = p.bias ? p.bias[nc] : 0.f;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int mb = m0 + wm * 64 + i * 32 + 4 * (lane >> 5);
+    for (int i = 0; i < TM; ++i) {
+      const int mb = m0 + wm * TM * 32 + i * 32 + 4 * (lane >> 5);
       float v[16];
       if (p.flags & FLAG_ACCUMULATE) {
         const float* o = (const float*)p.out;
@@ -240,7 +245,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16_tile_kernel(GemmArgs p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           v[r] = acc[i][j][r] + bias;
-          if (p.flags & FLAG_GELU) v[r] = gelu_tanh(v[r]);
+          if (p.flags & FLAG_GELU) v[r] = gelu_tanh_fast(v[r]);
         }
       }
       if (n >= p.N) continue;
@@ -354,7 +359,31 @@ static int check_args(const GemmArgs& p) {
   return 0;
 }
 
-// variant: 0 = choose, 1 = tile kernel, 2 = skinny kernel
+template <typename S>
+static void launch_tiles(const GemmArgs& p, hipStream_t stream) {
+  const int super_m = ((p.M + S::BM - 1) / S::BM + S::SUPER_M - 1) / S::SUPER_M;
+  const int super_n = ((p.N + S::BN - 1) / S::BN + S::SUPER_N - 1) / S::SUPER_N;
+  const int per_die = (super_m * super_n + 7) / 8;  // super-tiles a die works through
+  dim3 grid(per_die * 8 * S::SUPER_M * S::SUPER_N), block(S::THREADS);
+  hipLaunchKernelGGL(gemm_bf16_tile_kernel<S>, grid, block, 0, stream, p);
+}
+
+// Microseconds per k-block of the busiest CU, from what was measured at GPT-2 XL
+// sizes: two 128 x 128 blocks on a CU finish a k-block each in 1.15 us, one
+// alone in 1.3 us (its fetching and its arithmetic take turns; two blocks
+// overlap each other's), a 256 x 256 block (four times the work) in 2.2 us.
+static double cost_128(int M, int N) {
+  const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+  const long rest = tiles % 512;
+  // (a last round of few blocks finds the L2s idle: 1.0)
+  return (double)(tiles / 512) * 1.15 + (rest == 0 ? 0.0 : rest <= 128 ? 1.0 : rest <= 256 ? 1.3 : 1.15);
+}
+static double cost_256(int M, int N) {
+  const long tiles = (long)((M + 255) / 256) * ((N + 255) / 256);
+  return (double)((tiles + 255) / 256) * 2.2;
+}
+
+// variant: 0 = choose, 1 = 128 x 128 tiles, 2 = skinny kernel, 3 = 256 x 256 tiles
 extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* bias, int M, int N,
                          int K, int lda, int ldw, int ldo, int flags, int variant,
                          hipStream_t stream) {
@@ -368,7 +397,12 @@ extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* b
   p.flags = flags;
   if (check_args(p)) return 1;
   if (M == 0) return 0;
-  if (variant == 0) variant = (M <= SK_MAXM) ? 2 : 1;
+  if (variant == 0) {
+    if (M <= SK_MAXM)
+      variant = 2;
+    else
+      variant = cost_256(M, N) < cost_128(M, N) ? 3 : 1;
+  }
   if (variant == 2) {
     if (M > SK_MAXM) FAIL("gemm_bf16: the skinny kernel takes at most %d rows, got %d", SK_MAXM, M);
     dim3 grid((N + 15) / 16), block(256);
@@ -381,12 +415,11 @@ extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* b
       hipLaunchKernelGGL(gemm_bf16_skinny_kernel<3>, grid, block, 0, stream, p);
     else
       hipLaunchKernelGGL(gemm_bf16_skinny_kernel<4>, grid, block, 0, stream, p);
-  } else if (variant == 1) {
-    const int super_m = ((M + BM - 1) / BM + SUPER_M - 1) / SUPER_M;
-    const int super_n = ((N + BN - 1) / BN + SUPER_N - 1) / SUPER_N;
-    const int per_die = (super_m * super_n + 7) / 8;  // super-tiles a die works through
-    dim3 grid(per_die * 8 * SUPER_M * SUPER_N), block(256);
-    hipLaunchKernelGGL(gemm_bf16_tile_kernel, grid, block, 0, stream, p);
+  } else if (variant == 1 || variant == 3) {
+    if (variant == 1)
+      launch_tiles<Tile128>(p, stream);
+    else
+      launch_tiles<Tile256>(p, stream);
   } else {
     FAIL("gemm_bf16: unknown variant %d", variant);
   }

@@ -77,12 +77,6 @@ struct DecodeGemmArgs {
   int vec4;            // four outputs at a time: N, ldo and the scatter widths are multiples of 4, pointers aligned
 };
 
-__device__ __forceinline__ float gelu_tanh(float x) {
-  const float c = 0.7978845608028654f;
-  const float u = c * (x + 0.044715f * x * x * x);
-  return 0.5f * x * (1.0f + tanhf(u));
-}
-
 __device__ __forceinline__ uint32_t pack2(float a, float b) {
   return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
 }
@@ -95,7 +89,7 @@ union Frag {
 // bias, activation and where one output goes: the matrix, the residual stream or a cache page
 __device__ __forceinline__ void finish(const DecodeGemmArgs& p, int m, int n, float v) {
   if (p.bias) v += p.bias[n];
-  if (p.flags & FLAG_GELU) v = gelu_tanh(v);
+  if (p.flags & FLAG_GELU) v = gelu_tanh_fast(v);
   if ((p.flags & FLAG_KV) && n >= p.q_width) {
     const int c = n - p.q_width;
     const bool is_v = c >= p.kv_width;
@@ -123,7 +117,7 @@ __device__ __forceinline__ void finish4(const DecodeGemmArgs& p, int m, int n, f
     const float4 b = *(const float4*)(p.bias + n);
     v.x += b.x, v.y += b.y, v.z += b.z, v.w += b.w;
   }
-  if (p.flags & FLAG_GELU) v.x = gelu_tanh(v.x), v.y = gelu_tanh(v.y), v.z = gelu_tanh(v.z), v.w = gelu_tanh(v.w);
+  if (p.flags & FLAG_GELU) v.x = gelu_tanh_fast(v.x), v.y = gelu_tanh_fast(v.y), v.z = gelu_tanh_fast(v.z), v.w = gelu_tanh_fast(v.w);
   uint2 packed;
   packed.x = pack2(v.x, v.y), packed.y = pack2(v.z, v.w);
   if ((p.flags & FLAG_KV) && n >= p.q_width) {

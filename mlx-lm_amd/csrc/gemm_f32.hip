@@ -25,12 +25,6 @@ struct GemmArgs {
   int flags;
 };
 
-__device__ __forceinline__ float gelu_tanh(float x) {
-  const float c = 0.7978845608028654f;  // sqrt(2/pi)
-  const float u = c * (x + 0.044715f * x * x * x);
-  return 0.5f * x * (1.0f + tanhf(u));
-}
-
 #define BK 16
 #define LDS_STRIDE (BK + 1)
 
