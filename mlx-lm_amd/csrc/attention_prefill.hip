@@ -97,6 +97,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(PrefillArgs p) {
   const int kt0 = (k_lo / KT) * KT;
   // keys this wave's queries can see end here; later tiles it only helps to load
   const int wave_hi = min(k_hi, pos0 + wave * 32 + 32);
+  const int wave_q0 = pos0 + wave * 32;            // position of the wave's first query
+  const float c2 = p.scale * 1.4426950408889634f;  // scores to units of log 2
 
   float m = -INFINITY, l = 0.f;
   f32x16_t ot[DT];
@@ -178,21 +180,35 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(PrefillArgs p) {
         st[s] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, qf[dc].v, st[s], 0, 0, 0);
       }
     }
-    // element r of subtile s: key kt + 32 s + 16 (r / 8) + 8 g + r % 8
+    // element r of subtile s: key kt + 32 s + 16 (r / 8) + 8 g + r % 8.
+    // Scores are kept in units of log 2 (scale * log2(e) folded into one
+    // factor), so that a probability is one fused multiply-add and one
+    // v_exp_f32.  Tiles that every query of the wave sees whole (below the
+    // diagonal, inside the window) skip the masks: this arithmetic, not the
+    // MFMAs, is what the kernel's time goes to.
+    const bool whole = kt + KT - 1 <= wave_q0 && (p.window <= 0 || kt >= wave_q0 + 31 - p.window + 1);
     float tmax = -INFINITY;
+    if (whole) {
 #pragma unroll
-    for (int s = 0; s < 2; ++s)
+      for (int s = 0; s < 2; ++s)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int key = kt + 32 * s + 16 * (r >> 3) + 8 * g + (r & 7);
-        const bool ok = q_live && key <= qpos && key >= q_lo;
-        st[s][r] = ok ? st[s][r] * p.scale : -INFINITY;
-        tmax = fmaxf(tmax, st[s][r]);
-      }
+        for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, st[s][r]);
+      tmax *= c2;  // c2 > 0: the largest score stays the largest
+    } else {
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = kt + 32 * s + 16 * (r >> 3) + 8 * g + (r & 7);
+          const bool ok = q_live && key <= qpos && key >= q_lo;
+          st[s][r] = ok ? st[s][r] : -INFINITY;
+          tmax = fmaxf(tmax, st[s][r] * c2);
+        }
+    }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
     const float m_new = fmaxf(m, tmax);
     const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // a row with no key yet
-    const float alpha = __expf(m - m_use);
+    const float alpha = exp2f(m - m_use);
     float lsum = 0.f;
     Frag8 pf[2][2];
 #pragma unroll
@@ -202,21 +218,24 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(PrefillArgs p) {
         float e[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          e[i] = __expf(st[s][8 * c + i] - m_use);
+          e[i] = __builtin_amdgcn_exp2f(fmaf(st[s][8 * c + i], c2, -m_use));
           lsum += e[i];
         }
-        pf[s][c].u.x = (uint32_t)f32_to_bf16_bits(e[0]) | ((uint32_t)f32_to_bf16_bits(e[1]) << 16);
-        pf[s][c].u.y = (uint32_t)f32_to_bf16_bits(e[2]) | ((uint32_t)f32_to_bf16_bits(e[3]) << 16);
-        pf[s][c].u.z = (uint32_t)f32_to_bf16_bits(e[4]) | ((uint32_t)f32_to_bf16_bits(e[5]) << 16);
-        pf[s][c].u.w = (uint32_t)f32_to_bf16_bits(e[6]) | ((uint32_t)f32_to_bf16_bits(e[7]) << 16);
+        pf[s][c].u.x = pack_bf16x2(e[0], e[1]);
+        pf[s][c].u.y = pack_bf16x2(e[2], e[3]);
+        pf[s][c].u.z = pack_bf16x2(e[4], e[5]);
+        pf[s][c].u.w = pack_bf16x2(e[6], e[7]);
       }
     l = l * alpha + lsum;
     m = m_new;
     // ---- O^T = O^T * alpha + V^T P^T ---------------------------------------------
+    const bool rescale = __any(alpha != 1.0f);  // no row's maximum moved: nothing to scale
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
+      if (rescale) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) ot[dt][r] *= alpha;
+        for (int r = 0; r < 16; ++r) ot[dt][r] *= alpha;
+      }
       const uint16_t* vrow = Vt + (dt * 32 + ql) * VT_STRIDE + 8 * g;
 #pragma unroll
       for (int s = 0; s < 2; ++s)
@@ -240,10 +259,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(PrefillArgs p) {
       for (int j = 0; j < 4; ++j) {
         // accumulators 4j .. 4j+3: head columns dt*32 + 8j + 4g + (0..3)
         uint2 o;
-        o.x = (uint32_t)f32_to_bf16_bits(ot[dt][4 * j] * inv) |
-              ((uint32_t)f32_to_bf16_bits(ot[dt][4 * j + 1] * inv) << 16);
-        o.y = (uint32_t)f32_to_bf16_bits(ot[dt][4 * j + 2] * inv) |
-              ((uint32_t)f32_to_bf16_bits(ot[dt][4 * j + 3] * inv) << 16);
+        o.x = pack_bf16x2(ot[dt][4 * j] * inv, ot[dt][4 * j + 1] * inv);
+        o.y = pack_bf16x2(ot[dt][4 * j + 2] * inv, ot[dt][4 * j + 3] * inv);
         *(uint2*)(orow + dt * 32 + 8 * j + 4 * g) = o;
       }
   }

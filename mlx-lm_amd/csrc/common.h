@@ -29,12 +29,18 @@ __device__ __forceinline__ float bits_to_f32(uint16_t b) {
   return __uint_as_float(((uint32_t)b) << 16);
 }
 
-// round to nearest even, NaN kept quiet
+// Round to nearest even, NaN kept quiet: gfx950 has an instruction for it
+// (v_cvt_pk_bf16_f32, two values at a time), which the compiler picks for the
+// conversion of a float vector to __bf16.
+typedef __bf16 hw_bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float hw_f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  const hw_f32x2_t v = {lo, hi};
+  const hw_bf16x2_t b = __builtin_convertvector(v, hw_bf16x2_t);
+  return __builtin_bit_cast(uint32_t, b);
+}
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  return (uint16_t)(pack_bf16x2(f, 0.f) & 0xffffu);
 }
 
 template <typename T>

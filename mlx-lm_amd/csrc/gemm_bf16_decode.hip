@@ -77,9 +77,7 @@ struct DecodeGemmArgs {
   int vec4;            // four outputs at a time: N, ldo and the scatter widths are multiples of 4, pointers aligned
 };
 
-__device__ __forceinline__ uint32_t pack2(float a, float b) {
-  return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
-}
+__device__ __forceinline__ uint32_t pack2(float a, float b) { return pack_bf16x2(a, b); }
 
 union Frag {
   uint4 u;
@@ -593,7 +591,7 @@ extern "C" int gemm_bf16_decode_splits(int M, int N, int K, int with_norm, int f
     want = force;
   } else if (M <= 16) {
     const int n_blocks = (N + 15) / 16;
-    if (n_blocks >= 200) return 1;
+    if (n_blocks >= 200 || M < 4) return 1;  // (one to three rows: the next projection's norm prologue is cheaper than a second kernel)
     want = (512 + n_blocks - 1) / n_blocks;  // two blocks a CU (measured at N = 1600: K = 6400 is best in 5, K = 1600 in 2 to 6)
     if (want > n_chunks / 4) want = n_chunks / 4;  // at least four k-blocks a split
   } else {

@@ -738,6 +738,7 @@ def test_default_splits_fill_the_gpu():
     lib = k.build.load("gemm_bf16_decode")
     assert lib.gemm_bf16_decode_splits(8, 4800, 1600, 0, 0) == 1
     assert lib.gemm_bf16_decode_splits(8, 1600, 6400, 0, 0) > 1
+    assert lib.gemm_bf16_decode_splits(1, 1600, 6400, 0, 0) == 1  # a row or two: the norm prologue is cheaper
     assert lib.gemm_bf16_decode_splits(8, 1600, 1600, 1, 0) == 1  # the norm prologue needs whole rows
     assert lib.gemm_bf16_decode_splits(64, 1600, 6400, 0, 0) > 1
     assert lib.gemm_bf16_decode_splits(64, 50257, 1600, 0, 0) == 1
