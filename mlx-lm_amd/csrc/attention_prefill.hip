@@ -23,6 +23,7 @@
 //    eight 32-bit words (two keys each).
 //  * Online softmax in 32-bit per lane; outputs leave as O^T accumulators.
 #include "common.h"
+#include <type_traits>
 
 struct PrefillArgs {
   uint16_t* out;
@@ -55,7 +56,7 @@ __device__ __forceinline__ int key_of_row(int rho) {
 }
 
 template <int HD>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(PrefillArgs p) {
+__global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(PrefillArgs p) {
   constexpr int KS_STRIDE = HD + 8;
   constexpr int DC = HD / 16;           // 16-column chunks of a head (QK contraction steps)
   constexpr int DT = HD / 32;           // 32-row tiles of O^T
@@ -107,64 +108,83 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(PrefillArgs p) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) ot[dt][r] = 0.f;
 
-  uint4 kreg[K_PER_T], vreg[V_PER_T][2];
+  // two tiles on their way (the keys' two sets as arrays of their own: as one array
+  // indexed by the set they stayed in scratch memory)
+  uint4 kreg0[K_PER_T], kreg1[K_PER_T], vreg[2][V_PER_T][2];
 
-  auto address = [&](int key, int col) -> size_t {
-    const int kk = min(max(key, k_lo), k_hi - 1);  // pulled into range; zeroed by the caller
-    const int page = table[kk / p.page_size];
+  // The request's page numbers go to LDS once: a load of keys or values then
+  // depends on no other load from memory, and two tiles can be on their way
+  // while one is multiplied.  (Looked up from memory per load, every load
+  // waited for its page number first: eight trips to memory in a row per tile.)
+  extern __shared__ int page_of[];  // [max_blocks]
+  const int pg0 = k_lo / p.page_size;
+  const int n_pg = (k_hi - 1) / p.page_size - pg0 + 1;
+  for (int i = tid; i < n_pg; i += 256) page_of[i] = table[pg0 + i];
+  __syncthreads();
+
+  // Loads are never predicated and never zeroed: a key outside [k_lo, k_hi) is
+  // read from the nearest key inside (a valid address with finite numbers);
+  // its score is masked below, so its probability is zero.
+  auto address = [&](int key, int col) __attribute__((always_inline)) -> size_t {
+    const int kk = min(max(key, k_lo), k_hi - 1);
+    const int page = page_of[kk / p.page_size - pg0];
     return (size_t)page * p.page_stride + head_off + (size_t)(kk % p.page_size) * HD + col;
   };
-  auto fetch = [&](int kt) {
+  auto fetch = [&](int kt, const int set) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < K_PER_T; ++i) {
       const int c = min(tid + 256 * i, K_CHUNKS - 1);  // surplus threads repeat the last piece
-      const int key = kt + c / (HD / 8), col = (c % (HD / 8)) * 8;
-      const uint4 t = *(const uint4*)(p.k_pages + address(key, col));
-      kreg[i] = (key >= k_lo && key < k_hi) ? t : make_uint4(0u, 0u, 0u, 0u);
+      const uint4 t = *(const uint4*)(p.k_pages + address(kt + c / (HD / 8), (c % (HD / 8)) * 8));
+      if (set == 0) kreg0[i] = t; else kreg1[i] = t;
     }
 #pragma unroll
     for (int i = 0; i < V_PER_T; ++i) {
       const int it = min(tid + 256 * i, V_ITEMS - 1);
       const int jp = it % (KT / 2), col = (it / (KT / 2)) * 8;
 #pragma unroll
-      for (int e = 0; e < 2; ++e) {
-        const int key = kt + 2 * jp + e;
-        const uint4 t = *(const uint4*)(p.v_pages + address(key, col));
-        vreg[i][e] = (key >= k_lo && key < k_hi) ? t : make_uint4(0u, 0u, 0u, 0u);
-      }
+      for (int e = 0; e < 2; ++e) vreg[set][i][e] = *(const uint4*)(p.v_pages + address(kt + 2 * jp + e, col));
     }
   };
-  auto stage = [&]() {
+  auto stage = [&](const int set) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < K_PER_T; ++i) {
       const int c = tid + 256 * i;
       if (K_CHUNKS % 256 == 0 || c < K_CHUNKS)
-        *(uint4*)(Ks + (c / (HD / 8)) * KS_STRIDE + (c % (HD / 8)) * 8) = kreg[i];
+        *(uint4*)(Ks + (c / (HD / 8)) * KS_STRIDE + (c % (HD / 8)) * 8) = set == 0 ? kreg0[i] : kreg1[i];
     }
 #pragma unroll
     for (int i = 0; i < V_PER_T; ++i) {
       const int it = tid + 256 * i;
-      if (V_ITEMS % 256 != 0 && it >= V_ITEMS) continue;
-      const int jp = it % (KT / 2), col = (it / (KT / 2)) * 8;
-      const uint32_t a[4] = {vreg[i][0].x, vreg[i][0].y, vreg[i][0].z, vreg[i][0].w};
-      const uint32_t b[4] = {vreg[i][1].x, vreg[i][1].y, vreg[i][1].z, vreg[i][1].w};
-      uint32_t* dst = (uint32_t*)(Vt + col * VT_STRIDE + 2 * jp);
+      if (V_ITEMS % 256 == 0 || it < V_ITEMS) {
+        const int jp = it % (KT / 2), col = (it / (KT / 2)) * 8;
+        const uint32_t a[4] = {vreg[set][i][0].x, vreg[set][i][0].y, vreg[set][i][0].z, vreg[set][i][0].w};
+        const uint32_t b[4] = {vreg[set][i][1].x, vreg[set][i][1].y, vreg[set][i][1].z, vreg[set][i][1].w};
+        uint32_t* dst = (uint32_t*)(Vt + col * VT_STRIDE + 2 * jp);
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        // columns col+2w and col+2w+1 of keys 2jp (low half) and 2jp+1 (high half)
-        dst[(2 * w) * (VT_STRIDE / 2)] = (a[w] & 0xffffu) | (b[w] << 16);
-        dst[(2 * w + 1) * (VT_STRIDE / 2)] = (a[w] >> 16) | (b[w] & 0xffff0000u);
+        for (int w = 0; w < 4; ++w) {
+          // columns col+2w and col+2w+1 of keys 2jp (low half) and 2jp+1 (high half)
+          dst[(2 * w) * (VT_STRIDE / 2)] = (a[w] & 0xffffu) | (b[w] << 16);
+          dst[(2 * w + 1) * (VT_STRIDE / 2)] = (a[w] >> 16) | (b[w] & 0xffff0000u);
+        }
       }
     }
   };
 
-  fetch(kt0);
-  for (int kt = kt0; kt < k_hi; kt += KT) {
+  // One tile: its keys and values go from registers to LDS, the registers take
+  // the tile after the next, then the arithmetic.
+  // `steady` (a compile-time flag): the tile lies below every query of the block
+  // and there is no window, so no wave is idle and nothing is masked; a loop of
+  // such tiles has no branch inside, and the compiler lets the loads of the
+  // other register set stay in flight while this one is staged.
+  auto one_tile = [&](int kt, const int set, auto steady) __attribute__((always_inline)) {
+    constexpr bool STEADY = decltype(steady)::value;
     __syncthreads();  // the previous tile is no longer read
-    stage();
+    stage(set);
     __syncthreads();
-    if (kt + KT < k_hi) fetch(kt + KT);  // in flight during the arithmetic below
-    if (kt >= wave_hi || wave * 32 >= nq) continue;  // nothing here for this wave (uniform)
+    fetch(kt + 2 * KT, set);  // (beyond the last tile: harmless reads of the last key)
+    if constexpr (!STEADY) {
+      if (kt >= wave_hi || wave * 32 >= nq) return;  // nothing here for this wave (uniform)
+    }
 
     // ---- S^T = K Q^T for the two 32-key subtiles --------------------------------
     f32x16_t st[2];
@@ -186,7 +206,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(PrefillArgs p) {
     // v_exp_f32.  Tiles that every query of the wave sees whole (below the
     // diagonal, inside the window) skip the masks: this arithmetic, not the
     // MFMAs, is what the kernel's time goes to.
-    const bool whole = kt + KT - 1 <= wave_q0 && (p.window <= 0 || kt >= wave_q0 + 31 - p.window + 1);
+    const bool whole = STEADY || (kt + KT - 1 <= wave_q0 && (p.window <= 0 || kt >= wave_q0 + 31 - p.window + 1));
     float tmax = -INFINITY;
     if (whole) {
 #pragma unroll
@@ -246,6 +266,21 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(PrefillArgs p) {
           ot[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pf[s][c].v, ot[dt], 0, 0, 0);
         }
     }
+  };
+
+  fetch(kt0, 0);
+  fetch(kt0 + KT, 1);
+  int kt = kt0;
+  if (p.window <= 0) {
+    for (; kt + 2 * KT - 1 <= pos0; kt += 2 * KT) {
+      one_tile(kt, 0, std::true_type{});
+      one_tile(kt + KT, 1, std::true_type{});
+    }
+  }
+  for (; kt < k_hi; kt += 2 * KT) {  // the tiles around the diagonal, or all of them under a window
+    one_tile(kt, 0, std::false_type{});
+    if (kt + KT >= k_hi) break;  // uniform
+    one_tile(kt + KT, 1, std::false_type{});
   }
 
   // the two halves of the wave hold different keys of the same query
@@ -298,12 +333,16 @@ extern "C" int attn_prefill(void* out, const void* q, int ldq, int ldo, const vo
   p.n_heads = n_heads, p.n_kv_heads = n_kv_heads, p.page_size = page_size, p.window = window;
   p.scale = scale;
   dim3 grid(n_tiles, n_heads), block(256);
+  // a request's page numbers lie in LDS beside the tiles
+  if (max_blocks > 7168)
+    FAIL("attn_prefill: block tables of %d pages a request do not fit beside the tiles (at most 7168)", max_blocks);
+  const size_t lds = (size_t)max_blocks * sizeof(int);
   if (head_dim == 32)
-    hipLaunchKernelGGL(attn_prefill_kernel<32>, grid, block, 0, stream, p);
+    hipLaunchKernelGGL(attn_prefill_kernel<32>, grid, block, lds, stream, p);
   else if (head_dim == 64)
-    hipLaunchKernelGGL(attn_prefill_kernel<64>, grid, block, 0, stream, p);
+    hipLaunchKernelGGL(attn_prefill_kernel<64>, grid, block, lds, stream, p);
   else
-    hipLaunchKernelGGL(attn_prefill_kernel<128>, grid, block, 0, stream, p);
+    hipLaunchKernelGGL(attn_prefill_kernel<128>, grid, block, lds, stream, p);
   CHECK_LAUNCH("attn_prefill");
   return 0;
 }
