@@ -37,6 +37,7 @@ struct PrefillArgs {
   size_t page_stride;
   int ldq, ldo, max_blocks;
   int n_heads, n_kv_heads, page_size, window;
+  int page_shift;  // log2(page_size), or -1 if that is no power of two
   float scale;
 };
 
@@ -127,8 +128,11 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
   // its score is masked below, so its probability is zero.
   auto address = [&](int key, int col) __attribute__((always_inline)) -> size_t {
     const int kk = min(max(key, k_lo), k_hi - 1);
-    const int page = page_of[kk / p.page_size - pg0];
-    return (size_t)page * p.page_stride + head_off + (size_t)(kk % p.page_size) * HD + col;
+    // (a division by a run-time number costs some thirty instructions, and there are four
+    // addresses a thread and tile: page sizes that are powers of two take a shift instead)
+    const int idx = p.page_shift >= 0 ? kk >> p.page_shift : kk / p.page_size;
+    const int row = kk - idx * p.page_size;
+    return (size_t)page_of[idx - pg0] * p.page_stride + head_off + (size_t)(row * HD + col);
   };
   auto fetch = [&](int kt, const int set) __attribute__((always_inline)) {
 #pragma unroll
@@ -330,6 +334,9 @@ extern "C" int attn_prefill(void* out, const void* q, int ldq, int ldo, const vo
   p.k_pages = (const uint16_t*)k_pages, p.v_pages = (const uint16_t*)v_pages;
   p.block_table = block_table, p.token_req = token_req, p.positions = positions, p.tiles = tiles;
   p.page_stride = page_stride, p.ldq = ldq, p.ldo = ldo, p.max_blocks = max_blocks;
+  p.page_shift = -1;
+  for (int sh = 0; sh < 31; ++sh)
+    if ((1 << sh) == page_size) p.page_shift = sh;
   p.n_heads = n_heads, p.n_kv_heads = n_kv_heads, p.page_size = page_size, p.window = window;
   p.scale = scale;
   dim3 grid(n_tiles, n_heads), block(256);

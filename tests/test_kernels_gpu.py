@@ -304,6 +304,8 @@ PREFILL_CASES = [c for c in ATTN_CASES if c[2] in (32, 64, 128)] + [
     (4, 2, 32, 16, [5, 0], [260, 64], 0),
     (2, 1, 128, 32, [190, 0], [70, 200], 0),
     (5, 5, 64, 16, [0, 400], [333, 128], 90),
+    (2, 2, 64, 48, [30, 0], [200, 150], 0),  # a page size that is no power of two
+    (3, 1, 32, 80, [0, 77], [170, 40], 60),
 ]
 
 
