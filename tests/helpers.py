@@ -54,7 +54,7 @@ def round_matrices_to_bf16(weights):
     """What the engine's bfloat16 path holds: matrices rounded, vectors as they are."""
     out = {}
     for k, v in weights.items():
-        out[k] = v.to(torch.bfloat16).float() if v.dim() == 2 else v
+        out[k] = v.to(torch.bfloat16).float() if v.dim() >= 2 else v
     return out
 
 

@@ -154,14 +154,16 @@ def test_attention_part_and_block_in_portions(folder_b, dtype):
 
 
 # ---------------------------------------------------------------------------
-# toy parts: a mixer with state of its own, a rotating position encoding, grouped
-# key heads, a window, a layer that runs twice and a layer that reads another's cache
+# toy parts: a mixer with state of its own, a rotating position encoding, a feed-forward
+# with experts chosen per token, grouped key heads, a window, a layer that runs twice and a
+# layer that reads another's cache
 
 
 def _register_toys():
     from mlx_lm_amd.config import BaseModelArgs, LayerSpec, ModelPlan, PartSpec, RunEntry, StateNeed, register_model
-    from mlx_lm_amd.parts import (DecoderModel, Mixer, PositionEncoding, TensorSpec, register_mixer,
-                                  register_position_encoding)
+    from mlx_lm_amd.ops import kernels
+    from mlx_lm_amd.parts import (DecoderModel, FeedForward, Mixer, PositionEncoding, TensorSpec,
+                                  register_feed_forward, register_mixer, register_position_encoding)
 
     class DecayMixer(Mixer):
         """``s_t = decay * s_{t-1} + x_t``; adds ``s_t`` to the residual.  Its state
@@ -206,8 +208,39 @@ def _register_toys():
                 out = torch.cat([a * cos - b * sin, a * sin + b * cos], -1)
                 t.copy_(out.reshape(t.shape).to(t.dtype))
 
+    class HashedExperts(FeedForward):
+        """``n_experts`` GELU feed-forwards; a token goes to expert ``token_id % n_experts``
+        (routing by a hash of the token, so that rounding cannot change the choice).  The
+        tokens of an expert are gathered, run through the framework's ``linear`` and added
+        back into the residual stream."""
+
+        def __init__(self, width, inner, n_experts, prefix=""):
+            super().__init__(prefix)
+            self.width, self.inner, self.n_experts = width, inner, n_experts
+
+        def tensors(self):
+            return {self._name("up"): TensorSpec((self.n_experts, self.inner, self.width), "matrix"),
+                    self._name("down"): TensorSpec((self.n_experts, self.width, self.inner), "matrix")}
+
+        def load(self, tensors):
+            self.up, self.down = tensors[self._name("up")], tensors[self._name("down")]
+
+        def forward(self, ctx, x, residual):
+            expert = ctx.token_ids % self.n_experts
+            for e in range(self.n_experts):
+                rows = torch.nonzero(expert == e).flatten()
+                if rows.numel() == 0:
+                    continue
+                xe = x[rows].contiguous()
+                act = torch.empty((rows.numel(), self.inner), dtype=x.dtype, device=x.device)
+                kernels.linear(act, xe, self.up[e], gelu=True)
+                out = torch.empty((rows.numel(), self.width), dtype=torch.float32, device=x.device)
+                kernels.linear(out, act, self.down[e])
+                residual.index_add_(0, rows, out)
+
     register_mixer("toy_decay", DecayMixer)
     register_position_encoding("toy_pair_rotation", PairRotation)
+    register_feed_forward("toy_hashed_experts", HashedExperts)
 
     @dataclass
     class ToyArgs(BaseModelArgs):
@@ -222,6 +255,7 @@ def _register_toys():
         inner: int
         eps: float
         theta: float
+        experts: int
 
     class ToyModel:
         def __init__(self, args):
@@ -248,8 +282,11 @@ def _register_toys():
 
             mixers = [attention("l0.mix.", 0), attention("l1.mix.", a.window),
                       PartSpec("toy_decay", {"width": a.width}, "l2.mix.")]
-            layers = [LayerSpec("pre_norm", norm(f"l{i}.n1."), m, norm(f"l{i}.n2."), ffn(f"l{i}.ff."))
-                      for i, m in enumerate(mixers)]
+            ffns = [ffn("l0.ff."), PartSpec("toy_hashed_experts", {"width": a.width, "inner": a.inner,
+                                                                     "n_experts": a.experts}, "l1.ff."),
+                    ffn("l2.ff.")]
+            layers = [LayerSpec("pre_norm", norm(f"l{i}.n1."), m, norm(f"l{i}.n2."), f)
+                      for i, (m, f) in enumerate(zip(mixers, ffns))]
             # layer 0 runs twice (two cache slots); the last run of layer 1 reads the
             # keys and values that its first run wrote
             schedule = [RunEntry(0, 0), RunEntry(1, 1), RunEntry(2, 2), RunEntry(0, 3),
@@ -266,7 +303,7 @@ def _register_toys():
 
 
 TOY = dict(model_type="toy_hybrid", width=80, vocab=211, max_len=160, heads=6, kv_heads=2, head_dim=32,
-           window=24, inner=120, eps=1e-4, theta=100.0)
+           window=24, inner=120, eps=1e-4, theta=100.0, experts=3)
 
 
 def _toy_folder(path):
@@ -309,6 +346,12 @@ def _toy_plain(t, ids):
         return plain.layer_norm(x, w[p + "weight"], w[p + "bias"], a["eps"])
 
     def ffn(x, p):
+        if p + "up" in w:  # experts by token id
+            out = torch.zeros_like(x)
+            for i, tok in enumerate(ids):
+                e = tok % a["experts"]
+                out[i] = plain.linear(plain.gelu_tanh(plain.linear(x[i : i + 1], w[p + "up"][e])), w[p + "down"][e])[0]
+            return out
         return plain.mlp(x, w, p)
 
     kv_store = {}
