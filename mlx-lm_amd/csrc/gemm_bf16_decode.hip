@@ -592,6 +592,9 @@ extern "C" int gemm_bf16_decode_splits(int M, int N, int K, int with_norm, int f
   } else if (M <= 16) {
     const int n_blocks = (N + 15) / 16;
     if (n_blocks >= 200 || M < 4) return 1;  // (one to three rows: the next projection's norm prologue is cheaper than a second kernel)
+    // a small matrix streams in less time than the second kernel costs (measured at N = 1600:
+    // K = 1600 loses 2 us by the split, K = 6400 gains 4)
+    if ((long)N * K < 5000000L) return 1;
     want = (512 + n_blocks - 1) / n_blocks;  // two blocks a CU (measured at N = 1600: K = 6400 is best in 5, K = 1600 in 2 to 6)
     if (want > n_chunks / 4) want = n_chunks / 4;  // at least four k-blocks a split
   } else {
