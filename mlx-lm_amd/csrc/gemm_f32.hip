@@ -5,6 +5,13 @@
 // tanh-GELU, or accumulate into the residual stream.  Any M, N; K % 4 == 0.
 // The 32-bit twin of gemm_bf16.hip; replaces the same nn.Linear calls
 // (mlx_lm/models/gpt2.py:41-42,52,68,76-80,167).
+//
+// Up to 16 rows (decode steps) take a kernel of their own, which streams W
+// once with plain float FMAs: a 64 x 64 MFMA tile would spend its time on rows
+// that are not there.  A wave owns four features; its lanes stride along k in
+// float4 pieces, the rows sit in LDS in stretches of 512 columns; a lane sums
+// its share in the order of k and the 64 shares are added by a fixed tree, so
+// an output does not depend on the other rows of the step.
 #include "common.h"
 
 #define FLAG_GELU 1
@@ -155,9 +162,77 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs p) {
   }
 }
 
+#define SKF_FW 4     // features a wave
+#define SKF_KC 512   // columns of the rows held in LDS at a time
+
+template <int MR>  // rows, rounded up to a power of two (rows that are not there are zero)
+__global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(GemmArgs p) {
+  __shared__ float4 As[MR][SKF_KC / 4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n_base = blockIdx.x * (4 * SKF_FW) + wave * SKF_FW;
+  const float* wrow[SKF_FW];
+#pragma unroll
+  for (int f = 0; f < SKF_FW; ++f) wrow[f] = p.W + (size_t)min(n_base + f, p.N - 1) * p.ldw;
+
+  float acc[SKF_FW][MR];
+#pragma unroll
+  for (int f = 0; f < SKF_FW; ++f)
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[f][m] = 0.f;
+
+  for (int k0 = 0; k0 < p.K; k0 += SKF_KC) {
+    const int width = min(SKF_KC, p.K - k0);  // a multiple of 4
+    // the weights first: they are on their way while the rows are copied into LDS
+    // (columns beyond the stretch are read from inside it; they meet zeros in LDS)
+    float4 w[SKF_KC / 256][SKF_FW];
+#pragma unroll
+    for (int j = 0; j < SKF_KC / 256; ++j)
+#pragma unroll
+      for (int f = 0; f < SKF_FW; ++f) w[j][f] = *(const float4*)(wrow[f] + k0 + min((lane + 64 * j) * 4, width - 4));
+    __syncthreads();  // the stretch before is no longer read
+    for (int i = tid; i < MR * (SKF_KC / 4); i += 256) {
+      const int r = i / (SKF_KC / 4), c = i - r * (SKF_KC / 4);
+      const float4 t = *(const float4*)(p.A + (size_t)min(r, p.M - 1) * p.lda + k0 + min(c * 4, width - 4));
+      As[r][c] = (r < p.M && c * 4 < width) ? t : ZERO4;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < SKF_KC / 256; ++j) {
+      const int c = lane + 64 * j;
+#pragma unroll
+      for (int m = 0; m < MR; ++m) {
+        const float4 a = As[m][c];
+#pragma unroll
+        for (int f = 0; f < SKF_FW; ++f) {
+          acc[f][m] = fmaf(w[j][f].x, a.x, acc[f][m]);
+          acc[f][m] = fmaf(w[j][f].y, a.y, acc[f][m]);
+          acc[f][m] = fmaf(w[j][f].z, a.z, acc[f][m]);
+          acc[f][m] = fmaf(w[j][f].w, a.w, acc[f][m]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int f = 0; f < SKF_FW; ++f) {
+    const int n = n_base + f;
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+      float v = wave_sum(acc[f][m]);
+      if (lane == 0 && n < p.N && m < p.M) {
+        if (p.bias) v += p.bias[n];
+        const size_t idx = (size_t)m * p.ldo + n;
+        if (p.flags & FLAG_ACCUMULATE)
+          p.out[idx] += v;
+        else
+          p.out[idx] = (p.flags & FLAG_GELU) ? gelu_tanh(v) : v;
+      }
+    }
+  }
+}
+
 DEFINE_LAST_ERROR(mlxlm_last_error)
 
-// variant: 0 = choose, 1 = 128x128 block tile, 2 = 64x64 block tile
+// variant: 0 = choose, 1 = 128x128 block tile, 2 = 64x64 block tile, 3 = the kernel for up to 16 rows
 extern "C" int gemm_f32(void* out, const void* A, const void* W, const float* bias, int M, int N,
                         int K, int lda, int ldw, int ldo, int flags, int variant,
                         hipStream_t stream) {
@@ -180,13 +255,26 @@ extern "C" int gemm_f32(void* out, const void* A, const void* W, const float* bi
   if ((flags & FLAG_ACCUMULATE) && (flags & FLAG_GELU))
     FAIL("gemm_f32: GELU and accumulate cannot be combined");
   if (M == 0) return 0;
-  if (variant == 0) variant = (M <= 64 || (size_t)M * N < (size_t)128 * 128 * 128) ? 2 : 1;
+  if (variant == 0) variant = M <= 16 ? 3 : (M <= 64 || (size_t)M * N < (size_t)128 * 128 * 128) ? 2 : 1;
   if (variant == 1) {
     dim3 grid((N + 127) / 128, (M + 127) / 128), block(256);
     hipLaunchKernelGGL((gemm_f32_kernel<2, 2>), grid, block, 0, stream, p);
   } else if (variant == 2) {
     dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
     hipLaunchKernelGGL((gemm_f32_kernel<1, 1>), grid, block, 0, stream, p);
+  } else if (variant == 3) {
+    if (M > 16) FAIL("gemm_f32: the kernel for few rows takes at most 16, got %d", M);
+    dim3 grid((N + 4 * SKF_FW - 1) / (4 * SKF_FW)), block(256);
+    if (M <= 1)
+      hipLaunchKernelGGL(gemm_f32_skinny_kernel<1>, grid, block, 0, stream, p);
+    else if (M <= 2)
+      hipLaunchKernelGGL(gemm_f32_skinny_kernel<2>, grid, block, 0, stream, p);
+    else if (M <= 4)
+      hipLaunchKernelGGL(gemm_f32_skinny_kernel<4>, grid, block, 0, stream, p);
+    else if (M <= 8)
+      hipLaunchKernelGGL(gemm_f32_skinny_kernel<8>, grid, block, 0, stream, p);
+    else
+      hipLaunchKernelGGL(gemm_f32_skinny_kernel<16>, grid, block, 0, stream, p);
   } else {
     FAIL("gemm_f32: unknown variant %d", variant);
   }

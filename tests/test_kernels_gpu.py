@@ -67,6 +67,8 @@ def test_layernorm(out_dtype, width, eps):
 
 GEMM_SHAPES = [
     (1, 48, 64),
+    (3, 50, 1608),
+    (8, 1600, 6400),
     (7, 1000, 96),
     (16, 80, 200),
     (33, 257, 384),
@@ -85,7 +87,7 @@ def test_gemm_f32(M, N, K, mode):
     w = _rand((N, K), torch.float32, 11, 0.1)
     bias = _rand((N,), torch.float32, 12)
     ref = plain.linear(a.double().cpu(), w.double().cpu(), bias.double().cpu())
-    for variant in (1, 2):
+    for variant in (1, 2, 3) if M <= 16 else (1, 2):  # tiles of 128 and of 64, the kernel for few rows
         if mode == "accumulate":
             out = _rand((M, N), torch.float32, 13)
             want = out.double().cpu() + ref
