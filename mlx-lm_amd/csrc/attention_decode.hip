@@ -7,9 +7,12 @@
 // Replaces scaled_dot_product_attention with one query per sequence
 // (mlx_lm/models/base.py:132-139 with mask=None, mlx_lm/generate.py:1414).
 //
-// Work split: grid (rows, heads, n_splits), 256 threads.  The row's keys
-// [k_lo, k_hi) are cut into tiles of 64; the tiles are dealt to the splits in
-// runs and, inside a block, to the four waves in turn.  A wave reads a tile as
+// Work split: grid (rows, heads, n_splits), 4 to 16 waves a block.  The row's
+// keys [k_lo, k_hi) are cut into tiles of 64; the tiles are dealt to the splits
+// in runs and, inside a block, to the waves in turn.  With few rows in a step
+// it is the many waves of a block, joined through LDS, that give the GPU
+// enough to do: splits need a second kernel to join them, which at these sizes
+// costs as much as the attention itself.  A wave reads a tile as
 // CPK-lane groups: lane l holds 16 bytes (8 columns) l % CPK of key l / CPK of
 // each load, where CPK = head_dim / 8 lanes cover one key.  One load
 // instruction therefore reads 64 / CPK whole keys that lie back to back in a
@@ -35,6 +38,8 @@ struct DecodeArgs {
   float scale;
 };
 
+#define MAX_WAVES 16
+
 #define TILE 64
 
 __device__ __forceinline__ void unpack8(const uint4& v, float* f) {
@@ -45,14 +50,15 @@ __device__ __forceinline__ void unpack8(const uint4& v, float* f) {
 }
 
 template <int CPK>  // lanes per key: head_dim = 8 * CPK
-__global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs p) {
+__global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void attn_decode_kernel(DecodeArgs p) {
   constexpr int HD = 8 * CPK;
   constexpr int KPL = 64 / CPK;    // keys per load instruction
   constexpr int NL = TILE / KPL;   // loads per tile (= CPK)
-  __shared__ float Ms[4], Ls[4];
-  __shared__ float Os[4][HD];
+  __shared__ float Ms[MAX_WAVES], Ls[MAX_WAVES];
+  __shared__ float Os[MAX_WAVES][HD];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n_waves = blockDim.x >> 6;
   const int item = blockIdx.x, h = blockIdx.y, split = blockIdx.z;
   const int row = p.rows[item];
   const int kv_head = h / (p.n_heads / p.n_kv_heads);
@@ -83,7 +89,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs p) {
 
   const size_t head_off = (size_t)kv_head * p.page_size * HD;
 
-  for (int t = t_begin + wave; t < t_end; t += 4) {
+  for (int t = t_begin + wave; t < t_end; t += n_waves) {
     const int kt = kt0 + t * TILE;
     uint4 kv[NL], vv[NL];
     // all loads of the tile first; addresses of keys outside [k_lo, k_hi) are
@@ -149,15 +155,16 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(DecodeArgs p) {
   }
   __syncthreads();
 
-  const float M = fmaxf(fmaxf(Ms[0], Ms[1]), fmaxf(Ms[2], Ms[3]));
-  float w[4], L = 0.f;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    w[i] = (Ms[i] == -INFINITY) ? 0.f : __expf(Ms[i] - M);
-    L += Ls[i] * w[i];
+  // every thread joins the waves' results the same way, in the order of the waves
+  float M = -INFINITY;
+  for (int i = 0; i < n_waves; ++i) M = fmaxf(M, Ms[i]);
+  float L = 0.f, acc = 0.f;
+  for (int i = 0; i < n_waves; ++i) {
+    const float w = (Ms[i] == -INFINITY) ? 0.f : __expf(Ms[i] - M);
+    L += Ls[i] * w;
+    if (tid < HD) acc += Os[i][tid] * w;
   }
   if (tid < HD) {
-    const float acc = Os[0][tid] * w[0] + Os[1][tid] * w[1] + Os[2][tid] * w[2] + Os[3][tid] * w[3];
     if (p.n_splits == 1) {
       p.out[(size_t)row * p.ldo + h * HD + tid] = f32_to_bf16_bits(acc / L);
     } else {
@@ -191,8 +198,8 @@ __global__ void attn_decode_merge_kernel(DecodeArgs p) {
 DEFINE_LAST_ERROR(mlxlm_last_error)
 
 template <int CPK>
-static void launch(const DecodeArgs& p, int n_rows, hipStream_t stream) {
-  hipLaunchKernelGGL(attn_decode_kernel<CPK>, dim3(n_rows, p.n_heads, p.n_splits), dim3(256), 0, stream, p);
+static void launch(const DecodeArgs& p, int n_rows, int n_waves, hipStream_t stream) {
+  hipLaunchKernelGGL(attn_decode_kernel<CPK>, dim3(n_rows, p.n_heads, p.n_splits), dim3(64 * n_waves), 0, stream, p);
   if (p.n_splits > 1)
     hipLaunchKernelGGL(attn_decode_merge_kernel<CPK>, dim3(n_rows, p.n_heads), dim3(8 * CPK), 0, stream, p);
 }
@@ -204,8 +211,11 @@ extern "C" int attn_decode(void* out, const void* q, int ldq, int ldo, const voi
                            int max_blocks, const int* token_req, const int* positions,
                            const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
                            int page_size, int window, float scale, int n_splits, float* part_o,
-                           float* part_ml, hipStream_t stream) {
+                           float* part_ml, int n_waves, hipStream_t stream) {
   if (n_rows <= 0) return 0;
+  if (n_waves < 1 || n_waves > MAX_WAVES) FAIL("attn_decode: %d waves a block, must be 1 to %d", n_waves, MAX_WAVES);
+  if (head_dim > 64 * n_waves) FAIL("attn_decode: head_dim %d needs at least %d waves", head_dim, (head_dim + 63) / 64);
+  if (head_dim == 128 && n_waves > MAX_WAVES / 2) n_waves = MAX_WAVES / 2;  // (that kernel's registers allow eight)
   if (head_dim != 32 && head_dim != 64 && head_dim != 128)
     FAIL("attn_decode: head_dim %d is not 32, 64 or 128 (attn_row takes the others)", head_dim);
   const int kpl = 512 / head_dim;
@@ -230,11 +240,11 @@ extern "C" int attn_decode(void* out, const void* q, int ldq, int ldo, const voi
   p.n_heads = n_heads, p.n_kv_heads = n_kv_heads, p.page_size = page_size;
   p.window = window, p.n_splits = n_splits, p.scale = scale;
   if (head_dim == 32)
-    launch<4>(p, n_rows, stream);
+    launch<4>(p, n_rows, n_waves, stream);
   else if (head_dim == 64)
-    launch<8>(p, n_rows, stream);
+    launch<8>(p, n_rows, n_waves, stream);
   else
-    launch<16>(p, n_rows, stream);
+    launch<16>(p, n_rows, n_waves, stream);
   CHECK_LAUNCH("attn_decode");
   return 0;
 }

@@ -524,7 +524,7 @@ def attn_decode_takes(q_dtype, kv):
 
 
 def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_heads, scale,
-                window=0, n_splits=1, part_o=None, part_ml=None):
+                window=0, n_splits=1, part_o=None, part_ml=None, n_waves=4):
     """``attn_row`` for bfloat16 caches with head_dim 32, 64 or 128: keys stream into registers."""
     lib = build.load("attention_decode")
     ldq, ldo = _rows2d(q, "q"), _rows2d(out, "out")
@@ -544,7 +544,7 @@ def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_h
         _c_size_t(kv.page_stride), _ptr(block_table), _c_int(block_table.shape[1]),
         _ptr(token_req), _ptr(positions), _ptr(rows), _c_int(n_rows), _c_int(n_heads),
         _c_int(kv.n_kv_heads), _c_int(kv.head_dim), _c_int(kv.page_size), _c_int(window),
-        _c_float(scale), _c_int(n_splits), _ptr(part_o), _ptr(part_ml), _stream(),
+        _c_float(scale), _c_int(n_splits), _ptr(part_o), _ptr(part_ml), _c_int(n_waves), _stream(),
     )
     build.check(lib, rc, "attn_decode")
     return out

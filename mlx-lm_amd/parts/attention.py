@@ -109,15 +109,22 @@ class CausalSelfAttention(Mixer):
                 kernels.attn_tile(out, q, *args, plan.tiles, plan.n_tiles, self.n_heads, self.scale,
                                   self.window)
         if plan.n_rows:
-            n_splits = plan.row_splits(self.n_heads, self.window)
+            fast = kernels.attn_decode_takes(q.dtype, cache.kv)
+            if fast:
+                n_splits, n_waves = plan.row_work(self.n_heads, self.window)
+            else:
+                n_splits, n_waves = plan.row_splits(self.n_heads, self.window), 4
             part_o = part_ml = None
             if n_splits > 1:
                 n = plan.n_rows * self.n_heads * n_splits
                 part_o = ctx.scratch((n * self.head_dim,), "float32")
                 part_ml = ctx.scratch((n * 2,), "float32")
-            row_kernel = kernels.attn_decode if kernels.attn_decode_takes(q.dtype, cache.kv) else kernels.attn_row
-            row_kernel(out, q, *args, plan.rows, plan.n_rows, self.n_heads, self.scale,
-                       self.window, n_splits, part_o, part_ml)
+            if fast:
+                kernels.attn_decode(out, q, *args, plan.rows, plan.n_rows, self.n_heads, self.scale,
+                                    self.window, n_splits, part_o, part_ml, n_waves)
+            else:
+                kernels.attn_row(out, q, *args, plan.rows, plan.n_rows, self.n_heads, self.scale,
+                                 self.window, n_splits, part_o, part_ml)
 
 
 register_mixer("attention", CausalSelfAttention)

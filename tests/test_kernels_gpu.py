@@ -284,8 +284,8 @@ def test_attn_row(dtype, case, n_splits):
     (8, 2, 32, 16, [700, 15, 16], [1, 1, 3], 0),
     (4, 4, 128, 16, [63, 64, 1000], [1, 2, 1], 100),
 ])
-@pytest.mark.parametrize("n_splits", [1, 3, 8])
-def test_attn_decode(case, n_splits):
+@pytest.mark.parametrize("n_splits,n_waves", [(1, 4), (3, 4), (8, 4), (1, 16), (1, 8), (2, 16), (1, 2)])
+def test_attn_decode(case, n_splits, n_waves):
     k = _k()
     H, Hkv, hd, ps, ctx, ql, window = case
     c = PagedCase(torch.bfloat16, H, Hkv, hd, ps, ctx, ql, seed=hd + H + 2, window=window)
@@ -296,7 +296,7 @@ def test_attn_decode(case, n_splits):
     part_ml = torch.empty(c.T * H * n_splits * 2, dtype=torch.float32, device=DEV)
     out = torch.full((c.T, H * hd), float("nan")).to(torch.bfloat16).to(DEV)
     k.attn_decode(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, c.T, H,
-                  c.scale, window, n_splits, part_o, part_ml)
+                  c.scale, window, n_splits, part_o, part_ml, n_waves)
     err = (out.double().cpu() - c.reference()).abs().max().item()
     assert err < _attn_tol(torch.bfloat16), err
 
@@ -358,12 +358,12 @@ def test_attn_decode_far_key_stands_out():
         c.q[0, hd:] = (kf * (30.0 / (c.scale * float(kf.norm() ** 2)))).to(torch.bfloat16)
         k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
         rows = torch.zeros(1, dtype=torch.int32, device=DEV)
-        for n_splits in (1, 4):
+        for n_splits, n_waves in ((1, 4), (4, 4), (1, 16)):
             out = torch.empty(1, H * hd, dtype=torch.bfloat16, device=DEV)
             po = torch.empty(H * n_splits * hd, dtype=torch.float32, device=DEV)
             pm = torch.empty(H * n_splits * 2, dtype=torch.float32, device=DEV)
             k.attn_decode(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, 1,
-                          H, c.scale, 0, n_splits, po, pm)
+                          H, c.scale, 0, n_splits, po, pm, n_waves)
             v_far = c.v_full[0][far, 1].double()
             assert (out[0, hd:].double().cpu() - v_far).abs().max().item() < 0.1, (far, n_splits)
             assert (out.double().cpu() - c.reference()).abs().max().item() < _attn_tol(torch.bfloat16)
