@@ -20,7 +20,29 @@ __global__ __launch_bounds__(256) void embed_gather_add_kernel(
   }
 }
 
+// Tokens that a sampling kernel left on the device take their place among the
+// step's token ids without a trip through the host: ids[t] = src[index[t]]
+// where index[t] >= 0 (clamped into the vocabulary: nothing on the host has
+// seen these values).  This is what lets the next decode step be launched
+// before the host has read the tokens of this one, the job of mx.async_eval in
+// the reference's loops (mlx_lm/generate.py:446-451,1449-1456).
+__global__ void feed_tokens_kernel(int* __restrict__ ids, const int* __restrict__ src,
+                                   const int* __restrict__ index, int n, int vocab) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n) return;
+  const int i = index[t];
+  if (i >= 0) ids[t] = min(max(src[i], 0), vocab - 1);
+}
+
 DEFINE_LAST_ERROR(mlxlm_last_error)
+
+extern "C" int feed_tokens(int* ids, const int* src, const int* index, int n, int vocab, hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (!ids || !src || !index || vocab <= 0) FAIL("feed_tokens: null pointer or bad vocabulary %d", vocab);
+  hipLaunchKernelGGL(feed_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, ids, src, index, n, vocab);
+  CHECK_LAUNCH("feed_tokens");
+  return 0;
+}
 
 extern "C" int embed_gather_add(void* out, const void* table, const int* ids, const void* add_table,
                                 const int* add_ids, int n_tokens, int width, int dtype,

@@ -33,7 +33,8 @@ class DecodeGraph:
         cm = engine.cache
         B = batch
         self.max_blocks = cm.blocks_for(engine.decoder.max_positions)
-        sizes = [B] * 6 + [2 * B] + [B * self.max_blocks] * len(cm.groups)
+        sizes = [B] * 6 + [2 * B] + [B * self.max_blocks] * len(cm.groups) + [B]  # last: fed rows
+        self.fed_piece = len(sizes) - 1
         self.offsets, total = [], 0
         for s in sizes:
             self.offsets.append(total)
@@ -72,6 +73,13 @@ class DecodeGraph:
             ctx.block_tables.append(self._piece(7 + gi, B * self.max_blocks).view(B, self.max_blocks))
         return ctx
 
+    def _feed(self, ctx):
+        """Tokens fed on the device replace the placeholders (a row of -1s changes nothing)."""
+        from ..ops import kernels
+
+        kernels.feed_tokens(ctx.token_ids, self.engine.fed_src, self._piece(self.fed_piece, self.batch),
+                            self.engine.decoder.vocab_size)
+
     def _fill(self, entries):
         cm = self.engine.cache
         if self._copied is not None:
@@ -80,6 +88,7 @@ class DecodeGraph:
         for r, e in enumerate(entries):
             rc = cm.requests[e.request_id]
             h[off[0] + r] = int(e.tokens[0])
+            h[off[self.fed_piece] + r] = e.fed_row
             h[off[1] + r] = rc.length
             h[off[4] + r] = rc.state_slot
             for gi in range(len(cm.groups)):
@@ -98,6 +107,7 @@ class DecodeGraph:
             ctx = self._context()
             # once eagerly: libraries load, scratch memory grows to what the step needs
             self.dev.copy_(self.host, non_blocking=True)
+            self._feed(ctx)
             eng.scratch.reset()
             eng.decoder.forward(ctx)
             torch.cuda.synchronize()
@@ -106,12 +116,13 @@ class DecodeGraph:
             try:
                 with torch.cuda.graph(graph):
                     self.dev.copy_(self.host, non_blocking=True)
+                    self._feed(ctx)
                     eng.scratch.reset()
                     self.logits = eng.decoder.forward(ctx)
             finally:
                 eng.scratch.frozen = False
             self.graph = graph
-            self._keep = (eng.scratch.buffer, eng._logits)
+            self._keep = (eng.scratch.buffer, eng._logits, eng.fed_src)
             self._copied = torch.cuda.Event()
         self.graph.replay()
         self._copied.record()

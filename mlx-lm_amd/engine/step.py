@@ -19,6 +19,9 @@ class StepEntry:
     request_id: object
     tokens: Sequence[int]
     want: Sequence[int] = ()
+    # Row of the step's ``fed`` tokens (sampled tokens still on the device) that is
+    # this request's one token; ``tokens`` then holds a placeholder.  -1: ``tokens`` are the tokens.
+    fed_row: int = -1
 
 
 class _HostRing:
@@ -79,6 +82,8 @@ class Engine:
         self._meta_dev = None
         self._logits = None
         self.steps = 0
+        # sampled tokens that go into the next step without passing through the host
+        self.fed_src = torch.zeros(max(64, max_requests), dtype=torch.int32, device=self.device)
         # decode steps are recorded as graphs where every part launches kernels only
         self.use_graphs = use_graphs and all(getattr(p, "graph_safe", False) for p in self.decoder.parts())
         self._graphs = {}
@@ -128,6 +133,8 @@ class Engine:
             n = len(e.tokens)
             if n == 0:
                 raise ValueError(f"request {e.request_id!r} brings no tokens")
+            if e.fed_row >= 0 and n != 1:
+                raise ValueError(f"request {e.request_id!r}: a token fed on the device is one token")
             for t in e.tokens:
                 if not (0 <= int(t) < V):
                     raise ValueError(f"token id {t} of request {e.request_id!r} is outside [0, {V})")
@@ -141,14 +148,23 @@ class Engine:
                 if not (0 <= int(w) < n):
                     raise ValueError(f"wanted place {w} of request {e.request_id!r} is outside its {n} tokens")
 
-    def step(self, entries: List[StepEntry]):
+    def step(self, entries: List[StepEntry], fed=None):
         """Run one batch; returns float32 logits ``[n_wanted, vocab]`` (``None`` if nothing is wanted).
 
+        ``fed``: an int32 device tensor of sampled tokens; entries with
+        ``fed_row >= 0`` take their token from it on the device, so the step
+        can be launched before the host has read those tokens.
         The returned tensor is a view of a buffer that the next step overwrites.
         """
         if not entries:
             return None
         self._check(entries)
+        if any(e.fed_row >= 0 for e in entries):
+            if fed is None or fed.dtype != torch.int32 or not fed.is_cuda:
+                raise ValueError("entries with fed_row need the int32 device tensor `fed`")
+            if fed.numel() > self.fed_src.numel() or any(e.fed_row >= fed.numel() for e in entries):
+                raise ValueError(f"`fed` has {fed.numel()} tokens; at most {self.fed_src.numel()}, and every fed_row inside")
+            self.fed_src[: fed.numel()].copy_(fed.reshape(-1), non_blocking=True)
         cm = self.cache
         # pages first: all or nothing for the whole step
         done = []
@@ -215,7 +231,7 @@ class Engine:
         T = sum(len(e.tokens) for e in entries)
         ctx = StepContext(self)
         q_start = 0
-        token_ids, positions, token_req, wanted, slot_ids = [], [], [], [], []
+        token_ids, positions, token_req, wanted, slot_ids, fed_index = [], [], [], [], [], []
         tiles, rows, all_tiles, big = [], [], [], []
         plan = AttentionPlan()
         for r, e in enumerate(entries):
@@ -225,6 +241,7 @@ class Engine:
             ctx.q_lens.append(n)
             ctx.context_lens.append(rc.length)
             token_ids.extend(int(t) for t in e.tokens)
+            fed_index.extend([e.fed_row] if e.fed_row >= 0 else [-1] * n)
             positions.extend(range(rc.length, rc.length + n))
             token_req.extend([r] * n)
             wanted.extend(q_start + int(w) for w in e.want)
@@ -264,6 +281,7 @@ class Engine:
         # everything in one pinned buffer and one copy; pieces start on 4-int boundaries
         pieces = [token_ids, positions, token_req, wanted, slot_ids, tiles, rows, all_tiles, big_tiles]
         pieces += [flat for _, flat in tables]
+        pieces.append(fed_index)  # (last: the pieces before it keep their numbers)
         offsets, total = [], 0
         for p in pieces:
             offsets.append(total)
@@ -297,4 +315,8 @@ class Engine:
         ctx.attention_plan = plan
         for gi, (width, flat) in enumerate(tables):
             ctx.block_tables.append(piece(9 + gi, len(flat)).view(R, width))
+        if any(i >= 0 for i in fed_index):
+            from ..ops import kernels
+
+            kernels.feed_tokens(ctx.token_ids, self.fed_src, piece(9 + len(tables), T), self.decoder.vocab_size)
         return ctx

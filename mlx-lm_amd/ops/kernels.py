@@ -76,6 +76,17 @@ def embed_gather_add(out, table, ids, add_table=None, add_ids=None):
     return out
 
 
+def feed_tokens(ids, src, index, vocab):
+    """``ids[t] = src[index[t]]`` where ``index[t] >= 0``: sampled tokens that are still on the device."""
+    lib = build.load("embed")
+    for name, t in (("ids", ids), ("src", src), ("index", index)):
+        _dev(t, name, torch.int32)
+    _need(index.numel() >= ids.numel(), "feed_tokens: an index for every id")
+    rc = lib.feed_tokens(_ptr(ids), _ptr(src), _ptr(index), _c_int(ids.numel()), _c_int(vocab), _stream())
+    build.check(lib, rc, "feed_tokens")
+    return ids
+
+
 def layernorm(out, x, gamma, beta, eps, rows=None):
     """LayerNorm of float32 rows of ``x`` (all, or those listed in ``rows``) into ``out``."""
     lib = build.load("norm")

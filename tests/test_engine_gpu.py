@@ -419,3 +419,61 @@ def test_recorded_steps_of_repeating_shapes(folders, dtype):
         n = sum(x.shape[0] for x in got[r])
         want = _plain_logits(weights, config, toks[:n], dtype)
         _close(torch.cat(got[r]), want, dtype, f"recorded shapes, request {r}")
+
+
+@pytest.mark.parametrize("use_graphs", [True, False])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_tokens_fed_on_the_device(folders, dtype, use_graphs):
+    """A decode step may take its tokens from the sampler's device array (the host reads them a
+    step later): same logits, bit for bit, as with the tokens passed through the host.  Rows of the
+    fed array in another order than the entries, a host token beside fed ones, and a portion of a
+    prompt beside them (a step that is not replayed from a graph)."""
+    from mlx_lm_amd.engine import Engine, StepEntry
+    from mlx_lm_amd.sample_utils import Sampler
+    from mlx_lm_amd.sampling import sample_batch
+    from mlx_lm_amd.utils import load_model
+
+    folder, config, weights = folders[("B", 8.0)]
+    V = config["vocab_size"]
+    model, _ = load_model(folder, dtype=dtype)
+    prompts = {r: helpers.random_tokens(n, V, seed=90 + i) for i, (r, n) in enumerate([("a", 33), ("b", 70), ("c", 5)])}
+    late = helpers.random_tokens(40, V, seed=99)
+    greedy = [Sampler()] * 3
+
+    def run(feed):
+        eng = Engine(model, dtype=dtype, page_size=16, n_pages=40, max_requests=4, use_graphs=use_graphs)
+        rows = []
+        for r, toks in prompts.items():
+            eng.add_request(r)
+            rows.append(eng.step([StepEntry(r, toks, [len(toks) - 1])])[0].clone())
+        logits = torch.stack(rows)
+        history, kept = [], []
+        for step in range(24):
+            tokens, _ = sample_batch(logits, greedy, [0, 1, 2], [step] * 3)
+            order = ["c", "a", "b"] if step % 2 else ["a", "b", "c"]  # entries in another order than the rows
+            row_of = {"a": 0, "b": 1, "c": 2}
+            if feed:
+                entries = [StepEntry(r, [0], [0], fed_row=row_of[r]) for r in order]
+                if step % 5 == 4:  # one token through the host beside fed ones
+                    r = order[1]
+                    entries[1] = StepEntry(r, [int(tokens[row_of[r]])], [0])
+            else:
+                host = tokens.tolist()
+                entries = [StepEntry(r, [host[row_of[r]]], [0]) for r in order]
+            if step == 10:  # a portion of a new prompt beside the decoding requests: an eager step
+                eng.add_request("late")
+                entries.append(StepEntry("late", late, []))
+            out = eng.step(entries, fed=tokens if feed else None)
+            history.append(tokens.clone())
+            logits = torch.stack([out[order.index(r)] for r in ("a", "b", "c")]).clone()
+            kept.append(logits)
+        return torch.stack(history), torch.stack(kept)
+
+    tokens_host, logits_host = run(False)
+    tokens_fed, logits_fed = run(True)
+    assert torch.equal(tokens_host, tokens_fed)
+    assert torch.equal(logits_host, logits_fed)
+    # and the tokens are what the plain model decodes greedily
+    want = plain.greedy_generate(helpers.round_matrices_to_bf16(weights) if dtype == "bfloat16" else weights,
+                                 config, prompts["c"], 6)
+    assert tokens_host[:6, 2].tolist() == want
