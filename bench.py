@@ -73,50 +73,40 @@ def prefill_flops(args, n_seqs, seq_len):
     return per_token * n_seqs * seq_len + attn + head
 
 
-def run_decode(engine, sample, batch, prompt_len, steps, warmup, vocab, seed):
-    """Fill `batch` requests with `prompt_len` tokens, then time `steps` decode steps."""
+def run_decode(engine, batch, prompt_len, steps, warmup, vocab, seed):
+    """`batch` requests of `prompt_len` tokens through the scheduler (the loop that generation uses:
+    a step is launched while the host reads the tokens of the one before); times `steps` decode steps."""
     import torch
 
-    from mlx_lm_amd.engine import StepEntry
-    from mlx_lm_amd.sample_utils import Sampler
+    from mlx_lm_amd.engine.scheduler import Request, Scheduler
+    from mlx_lm_amd.generate import make_sample_fn
 
     g = torch.Generator().manual_seed(seed)
-    rids = [("bench", batch, i) for i in range(batch)]
-    for rid in rids:
-        engine.add_request(rid)
     prompts = torch.randint(0, vocab, (batch, prompt_len), generator=g).tolist()
-    # prompts go in a few at a time to bound the step's scratch memory
-    logits_rows = {}
-    for i in range(0, batch, 4):
-        part = rids[i : i + 4]
-        out = engine.step([StepEntry(r, prompts[i + j], [prompt_len - 1]) for j, r in enumerate(part)])
-        for j, r in enumerate(part):
-            logits_rows[r] = out[j].clone()
-    logits = torch.stack([logits_rows[r] for r in rids])
-    greedy = [Sampler()] * batch
-    seeds = list(range(batch))
-
-    def one(logits, n):
-        tokens, _ = sample(logits, greedy, seeds, [n] * batch)
-        toks = tokens.tolist()  # the host reads every token, as generation does (the step's only wait)
-        return engine.step([StepEntry(r, [t], [0]) for r, t in zip(rids, toks)])
-
-    n = 0
+    # prompts go in four at a time to bound the step's scratch memory
+    sched = Scheduler(engine, make_sample_fn(), max_num_seqs=batch,
+                      max_num_batched_tokens=4 * prompt_len + batch, prefill_step_size=prompt_len)
+    rids = [("bench", batch, i) for i in range(batch)]
+    for i, rid in enumerate(rids):
+        sched.add(Request(rid, prompts[i], max_tokens=10**6, seed=i))  # greedy; the timed steps end it
+    while sched.waiting or not all(r.decoding for r in sched.running):
+        sched.step()
     for _ in range(warmup):
-        logits = one(logits, n)
-        n += 1
+        sched.step()
     torch.cuda.synchronize()
+    ctx0 = sum(engine.context_len(rid) for rid in rids) / batch
     t0 = time.perf_counter()
-    ctx0 = prompt_len + n
+    n_out = 0
     for _ in range(steps):
-        logits = one(logits, n)
-        n += 1
+        n_out += len(sched.step())  # every step hands out one token per request
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    ctx1 = sum(engine.context_len(rid) for rid in rids) / batch
+    if n_out != batch * steps:
+        raise RuntimeError(f"{n_out} tokens came out of {steps} steps of {batch} requests")
     for rid in rids:
-        engine.end_request(rid)
-    mean_ctx = ctx0 + (steps - 1) / 2 + 1
-    return dt, mean_ctx
+        sched.abort(rid)
+    return dt, (ctx0 + ctx1) / 2
 
 
 def main():
@@ -137,7 +127,6 @@ def main():
     import torch
 
     from mlx_lm_amd.engine import Engine, StepEntry
-    from mlx_lm_amd.sampling import sample_batch
 
     config = dict(XL)
     config["n_layer"] = a.layers
@@ -176,7 +165,7 @@ def main():
     batches = [a.batch] if a.no_points else sorted({1, a.batch, 64})
     for b in batches:
         k = steps if b == a.batch else min(steps, 64)
-        dt, mean_ctx = run_decode(engine, sample_batch, b, a.prompt_len, k, a.warmup, V, seed=b)
+        dt, mean_ctx = run_decode(engine, b, a.prompt_len, k, a.warmup, V, seed=b)
         results[b] = (b * k / dt, dt / k * 1e3, mean_ctx, k)
         print(f"[bench] decode batch {b}: {results[b][0]:.1f} tok/s, {results[b][1]:.3f} ms/step",
               file=sys.stderr, flush=True)

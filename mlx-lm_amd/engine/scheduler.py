@@ -22,6 +22,17 @@ when it is added.
 
 Decisions (``plan_step``) are pure bookkeeping on the host and can be tested
 without a GPU; ``step`` runs a plan through the engine and the sampler.
+
+Where the sampler can work in two phases (``launch`` / ``finish``), steps
+overlap the way the reference's loops do with ``mx.async_eval``
+(mlx_lm/generate.py:446-451,1449-1456): step t is planned and launched while
+the tokens of step t-1 are still on the device (decoding requests get them
+fed there), then the host reads the tokens of step t-1, decides who has
+finished, and queues the sampling of step t.  ``step`` therefore returns the
+outputs of the step before the one it launches.  What cannot be known without
+the token -- a stop sequence -- is found a step late: the request has then
+taken part in one step too many, whose result is dropped.  What can be known
+(``max_tokens``, the model's positions) is: such a request is left out.
 """
 
 from collections import deque
@@ -49,6 +60,8 @@ class Request:
     finish_reason: Optional[str] = None
     preemptions: int = 0
     order: int = 0
+    # row of the sampling call in flight that holds this request's newest token (not yet in ``generated``)
+    inflight_row: Optional[int] = None
 
     @property
     def tokens(self):
@@ -61,6 +74,8 @@ class Request:
     @property
     def decoding(self):
         """All but the newest token are computed: the next step brings one token."""
+        if self.inflight_row is not None:  # the newest token is still on the device
+            return self.num_computed == self.num_tokens
         return self.num_computed == self.num_tokens - 1 and len(self.generated) > 0
 
 
@@ -122,6 +137,8 @@ class Scheduler:
         self.running: List[Request] = []
         self.stats = SchedulerStats()
         self._order = 0
+        self.pipelined = hasattr(sample, "launch") and hasattr(sample, "finish")
+        self._inflight = None  # the sampling call whose tokens the host has not read yet
 
     # -- requests ----------------------------------------------------------------
 
@@ -161,12 +178,20 @@ class Scheduler:
 
     @property
     def has_work(self):
-        return bool(self.waiting or self.running)
+        return bool(self.waiting or self.running or self._inflight is not None)
 
     def _drop(self, r):
-        self.running.remove(r)
+        if r in self.running:
+            self.running.remove(r)
+        elif r in self.waiting:  # pre-empted, and finished by the token that was in flight
+            self.waiting.remove(r)
         if self.engine.has_request(r.request_id):
             self.engine.end_request(r.request_id)
+
+    def _ends_with_token_in_flight(self, r):
+        """The token in flight is the request's last, whatever it is."""
+        return r.inflight_row is not None and (
+            len(r.generated) + 1 >= r.max_tokens or r.num_tokens + 1 >= self.max_positions)
 
     def _preempt(self, r):
         self._drop(r)
@@ -189,7 +214,7 @@ class Scheduler:
         plan = []
 
         # 1. one token for every decoding request; pre-empt from the newest if pages run short
-        decoding = [r for r in self.running if r.decoding]
+        decoding = [r for r in self.running if r.decoding and not self._ends_with_token_in_flight(r)]
         decoding.sort(key=lambda r: r.order)
         while decoding:
             need = sum(self._pages_for(r, 1) for r in decoding)
@@ -222,6 +247,8 @@ class Scheduler:
         # 3. admit waiting requests while their whole prompt fits
         while self.waiting and len(self.running) < self.max_num_seqs and budget > 0:
             r = self.waiting[0]
+            if r.inflight_row is not None:
+                break  # pre-empted with a token in flight: it is read as a prompt once that token is known
             whole = self.cache.blocks_for(min(r.num_tokens + 1, self.max_positions))
             if whole > free:
                 break
@@ -250,44 +277,93 @@ class Scheduler:
     # -- running a plan ------------------------------------------------------------
 
     def step(self):
-        """Plan, run and sample one step; returns the ``StepOutput`` of every sampled token."""
+        """Plan, run and sample one step; returns the ``StepOutput`` of every sampled token
+        (of this step, or of the step before where steps overlap)."""
+        if not self.pipelined:
+            return self._step_in_turn()
+        prev, self._inflight = self._inflight, None
+        outputs = []
+        if prev is not None and not prev.feedable:
+            outputs = self._finish(prev)  # tokens made on the host: nothing to overlap
+            prev = None
         plan = self.plan_step()
-        if not plan:
-            if self.has_work and not self.running:
-                raise RuntimeError("requests are waiting but none can be admitted")
-            return []
+        logits = None
+        if plan:
+            logits = self._run(plan, prev)
+        elif prev is None and self.has_work and not self.running:
+            raise RuntimeError("requests are waiting but none can be admitted")
+        if prev is not None:
+            outputs = self._finish(prev)  # the GPU is busy with this step meanwhile
+        sampled = [p.request for p in plan if p.samples]
+        if sampled:
+            job = self.sample.launch(logits, sampled)
+            for i, r in enumerate(sampled):
+                r.inflight_row = i
+            self._inflight = job
+        return outputs
+
+    def _run(self, plan, prev=None):
+        """Launch the planned step; decoding requests whose token is in flight get it fed on the device."""
         entries = []
         for p in plan:
             r = p.request
-            toks = r.tokens[r.num_computed : r.num_computed + p.n_tokens]
-            entries.append(StepEntry(r.request_id, toks, [p.n_tokens - 1] if p.samples else []))
-        logits = self.engine.step(entries)
+            if r.inflight_row is not None:
+                entries.append(StepEntry(r.request_id, [0], [0] if p.samples else [], fed_row=r.inflight_row))
+            else:
+                toks = r.tokens[r.num_computed : r.num_computed + p.n_tokens]
+                entries.append(StepEntry(r.request_id, toks, [p.n_tokens - 1] if p.samples else []))
+        if prev is not None and any(e.fed_row >= 0 for e in entries):
+            logits = self.engine.step(entries, fed=prev.tokens)
+        else:
+            logits = self.engine.step(entries)
         for p in plan:
             r = p.request
-            if not r.generated:
+            if not r.generated and r.inflight_row is None:
                 self.stats.prompt_tokens += p.n_tokens
             r.num_computed += p.n_tokens
         self.stats.steps += 1
         self.stats.pages_high_water = max(
             self.stats.pages_high_water, max((g.pool.high_water for g in self.cache.groups), default=0)
         )
+        return logits
+
+    def _finish(self, job):
+        """Read a sampling call's tokens and give them to their requests."""
+        results = self.sample.finish(job)
+        outputs = []
+        for r, (token, logprob, logprobs) in zip(job.requests, results):
+            r.inflight_row = None
+            if r.finish_reason is not None or not (r in self.running or r in self.waiting):
+                continue  # finished a step ago (this token is one too many), or taken out meanwhile
+            outputs.append(self._take(r, token, logprob, logprobs))
+        return outputs
+
+    def _take(self, r, token, logprob, logprobs):
+        r.generated.append(int(token))
+        self.stats.generation_tokens += 1
+        # "length" at max_tokens or when the model's positions are used up;
+        # "stop" is checked second and wins (mlx_lm/generate.py:1501-1514)
+        reason = None
+        if len(r.generated) >= r.max_tokens or r.num_tokens >= self.max_positions:
+            reason = "length"
+        if stops(r.generated, r.stop_sequences):
+            reason = "stop"
+        r.finish_reason = reason
+        if reason is not None:
+            self._drop(r)
+        return StepOutput(r.request_id, int(token), float(logprob), reason, logprobs)
+
+    def _step_in_turn(self):
+        """One step and its sampling, the host waiting for the tokens before it goes on."""
+        plan = self.plan_step()
+        if not plan:
+            if self.has_work and not self.running:
+                raise RuntimeError("requests are waiting but none can be admitted")
+            return []
+        logits = self._run(plan)
         sampled = [p.request for p in plan if p.samples]
         if not sampled:
             return []
         results = self.sample(logits, sampled)
-        outputs = []
-        for r, (token, logprob, logprobs) in zip(sampled, results):
-            r.generated.append(int(token))
-            self.stats.generation_tokens += 1
-            # "length" at max_tokens or when the model's positions are used up;
-            # "stop" is checked second and wins (mlx_lm/generate.py:1501-1514)
-            reason = None
-            if len(r.generated) >= r.max_tokens or r.num_tokens >= self.max_positions:
-                reason = "length"
-            if stops(r.generated, r.stop_sequences):
-                reason = "stop"
-            r.finish_reason = reason
-            outputs.append(StepOutput(r.request_id, int(token), float(logprob), reason, logprobs))
-            if reason is not None:
-                self._drop(r)
-        return outputs
+        return [self._take(r, token, logprob, logprobs)
+                for r, (token, logprob, logprobs) in zip(sampled, results)]

@@ -20,7 +20,7 @@ from . import sample_utils
 from .engine.scheduler import Request, Scheduler
 from .engine.step import Engine
 from .sample_utils import Sampler, make_logits_processors, make_sampler
-from .sampling import apply_processors, read_sampled, sample_batch
+from .sampling import PendingRead, apply_processors, read_sampled, sample_batch
 
 DEFAULT_PROMPT = "hello"
 DEFAULT_MAX_TOKENS = 100
@@ -66,14 +66,28 @@ def engine_for(model, page_size=16, max_requests=64, max_cache_tokens=None):
     return eng
 
 
-def make_sample_fn():
+class SampleJob:
+    """A sampling call whose tokens are on their way to the host."""
+
+    def __init__(self, requests, tokens, read, logprobs, custom):
+        self.requests = requests
+        self.tokens = tokens      # int32 device array, a row per request: what the next step can be fed
+        self.read = read          # PendingRead
+        self.logprobs = logprobs  # float32 [rows, vocab] on the device, or None
+        self.custom = custom      # requests whose sampler is a callable: their token is made on the host
+        self.feedable = not custom
+
+
+class _SampleFn:
     """The scheduler's sampling callback: processors, log-probabilities, one draw per row.
 
     ``logits processors -> logprobs = logits - logsumexp -> sampler`` as in
     mlx_lm/generate.py:400-412,1417-1445, for all rows in one launch each.
+    ``launch`` queues the work and returns at once; ``finish`` waits for the
+    tokens; calling the object does both.
     """
 
-    def sample(logits, requests):
+    def launch(self, logits, requests):
         if any(r.logits_processors for r in requests):
             apply_processors(logits, [r.logits_processors or [] for r in requests],
                              [r.tokens for r in requests])
@@ -82,18 +96,25 @@ def make_sample_fn():
         want = bool(custom) or any(r.want_logprobs for r in requests)
         out = sample_batch(logits, samplers, [r.seed for r in requests],
                            [len(r.generated) for r in requests], want_logprobs=want)
-        tokens, token_lp = read_sampled(out[0], out[1])
-        logprobs = out[2] if want else None
+        return SampleJob(list(requests), out[0], PendingRead(out[0], out[1]), out[2] if want else None, custom)
+
+    def finish(self, job):
+        tokens, token_lp = job.read.wait()
         results = []
-        for i, r in enumerate(requests):
+        for i, r in enumerate(job.requests):
             tok, lp = tokens[i], token_lp[i]
-            if r in custom:  # any callable on log-probabilities, as the reference allows
-                tok = int(torch.as_tensor(r.sampler(logprobs[i : i + 1])).reshape(-1)[0])
-                lp = float(logprobs[i, tok])
-            results.append((tok, lp, logprobs[i] if (want and r.want_logprobs) else None))
+            if r in job.custom:  # any callable on log-probabilities, as the reference allows
+                tok = int(torch.as_tensor(r.sampler(job.logprobs[i : i + 1])).reshape(-1)[0])
+                lp = float(job.logprobs[i, tok])
+            results.append((tok, lp, job.logprobs[i] if (job.logprobs is not None and r.want_logprobs) else None))
         return results
 
-    return sample
+    def __call__(self, logits, requests):
+        return self.finish(self.launch(logits, requests))
+
+
+def make_sample_fn():
+    return _SampleFn()
 
 
 # ---------------------------------------------------------------------------

@@ -169,6 +169,56 @@ class SampledRows:
         self.token_logprob = both[rows:].view(torch.float32)
 
 
+class _ReadRing:
+    """Pinned host arrays that sampled tokens are copied into, reused in turn."""
+
+    def __init__(self, n=4):
+        self.bufs = [None] * n
+        self.i = 0
+
+    def get(self, n_words):
+        self.i = (self.i + 1) % len(self.bufs)
+        b = self.bufs[self.i]
+        if b is None or b.numel() < n_words:
+            b = self.bufs[self.i] = torch.empty(max(n_words, 256), dtype=torch.int32, pin_memory=True)
+        return b
+
+
+_READ_RING = _ReadRing()
+
+
+class PendingRead:
+    """Tokens and log-probabilities on their way to the host.
+
+    ``start`` queues the copy behind the sampling kernel and returns at once;
+    ``wait`` blocks until that copy (and nothing queued after it) is done, so a
+    step launched in between keeps the GPU busy while the host reads.  Up to
+    four reads may be pending.
+    """
+
+    def __init__(self, tokens, token_logprob):
+        R = tokens.numel()
+        self.rows = R
+        adjacent = (token_logprob.data_ptr() == tokens.data_ptr() + 4 * R and tokens.dtype == torch.int32
+                    and tokens.is_contiguous() and token_logprob.is_contiguous())
+        self.host = _READ_RING.get(2 * R)
+        if adjacent:
+            self.host[: 2 * R].copy_(torch.as_strided(tokens, (2 * R,), (1,)), non_blocking=True)
+        else:
+            self.host[:R].copy_(tokens, non_blocking=True)
+            self.host[R : 2 * R].copy_(token_logprob.view(torch.int32), non_blocking=True)
+        self.event = torch.cuda.Event()
+        self.event.record()
+
+    def wait(self):
+        """``(tokens, logprobs)`` as Python lists."""
+        import numpy as np
+
+        self.event.synchronize()
+        both = self.host.numpy()[: 2 * self.rows]
+        return both[: self.rows].tolist(), both[self.rows :].view(np.float32).tolist()
+
+
 def read_sampled(tokens, token_logprob):
     """``(tokens, logprobs)`` as Python lists with a single device-to-host copy
     when the two came from one ``sample_batch`` call."""

@@ -17,6 +17,7 @@ class FakeEngine:
         self.cache = CacheManager([CacheNeed(2, 16, 0)], page_size, n_pages, max_requests)
         self.decoder = SimpleNamespace(max_positions=max_positions)
         self.log = []
+        self.fed = 0
 
     def add_request(self, rid):
         return self.cache.add(rid)
@@ -27,9 +28,12 @@ class FakeEngine:
     def has_request(self, rid):
         return rid in self.cache.requests
 
-    def step(self, entries):
+    def step(self, entries, fed=None):
         for e in entries:
             self.cache.reserve(e.request_id, len(e.tokens))
+            if e.fed_row >= 0:  # the token comes from the sampling call in flight: the right row of it
+                assert fed is not None and fed[e.fed_row][0] == e.request_id and len(e.tokens) == 1
+                self.fed += 1
         rows = []
         for e in entries:
             start = self.cache.requests[e.request_id].length
@@ -51,6 +55,25 @@ def fake_sample(rows, requests):
         assert rid == r.request_id and pos == r.num_tokens - 1  # the row of the newest token
         out.append((token_for(rid, len(r.generated)), -1.0, None))
     return out
+
+
+class TwoPhaseSample:
+    """The same sampler in two phases, as the GPU's: ``launch`` returns at once, ``finish`` hands out
+    the tokens; a scheduler given this overlaps its steps."""
+
+    def launch(self, rows, requests):
+        results = fake_sample(rows, requests)
+        return SimpleNamespace(requests=list(requests), results=results, feedable=True,
+                               tokens=[(r.request_id, t) for r, (t, _, _) in zip(requests, results)])
+
+    def finish(self, job):
+        return job.results
+
+    def __call__(self, rows, requests):
+        return self.finish(self.launch(rows, requests))
+
+
+SAMPLERS = {"in turn": lambda: fake_sample, "overlapped": TwoPhaseSample}
 
 
 def run_all(sched, limit=10000):
@@ -83,9 +106,10 @@ def test_portions_under_a_token_budget_beside_decoding():
     assert eng.cache.free_pages() == 64 and not eng.cache.requests
 
 
-def test_max_tokens_stop_and_positions():
+@pytest.mark.parametrize("mode", SAMPLERS)
+def test_max_tokens_stop_and_positions(mode):
     eng = FakeEngine(n_pages=64, max_positions=40)
-    s = Scheduler(eng, fake_sample)
+    s = Scheduler(eng, SAMPLERS[mode]())
     for rid, n, mt in (("a", 5, 2), ("b", 7, 3), ("c", 3, 4), ("d", 9, 5)):
         s.add(Request(rid, list(range(1, n + 1)), mt))
     s.add(Request("stop", [1, 2, 3], 50, stop_sequences=[[token_for("stop", 1), token_for("stop", 2)]]))
@@ -100,9 +124,10 @@ def test_max_tokens_stop_and_positions():
     assert stops([4, 5, 6], [[5, 6]]) and not stops([5, 6, 4], [[5, 6]]) and not stops([6], [[5, 6]])
 
 
-def test_admission_waits_for_pages_and_keeps_order():
+@pytest.mark.parametrize("mode", SAMPLERS)
+def test_admission_waits_for_pages_and_keeps_order(mode):
     eng = FakeEngine(n_pages=6)
-    s = Scheduler(eng, fake_sample, max_num_seqs=8)
+    s = Scheduler(eng, SAMPLERS[mode](), max_num_seqs=8)
     s.add(Request("a", list(range(1, 50)), 4))  # 4 pages
     s.add(Request("b", list(range(1, 40)), 4))  # 3 pages: has to wait
     s.add(Request("c", [1, 2], 4))  # would fit, but b is first
@@ -115,9 +140,10 @@ def test_admission_waits_for_pages_and_keeps_order():
     assert first_step["a"] < first_step["b"] <= first_step["c"]
 
 
-def test_preemption_when_pages_run_out():
+@pytest.mark.parametrize("mode", SAMPLERS)
+def test_preemption_when_pages_run_out(mode):
     eng = FakeEngine(n_pages=5, max_positions=200)
-    s = Scheduler(eng, fake_sample, max_num_seqs=4)
+    s = Scheduler(eng, SAMPLERS[mode](), max_num_seqs=4)
     s.add(Request("old", list(range(1, 31)), 40))  # 2 pages, grows to 5
     s.add(Request("new", list(range(1, 17)), 40))  # 2 pages with its first token
     done = run_all(s)
@@ -147,9 +173,10 @@ def test_what_cannot_fit_is_refused_at_once():
         s.add(Request("ok", [1], 1))
 
 
-def test_abort_frees_everything():
+@pytest.mark.parametrize("mode", SAMPLERS)
+def test_abort_frees_everything(mode):
     eng = FakeEngine(n_pages=16)
-    s = Scheduler(eng, fake_sample, max_num_batched_tokens=16, prefill_step_size=16)
+    s = Scheduler(eng, SAMPLERS[mode](), max_num_batched_tokens=16, prefill_step_size=16)
     s.add(Request("a", list(range(1, 60)), 5))
     s.add(Request("b", list(range(1, 20)), 5))
     s.step()
@@ -160,12 +187,13 @@ def test_abort_frees_everything():
         s.abort("a")
 
 
+@pytest.mark.parametrize("mode", SAMPLERS)
 @pytest.mark.parametrize("seed", range(5))
-def test_random_load_every_request_finishes_with_its_own_tokens(seed):
+def test_random_load_every_request_finishes_with_its_own_tokens(seed, mode):
     rng = random.Random(seed)
     P = 128
     eng = FakeEngine(n_pages=rng.choice([8, 12, 30]), max_positions=P, max_requests=6)
-    s = Scheduler(eng, fake_sample, max_num_seqs=rng.choice([2, 4, 6]),
+    s = Scheduler(eng, SAMPLERS[mode](), max_num_seqs=rng.choice([2, 4, 6]),
                   max_num_batched_tokens=rng.choice([8, 33, 256]), prefill_step_size=rng.choice([5, 64]))
     want, done, added = {}, {}, 0
     for _ in range(3000):
@@ -188,3 +216,59 @@ def test_random_load_every_request_finishes_with_its_own_tokens(seed):
         assert [o.token for o in outs] == [token_for(rid, i) for i in range(len(outs))]
         assert outs[-1].finish_reason == "length" and all(o.finish_reason is None for o in outs[:-1])
     assert eng.cache.free_pages() == eng.cache.n_pages
+    assert (eng.fed > 0) == (mode == "overlapped")
+
+
+def test_overlapped_steps_what_is_known_early_and_what_is_found_late():
+    """Steps overlap: a step is launched while the tokens of the one before are still on the device.
+    A request whose token in flight is its last (max_tokens) is left out of that step; a stop
+    sequence is only seen when the token is read, so the request takes part in one step too many,
+    whose token is dropped; outputs come a step late."""
+    eng = FakeEngine(n_pages=64)
+    s = Scheduler(eng, TwoPhaseSample(), max_num_seqs=4)
+    s.add(Request("len", [1, 2, 3], 2))
+    s.add(Request("stop", [4, 5], 50, stop_sequences=[[token_for("stop", 1)]]))
+    s.add(Request("on", [6], 6))
+    assert s.step() == []  # the prompts run, sampling is in flight
+    assert eng.log[-1] == [("len", 3, [2]), ("stop", 2, [1]), ("on", 1, [0])]
+    outs = s.step()  # launches the first decode step, then reads the first tokens
+    assert eng.log[-1] == [("len", 1, [0]), ("stop", 1, [0]), ("on", 1, [0])] and eng.fed == 3
+    assert [(o.request_id, o.token, o.finish_reason) for o in outs] == [
+        (r, token_for(r, 0), None) for r in ("len", "stop", "on")]
+    outs = s.step()  # "len" is left out: its second token, in flight, is its last
+    assert eng.log[-1] == [("stop", 1, [0]), ("on", 1, [0])]
+    assert [(o.request_id, o.finish_reason) for o in outs] == [("len", "length"), ("stop", "stop"), ("on", None)]
+    assert [r.request_id for r in s.running] == ["on"]  # "stop" is gone, though it was in the step just launched
+    outs = s.step()
+    assert eng.log[-1] == [("on", 1, [0])]
+    assert [(o.request_id, o.token) for o in outs] == [("on", token_for("on", 2))]  # the token too many is dropped
+    done = run_all(s)
+    assert [o.token for o in done["on"]] == [token_for("on", i) for i in range(3, 6)]
+    assert done["on"][-1].finish_reason == "length"
+    assert eng.cache.free_pages() == 64 and not eng.cache.requests and not s.has_work
+
+
+def test_overlapped_steps_abort_and_preemption_with_a_token_in_flight():
+    eng = FakeEngine(n_pages=16)
+    s = Scheduler(eng, TwoPhaseSample(), max_num_seqs=4)
+    s.add(Request("a", [1, 2, 3], 10))
+    s.add(Request("b", [4, 5, 6], 10))
+    s.step()
+    s.step()
+    s.abort("a")  # its token is in flight: dropped when it is read
+    outs = s.step()
+    assert [o.request_id for o in outs] == ["b"]
+    done = run_all(s)
+    assert [o.token for o in outs + done["b"]] == [token_for("b", i) for i in range(1, 10)]
+    assert eng.cache.free_pages() == 16
+    # pre-emption of a request whose token is in flight: the token is kept, the request waits a
+    # step and then reads prompt and generated tokens as one prompt
+    eng = FakeEngine(n_pages=5, max_positions=200)
+    s = Scheduler(eng, TwoPhaseSample(), max_num_seqs=4)
+    s.add(Request("old", list(range(1, 31)), 40))
+    s.add(Request("new", list(range(1, 17)), 40))
+    done = run_all(s)
+    assert s.stats.preemptions >= 1
+    for rid in ("old", "new"):
+        assert [o.token for o in done[rid]] == [token_for(rid, i) for i in range(40)]
+    assert eng.cache.free_pages() == 5
