@@ -57,6 +57,10 @@ def main(argv=None, stdin=None, stdout=None):
         step = rec["step"]
         entries = []
         for e in rec.get("entries", []):
+            if not e.get("tokens"):
+                if e.get("want"):
+                    raise SystemExit(f"step {step}: request {e['id']!r} wants logits but brings no tokens")
+                continue  # a request that sits this step out
             if not engine.has_request(e["id"]):
                 engine.add_request(e["id"])
             entries.append(StepEntry(e["id"], e["tokens"], e.get("want", [])))
