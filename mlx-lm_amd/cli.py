@@ -8,6 +8,7 @@ from . import __version__
 SUBCOMMANDS = {
     "generate": ("mlx_lm_amd.generate", "main"),
     "trace_run": ("mlx_lm_amd.engine.replay", "main"),
+    "random_weights": ("mlx_lm_amd.weights.random_init", "main"),
 }
 
 

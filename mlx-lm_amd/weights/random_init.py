@@ -31,3 +31,23 @@ def write_model_folder(path, config, seed, scheme="a", dtype="float32", get_mode
         json.dump(config, fh, indent=1)
     save_file(tensors, os.path.join(path, "model.safetensors"))
     return path
+
+
+def main(argv=None):
+    """``python -m mlx_lm_amd random_weights --config config.json --seed 2 --out DIR``."""
+    import argparse
+
+    p = argparse.ArgumentParser(prog="mlx_lm_amd random_weights",
+                                description="Write a model folder with seeded random weights.")
+    p.add_argument("--config", required=True, help="a config.json (its model_type chooses the architecture)")
+    p.add_argument("--seed", type=int, required=True)
+    p.add_argument("--out", required=True, help="folder to write config.json and model.safetensors into")
+    p.add_argument("--scheme", choices=["a", "b"], default="a",
+                   help="a: biases 0, norm scale 1; b: random biases and norm scales")
+    p.add_argument("--dtype", choices=["float32", "bfloat16"], default="float32")
+    a = p.parse_args(argv)
+    with open(a.config) as fh:
+        config = json.load(fh)
+    write_model_folder(a.out, config, a.seed, a.scheme, a.dtype)
+    print(a.out)
+    return 0

@@ -186,3 +186,27 @@ def test_plan_validation():
     plan.schedule = [RunEntry(5, 0)]
     with pytest.raises(ValueError, match="names layer 5"):
         plan.validate()
+
+
+def test_random_weights_from_the_command_line(tmp_path):
+    """``python -m mlx_lm_amd random_weights`` writes the folder that the function writes."""
+    import json
+    import subprocess
+    import sys
+
+    from safetensors.torch import load_file
+
+    from mlx_lm_amd.weights import write_model_folder
+
+    config = dict(model_type="gpt2", n_layer=2, n_embd=48, n_head=3, n_positions=40, vocab_size=77,
+                  layer_norm_epsilon=1e-6, n_inner=100)
+    cfg = tmp_path / "c.json"
+    cfg.write_text(json.dumps(config))
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-m", "mlx_lm_amd", "random_weights", "--config", str(cfg), "--seed", "5",
+                        "--scheme", "b", "--out", str(tmp_path / "cli")], cwd=root, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    write_model_folder(str(tmp_path / "fn"), config, 5, "b")
+    a, b = load_file(str(tmp_path / "cli" / "model.safetensors")), load_file(str(tmp_path / "fn" / "model.safetensors"))
+    assert sorted(a) == sorted(b) and all(torch.equal(a[k], b[k]) for k in a)
+    assert json.loads((tmp_path / "cli" / "config.json").read_text()) == config
