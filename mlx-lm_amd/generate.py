@@ -20,7 +20,7 @@ from . import sample_utils
 from .engine.scheduler import Request, Scheduler
 from .engine.step import Engine
 from .sample_utils import Sampler, make_logits_processors, make_sampler
-from .sampling import PendingRead, apply_processors, read_sampled, sample_batch
+from .sampling import PendingRead, apply_processors, sample_batch
 
 DEFAULT_PROMPT = "hello"
 DEFAULT_MAX_TOKENS = 100

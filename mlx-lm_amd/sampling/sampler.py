@@ -220,13 +220,6 @@ class PendingRead:
 
 
 def read_sampled(tokens, token_logprob):
-    """``(tokens, logprobs)`` as Python lists with a single device-to-host copy
-    when the two came from one ``sample_batch`` call."""
-    import numpy as np
-
-    R = tokens.numel()
-    if (token_logprob.data_ptr() == tokens.data_ptr() + 4 * R and tokens.dtype == torch.int32
-            and tokens.is_contiguous() and token_logprob.is_contiguous()):
-        both = torch.as_strided(tokens, (2 * R,), (1,)).cpu().numpy()
-        return both[:R].tolist(), both[R:].view(np.float32).tolist()
-    return tokens.tolist(), token_logprob.tolist()
+    """``(tokens, logprobs)`` as Python lists, waiting for them (one copy when the two came from one
+    ``sample_batch`` call)."""
+    return PendingRead(tokens, token_logprob).wait()
