@@ -130,9 +130,11 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
 
   uint4 ra[2][PA], rb[2][PB];
   auto load_global = [&](uint4 (&xa)[PA], uint4 (&xb)[PB], int k0) {
-    // a piece beyond K is read from where it still fits and zeroed when it goes to LDS
-    // (zeroing it here would make the loads wait at once)
-    const int kk = (k0 + kc_mine < p.K) ? k0 : 0;
+    // a piece beyond K is read from the row's last eight columns instead (K may be
+    // smaller than a k-block, so no earlier k-block is sure to hold this piece's
+    // columns) and zeroed when it goes to LDS: zeroing it here would make the
+    // loads wait at once
+    const int kk = (k0 + kc_mine < p.K) ? k0 : p.K - 8 - kc_mine;
 #pragma unroll
     for (int i = 0; i < PA; ++i) xa[i] = *(const uint4*)(p.A + a_off[i] + kk);
 #pragma unroll

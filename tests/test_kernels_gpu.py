@@ -76,6 +76,9 @@ GEMM_SHAPES = [
     (130, 300, 72),
     (300, 513, 1608),
     (700, 520, 200),
+    (130, 48, 16),  # K shorter than a k-block of the tile kernels
+    (100, 96, 32),
+    (70, 100, 48),
 ]
 
 
