@@ -85,17 +85,20 @@ class AttentionPlan:
         return max(1, min(most, want, 64))
 
     def row_work(self, n_heads, window=0, max_waves=16):
-        """``(n_splits, n_waves)`` for a decode kernel whose blocks take 4 to ``max_waves`` waves.
+        """``(n_splits, n_waves)`` for a decode kernel whose blocks take 2 to ``max_waves`` waves.
 
         Few rows: many waves a block (a tile of 64 keys each) keep the GPU busy
-        without the second kernel that joining splits needs.  Splits only where
-        sixteen waves would still take several tiles each and blocks are few.
+        without the second kernel that joining splits needs.  Many rows: few
+        waves a block, each with several tiles, so that a block's fixed cost
+        (its way to the first key, joining its waves) is spread over more keys.
+        Splits only where sixteen waves would still take several tiles each and
+        blocks are few.
         """
         ctx = self.max_row_context if window <= 0 else min(self.max_row_context, window + 63)
         tiles = max(1, (ctx + 63) // 64)
         blocks = max(1, self.n_rows * n_heads)
         want = (8 * self.n_compute_units + blocks - 1) // blocks  # eight waves a CU in all
-        n_waves = 4
+        n_waves = 2
         while n_waves < max_waves and n_waves < want and n_waves < tiles:
             n_waves *= 2
         rounds = (tiles + n_waves - 1) // n_waves
