@@ -21,7 +21,9 @@
 // wave takes every eighth 64-wide k-block of the 16 weight rows as the
 // A-operand of two v_mfma_f32_16x16x32_bf16 (lane l reads 32 contiguous bytes
 // of row l % 16 at k offset (l / 16) * 16).  Weight loads run two passes ahead
-// of the MFMAs; the eight partial tiles are summed in a fixed order.
+// of the MFMAs; the eight partial tiles are summed in a fixed order.  Where
+// the matrix has few features and K is not split, a block owns only eight of
+// them (lanes 8..15 of a group repeat the eighth): twice as many blocks.
 //
 // 17 to 64 rows: every block re-reading all activations would cost more than
 // the weights, so a block takes 64 or 128 features (16 a wave) and a slice of
@@ -72,7 +74,7 @@ struct DecodeGemmArgs {
   int max_blocks, q_width, kv_width, head_dim, page_size;
   // split of K over blockIdx.y
   int n_splits, chunks_per_split;
-  int rows;            // output features a block of the 16-row kernel owns (16)
+  int rows;            // output features a block of the 16-row kernel owns (16, or 8 where features are few)
   float* ws;           // [n_splits][M][N] partial sums, when n_splits > 1
   int vec4;            // four outputs at a time: N, ldo and the scatter widths are multiples of 4, pointers aligned
 };
@@ -184,7 +186,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArg
   // packed weights (ldw == 0): the 16 x 64 tile of block b and k-block c lies at
   // (b * n_chunks_all + c) * 1024 elements, first halves of the lanes' 16 values, then second halves
   const bool packed = p.ldw == 0;
-  const uint16_t* wtile = p.W + (size_t)blockIdx.x * ((p.K + 63) / 64) * 1024 + lane * 8;
+  const int fpk = n0 + min(lane & 15, p.rows - 1);  // this lane's feature (inside the padded matrix)
+  const uint16_t* wtile = p.W + (size_t)(fpk >> 4) * ((p.K + 63) / 64) * 1024 + ((lane & 48) | (fpk & 15)) * 8;
   const int n_chunks_all = (p.K + 63) / 64;
   const int c_begin = blockIdx.y * p.chunks_per_split;  // this split's k-blocks
   const int n_chunks = min(n_chunks_all, c_begin + p.chunks_per_split) - c_begin;
@@ -564,6 +567,7 @@ DEFINE_LAST_ERROR(mlxlm_last_error)
 
 #define MAX_LDS_BYTES (120 * 1024)
 #define MID_WAVES 4
+#define FEW_BLOCKS 150  // fewer blocks of 16 features than this leave many CUs idle
 
 // LDS row stride: rows of 16-byte reads from 16 lanes must fall on distinct
 // banks, which holds when the stride in 32-bit words is 4 mod 32.
@@ -672,7 +676,9 @@ extern "C" int gemm_bf16_decode(
   p.W = (const uint16_t*)W, p.A = (const uint16_t*)A, p.X = X;
   p.gamma = gamma, p.beta = beta, p.eps = eps;
   p.K = K, p.lda = lda, p.ldx = ldx, p.ldw = ldw;
-  p.rows = 16;
+  // Few features and no split of K: blocks of eight features (half of each MFMA
+  // tile is idle, which costs nothing here) put twice as many CUs to work.
+  p.rows = (M <= 16 && n_splits == 1 && (N + 15) / 16 < FEW_BLOCKS) ? 8 : 16;
   p.n_splits = n_splits, p.chunks_per_split = chunks_per_split(K, n_splits);
   p.ws = ws;
   if (n_splits > 1) {
