@@ -33,6 +33,9 @@ struct GemmArgs {
   int M, N, K;
   int lda, ldw, ldo;
   int flags;
+  // K split over blockIdx.y (tile kernel, 128 x 128): partial sums [n_splits][M][N] go to ws
+  float* ws;
+  int n_splits, blocks_per_split;
 };
 
 __device__ __forceinline__ void store_out(const GemmArgs& p, int m, int n, float v) {
@@ -127,6 +130,14 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
 #pragma unroll
   for (int i = 0; i < PB; ++i) b_off[i] = min(n0 + (tid >> 3) + ROW_STEP * i, p.N - 1) * p.ldw + (tid & 7) * 8;
   const int kc_mine = (tid & 7) * 8;
+  // this split's k-blocks (all of them without a split); the offsets start at its first column
+  const int kb_lo = blockIdx.y * p.blocks_per_split;
+  const int n_blocks = min((p.K + BK - 1) / BK, kb_lo + p.blocks_per_split) - kb_lo;
+  const int k_lo = kb_lo * BK;
+#pragma unroll
+  for (int i = 0; i < PA; ++i) a_off[i] += k_lo;
+#pragma unroll
+  for (int i = 0; i < PB; ++i) b_off[i] += k_lo;
 
   uint4 ra[2][PA], rb[2][PB];
   auto load_global = [&](uint4 (&xa)[PA], uint4 (&xb)[PB], int k0) {
@@ -134,21 +145,20 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
     // smaller than a k-block, so no earlier k-block is sure to hold this piece's
     // columns) and zeroed when it goes to LDS: zeroing it here would make the
     // loads wait at once
-    const int kk = (k0 + kc_mine < p.K) ? k0 : p.K - 8 - kc_mine;
+    const int kk = (k_lo + k0 + kc_mine < p.K) ? k0 : p.K - 8 - kc_mine - k_lo;
 #pragma unroll
     for (int i = 0; i < PA; ++i) xa[i] = *(const uint4*)(p.A + a_off[i] + kk);
 #pragma unroll
     for (int i = 0; i < PB; ++i) xb[i] = *(const uint4*)(p.W + b_off[i] + kk);
   };
   auto store_lds = [&](int stage, const uint4 (&xa)[PA], const uint4 (&xb)[PB], int k0) {
-    const bool in = k0 + kc_mine < p.K;
+    const bool in = k_lo + k0 + kc_mine < p.K;
 #pragma unroll
     for (int i = 0; i < PA; ++i) *(uint4*)(As[stage] + lds_off0 + i * ROW_STEP * LDS_STRIDE) = in ? xa[i] : ZERO4;
 #pragma unroll
     for (int i = 0; i < PB; ++i) *(uint4*)(Bs[stage] + lds_off0 + i * ROW_STEP * LDS_STRIDE) = in ? xb[i] : ZERO4;
   };
 
-  const int n_blocks = (p.K + BK - 1) / BK;
   load_global(ra[0], rb[0], 0);
   if (n_blocks > 1) load_global(ra[1], rb[1], BK);
   store_lds(0, ra[0], rb[0], 0);
@@ -194,7 +204,7 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
     for (int i = 0; i < PB; ++i) *(uint4*)(Bs[stage] + lds_off0 + i * ROW_STEP * LDS_STRIDE) = xb[i];
   };
   int kb = 0;
-  const int whole_blocks = p.K / BK;  // k-blocks that need no masking
+  const int whole_blocks = min(n_blocks, p.K / BK - kb_lo);  // k-blocks that need no masking
   for (; kb + 4 <= whole_blocks; kb += 2) {
     load_whole(ra[0], rb[0], (kb + 2) * BK);
     __builtin_amdgcn_sched_barrier(0);  // the loads go out before the arithmetic, not after it
@@ -218,6 +228,25 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
     multiply(1);
     if (kb + 2 < n_blocks) store_lds(0, ra[0], rb[0], (kb + 2) * BK);
     __syncthreads();
+  }
+
+  if (p.n_splits > 1) {  // the partial sums as they are; sum_partials adds them and runs the epilogue
+    float* ws = p.ws + (size_t)blockIdx.y * p.M * p.N;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + wn * TN * 32 + j * 32 + (lane & 31);
+      if (n >= p.N) continue;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int mb = m0 + wm * TM * 32 + i * 32 + 4 * (lane >> 5);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = mb + 8 * (r >> 2) + (r & 3);
+          if (m < p.M) ws[(size_t)m * p.N + n] = acc[i][j][r];
+        }
+      }
+    }
+    return;
   }
 
   // Epilogue.  Accumulator r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4,
@@ -366,7 +395,7 @@ static void launch_tiles(const GemmArgs& p, hipStream_t stream) {
   const int super_m = ((p.M + S::BM - 1) / S::BM + S::SUPER_M - 1) / S::SUPER_M;
   const int super_n = ((p.N + S::BN - 1) / S::BN + S::SUPER_N - 1) / S::SUPER_N;
   const int per_die = (super_m * super_n + 7) / 8;  // super-tiles a die works through
-  dim3 grid(per_die * 8 * S::SUPER_M * S::SUPER_N), block(S::THREADS);
+  dim3 grid(per_die * 8 * S::SUPER_M * S::SUPER_N, p.n_splits), block(S::THREADS);
   hipLaunchKernelGGL(gemm_bf16_tile_kernel<S>, grid, block, 0, stream, p);
 }
 
@@ -385,10 +414,32 @@ static double cost_256(int M, int N) {
   return (double)((tiles + 255) / 256) * 2.2;
 }
 
-// variant: 0 = choose, 1 = 128 x 128 tiles, 2 = skinny kernel, 3 = 256 x 256 tiles
+// Into how many parts the 128 x 128 kernel should split K (1: no split).  Few rows
+// give few tiles: 65 to 128 rows of GPT-2 XL's projections are 13 to 50 tiles
+// for 256 CUs, and a tile's walk through K takes the same time whether 50 or
+// 500 of them run.  Measured at those sizes (65 to 640 rows): two parts win up
+// to some 160 tiles, four where the output is narrow (N = 1600) up to some 56;
+// beyond, the partial sums ([parts][M][N] floats, written and read once) cost
+// more than the idle CUs.
+// A part keeps at least six k-blocks: a block's prologue and epilogue cost two.
+// `force` > 0 asks for that many parts wherever K has them (for tests of small sizes).
+extern "C" int gemm_bf16_splits(int M, int N, int K, int force) {
+  if (M <= SK_MAXM) return 1;
+  const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+  const int n_blocks = (K + BK - 1) / BK;
+  int want = (tiles <= 56 && N <= 2048) ? 4 : tiles <= 160 ? 2 : 1;
+  if (want > n_blocks / 6) want = n_blocks / 6;
+  if (force > 0) want = force < n_blocks ? force : n_blocks;
+  if (want <= 1) return 1;
+  const int per = (n_blocks + want - 1) / want;
+  return (n_blocks + per - 1) / per;  // no empty part
+}
+
+// variant: 0 = choose, 1 = 128 x 128 tiles, 2 = skinny kernel, 3 = 256 x 256 tiles.
+// n_splits > 1 (128 x 128 tiles only): no epilogue, the partial sums go to ws.
 extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* bias, int M, int N,
-                         int K, int lda, int ldw, int ldo, int flags, int variant,
-                         hipStream_t stream) {
+                         int K, int lda, int ldw, int ldo, int flags, int variant, int n_splits,
+                         float* ws, size_t ws_floats, hipStream_t stream) {
   GemmArgs p;
   p.A = (const uint16_t*)A;
   p.W = (const uint16_t*)W;
@@ -399,6 +450,16 @@ extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* b
   p.flags = flags;
   if (check_args(p)) return 1;
   if (M == 0) return 0;
+  const int n_blocks = (K + BK - 1) / BK;
+  if (n_splits < 1 || n_splits > n_blocks) FAIL("gemm_bf16: %d splits of K=%d", n_splits, K);
+  p.ws = ws, p.n_splits = n_splits, p.blocks_per_split = (n_blocks + n_splits - 1) / n_splits;
+  if (n_splits > 1) {
+    if (variant == 0) variant = 1;
+    if (variant != 1) FAIL("gemm_bf16: only the 128 x 128 kernel splits K");
+    if (p.blocks_per_split * (n_splits - 1) >= n_blocks) FAIL("gemm_bf16: %d splits of K=%d leave one empty", n_splits, K);
+    if (!ws || ((uintptr_t)ws & 15) || ws_floats < (size_t)n_splits * M * N)
+      FAIL("gemm_bf16: %d splits of %d x %d need an aligned workspace of that many floats", n_splits, M, N);
+  }
   if (variant == 0) {
     if (M <= SK_MAXM)
       variant = 2;

@@ -15,6 +15,10 @@ records such a step; its integer arrays are built as for an eager step, but
 into a device buffer of the graph's own.
 """
 
+import contextlib
+import gc
+import weakref
+
 import numpy as np
 import torch
 
@@ -25,11 +29,33 @@ def _pad4(n):
     return (n + 3) // 4 * 4
 
 
+@contextlib.contextmanager
+def _recording(graph):
+    """``torch.cuda.graph(graph)`` with the cyclic garbage collector switched off.
+
+    The collector may run at any allocation.  If it then frees a recorded graph
+    that is garbage (an engine that was dropped), that graph is destroyed
+    inside this capture, which HIP refuses; the error is raised in a
+    destructor and ends the process.  (``torch.cuda.graph`` collects once
+    before the capture begins; this keeps it from happening again within.)
+    """
+    was_enabled = gc.isenabled()
+    gc.disable()
+    try:
+        with torch.cuda.graph(graph):
+            yield
+    finally:
+        if was_enabled:
+            gc.enable()
+
+
 class DecodeGraph:
     """The recorded decode step for one batch size."""
 
     def __init__(self, engine, batch):
-        self.engine, self.batch = engine, batch
+        # (a weak reference: the engine owns its graphs, and without a cycle they are freed
+        # the moment the engine is dropped, not whenever the collector next runs)
+        self.engine, self.batch = weakref.proxy(engine), batch
         cm = engine.cache
         B = batch
         self.max_blocks = cm.blocks_for(engine.decoder.max_positions)
@@ -114,7 +140,7 @@ class DecodeGraph:
             graph = torch.cuda.CUDAGraph()
             eng.scratch.frozen = True
             try:
-                with torch.cuda.graph(graph):
+                with _recording(graph):
                     self.dev.copy_(self.host, non_blocking=True)
                     self._feed(ctx)
                     eng.scratch.reset()
@@ -133,11 +159,12 @@ class StepGraph:
     """A recorded step of one shape (tokens per request, number of wanted places)."""
 
     def __init__(self, engine):
-        self.engine = engine
+        self.engine = weakref.proxy(engine)
         self.dev = None  # the step's integer arrays, at the same offsets every time
         self.graph = None
         self.logits = None
         self.failed = False
+        self.error = None  # why recording failed, if it did
         self._keep = None
 
     def run(self, entries):
@@ -148,11 +175,12 @@ class StepGraph:
             graph = torch.cuda.CUDAGraph()
             eng.scratch.frozen = True
             try:
-                with torch.cuda.graph(graph):
+                with _recording(graph):
                     eng.scratch.reset()
                     self.logits = eng.decoder.forward(ctx)
-            except Exception:
+            except Exception as e:
                 self.failed = True  # this shape stays eager (an error of the step itself comes again below)
+                self.error = e
             finally:
                 eng.scratch.frozen = False
             if self.failed:

@@ -88,13 +88,8 @@ class Engine:
         self.use_graphs = use_graphs and all(getattr(p, "graph_safe", False) for p in self.decoder.parts())
         self._graphs = {}
         # Other steps whose shape keeps coming back (portions of prompts of the scheduler's size, with
-        # or without decoding requests beside them) could be recorded too.  Switched off: the first
-        # run of it ended in an abort of the process whose message was lost, and no cause has been
-        # shown since; asking for it raises until one has.
-        if record_prompt_steps:
-            raise NotImplementedError("recording steps other than decode steps is switched off: "
-                                      "its first run aborted and the cause is not known")
-        self.record_prompt_steps = False
+        # or without decoding requests beside them) are recorded too, if asked for.
+        self.record_prompt_steps = bool(record_prompt_steps) and self.use_graphs
         self._step_graphs = OrderedDict()
         self._shape_seen = {}
 

@@ -25,7 +25,16 @@ GEMM_OUT_F32 = 4
 GEMM_KV = 8
 
 
+# torch's current stream as a raw handle.  torch.cuda.current_stream() builds a Stream object
+# through several Python layers (some 4 us a call, once per launch); the binding below is what
+# that ends in.
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_current_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream():
+    if _raw_stream is not None and _current_device is not None:
+        return _vp(_raw_stream(_current_device()))
     return _vp(torch.cuda.current_stream().cuda_stream)
 
 
@@ -38,17 +47,22 @@ def _need(cond, msg):
         raise ValueError(msg)
 
 
+def _fail(msg):
+    """``cond or _fail(f"...")``: the message is put together only when the check fails."""
+    raise ValueError(msg)
+
+
 def _dev(t, name, dtype=None):
-    _need(t.is_cuda, f"{name} must be on the GPU")
-    _need(t.is_contiguous(), f"{name} must be contiguous")
+    t.is_cuda or _fail(f"{name} must be on the GPU")
+    t.is_contiguous() or _fail(f"{name} must be contiguous")
     if dtype is not None:
-        _need(t.dtype == dtype, f"{name} must be {dtype}, is {t.dtype}")
+        t.dtype == dtype or _fail(f"{name} must be {dtype}, is {t.dtype}")
 
 
 def _rows2d(t, name):
     """A 2-D tensor whose rows are contiguous; returns its row stride."""
-    _need(t.is_cuda, f"{name} must be on the GPU")
-    _need(t.dim() == 2 and t.stride(1) == 1, f"{name} must be 2-D with contiguous rows")
+    t.is_cuda or _fail(f"{name} must be on the GPU")
+    (t.dim() == 2 and t.stride(1) == 1) or _fail(f"{name} must be 2-D with contiguous rows")
     return t.stride(0)
 
 
@@ -62,7 +76,7 @@ def embed_gather_add(out, table, ids, add_table=None, add_ids=None):
     _dev(out, "out", torch.float32)
     _dev(table, "table")
     _dev(ids, "ids", torch.int32)
-    _need(table.dtype in DT, f"table dtype {table.dtype} not supported")
+    table.dtype in DT or _fail(f"table dtype {table.dtype} not supported")
     _need(table.shape[1] == width and ids.numel() >= n, "embed_gather_add: shapes disagree")
     if add_table is not None:
         _dev(add_table, "add_table", table.dtype)
@@ -93,7 +107,7 @@ def layernorm(out, x, gamma, beta, eps, rows=None):
     n, width = out.shape
     _dev(out, "out")
     _dev(x, "x", torch.float32)
-    _need(out.dtype in DT, f"out dtype {out.dtype} not supported")
+    out.dtype in DT or _fail(f"out dtype {out.dtype} not supported")
     _need(x.shape[-1] == width, "layernorm: widths disagree")
     if rows is None:
         _need(x.shape[0] >= n, "layernorm: fewer input rows than output rows")
@@ -103,7 +117,7 @@ def layernorm(out, x, gamma, beta, eps, rows=None):
     for name, v in (("gamma", gamma), ("beta", beta)):
         if v is not None:
             _dev(v, name, torch.float32)
-            _need(v.numel() == width, f"layernorm: {name} has {v.numel()} elements, width is {width}")
+            v.numel() == width or _fail(f"layernorm: {name} has {v.numel()} elements, width is {width}")
     rc = lib.layernorm(
         _ptr(out), _ptr(x), _ptr(rows), _ptr(gamma), _ptr(beta), _c_float(eps),
         _c_int(n), _c_int(width), _c_int(DT[out.dtype]), _stream(),
@@ -279,7 +293,7 @@ def sum_partials_norm(h, ws, n_splits, bias, gamma, beta, eps, out):
     for name, v in (("bias", bias), ("gamma", gamma), ("beta", beta)):
         if v is not None:
             _dev(v, name, torch.float32)
-            _need(v.numel() == N, f"sum_partials_norm: {name} has {v.numel()} elements, width is {N}")
+            v.numel() == N or _fail(f"sum_partials_norm: {name} has {v.numel()} elements, width is {N}")
     rc = lib.sum_partials_norm(_ptr(h), _c_int(_rows2d(h, "h")), _ptr(ws), _c_int(n_splits), _ptr(bias),
                                _ptr(gamma), _ptr(beta), _c_float(eps), _ptr(out), _c_int(DT[out.dtype]),
                                _c_int(M), _c_int(N), _stream())
@@ -311,8 +325,8 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
     M, K = a.shape
     N = w.shape[0]
     ldw, ldo = _rows2d(w, "w"), _rows2d(out, "out")
-    _need(w.shape[1] == K, f"linear: a is [{M},{K}] but w is {list(w.shape)}")
-    _need(tuple(out.shape) == (M, N), f"linear: out is {list(out.shape)}, want [{M},{N}]")
+    w.shape[1] == K or _fail(f"linear: a is [{M},{K}] but w is {list(w.shape)}")
+    tuple(out.shape) == (M, N) or _fail(f"linear: out is {list(out.shape)}, want [{M},{N}]")
     _need(a.dtype == w.dtype and w.dtype in DT, "linear: a and w must share float32 or bfloat16")
     if bias is not None:
         _dev(bias, "bias", torch.float32)
@@ -381,15 +395,44 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
     lda = _rows2d(a, "a")
     if w.dtype == torch.float32:
         lib = build.load("gemm_f32")
-        fn = lib.gemm_f32
+        rc = lib.gemm_f32(
+            _ptr(out), _ptr(a), _ptr(w), _ptr(bias), _c_int(M), _c_int(N), _c_int(K),
+            _c_int(lda), _c_int(ldw), _c_int(ldo), _c_int(flags), _c_int(variant), _stream(),
+        )
+        build.check(lib, rc, "linear")
     else:
+        # Few rows give the tile kernel few tiles: K is split then as for the decode kernels,
+        # and the same second kernels add the parts and run the epilogue.
         lib = build.load("gemm_bf16")
-        fn = lib.gemm_bf16
-    rc = fn(
-        _ptr(out), _ptr(a), _ptr(w), _ptr(bias), _c_int(M), _c_int(N), _c_int(K),
-        _c_int(lda), _c_int(ldw), _c_int(ldo), _c_int(flags), _c_int(variant), _stream(),
-    )
-    build.check(lib, rc, "linear")
+        n_splits, ws = 1, None
+        if variant in (0, 1) and M > 0:
+            n_blocks = (K + 63) // 64
+            if splits is None:
+                n_splits = lib.gemm_bf16_splits(_c_int(M), _c_int(N), _c_int(K), _c_int(force_splits))
+            else:
+                per_split = -(-n_blocks // max(1, min(splits, n_blocks)))
+                n_splits = -(-n_blocks // per_split)
+            if n_splits > 1:
+                ws = split_workspace(w.device)
+                n_splits = min(n_splits, ws.numel() // (M * N))
+                if n_splits > 1:  # (again without an empty part)
+                    per_split = -(-n_blocks // n_splits)
+                    n_splits = -(-n_blocks // per_split)
+            if n_splits > 1 and pending is not None:
+                pending.settle()  # the workspace is about to be written again
+        rc = lib.gemm_bf16(
+            _ptr(out), _ptr(a), _ptr(w), _ptr(bias), _c_int(M), _c_int(N), _c_int(K),
+            _c_int(lda), _c_int(ldw), _c_int(ldo), _c_int(flags), _c_int(variant),
+            _c_int(max(1, n_splits)), _ptr(ws if n_splits > 1 else None),
+            _c_size_t(ws.numel() if n_splits > 1 else 0), _stream(),
+        )
+        build.check(lib, rc, "linear")
+        if n_splits > 1:
+            if accumulate and pending is not None and pending.allowed:
+                pending.target, pending.ws, pending.n_splits, pending.bias = out, ws, n_splits, bias
+            else:
+                sum_partials(out, ws, n_splits, bias, gelu=gelu, accumulate=accumulate, scatter=scatter)
+            return out
     if scatter is not None:
         q, kw = scatter.q_width, scatter.kv_width
         kv_write(out[:, q : q + kw], out[:, q + kw :], scatter.kv, scatter.block_table,
@@ -579,7 +622,7 @@ def sample_rows(tokens, token_logprob, logits, temp, top_p, min_p, min_keep, top
                         ("xtc_thr", xtc_thr, torch.float32), ("seed", seed, torch.int64),
                         ("counter", counter, torch.int32)):
         _dev(t, name, dt)
-        _need(t.numel() >= n, f"sample_rows: {name} shorter than the rows")
+        t.numel() >= n or _fail(f"sample_rows: {name} shorter than the rows")
     _need(tokens.numel() >= n and token_logprob.numel() >= n, "sample_rows: outputs too short")
     n_special = 0
     if xtc_special is not None and xtc_special.numel() > 0:
@@ -624,7 +667,7 @@ def apply_penalties(logits, offsets, hist, rep, rep_ctx, pres, pres_ctx, freq, f
                         ("freq", freq, torch.float32), ("rep_ctx", rep_ctx, torch.int32),
                         ("pres_ctx", pres_ctx, torch.int32), ("freq_ctx", freq_ctx, torch.int32)):
         _dev(t, name, dt)
-        _need(t.numel() >= n, f"apply_penalties: {name} shorter than the rows")
+        t.numel() >= n or _fail(f"apply_penalties: {name} shorter than the rows")
     rc = lib.apply_penalties(_ptr(logits), _c_int(ld), _c_int(n), _ptr(offsets), _ptr(hist),
                              _ptr(rep), _ptr(rep_ctx), _ptr(pres), _ptr(pres_ctx), _ptr(freq),
                              _ptr(freq_ctx), _stream())

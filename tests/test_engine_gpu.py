@@ -375,8 +375,6 @@ def test_recorded_decode_steps_equal_eager_ones(folders, dtype):
         assert torch.equal(results[True][r], results[False][r]), r
 
 
-@pytest.mark.skip(reason="recording prompt steps is switched off: its first run aborted the process, the "
-                         "message was lost and no cause has been shown; Engine(record_prompt_steps=True) raises")
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_recorded_steps_of_repeating_shapes(folders, dtype):
     """Portions of one size, alone and beside a decoding request, come back with the same shape: from
@@ -419,6 +417,35 @@ def test_recorded_steps_of_repeating_shapes(folders, dtype):
         n = sum(x.shape[0] for x in got[r])
         want = _plain_logits(weights, config, toks[:n], dtype)
         _close(torch.cat(got[r]), want, dtype, f"recorded shapes, request {r}")
+
+
+def test_a_dropped_engine_frees_its_graphs_at_once(folders):
+    """An engine and its recorded graphs form no reference cycle: dropping the engine frees them
+    there and then.  (Left to the cycle collector, a graph could be destroyed while another
+    engine records one, which HIP refuses with an error that ends the process.)"""
+    import gc
+    import weakref
+
+    from mlx_lm_amd.engine import Engine, StepEntry
+    from mlx_lm_amd.utils import load_model
+
+    folder, config, _ = folders[("A", 8.0)]
+    model, _ = load_model(folder, dtype="bfloat16")
+    gc.collect()
+    gc.disable()
+    try:
+        eng = Engine(model, dtype="bfloat16", page_size=16, n_pages=8, max_requests=4, record_prompt_steps=True)
+        eng.add_request("a")
+        for at in range(0, 12, 3):  # the shape (3,) four times: recorded from the third on
+            eng.step([StepEntry("a", [1 + at, 2 + at, 3 + at], [2])])
+        for t in range(3):
+            eng.step([StepEntry("a", [20 + t], [0])])
+        refs = [weakref.ref(eng), weakref.ref(eng._graphs[1])] + [weakref.ref(g) for g in eng._step_graphs.values()]
+        assert len(refs) == 3 and eng._graphs[1].graph is not None
+        del eng
+        assert all(r() is None for r in refs)
+    finally:
+        gc.enable()
 
 
 @pytest.mark.parametrize("use_graphs", [True, False])

@@ -650,11 +650,13 @@ def test_gemm_bf16_decode_mid(M, N, K, mode, packed):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 48, 1024), (8, 1600, 6400), (16, 80, 200), (16, 1600, 6400), (11, 333, 1608),
-                                   (17, 48, 1024), (64, 1600, 6400), (40, 333, 1608), (33, 4800, 1600)])
+                                   (17, 48, 1024), (64, 1600, 6400), (40, 333, 1608), (33, 4800, 1600),
+                                   (65, 257, 1608), (130, 300, 200), (300, 1600, 1600), (72, 96, 128)])
 @pytest.mark.parametrize("mode", ["plain", "accumulate", "gelu"])
 def test_gemm_bf16_decode_split_k(M, N, K, mode):
-    """K split over blocks: partial sums in the workspace, added in the order of the splits by a
-    second kernel, so a number of splits gives the same bits run after run."""
+    """K split over blocks (the decode kernels up to 64 rows, the tile kernel beyond): partial sums
+    in the workspace, added in the order of the splits by a second kernel, so a number of splits
+    gives the same bits run after run."""
     k = _k()
     a = _rand((M, K), torch.bfloat16, 10)
     w = _rand((N, K), torch.bfloat16, 11, 0.1)
@@ -685,7 +687,7 @@ def test_gemm_bf16_decode_split_k(M, N, K, mode):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 256), (8, 1600, 6400), (16, 96, 384), (40, 240, 200), (64, 1600, 1600),
-                                   (5, 4100, 512)])
+                                   (5, 4100, 512), (100, 1600, 1600), (200, 240, 456)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_pending_sum_is_added_by_the_norm(M, N, K, out_dtype):
     """A split projection into the residual stream may stop at its partial sums; the norm that reads the
@@ -752,6 +754,13 @@ def test_default_splits_fill_the_gpu():
     assert lib.gemm_bf16_decode_splits(8, 64, 64, 0, 0) == 1
     assert lib.gemm_bf16_decode_splits(8, 64, 64, 0, 2) == 1  # one k-block cannot be split
     assert lib.gemm_bf16_decode_splits(8, 64, 200, 0, 2) == 2
+    tiles = k.build.load("gemm_bf16")
+    assert tiles.gemm_bf16_splits(64, 1600, 6400, 0) == 1  # (the decode kernels' rows)
+    assert tiles.gemm_bf16_splits(72, 1600, 6400, 0) == 4
+    assert tiles.gemm_bf16_splits(128, 4800, 1600, 0) == 2
+    assert tiles.gemm_bf16_splits(2048, 4800, 1600, 0) == 1
+    assert tiles.gemm_bf16_splits(100, 96, 128, 0) == 1  # too few k-blocks to share out
+    assert tiles.gemm_bf16_splits(100, 96, 128, 3) == 2
 
 
 @pytest.mark.parametrize("M", [1, 5, 16, 40, 80])
