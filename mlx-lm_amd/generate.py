@@ -60,8 +60,10 @@ def engine_for(model, page_size=16, max_requests=64, max_cache_tokens=None):
             free, _ = torch.cuda.mem_get_info(torch.device(model.device))
             max_cache_tokens = min(max_requests * dec.max_positions, int(free * 0.6) // per_token)
             max_cache_tokens = max(max_cache_tokens, dec.max_positions)
+        # (a scheduler's steps keep coming back in the same shapes: portions of one size beside
+        # the requests that decode; those are recorded as the decode steps are)
         eng = Engine(model, dtype=model.dtype, device=model.device, page_size=page_size,
-                     max_tokens=max_cache_tokens, max_requests=max_requests)
+                     max_tokens=max_cache_tokens, max_requests=max_requests, record_prompt_steps=True)
         engines[key] = eng
     return eng
 

@@ -388,35 +388,38 @@ def test_recorded_steps_of_repeating_shapes(folders, dtype):
     model, _ = load_model(folder, dtype=dtype)
     seqs = {r: helpers.random_tokens(n, V, seed=80 + i) for i, (r, n) in enumerate(
         [("a", 230), ("b", 200), ("c", 160)])}
-    eng = Engine(model, dtype=dtype, page_size=16, n_pages=30, max_requests=4, record_prompt_steps=True)
-    got = {r: [] for r in seqs}
-
     def portion(r, at, n):
         return StepEntry(r, seqs[r][at : at + n], list(range(n)))
 
-    eng.add_request("a")
-    for at in range(0, 200, 40):  # five steps of shape (40,)
-        got["a"].append(eng.step([portion("a", at, 40)]).clone())
-    eng.add_request("b")
-    for i in range(5):  # five of shape (1, 40)
-        out = eng.step([portion("a", 200 + i, 1), portion("b", 40 * i, 40)])
-        got["a"].append(out[:1].clone())
-        got["b"].append(out[1:].clone())
-    for i in range(5, 30):  # decode steps
-        got["a"].append(eng.step([portion("a", 200 + i, 1)]).clone())
-    eng.end_request("a")
-    eng.end_request("b")
-    eng.cache.poison_free_pages()
-    eng.add_request("c")
-    for at in range(0, 160, 40):  # shape (40,) again, replayed, on pages that a and b held
-        got["c"].append(eng.step([portion("c", at, 40)]).clone())
-    eng.cache.check()
-    recorded = {k: g for k, g in eng._step_graphs.items() if g.graph is not None}
-    assert set(recorded) == {((40,), 40, True), ((1, 40), 41, True)}
+    results = {}
+    for record in (True, False):
+        eng = Engine(model, dtype=dtype, page_size=16, n_pages=30, max_requests=4, record_prompt_steps=record)
+        got = {r: [] for r in seqs}
+        eng.add_request("a")
+        for at in range(0, 200, 40):  # five steps of shape (40,)
+            got["a"].append(eng.step([portion("a", at, 40)]).clone())
+        eng.add_request("b")
+        for i in range(5):  # five of shape (1, 40)
+            out = eng.step([portion("a", 200 + i, 1), portion("b", 40 * i, 40)])
+            got["a"].append(out[:1].clone())
+            got["b"].append(out[1:].clone())
+        for i in range(5, 30):  # decode steps
+            got["a"].append(eng.step([portion("a", 200 + i, 1)]).clone())
+        eng.end_request("a")
+        eng.end_request("b")
+        eng.cache.poison_free_pages()
+        eng.add_request("c")
+        for at in range(0, 160, 40):  # shape (40,) again, replayed, on pages that a and b held
+            got["c"].append(eng.step([portion("c", at, 40)]).clone())
+        eng.cache.check()
+        recorded = {k: g for k, g in eng._step_graphs.items() if g.graph is not None}
+        assert set(recorded) == ({((40,), 40, True), ((1, 40), 41, True)} if record else set())
+        results[record] = {r: torch.cat(v) for r, v in got.items()}
     for r, toks in seqs.items():
-        n = sum(x.shape[0] for x in got[r])
+        n = results[True][r].shape[0]
         want = _plain_logits(weights, config, toks[:n], dtype)
-        _close(torch.cat(got[r]), want, dtype, f"recorded shapes, request {r}")
+        _close(results[True][r], want, dtype, f"recorded shapes, request {r}")
+        assert torch.equal(results[True][r], results[False][r]), r  # the same launches, replayed
 
 
 def test_a_dropped_engine_frees_its_graphs_at_once(folders):
