@@ -171,7 +171,11 @@ class StepGraph:
         eng = self.engine
         ctx = eng._build_context(entries, static=self)
         if self.graph is None:
-            # the shape has run eagerly before: libraries are loaded and scratch memory is large enough
+            # once eagerly with this context (its block tables are wider, its keys may be split
+            # further than in the eager steps before): scratch memory grows to what it needs
+            eng.scratch.reset()
+            eng.decoder.forward(ctx)
+            torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             eng.scratch.frozen = True
             try:
