@@ -95,7 +95,9 @@ using Tile256 = TileShape<2, 4, 4, 2, 4, 2, 1>;
 // iteration i the loads of k-block i+2 are issued, k-block i is multiplied
 // out of LDS, then k-block i+1 (loaded an iteration ago) goes from registers
 // to the other half of LDS; one barrier an iteration.
-template <typename S>
+// SPLIT: K is shared out over blockIdx.y and the partial sums go to the workspace (a kernel of
+// its own, so that the unsplit one carries none of it).
+template <typename S, bool SPLIT>
 __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_kernel(GemmArgs p) {
   constexpr int BM = S::BM, BN = S::BN, TM = S::TM, TN = S::TN, PA = S::PA, PB = S::PB;
   __shared__ __attribute__((aligned(16))) uint16_t As[2][BM * LDS_STRIDE];
@@ -131,13 +133,15 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
   for (int i = 0; i < PB; ++i) b_off[i] = min(n0 + (tid >> 3) + ROW_STEP * i, p.N - 1) * p.ldw + (tid & 7) * 8;
   const int kc_mine = (tid & 7) * 8;
   // this split's k-blocks (all of them without a split); the offsets start at its first column
-  const int kb_lo = blockIdx.y * p.blocks_per_split;
-  const int n_blocks = min((p.K + BK - 1) / BK, kb_lo + p.blocks_per_split) - kb_lo;
+  const int kb_lo = SPLIT ? blockIdx.y * p.blocks_per_split : 0;
+  const int n_blocks = SPLIT ? min((p.K + BK - 1) / BK, kb_lo + p.blocks_per_split) - kb_lo : (p.K + BK - 1) / BK;
   const int k_lo = kb_lo * BK;
+  if constexpr (SPLIT) {
 #pragma unroll
-  for (int i = 0; i < PA; ++i) a_off[i] += k_lo;
+    for (int i = 0; i < PA; ++i) a_off[i] += k_lo;
 #pragma unroll
-  for (int i = 0; i < PB; ++i) b_off[i] += k_lo;
+    for (int i = 0; i < PB; ++i) b_off[i] += k_lo;
+  }
 
   uint4 ra[2][PA], rb[2][PB];
   auto load_global = [&](uint4 (&xa)[PA], uint4 (&xb)[PB], int k0) {
@@ -204,7 +208,7 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
     for (int i = 0; i < PB; ++i) *(uint4*)(Bs[stage] + lds_off0 + i * ROW_STEP * LDS_STRIDE) = xb[i];
   };
   int kb = 0;
-  const int whole_blocks = min(n_blocks, p.K / BK - kb_lo);  // k-blocks that need no masking
+  const int whole_blocks = SPLIT ? min(n_blocks, p.K / BK - kb_lo) : p.K / BK;  // k-blocks that need no masking
   for (; kb + 4 <= whole_blocks; kb += 2) {
     load_whole(ra[0], rb[0], (kb + 2) * BK);
     __builtin_amdgcn_sched_barrier(0);  // the loads go out before the arithmetic, not after it
@@ -230,7 +234,7 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
     __syncthreads();
   }
 
-  if (p.n_splits > 1) {  // the partial sums as they are; sum_partials adds them and runs the epilogue
+  if constexpr (SPLIT) {  // the partial sums as they are; sum_partials adds them and runs the epilogue
     float* ws = p.ws + (size_t)blockIdx.y * p.M * p.N;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
@@ -396,7 +400,10 @@ static void launch_tiles(const GemmArgs& p, hipStream_t stream) {
   const int super_n = ((p.N + S::BN - 1) / S::BN + S::SUPER_N - 1) / S::SUPER_N;
   const int per_die = (super_m * super_n + 7) / 8;  // super-tiles a die works through
   dim3 grid(per_die * 8 * S::SUPER_M * S::SUPER_N, p.n_splits), block(S::THREADS);
-  hipLaunchKernelGGL(gemm_bf16_tile_kernel<S>, grid, block, 0, stream, p);
+  if (p.n_splits > 1)
+    hipLaunchKernelGGL((gemm_bf16_tile_kernel<S, true>), grid, block, 0, stream, p);
+  else
+    hipLaunchKernelGGL((gemm_bf16_tile_kernel<S, false>), grid, block, 0, stream, p);
 }
 
 // Microseconds per k-block of the busiest CU, from what was measured at GPT-2 XL
