@@ -6,7 +6,9 @@ Prints one JSON line.  ``value`` is decoded tokens a second at the given batch
 (default 8): K timed decode steps after W untimed ones, every request starting
 from a 512-token prompt (the reference's benchmark draws uniform random
 prompts and switches end-of-sequence off, mlx_lm/benchmark.py:118-124).
-``prefill`` is one step of 2 x 1,024 prompt tokens; ``points`` holds decode at
+``prefill`` is one step of 2 x 1,024 prompt tokens (the best of five: a step
+whose shape keeps coming back is replayed from its recorded graph, as in the
+serving path); ``points`` holds decode at
 batch 1 and 64; ``roofline`` the bytes a decode step has to read over its time.
 Weights are random (seeded), data synthetic.
 """
@@ -135,7 +137,8 @@ def main():
     print(f"[bench] model built in {time.perf_counter() - t_build:.1f} s", file=sys.stderr, flush=True)
     P, V = args.n_positions, args.vocab_size
     steps = min(a.steps, P - a.prompt_len - a.warmup)
-    engine = Engine(model, dtype=a.dtype, page_size=16, max_tokens=64 * P, max_requests=64)
+    # (as the serving path makes it, generate.engine_for: steps of a shape that keeps coming back are recorded)
+    engine = Engine(model, dtype=a.dtype, page_size=16, max_tokens=64 * P, max_requests=64, record_prompt_steps=True)
     esize = 2 if a.dtype == "bfloat16" else 4
     kv_bytes_per_token = 2 * args.n_embd * args.n_layer * esize
     w_bytes = weight_bytes(model)
@@ -145,7 +148,7 @@ def main():
     n_seqs, seq_len = 2, 1024
     prompts = torch.randint(0, V, (n_seqs, seq_len), generator=g).tolist()
     pre_ms = []
-    for trial in range(3):
+    for trial in range(5):  # the third records the step, the later ones replay it
         for i in range(n_seqs):
             engine.add_request(("pre", i))
         torch.cuda.synchronize()
@@ -159,7 +162,7 @@ def main():
     flops = prefill_flops(args, n_seqs, seq_len)
     prefill = {"value": round(n_seqs * seq_len / (pre / 1e3), 1), "tokens": n_seqs * seq_len,
                "ms": round(pre, 3), "frac": round(flops / (pre / 1e3) / PEAK_FLOPS[a.dtype], 4)}
-    print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
+    print(f"[bench] prefill {prefill} (trials, ms: {[round(t, 2) for t in pre_ms]})", file=sys.stderr, flush=True)
 
     results = {}
     batches = [a.batch] if a.no_points else sorted({1, a.batch, 64})
