@@ -52,9 +52,16 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(T* __restrict__ out
   const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (r >= n_rows) return;  // whole waves leave; no barrier follows
   const float* xr = x + (size_t)(rows ? rows[r] : r) * width;
-  float4 v[NV];
+  float4 v[NV], g[NV], b[NV];
 #pragma unroll
   for (int i = 0; i < NV; ++i) v[i] = *(const float4*)(xr + min((lane + 64 * i) * 4, width - 4));
+  // scale and shift come in beside the row, not after its statistics
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int k = min((lane + 64 * i) * 4, width - 4);
+    g[i] = gamma ? *(const float4*)(gamma + k) : make_float4(1.f, 1.f, 1.f, 1.f);
+    b[i] = beta ? *(const float4*)(beta + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
@@ -74,16 +81,8 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(T* __restrict__ out
   for (int i = 0; i < NV; ++i) {
     const int k = (lane + 64 * i) * 4;
     if (k >= width) continue;
-    float y[4] = {(v[i].x - mean) * rstd, (v[i].y - mean) * rstd, (v[i].z - mean) * rstd,
-                  (v[i].w - mean) * rstd};
-    if (gamma) {
-      const float4 g = *(const float4*)(gamma + k);
-      y[0] *= g.x, y[1] *= g.y, y[2] *= g.z, y[3] *= g.w;
-    }
-    if (beta) {
-      const float4 b = *(const float4*)(beta + k);
-      y[0] += b.x, y[1] += b.y, y[2] += b.z, y[3] += b.w;
-    }
+    const float y[4] = {(v[i].x - mean) * rstd * g[i].x + b[i].x, (v[i].y - mean) * rstd * g[i].y + b[i].y,
+                        (v[i].z - mean) * rstd * g[i].z + b[i].z, (v[i].w - mean) * rstd * g[i].w + b[i].w};
     if constexpr (sizeof(T) == 4) {
       *(float4*)((float*)o + k) = make_float4(y[0], y[1], y[2], y[3]);
     } else {
