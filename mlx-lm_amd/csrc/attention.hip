@@ -123,6 +123,35 @@ __global__ __launch_bounds__(256) void kv_write_kernel(const T* __restrict__ k_s
   }
 }
 
+// The same, 16 bytes a thread (head_dim a multiple of the vector, rows and pages aligned).
+template <typename T>
+__global__ __launch_bounds__(256) void kv_write_vec_kernel(const T* __restrict__ k_src,
+                                                           const T* __restrict__ v_src, int ld_src,
+                                                           T* __restrict__ k_pages,
+                                                           T* __restrict__ v_pages, size_t page_stride,
+                                                           const int* __restrict__ block_table,
+                                                           int max_blocks,
+                                                           const int* __restrict__ token_req,
+                                                           const int* __restrict__ positions,
+                                                           int n_kv_heads, int head_dim,
+                                                           int page_size) {
+  constexpr int VN = 16 / sizeof(T);
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  const int page = block_table[(size_t)token_req[t] * max_blocks + pos / page_size];
+  const int row = pos % page_size;
+  const int chunks = n_kv_heads * head_dim / VN;
+  for (int c = threadIdx.x; c < chunks; c += blockDim.x) {
+    const int col = c * VN;
+    const int h = col / head_dim, d = col - h * head_dim;
+    const size_t dst = (size_t)page * page_stride + ((size_t)h * page_size + row) * head_dim + d;
+    const uint4 kk = *(const uint4*)(k_src + (size_t)t * ld_src + col);
+    const uint4 vv = *(const uint4*)(v_src + (size_t)t * ld_src + col);
+    *(uint4*)(k_pages + dst) = kk;
+    *(uint4*)(v_pages + dst) = vv;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // attn_tile: grid (n_tiles, n_heads), 256 threads.  Wave w owns queries
 // 4w .. 4w+3 of the tile.  In the score phase a lane is a key, in the
@@ -400,6 +429,22 @@ extern "C" int kv_write(const void* k_src, const void* v_src, int ld_src, void* 
   if (page_stride < (size_t)n_kv_heads * page_size * head_dim)
     FAIL("kv_write: page stride smaller than a page");
   dim3 grid(n_tokens), block(256);
+  const int vn = dtype == DT_F32 ? 4 : 8;
+  const uintptr_t all = (uintptr_t)k_src | (uintptr_t)v_src | (uintptr_t)k_pages | (uintptr_t)v_pages;
+  if (head_dim % vn == 0 && ld_src % vn == 0 && page_stride % vn == 0 && (all & 15) == 0) {
+    if (dtype == DT_F32)
+      hipLaunchKernelGGL(kv_write_vec_kernel<float>, grid, block, 0, stream, (const float*)k_src,
+                         (const float*)v_src, ld_src, (float*)k_pages, (float*)v_pages, page_stride,
+                         block_table, max_blocks, token_req, positions, n_kv_heads, head_dim,
+                         page_size);
+    else
+      hipLaunchKernelGGL(kv_write_vec_kernel<bf16>, grid, block, 0, stream, (const bf16*)k_src,
+                         (const bf16*)v_src, ld_src, (bf16*)k_pages, (bf16*)v_pages, page_stride,
+                         block_table, max_blocks, token_req, positions, n_kv_heads, head_dim,
+                         page_size);
+    CHECK_LAUNCH("kv_write");
+    return 0;
+  }
   if (dtype == DT_F32)
     hipLaunchKernelGGL(kv_write_kernel<float>, grid, block, 0, stream, (const float*)k_src,
                        (const float*)v_src, ld_src, (float*)k_pages, (float*)v_pages, page_stride,

@@ -265,6 +265,27 @@ def test_kv_write_and_attn_tile(dtype, case):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_kv_write_from_rows_that_are_not_aligned(dtype):
+    """Sources that start in the middle of a 16-byte piece take the element-wise kernel: same pages."""
+    k = _k()
+    H, Hkv, hd, ps, ctx, ql, window = ATTN_CASES[0]
+    c = PagedCase(dtype, H, Hkv, hd, ps, ctx, ql, seed=3, window=window)
+    start = c.pool.clone()  # (holds the keys and values of the tokens before)
+    k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
+    want = c.pool.clone()
+    bits = torch.int32 if dtype == torch.float32 else torch.int16  # (free slots hold NaN: compare bits)
+    assert not torch.equal(want.view(bits), start.view(bits))
+    c.pool.copy_(start)
+    width = c.k_new.shape[1]
+    wide = torch.zeros(c.T, 2 * width + 8, dtype=dtype, device=DEV)
+    wide[:, 1 : 1 + width] = c.k_new.to(DEV)
+    wide[:, 1 + width : 1 + 2 * width] = c.v_new.to(DEV)
+    k.kv_write(wide[:, 1 : 1 + width], wide[:, 1 + width : 1 + 2 * width], c.kv, c.block_table_dev, c.token_req,
+               c.positions)
+    assert torch.equal(c.pool.view(bits), want.view(bits))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", ATTN_CASES)
 @pytest.mark.parametrize("n_splits", [1, 3, 8])
 def test_attn_row(dtype, case, n_splits):
