@@ -8,13 +8,16 @@
 //
 // Two kernels:
 //  * gemm_bf16_tile: 128x128x64 block tile, 4 waves in 2x2, each wave a 64x64
-//    tile of four v_mfma_f32_32x32x16_bf16 accumulators; two k-blocks in LDS,
-//    two more in registers; tiles dealt to the dies in super-tiles that share
-//    their operands in a die's L2.  Any M, N; K % 8 == 0.
+//    tile of four v_mfma_f32_32x32x16_bf16 accumulators (or 256x256x64 with 8
+//    waves); two k-blocks in LDS, two more in registers; each die gets a run
+//    of neighbouring tiles that share their operands in its L2; K may be
+//    split over blocks where rows are few.  Any M, N; K % 8 == 0.
 //  * gemm_bf16_skinny: M <= 64 rows (decode).  A block of four waves owns 16
 //    output features and splits K among its waves; W streams from HBM once
 //    as the MFMA A-operand, the activations are the B-operand.
 #include "common.h"
+
+#include <algorithm>
 
 #define FLAG_GELU 1
 #define FLAG_ACCUMULATE 2
@@ -54,24 +57,37 @@ __device__ __forceinline__ void store_out(const GemmArgs& p, int m, int n, float
 
 // ---------------------------------------------------------------------------
 
+// Rows of a tile beyond the matrix read some row inside it (what they give is
+// never stored), and not all the same one: a tile of which only a few rows
+// exist would read that one row from hundreds of lanes at once, as would every
+// block of that row of tiles, and the cache channel that holds it serves them
+// one after another (a step of 2,056 rows took half as long again as one of 2,048).
+__device__ __forceinline__ int row_inside(int r, int n) { return r < n ? r : r % n; }
+
 #define BK 64
 #define LDS_STRIDE (BK + 8)  // 144 bytes a row: 16-byte reads of 16 rows hit distinct banks
 
 // Which tile a block works on.  Blocks go to the eight dies (each with an L2 of
-// its own) in turn, so block b runs on die b % 8.  Tiles are grouped in
-// super-tiles of SUPER_M x SUPER_N that share their rows of A and of W; a die
-// works through whole super-tiles, so what one of its blocks brings into the
-// L2 the others find there.  Returns false for the padding blocks of the grid.
-template <int SUPER_M, int SUPER_N>
+// its own) in turn, so block b runs on die b % 8.  The tiles are put in an
+// order in which neighbours share operands (panels of PANEL rows of tiles; in
+// a panel column after column) and that sequence is cut into eight runs of
+// equal length, one a die.  So every die gets the same number of tiles to
+// within one (dealing whole groups of tiles left a die with 40 tiles and
+// another with 4 at 2,056 rows), and the blocks at work on a die at one time
+// are a few columns of one panel: what one brings into the L2 the others find
+// there.  Returns false for the padding blocks of the grid.
+template <int PANEL>
 __device__ __forceinline__ bool tile_of_block(int tiles_m, int tiles_n, int& tm, int& tn) {
-  const int super_m = (tiles_m + SUPER_M - 1) / SUPER_M, super_n = (tiles_n + SUPER_N - 1) / SUPER_N;
+  const int total = tiles_m * tiles_n, run = (total + 7) / 8;
   const int die = blockIdx.x & 7, local = blockIdx.x >> 3;
-  const int st = (local / (SUPER_M * SUPER_N)) * 8 + die;
-  const int pos = local % (SUPER_M * SUPER_N);
-  if (st >= super_m * super_n) return false;
-  tm = (st % super_m) * SUPER_M + pos % SUPER_M;
-  tn = (st / super_m) * SUPER_N + pos / SUPER_M;
-  return tm < tiles_m && tn < tiles_n;
+  const int idx = die * run + local;
+  if (local >= run || idx >= total) return false;
+  const int panel = min(idx / (PANEL * tiles_n), (tiles_m + PANEL - 1) / PANEL - 1);  // (only the last is short)
+  const int rem = idx - panel * PANEL * tiles_n;
+  const int h = min(PANEL, tiles_m - panel * PANEL);
+  tn = rem / h;
+  tm = panel * PANEL + rem % h;
+  return true;
 }
 
 // The shape of a block: WAVES_M x WAVES_N waves, each with TM x TN MFMA tiles of
@@ -79,17 +95,17 @@ __device__ __forceinline__ bool tile_of_block(int tiles_m, int tiles_n, int& tm,
 // the larger the block's tile, the fewer bytes per product: 128 x 128 (two
 // blocks a CU) where the matrix gives few tiles, 256 x 256 (one block a CU,
 // half the bytes) where it gives enough of them.
-template <int WAVES_M_, int WAVES_N_, int TM_, int TN_, int SUPER_M_, int SUPER_N_, int BLOCKS_PER_CU_>
+template <int WAVES_M_, int WAVES_N_, int TM_, int TN_, int PANEL_, int BLOCKS_PER_CU_>
 struct TileShape {
   static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, TM = TM_, TN = TN_;
-  static constexpr int SUPER_M = SUPER_M_, SUPER_N = SUPER_N_, BLOCKS_PER_CU = BLOCKS_PER_CU_;
+  static constexpr int PANEL = PANEL_, BLOCKS_PER_CU = BLOCKS_PER_CU_;  // PANEL: rows of tiles that share a die's L2
   static constexpr int THREADS = 64 * WAVES_M * WAVES_N;
   static constexpr int BM = WAVES_M * TM * 32, BN = WAVES_N * TN * 32;
   static constexpr int PA = BM * 8 / THREADS, PB = BN * 8 / THREADS;  // 16-byte pieces a thread moves per k-block
   static constexpr int ROW_STEP = THREADS / 8;                          // rows between a thread's pieces
 };
-using Tile128 = TileShape<2, 2, 2, 2, 8, 4, 2>;
-using Tile256 = TileShape<2, 4, 4, 2, 4, 2, 1>;
+using Tile128 = TileShape<2, 2, 2, 2, 8, 2>;
+using Tile256 = TileShape<2, 4, 4, 2, 4, 1>;
 
 // Pipeline: LDS holds two k-blocks; registers hold two more on their way.  In
 // iteration i the loads of k-block i+2 are issued, k-block i is multiplied
@@ -104,7 +120,7 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
   __shared__ __attribute__((aligned(16))) uint16_t Bs[2][BN * LDS_STRIDE];
 
   int tm, tn;
-  if (!tile_of_block<S::SUPER_M, S::SUPER_N>((p.M + BM - 1) / BM, (p.N + BN - 1) / BN, tm, tn)) return;
+  if (!tile_of_block<S::PANEL>((p.M + BM - 1) / BM, (p.N + BN - 1) / BN, tm, tn)) return;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -121,16 +137,16 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   // each thread moves PA 16-byte pieces of A and PB of W per k-block: piece c
-  // is row c / 8, columns (c % 8) * 8 ..; rows beyond the matrix repeat its
-  // last row (their products land in rows or columns that are never stored)
+  // is row c / 8, columns (c % 8) * 8 ..; rows beyond the matrix read rows
+  // inside it (their products land in rows or columns that are never stored)
   // (32-bit element offsets and one LDS offset: registers are scarce here)
   constexpr int ROW_STEP = S::ROW_STEP;
   int a_off[PA], b_off[PB];
   const int lds_off0 = (tid >> 3) * LDS_STRIDE + (tid & 7) * 8;  // piece i lies ROW_STEP rows further down
 #pragma unroll
-  for (int i = 0; i < PA; ++i) a_off[i] = min(m0 + (tid >> 3) + ROW_STEP * i, p.M - 1) * p.lda + (tid & 7) * 8;
+  for (int i = 0; i < PA; ++i) a_off[i] = row_inside(m0 + (tid >> 3) + ROW_STEP * i, p.M) * p.lda + (tid & 7) * 8;
 #pragma unroll
-  for (int i = 0; i < PB; ++i) b_off[i] = min(n0 + (tid >> 3) + ROW_STEP * i, p.N - 1) * p.ldw + (tid & 7) * 8;
+  for (int i = 0; i < PB; ++i) b_off[i] = row_inside(n0 + (tid >> 3) + ROW_STEP * i, p.N) * p.ldw + (tid & 7) * 8;
   const int kc_mine = (tid & 7) * 8;
   // this split's k-blocks (all of them without a split); the offsets start at its first column
   const int kb_lo = SPLIT ? blockIdx.y * p.blocks_per_split : 0;
@@ -396,46 +412,49 @@ static int check_args(const GemmArgs& p) {
 
 template <typename S>
 static void launch_tiles(const GemmArgs& p, hipStream_t stream) {
-  const int super_m = ((p.M + S::BM - 1) / S::BM + S::SUPER_M - 1) / S::SUPER_M;
-  const int super_n = ((p.N + S::BN - 1) / S::BN + S::SUPER_N - 1) / S::SUPER_N;
-  const int per_die = (super_m * super_n + 7) / 8;  // super-tiles a die works through
-  dim3 grid(per_die * 8 * S::SUPER_M * S::SUPER_N, p.n_splits), block(S::THREADS);
+  const long tiles = (long)((p.M + S::BM - 1) / S::BM) * ((p.N + S::BN - 1) / S::BN);
+  dim3 grid((unsigned)((tiles + 7) / 8 * 8), p.n_splits), block(S::THREADS);  // a run of tiles for each die
   if (p.n_splits > 1)
     hipLaunchKernelGGL((gemm_bf16_tile_kernel<S, true>), grid, block, 0, stream, p);
   else
     hipLaunchKernelGGL((gemm_bf16_tile_kernel<S, false>), grid, block, 0, stream, p);
 }
 
-// Microseconds per k-block of the busiest CU, from what was measured at GPT-2 XL
+// How many tiles a die gets (tile_of_block shares them out evenly).
+template <typename S>
+static int busiest_die(int M, int N) {
+  const long tiles = (long)((M + S::BM - 1) / S::BM) * ((N + S::BN - 1) / S::BN);
+  return (int)((tiles + 7) / 8);
+}
+
+// Microseconds per k-block of the busiest die, from what was measured at GPT-2 XL
 // sizes: two 128 x 128 blocks on a CU finish a k-block each in 1.15 us, one
 // alone in 1.3 us (its fetching and its arithmetic take turns; two blocks
-// overlap each other's), a 256 x 256 block (four times the work) in 2.2 us.
+// overlap each other's), a 256 x 256 block (four times the work) in 2.2 us.  A
+// die has 32 CUs.
 static double cost_128(int M, int N) {
-  const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-  const long rest = tiles % 512;
-  // (a last round of few blocks finds the L2s idle: 1.0)
-  return (double)(tiles / 512) * 1.15 + (rest == 0 ? 0.0 : rest <= 128 ? 1.0 : rest <= 256 ? 1.3 : 1.15);
+  const int tiles = busiest_die<Tile128>(M, N);
+  const int rest = tiles % 64;
+  // (a last round of few blocks finds the L2 idle: 1.0)
+  return (double)(tiles / 64) * 1.15 + (rest == 0 ? 0.0 : rest <= 16 ? 1.0 : rest <= 32 ? 1.3 : 1.15);
 }
-static double cost_256(int M, int N) {
-  const long tiles = (long)((M + 255) / 256) * ((N + 255) / 256);
-  return (double)((tiles + 255) / 256) * 2.2;
-}
+static double cost_256(int M, int N) { return (double)((busiest_die<Tile256>(M, N) + 31) / 32) * 2.2; }
 
 // Into how many parts the 128 x 128 kernel should split K (1: no split).  Few rows
 // give few tiles: 65 to 128 rows of GPT-2 XL's projections are 13 to 50 tiles
 // for 256 CUs, and a tile's walk through K takes the same time whether 50 or
-// 500 of them run.  Measured at those sizes (65 to 640 rows): two parts win up
-// to some 160 tiles, four where the output is narrow (N = 1600) up to some 56;
-// beyond, the partial sums ([parts][M][N] floats, written and read once) cost
-// more than the idle CUs.
-// A part keeps at least six k-blocks: a block's prologue and epilogue cost two.
+// 500 of them run.  Measured at those sizes (65 to 640 rows), the best number
+// of parts brings the blocks to some 220, as long as a part keeps three
+// k-blocks or more; from 150 tiles on the partial sums ([parts][M][N] floats,
+// written and read once) cost more than the idle CUs.
 // `force` > 0 asks for that many parts wherever K has them (for tests of small sizes).
 extern "C" int gemm_bf16_splits(int M, int N, int K, int force) {
   if (M <= SK_MAXM) return 1;
   const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
   const int n_blocks = (K + BK - 1) / BK;
-  int want = (tiles <= 56 && N <= 2048) ? 4 : tiles <= 160 ? 2 : 1;
-  if (want > n_blocks / 6) want = n_blocks / 6;
+  int want = (int)((220 + tiles / 2) / tiles);
+  if (want > n_blocks / 3) want = n_blocks / 3;
+  if (want > 16) want = 16;
   if (force > 0) want = force < n_blocks ? force : n_blocks;
   if (want <= 1) return 1;
   const int per = (n_blocks + want - 1) / want;

@@ -35,6 +35,14 @@ struct GemmArgs {
 #define BK 16
 #define LDS_STRIDE (BK + 1)
 
+// Rows of a tile beyond the matrix read a row inside it (their products are
+// never stored): the row one tile back where there is one, so that they do not
+// all read the matrix's last row at once, which one cache channel would have
+// to serve to every block of that row of tiles.
+__device__ __forceinline__ int row_inside(int r, int n, int tile) {
+  return r < n ? r : (r - tile >= 0 && r - tile < n ? r - tile : n - 1);
+}
+
 // WM x WN waves of 64x64 (BIG) or 32x32 (small) wave tiles
 template <int TM, int TN>  // 32x32 MFMA tiles per wave along m and n
 __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs p) {
@@ -68,14 +76,14 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs p) {
     for (int i = 0; i < PA; ++i) {
       const int c = tid + 256 * i;
       const int row = c >> 2, gk = k0 + (c & 3) * 4, gm = m0 + row;
-      const float4 t = *(const float4*)(p.A + (size_t)min(gm, p.M - 1) * p.lda + min(gk, p.K - 4));
+      const float4 t = *(const float4*)(p.A + (size_t)row_inside(gm, p.M, BM_) * p.lda + min(gk, p.K - 4));
       ra[i] = (gm < p.M && gk < p.K) ? t : ZERO4;
     }
 #pragma unroll
     for (int i = 0; i < PB; ++i) {
       const int c = tid + 256 * i;
       const int row = c >> 2, gk = k0 + (c & 3) * 4, gn = n0 + row;
-      const float4 t = *(const float4*)(p.W + (size_t)min(gn, p.N - 1) * p.ldw + min(gk, p.K - 4));
+      const float4 t = *(const float4*)(p.W + (size_t)row_inside(gn, p.N, BN_) * p.ldw + min(gk, p.K - 4));
       rb[i] = (gn < p.N && gk < p.K) ? t : ZERO4;
     }
   };
