@@ -24,6 +24,10 @@ GEMM_ACCUMULATE = 2
 GEMM_OUT_F32 = 4
 GEMM_KV = 8
 
+# Up to this many rows a bfloat16 product goes to the decode kernels (which take up to 64); from
+# 57 on the tile kernel with K split over blocks is faster.
+DECODE_MAX_ROWS = 56
+
 
 # torch's current stream as a raw handle.  torch.cuda.current_stream() builds a Stream object
 # through several Python layers (some 4 us a call, once per launch); the binding below is what
@@ -310,13 +314,13 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
     float32 or both bfloat16; ``bias`` float32.  ``accumulate`` adds into a
     float32 ``out`` (the residual stream); otherwise ``out`` is float32 or the
     operands' dtype.  With ``scatter`` (a ``KVScatter``) the columns from
-    ``scatter.q_width`` on are also written to the key/value pages.  Up to 64
+    ``scatter.q_width`` on are also written to the key/value pages.  Up to 56
     bfloat16 rows go to the decode kernels, which fuse the norm (up to 16
-    rows) and the scatter and, where the output is too narrow to fill the GPU,
-    split K over ``splits`` blocks and add the partial sums in a second
-    kernel; with ``accumulate`` and a ``pending`` that allows it, that second
-    step is left to the next reader of ``out``.  Everything else is composed
-    from the general kernels.
+    rows) and the scatter; more go to the tile kernels.  Where the launch
+    would not fill the GPU, both split K over ``splits`` blocks and add the
+    partial sums in a second kernel; with ``accumulate`` and a ``pending``
+    that allows it, that second step is left to the next reader of ``out``.
+    Everything else is composed from the general kernels.
     """
     lazy = a if isinstance(a, NormedInput) else None
     packed = w if isinstance(w, PackedWeight) else None
@@ -350,7 +354,7 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
     else:
         _need(out.dtype == torch.bfloat16, "linear: out must be float32 or bfloat16")
 
-    if w.dtype == torch.bfloat16 and variant == 0 and 0 < M <= 64:
+    if w.dtype == torch.bfloat16 and variant == 0 and 0 < M <= DECODE_MAX_ROWS:
         lib = build.load("gemm_bf16_decode")
         if M > 16 and lazy:
             a, lazy = lazy.materialize(), None  # only the 16-row kernel norms its rows itself
