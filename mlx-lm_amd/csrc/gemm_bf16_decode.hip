@@ -228,8 +228,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArg
       const bool row_live = r < p.M;
       const float* x = p.X + (size_t)min(r, p.M - 1) * p.ldx;
       float4 v[NV];
+      if (row_live) {  // (uniform over the wave; a wave without a row still shares in scale and shift below)
 #pragma unroll
-      for (int i = 0; i < NV; ++i) v[i] = *(const float4*)(x + min((lane + 64 * i) * 4, p.K - 4));
+        for (int i = 0; i < NV; ++i) v[i] = *(const float4*)(x + min((lane + 64 * i) * 4, p.K - 4));
+      } else {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+      }
       float4 g4, b4;
       const int gk = min(tid * 4, p.K - 4);  // K / 4 <= 512 pieces: one a thread, surplus threads repeat the last
       if (first) {
