@@ -56,15 +56,47 @@ __device__ __forceinline__ bf16 from_f32<bf16>(float v) {
   return r;
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+// Reductions over a wave.  Inside a row of 16 lanes the values move through the
+// data-parallel primitives of the vector unit (swaps within quads, a mirror of
+// 8 lanes, a mirror of 16), which cost an instruction each; a shuffle through
+// __shfl_xor goes through the LDS crossbar and takes some 60 ns, six of them in
+// a row for a sum.  The four rows' results are read as scalars and joined in a
+// fixed order.  Every lane gets the result.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+#define DPP_QUAD_SWAP1 0xB1     // quad_perm [1, 0, 3, 2]
+#define DPP_QUAD_SWAP2 0x4E     // quad_perm [2, 3, 0, 1]
+#define DPP_HALF_MIRROR 0x141   // lane i of each 8 reads lane 7 - i
+#define DPP_ROW_MIRROR 0x140    // lane i of each 16 reads lane 15 - i
+__device__ __forceinline__ float lane_value(float v, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+// sum (max) over each group of 4, 8 or 16 neighbouring lanes, in every lane of the group
+template <int GROUP>
+__device__ __forceinline__ float group_sum(float v) {
+  v += dpp_move<DPP_QUAD_SWAP1>(v);
+  v += dpp_move<DPP_QUAD_SWAP2>(v);
+  if (GROUP >= 8) v += dpp_move<DPP_HALF_MIRROR>(v);
+  if (GROUP >= 16) v += dpp_move<DPP_ROW_MIRROR>(v);
   return v;
 }
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+template <int GROUP>
+__device__ __forceinline__ float group_max(float v) {
+  v = fmaxf(v, dpp_move<DPP_QUAD_SWAP1>(v));
+  v = fmaxf(v, dpp_move<DPP_QUAD_SWAP2>(v));
+  if (GROUP >= 8) v = fmaxf(v, dpp_move<DPP_HALF_MIRROR>(v));
+  if (GROUP >= 16) v = fmaxf(v, dpp_move<DPP_ROW_MIRROR>(v));
   return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+  v = group_sum<16>(v);
+  return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = group_max<16>(v);
+  return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)), fmaxf(lane_value(v, 32), lane_value(v, 48)));
 }
 
 // tanh-GELU: 0.5 x (1 + tanh(u)) with u = sqrt(2/pi) (x + 0.044715 x^3), written
