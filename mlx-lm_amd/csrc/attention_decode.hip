@@ -113,14 +113,12 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
       float d = 0.f;
 #pragma unroll
       for (int i = 0; i < 8; ++i) d += qf[i] * kf[i];
-#pragma unroll
-      for (int x = 1; x < CPK; x <<= 1) d += __shfl_xor(d, x, WAVE);
+      d = group_sum<CPK>(d);  // over the key's lanes
       const int key = kt + j * KPL + kin;
       s[j] = (key >= k_lo && key < k_hi) ? d : -INFINITY;
       tmax = fmaxf(tmax, s[j]);
     }
-#pragma unroll
-    for (int x = CPK; x < 64; x <<= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, x, WAVE));
+    tmax = wave_max(tmax);
     const float m_new = fmaxf(m, tmax);  // finite: every tile holds at least one live key
     const float alpha = __expf(m - m_new);
     l *= alpha;
