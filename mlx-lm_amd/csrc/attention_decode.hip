@@ -137,14 +137,18 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
   }
 
   // join the lane groups: lanes with the same `sub` hold the same columns
+  // (rotations of the row of 16 by 4 and by 8 through DPP moves; rows and halves of the wave
+  // through shuffles)
+  auto over_groups = [](float v) {
+    if (CPK <= 4) v += dpp_move<0x124>(v);  // row_ror:4
+    if (CPK <= 8) v += dpp_move<0x128>(v);  // row_ror:8
+    v += __shfl_xor(v, 16, WAVE);
+    return v + __shfl_xor(v, 32, WAVE);
+  };
+  l = over_groups(l);
 #pragma unroll
-  for (int x = CPK; x < 64; x <<= 1) {
-    l += __shfl_xor(l, x, WAVE);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) o[i] += __shfl_xor(o[i], x, WAVE);
-  }
-#pragma unroll
-  for (int x = 1; x < CPK; x <<= 1) l += __shfl_xor(l, x, WAVE);
+  for (int i = 0; i < 8; ++i) o[i] = over_groups(o[i]);
+  l = group_sum<CPK>(l);
 
   if (lane == 0) Ms[wave] = m, Ls[wave] = l;
   if (lane < CPK) {
