@@ -24,9 +24,10 @@ GEMM_ACCUMULATE = 2
 GEMM_OUT_F32 = 4
 GEMM_KV = 8
 
-# Up to this many rows a bfloat16 product goes to the decode kernels (which take up to 64); from
-# 57 on the tile kernel with K split over blocks is faster.
-DECODE_MAX_ROWS = 56
+# Up to this many rows a bfloat16 product goes to the decode kernels, except that from 57 rows on
+# the tile kernel is faster where it splits K over blocks (few tiles: not the vocabulary's head).
+DECODE_MAX_ROWS = 64
+TILE_SPLIT_MIN_ROWS = 57
 
 
 # torch's current stream as a raw handle.  torch.cuda.current_stream() builds a Stream object
@@ -314,9 +315,10 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
     float32 or both bfloat16; ``bias`` float32.  ``accumulate`` adds into a
     float32 ``out`` (the residual stream); otherwise ``out`` is float32 or the
     operands' dtype.  With ``scatter`` (a ``KVScatter``) the columns from
-    ``scatter.q_width`` on are also written to the key/value pages.  Up to 56
+    ``scatter.q_width`` on are also written to the key/value pages.  Up to 64
     bfloat16 rows go to the decode kernels, which fuse the norm (up to 16
-    rows) and the scatter; more go to the tile kernels.  Where the launch
+    rows) and the scatter; more go to the tile kernels (and 57 to 64 where
+    those split K).  Where the launch
     would not fill the GPU, both split K over ``splits`` blocks and add the
     partial sums in a second kernel; with ``accumulate`` and a ``pending``
     that allows it, that second step is left to the next reader of ``out``.
@@ -354,7 +356,10 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
     else:
         _need(out.dtype == torch.bfloat16, "linear: out must be float32 or bfloat16")
 
-    if w.dtype == torch.bfloat16 and variant == 0 and 0 < M <= DECODE_MAX_ROWS:
+    to_decode = w.dtype == torch.bfloat16 and variant == 0 and 0 < M <= DECODE_MAX_ROWS
+    if to_decode and M >= TILE_SPLIT_MIN_ROWS and splits is None:
+        to_decode = build.load("gemm_bf16").gemm_bf16_splits(_c_int(M), _c_int(N), _c_int(K), _c_int(force_splits)) <= 1
+    if to_decode:
         lib = build.load("gemm_bf16_decode")
         if M > 16 and lazy:
             a, lazy = lazy.materialize(), None  # only the 16-row kernel norms its rows itself
