@@ -108,9 +108,11 @@ using Tile128 = TileShape<2, 2, 2, 2, 8, 2>;
 using Tile256 = TileShape<2, 4, 4, 2, 4, 1>;
 
 // Pipeline: LDS holds two k-blocks; registers hold two more on their way.  In
-// iteration i the loads of k-block i+2 are issued, k-block i is multiplied
-// out of LDS, then k-block i+1 (loaded an iteration ago) goes from registers
-// to the other half of LDS; one barrier an iteration.
+// iteration i the loads of k-block i+2 are issued and k-block i is multiplied
+// out of LDS; between the MFMAs of its four steps k-block i+1 (loaded an
+// iteration ago) goes from registers to the other half of LDS, a quarter at a
+// time (all at the end, the LDS writes of all waves came in one burst with the
+// MFMA units idle: 8 % slower); one barrier an iteration.
 // SPLIT: K is shared out over blockIdx.y and the partial sums go to the workspace (a kernel of
 // its own, so that the unsplit one carries none of it).
 template <typename S, bool SPLIT>
@@ -217,24 +219,42 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
 #pragma unroll
     for (int i = 0; i < PB; ++i) xb[i] = *(const uint4*)(p.W + b_off[i] + k0);
   };
-  auto store_whole = [&](int stage, const uint4 (&xa)[PA], const uint4 (&xb)[PB]) {
+  // multiply out of `stage` and, a quarter with each 16 columns, move the next k-block (in
+  // registers since the iteration before) into the other stage, which nobody reads any more
+  auto multiply_store = [&](int stage, const uint4 (&xa)[PA], const uint4 (&xb)[PB]) {
+    const uint16_t* af = a_frag + stage * (BM * LDS_STRIDE);
+    const uint16_t* bf = b_frag + stage * (BN * LDS_STRIDE);
+    uint16_t* an = As[stage ^ 1] + lds_off0;
+    uint16_t* bn = Bs[stage ^ 1] + lds_off0;
 #pragma unroll
-    for (int i = 0; i < PA; ++i) *(uint4*)(As[stage] + lds_off0 + i * ROW_STEP * LDS_STRIDE) = xa[i];
+    for (int q = 0; q < 4; ++q) {
+      const int ks = q * 16;
+      bf16x8_t a[TM], b[TN];
 #pragma unroll
-    for (int i = 0; i < PB; ++i) *(uint4*)(Bs[stage] + lds_off0 + i * ROW_STEP * LDS_STRIDE) = xb[i];
+      for (int i = 0; i < TM; ++i) a[i] = *(const bf16x8_t*)(af + i * 32 * LDS_STRIDE + ks);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) b[j] = *(const bf16x8_t*)(bf + j * 32 * LDS_STRIDE + ks);
+#pragma unroll
+      for (int i = q * PA / 4; i < (q + 1) * PA / 4; ++i) *(uint4*)(an + i * ROW_STEP * LDS_STRIDE) = xa[i];
+#pragma unroll
+      for (int i = q * PB / 4; i < (q + 1) * PB / 4; ++i) *(uint4*)(bn + i * ROW_STEP * LDS_STRIDE) = xb[i];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
   };
   int kb = 0;
   const int whole_blocks = SPLIT ? min(n_blocks, p.K / BK - kb_lo) : p.K / BK;  // k-blocks that need no masking
   for (; kb + 4 <= whole_blocks; kb += 2) {
     load_whole(ra[0], rb[0], (kb + 2) * BK);
     __builtin_amdgcn_sched_barrier(0);  // the loads go out before the arithmetic, not after it
-    multiply(0);
-    store_whole(1, ra[1], rb[1]);
+    multiply_store(0, ra[1], rb[1]);
     __syncthreads();
     load_whole(ra[1], rb[1], (kb + 3) * BK);
     __builtin_amdgcn_sched_barrier(0);
-    multiply(1);
-    store_whole(0, ra[0], rb[0]);
+    multiply_store(1, ra[0], rb[0]);
     __syncthreads();
   }
   // the last few k-blocks, with every guard
@@ -433,7 +453,7 @@ static int busiest_die(int M, int N) {
 // Microseconds per k-block of the busiest die, from what was measured at GPT-2 XL
 // sizes: two 128 x 128 blocks on a CU finish a k-block each in 1.15 us, one
 // alone in 1.3 us (its fetching and its arithmetic take turns; two blocks
-// overlap each other's), a 256 x 256 block (four times the work) in 2.2 us.  A
+// overlap each other's), a 256 x 256 block (four times the work) in 2.0 us.  A
 // die has 32 CUs.
 static double cost_128(int M, int N) {
   const int tiles = busiest_die<Tile128>(M, N);
@@ -441,7 +461,7 @@ static double cost_128(int M, int N) {
   // (a last round of few blocks finds the L2 idle: 1.0)
   return (double)(tiles / 64) * 1.15 + (rest == 0 ? 0.0 : rest <= 16 ? 1.0 : rest <= 32 ? 1.3 : 1.15);
 }
-static double cost_256(int M, int N) { return (double)((busiest_die<Tile256>(M, N) + 31) / 32) * 2.2; }
+static double cost_256(int M, int N) { return (double)((busiest_die<Tile256>(M, N) + 31) / 32) * 2.0; }
 
 // Into how many parts the 128 x 128 kernel should split K (1: no split).  Few rows
 // give few tiles: 65 to 128 rows of GPT-2 XL's projections are 13 to 50 tiles
