@@ -106,6 +106,7 @@ struct TileShape {
 };
 using Tile128 = TileShape<2, 2, 2, 2, 8, 2>;
 using Tile256 = TileShape<2, 4, 4, 2, 4, 1>;
+using Tile256x192 = TileShape<4, 2, 2, 3, 4, 1>;
 
 // Pipeline: LDS holds two k-blocks; registers hold two more on their way.  In
 // iteration i the loads of k-block i+2 are issued and k-block i is multiplied
@@ -462,6 +463,8 @@ static double cost_128(int M, int N) {
   return (double)(tiles / 64) * 1.15 + (rest == 0 ? 0.0 : rest <= 16 ? 1.0 : rest <= 32 ? 1.3 : 1.15);
 }
 static double cost_256(int M, int N) { return (double)((busiest_die<Tile256>(M, N) + 31) / 32) * 2.0; }
+// (256 x 192: three quarters of the arithmetic, seven eighths of the bytes; its tiles fit N = 4800)
+static double cost_256x192(int M, int N) { return (double)((busiest_die<Tile256x192>(M, N) + 31) / 32) * 1.6; }
 
 // Into how many parts the 128 x 128 kernel should split K (1: no split).  Few rows
 // give few tiles: 65 to 128 rows of GPT-2 XL's projections are 13 to 50 tiles
@@ -484,7 +487,7 @@ extern "C" int gemm_bf16_splits(int M, int N, int K, int force) {
   return (n_blocks + per - 1) / per;  // no empty part
 }
 
-// variant: 0 = choose, 1 = 128 x 128 tiles, 2 = skinny kernel, 3 = 256 x 256 tiles.
+// variant: 0 = choose, 1 = 128 x 128 tiles, 2 = skinny kernel, 3 = 256 x 256 tiles, 4 = 256 x 192 tiles.
 // n_splits > 1 (128 x 128 tiles only): no epilogue, the partial sums go to ws.
 extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* bias, int M, int N,
                          int K, int lda, int ldw, int ldo, int flags, int variant, int n_splits,
@@ -512,8 +515,10 @@ extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* b
   if (variant == 0) {
     if (M < TILE_MIN_ROWS)
       variant = 2;
-    else
-      variant = cost_256(M, N) < cost_128(M, N) ? 3 : 1;
+    else {
+      const double c1 = cost_128(M, N), c3 = cost_256(M, N), c4 = cost_256x192(M, N);
+      variant = c4 < c3 && c4 < c1 ? 4 : c3 < c1 ? 3 : 1;
+    }
   }
   if (variant == 2) {
     if (M > SK_MAXM) FAIL("gemm_bf16: the skinny kernel takes at most %d rows, got %d", SK_MAXM, M);
@@ -527,11 +532,13 @@ extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* b
       hipLaunchKernelGGL(gemm_bf16_skinny_kernel<3>, grid, block, 0, stream, p);
     else
       hipLaunchKernelGGL(gemm_bf16_skinny_kernel<4>, grid, block, 0, stream, p);
-  } else if (variant == 1 || variant == 3) {
+  } else if (variant == 1 || variant == 3 || variant == 4) {
     if (variant == 1)
       launch_tiles<Tile128>(p, stream);
-    else
+    else if (variant == 3)
       launch_tiles<Tile256>(p, stream);
+    else
+      launch_tiles<Tile256x192>(p, stream);
   } else {
     FAIL("gemm_bf16: unknown variant %d", variant);
   }

@@ -111,7 +111,7 @@ def test_gemm_bf16(M, N, K, mode):
     w = _rand((N, K), torch.bfloat16, 11, 0.1)
     bias = _rand((N,), torch.float32, 12)
     ref = plain.linear(a.double().cpu(), w.double().cpu(), bias.double().cpu())
-    variants = (1, 2, 3) if M <= 64 else (1, 3)  # 128 x 128 tiles, skinny, 256 x 256 tiles
+    variants = (1, 2, 3, 4) if M <= 64 else (1, 3, 4)  # 128 x 128 tiles, skinny, 256 x 256 and 256 x 192 tiles
     for variant in variants:
         if mode == "accumulate":
             out = _rand((M, N), torch.float32, 13)
