@@ -4,6 +4,7 @@ from collections import OrderedDict
 from dataclasses import dataclass
 from typing import List, Sequence
 
+import numpy as np
 import torch
 
 from ..cache import CacheManager
@@ -44,6 +45,9 @@ class _HostRing:
             b = torch.empty(max(n_ints, 4096), dtype=torch.int32, pin_memory=True)
             self.bufs[self.i] = b
         return b
+
+    def current(self):
+        return self.bufs[self.i]
 
     def mark(self):
         ev = self.events[self.i] or torch.cuda.Event()
@@ -130,17 +134,20 @@ class Engine:
                 raise ValueError(f"request {e.request_id!r} brings no tokens")
             if e.fed_row >= 0 and n != 1:
                 raise ValueError(f"request {e.request_id!r}: a token fed on the device is one token")
-            for t in e.tokens:
-                if not (0 <= int(t) < V):
-                    raise ValueError(f"token id {t} of request {e.request_id!r} is outside [0, {V})")
+            toks = np.asarray(e.tokens, dtype=np.int64)
+            if toks.ndim != 1 or int(toks.min()) < 0 or int(toks.max()) >= V:
+                bad = [int(t) for t in np.ravel(toks) if not 0 <= int(t) < V][:1]
+                raise ValueError(f"token id {bad[0] if bad else '?'} of request {e.request_id!r} is outside [0, {V})")
             length = self.cache.requests[e.request_id].length
             if length + n > P:
                 raise ValueError(
                     f"request {e.request_id!r} would reach {length + n} tokens, the model "
                     f"has {P} positions"
                 )
-            for w in e.want:
-                if not (0 <= int(w) < n):
+            if len(e.want):
+                want = np.asarray(e.want, dtype=np.int64)
+                if int(want.min()) < 0 or int(want.max()) >= n:
+                    w = next(int(w) for w in want if not 0 <= int(w) < n)
                     raise ValueError(f"wanted place {w} of request {e.request_id!r} is outside its {n} tokens")
 
     def step(self, entries: List[StepEntry], fed=None):
@@ -235,11 +242,11 @@ class Engine:
             ctx.q_starts.append(q_start)
             ctx.q_lens.append(n)
             ctx.context_lens.append(rc.length)
-            token_ids.extend(int(t) for t in e.tokens)
-            fed_index.extend([e.fed_row] if e.fed_row >= 0 else [-1] * n)
-            positions.extend(range(rc.length, rc.length + n))
-            token_req.extend([r] * n)
-            wanted.extend(q_start + int(w) for w in e.want)
+            token_ids.append(np.asarray(e.tokens, dtype=np.int32))
+            fed_index.append(np.full(n, e.fed_row if e.fed_row >= 0 else -1, dtype=np.int32))
+            positions.append(np.arange(rc.length, rc.length + n, dtype=np.int32))
+            token_req.append(np.full(n, r, dtype=np.int32))
+            wanted.append(q_start + np.asarray(e.want, dtype=np.int32))
             slot_ids.append(rc.state_slot)
             ctx.state_slots.append(rc.state_slot)
             for s in range(0, n, TILE_Q):
@@ -274,6 +281,8 @@ class Engine:
             tables.append((width, flat))
 
         # everything in one pinned buffer and one copy; pieces start on 4-int boundaries
+        token_ids, positions, token_req = (np.concatenate(x) for x in (token_ids, positions, token_req))
+        wanted, fed_index = np.concatenate(wanted), np.concatenate(fed_index)
         pieces = [token_ids, positions, token_req, wanted, slot_ids, tiles, rows, all_tiles, big_tiles]
         pieces += [flat for _, flat in tables]
         pieces.append(fed_index)  # (last: the pieces before it keep their numbers)
@@ -281,10 +290,10 @@ class Engine:
         for p in pieces:
             offsets.append(total)
             total += (len(p) + 3) // 4 * 4
-        host = self._ring.get(total)
+        host = self._ring.get(total).numpy()
         for off, p in zip(offsets, pieces):
-            if p:
-                host[off : off + len(p)] = torch.tensor(p, dtype=torch.int32)
+            if len(p):
+                host[off : off + len(p)] = p
         if static is not None:
             if static.dev is None:
                 static.dev = torch.empty(total, dtype=torch.int32, device=self.device)
@@ -295,14 +304,14 @@ class Engine:
             if self._meta_dev is None or self._meta_dev.numel() < total:
                 self._meta_dev = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
             dev = self._meta_dev
-        dev[:total].copy_(host[:total], non_blocking=True)
+        dev[:total].copy_(self._ring.current()[:total], non_blocking=True)
         self._ring.mark()
 
         def piece(i, n):
             return dev[offsets[i] : offsets[i] + n]
 
         ctx.n_tokens, ctx.n_requests, ctx.n_wanted = T, R, len(wanted)
-        ctx.wants_every_row = wanted == list(range(T))
+        ctx.wants_every_row = len(wanted) == T and bool((wanted == np.arange(T, dtype=np.int32)).all())
         ctx.token_ids, ctx.positions, ctx.token_req = piece(0, T), piece(1, T), piece(2, T)
         ctx.wanted_rows, ctx.slot_ids = piece(3, len(wanted)), piece(4, R)
         plan.tiles, plan.rows, plan.all_tiles = piece(5, len(tiles)), piece(6, len(rows)), piece(7, len(all_tiles))
@@ -310,7 +319,7 @@ class Engine:
         ctx.attention_plan = plan
         for gi, (width, flat) in enumerate(tables):
             ctx.block_tables.append(piece(9 + gi, len(flat)).view(R, width))
-        if any(i >= 0 for i in fed_index):
+        if bool((fed_index >= 0).any()):
             from ..ops import kernels
 
             kernels.feed_tokens(ctx.token_ids, self.fed_src, piece(9 + len(tables), T), self.decoder.vocab_size)
