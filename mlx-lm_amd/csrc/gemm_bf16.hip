@@ -107,6 +107,7 @@ struct TileShape {
 using Tile128 = TileShape<2, 2, 2, 2, 8, 2>;
 using Tile256 = TileShape<2, 4, 4, 2, 4, 1>;
 using Tile256x192 = TileShape<4, 2, 2, 3, 4, 1>;
+using Tile64x128 = TileShape<1, 4, 2, 1, 8, 2>;
 
 // Pipeline: LDS holds two k-blocks; registers hold two more on their way.  In
 // iteration i the loads of k-block i+2 are issued and k-block i is multiplied
@@ -343,9 +344,10 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
 
 #define SK_WAVES 4
 #define SK_MAXM 64
-// From this many rows on the tile kernel with K split is faster than the streaming kernels
-// for 17 to 64 rows (measured at GPT-2 XL's four projections: level at 56, 5 % ahead at 64).
-#define TILE_MIN_ROWS 57
+// From this many rows on tiles of 64 x 128 with K split over blocks are faster than the
+// streaming kernels for 17 to 64 rows (measured at GPT-2 XL's four projections: level at 32
+// rows, 9 % ahead at 40, 17 % at 64).
+#define TILE_MIN_ROWS 33
 
 template <int MT>  // number of 16-row groups of activations (1..4)
 __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(GemmArgs p) {
@@ -466,8 +468,8 @@ static double cost_256(int M, int N) { return (double)((busiest_die<Tile256>(M, 
 // (256 x 192: three quarters of the arithmetic, seven eighths of the bytes; its tiles fit N = 4800)
 static double cost_256x192(int M, int N) { return (double)((busiest_die<Tile256x192>(M, N) + 31) / 32) * 1.6; }
 
-// Into how many parts the 128 x 128 kernel should split K (1: no split).  Few rows
-// give few tiles: 65 to 128 rows of GPT-2 XL's projections are 13 to 50 tiles
+// Into how many parts the 128 x 128 kernel (the 64 x 128 one up to 64 rows) should split K
+// (1: no split).  Few rows give few tiles: up to 128 rows of GPT-2 XL's projections are 13 to 50 tiles
 // for 256 CUs, and a tile's walk through K takes the same time whether 50 or
 // 500 of them run.  Measured at those sizes (65 to 640 rows), the best number
 // of parts brings the blocks to some 220, as long as a part keeps three
@@ -476,7 +478,7 @@ static double cost_256x192(int M, int N) { return (double)((busiest_die<Tile256x
 // `force` > 0 asks for that many parts wherever K has them (for tests of small sizes).
 extern "C" int gemm_bf16_splits(int M, int N, int K, int force) {
   if (M < TILE_MIN_ROWS) return 1;
-  const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+  const long tiles = M <= 64 ? (N + 127) / 128 : (long)((M + 127) / 128) * ((N + 127) / 128);
   const int n_blocks = (K + BK - 1) / BK;
   int want = (int)((220 + tiles / 2) / tiles);
   if (want > n_blocks / 3) want = n_blocks / 3;
@@ -487,8 +489,9 @@ extern "C" int gemm_bf16_splits(int M, int N, int K, int force) {
   return (n_blocks + per - 1) / per;  // no empty part
 }
 
-// variant: 0 = choose, 1 = 128 x 128 tiles, 2 = skinny kernel, 3 = 256 x 256 tiles, 4 = 256 x 192 tiles.
-// n_splits > 1 (128 x 128 tiles only): no epilogue, the partial sums go to ws.
+// variant: 0 = choose, 1 = 128 x 128 tiles, 2 = skinny kernel, 3 = 256 x 256 tiles, 4 = 256 x 192
+// tiles, 5 = 64 x 128 tiles.  n_splits > 1 (tiles of 128 x 128 and 64 x 128 only): no epilogue, the
+// partial sums go to ws.
 extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* bias, int M, int N,
                          int K, int lda, int ldw, int ldo, int flags, int variant, int n_splits,
                          float* ws, size_t ws_floats, hipStream_t stream) {
@@ -506,8 +509,8 @@ extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* b
   if (n_splits < 1 || n_splits > n_blocks) FAIL("gemm_bf16: %d splits of K=%d", n_splits, K);
   p.ws = ws, p.n_splits = n_splits, p.blocks_per_split = (n_blocks + n_splits - 1) / n_splits;
   if (n_splits > 1) {
-    if (variant == 0) variant = 1;
-    if (variant != 1) FAIL("gemm_bf16: only the 128 x 128 kernel splits K");
+    if (variant == 0) variant = M <= 64 ? 5 : 1;
+    if (variant != 1 && variant != 5) FAIL("gemm_bf16: only the 128 x 128 and 64 x 128 kernels split K");
     if (p.blocks_per_split * (n_splits - 1) >= n_blocks) FAIL("gemm_bf16: %d splits of K=%d leave one empty", n_splits, K);
     if (!ws || ((uintptr_t)ws & 15) || ws_floats < (size_t)n_splits * M * N)
       FAIL("gemm_bf16: %d splits of %d x %d need an aligned workspace of that many floats", n_splits, M, N);
@@ -515,6 +518,8 @@ extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* b
   if (variant == 0) {
     if (M < TILE_MIN_ROWS)
       variant = 2;
+    else if (M <= 64)
+      variant = 5;
     else {
       const double c1 = cost_128(M, N), c3 = cost_256(M, N), c4 = cost_256x192(M, N);
       variant = c4 < c3 && c4 < c1 ? 4 : c3 < c1 ? 3 : 1;
@@ -532,13 +537,15 @@ extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* b
       hipLaunchKernelGGL(gemm_bf16_skinny_kernel<3>, grid, block, 0, stream, p);
     else
       hipLaunchKernelGGL(gemm_bf16_skinny_kernel<4>, grid, block, 0, stream, p);
-  } else if (variant == 1 || variant == 3 || variant == 4) {
+  } else if (variant == 1 || variant == 3 || variant == 4 || variant == 5) {
     if (variant == 1)
       launch_tiles<Tile128>(p, stream);
     else if (variant == 3)
       launch_tiles<Tile256>(p, stream);
-    else
+    else if (variant == 4)
       launch_tiles<Tile256x192>(p, stream);
+    else
+      launch_tiles<Tile64x128>(p, stream);
   } else {
     FAIL("gemm_bf16: unknown variant %d", variant);
   }

@@ -24,10 +24,10 @@ GEMM_ACCUMULATE = 2
 GEMM_OUT_F32 = 4
 GEMM_KV = 8
 
-# Up to this many rows a bfloat16 product goes to the decode kernels, except that from 57 rows on
+# Up to this many rows a bfloat16 product goes to the decode kernels, except that from 33 rows on
 # the tile kernel is faster where it splits K over blocks (few tiles: not the vocabulary's head).
 DECODE_MAX_ROWS = 64
-TILE_SPLIT_MIN_ROWS = 57
+TILE_SPLIT_MIN_ROWS = 33
 
 
 # torch's current stream as a raw handle.  torch.cuda.current_stream() builds a Stream object
@@ -317,7 +317,7 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
     operands' dtype.  With ``scatter`` (a ``KVScatter``) the columns from
     ``scatter.q_width`` on are also written to the key/value pages.  Up to 64
     bfloat16 rows go to the decode kernels, which fuse the norm (up to 16
-    rows) and the scatter; more go to the tile kernels (and 57 to 64 where
+    rows) and the scatter; more go to the tile kernels (and 33 to 64 where
     those split K).  Where the launch
     would not fill the GPU, both split K over ``splits`` blocks and add the
     partial sums in a second kernel; with ``accumulate`` and a ``pending``
@@ -414,7 +414,7 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
         # and the same second kernels add the parts and run the epilogue.
         lib = build.load("gemm_bf16")
         n_splits, ws = 1, None
-        if variant in (0, 1) and M > 0:
+        if variant in (0, 1, 5) and M > 0:
             n_blocks = (K + 63) // 64
             if splits is None:
                 n_splits = lib.gemm_bf16_splits(_c_int(M), _c_int(N), _c_int(K), _c_int(force_splits))

@@ -111,7 +111,7 @@ def test_gemm_bf16(M, N, K, mode):
     w = _rand((N, K), torch.bfloat16, 11, 0.1)
     bias = _rand((N,), torch.float32, 12)
     ref = plain.linear(a.double().cpu(), w.double().cpu(), bias.double().cpu())
-    variants = (1, 2, 3, 4) if M <= 64 else (1, 3, 4)  # 128 x 128 tiles, skinny, 256 x 256 and 256 x 192 tiles
+    variants = (1, 2, 3, 4, 5) if M <= 64 else (1, 3, 4, 5)  # 128 x 128 tiles, skinny, 256 x 256, 256 x 192, 64 x 128
     for variant in variants:
         if mode == "accumulate":
             out = _rand((M, N), torch.float32, 13)
@@ -707,6 +707,34 @@ def test_gemm_bf16_decode_split_k(M, N, K, mode):
         assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2]), splits
 
 
+@pytest.mark.parametrize("M,N,K", [(33, 257, 1608), (64, 1600, 1600), (50, 96, 128), (40, 333, 200)])
+@pytest.mark.parametrize("mode", ["plain", "accumulate", "gelu"])
+def test_gemm_bf16_small_tiles_split_k(M, N, K, mode):
+    """33 to 64 rows: tiles of 64 x 128 with K split over blocks, summed by the second kernel."""
+    k = _k()
+    a = _rand((M, K), torch.bfloat16, 20)
+    w = _rand((N, K), torch.bfloat16, 21, 0.1)
+    bias = _rand((N,), torch.float32, 22)
+    ref = plain.linear(a.double().cpu(), w.double().cpu(), bias.double().cpu())
+    for splits in (1, 2, 5):
+        if splits > (K + 63) // 64:
+            continue
+        if mode == "accumulate":
+            out = _rand((M, N), torch.float32, 23)
+            k.linear(out, a, w, bias, accumulate=True, variant=5, splits=splits)
+            want, tol = _rand((M, N), torch.float32, 23).double().cpu() + ref, 1e-4 * math.sqrt(K)
+        elif mode == "gelu":
+            out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+            k.linear(out, a, w, bias, gelu=True, variant=5, splits=splits)
+            want = plain.gelu_tanh(ref)
+            tol = 2**-7 * float(want.abs().max()) + 1e-3
+        else:
+            out = torch.empty(M, N, dtype=torch.float32, device=DEV)
+            k.linear(out, a, w, bias, variant=5, splits=splits)
+            want, tol = ref, 1e-4 * math.sqrt(K)
+        assert (out.double().cpu() - want).abs().max().item() < tol, splits
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 64, 256), (8, 1600, 6400), (16, 96, 384), (40, 240, 200), (64, 1600, 1600),
                                    (5, 4100, 512), (100, 1600, 1600), (200, 240, 456)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
@@ -776,7 +804,8 @@ def test_default_splits_fill_the_gpu():
     assert lib.gemm_bf16_decode_splits(8, 64, 64, 0, 2) == 1  # one k-block cannot be split
     assert lib.gemm_bf16_decode_splits(8, 64, 200, 0, 2) == 2
     tiles = k.build.load("gemm_bf16")
-    assert tiles.gemm_bf16_splits(56, 1600, 6400, 0) == 1  # (the decode kernels' rows)
+    assert tiles.gemm_bf16_splits(32, 1600, 6400, 0) == 1  # (the decode kernels' rows)
+    assert tiles.gemm_bf16_splits(64, 50257, 1600, 0) == 1  # (many tiles: the streaming kernel's)
     assert tiles.gemm_bf16_splits(64, 1600, 6400, 0) > 8
     assert tiles.gemm_bf16_splits(72, 1600, 6400, 0) > 8
     assert 3 <= tiles.gemm_bf16_splits(128, 4800, 1600, 0) <= 8
