@@ -807,7 +807,7 @@ def test_default_splits_fill_the_gpu():
     assert tiles.gemm_bf16_splits(32, 1600, 6400, 0) == 1  # (the decode kernels' rows)
     assert tiles.gemm_bf16_splits(64, 50257, 1600, 0) == 1  # (many tiles: the streaming kernel's)
     assert tiles.gemm_bf16_splits(64, 1600, 6400, 0) > 8
-    assert tiles.gemm_bf16_splits(72, 1600, 6400, 0) > 8
+    assert tiles.gemm_bf16_splits(72, 1600, 6400, 0) >= 8
     assert 3 <= tiles.gemm_bf16_splits(128, 4800, 1600, 0) <= 8
     assert tiles.gemm_bf16_splits(512, 4800, 1600, 0) == 1
     assert tiles.gemm_bf16_splits(2048, 4800, 1600, 0) == 1
