@@ -348,6 +348,10 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
 // streaming kernels for 17 to 64 rows (measured at GPT-2 XL's four projections: level at 32
 // rows, 9 % ahead at 40, 17 % at 64).
 #define TILE_MIN_ROWS 33
+// A matrix this many tiles wide (the vocabulary's head) fills the GPU without a split, and tiles
+// of 64 x 128 beat the streaming kernels from 17 rows on (35 us against 39 at 17 rows, 38 against
+// 83 at 64).
+#define WIDE_TILES 160
 
 template <int MT>  // number of 16-row groups of activations (1..4)
 __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(GemmArgs p) {
@@ -481,6 +485,8 @@ static bool small_tiles(int M, int N) { return (long)((M + 127) / 128) * ((N + 1
 // k-blocks or more; from 150 tiles on the partial sums ([parts][M][N] floats,
 // written and read once) cost more than the idle CUs.
 // `force` > 0 asks for that many parts wherever K has them (for tests of small sizes).
+extern "C" int gemm_bf16_wide(int N) { return (N + 127) / 128 >= WIDE_TILES; }
+
 extern "C" int gemm_bf16_splits(int M, int N, int K, int force) {
   if (M < TILE_MIN_ROWS) return 1;
   const long cols = (N + 127) / 128;
@@ -522,9 +528,9 @@ extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* b
       FAIL("gemm_bf16: %d splits of %d x %d need an aligned workspace of that many floats", n_splits, M, N);
   }
   if (variant == 0) {
-    if (M < TILE_MIN_ROWS)
+    if (M < TILE_MIN_ROWS && (N + 127) / 128 < WIDE_TILES)
       variant = 2;
-    else if (small_tiles(M, N))
+    else if (M <= 64 || small_tiles(M, N))
       variant = 5;
     else {
       const double c1 = cost_128(M, N), c3 = cost_256(M, N), c4 = cost_256x192(M, N);

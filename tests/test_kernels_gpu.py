@@ -805,7 +805,8 @@ def test_default_splits_fill_the_gpu():
     assert lib.gemm_bf16_decode_splits(8, 64, 200, 0, 2) == 2
     tiles = k.build.load("gemm_bf16")
     assert tiles.gemm_bf16_splits(32, 1600, 6400, 0) == 1  # (the decode kernels' rows)
-    assert tiles.gemm_bf16_splits(64, 50257, 1600, 0) == 1  # (many tiles: the streaming kernel's)
+    assert tiles.gemm_bf16_splits(64, 50257, 1600, 0) == 1  # (many tiles fill the GPU as they are)
+    assert tiles.gemm_bf16_wide(50257) == 1 and tiles.gemm_bf16_wide(6400) == 0
     assert tiles.gemm_bf16_splits(64, 1600, 6400, 0) > 8
     assert tiles.gemm_bf16_splits(72, 1600, 6400, 0) >= 8
     assert 3 <= tiles.gemm_bf16_splits(128, 4800, 1600, 0) <= 8
