@@ -108,6 +108,7 @@ using Tile128 = TileShape<2, 2, 2, 2, 8, 2>;
 using Tile256 = TileShape<2, 4, 4, 2, 4, 1>;
 using Tile256x192 = TileShape<4, 2, 2, 3, 4, 1>;
 using Tile64x128 = TileShape<1, 4, 2, 1, 8, 2>;
+using Tile32x128 = TileShape<1, 4, 1, 1, 8, 2>;
 
 // Pipeline: LDS holds two k-blocks; registers hold two more on their way.  In
 // iteration i the loads of k-block i+2 are issued and k-block i is multiplied
@@ -344,14 +345,12 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
 
 #define SK_WAVES 4
 #define SK_MAXM 64
-// From this many rows on tiles of 64 x 128 with K split over blocks are faster than the
-// streaming kernels for 17 to 64 rows (measured at GPT-2 XL's four projections: level at 32
-// rows, 9 % ahead at 40, 17 % at 64).
-#define TILE_MIN_ROWS 33
-// A matrix this many tiles wide (the vocabulary's head) fills the GPU without a split, and tiles
-// of 64 x 128 beat the streaming kernels from 17 rows on (35 us against 39 at 17 rows, 38 against
-// 83 at 64).
-#define WIDE_TILES 160
+// From 17 rows on this file's kernels take the product: tiles of 32 x 128 up to 32 rows and of
+// 64 x 128 up to 64 (and beyond where 128 x 128 tiles would be few), with K split over blocks
+// where the tiles alone do not fill the GPU.  (A kernel that streamed the weights once for 17 to
+// 64 rows, 64 features a block, was 3 to 17 % slower than these at GPT-2 XL's projections and
+// twice as slow at the vocabulary's head.)
+#define TILE_MIN_ROWS 17
 
 template <int MT>  // number of 16-row groups of activations (1..4)
 __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(GemmArgs p) {
@@ -477,7 +476,7 @@ static double cost_256x192(int M, int N) { return (double)((busiest_die<Tile256x
 // 10 % ahead up to 384 rows and level at 512; the narrow ones (N = 1600) gain up to 1,024 rows.
 static bool small_tiles(int M, int N) { return (long)((M + 127) / 128) * ((N + 127) / 128) <= 160; }
 
-// Into how many parts the 128 x 128 kernel (or the 64 x 128 one) should split K
+// Into how many parts the kernels with tiles 128 wide should split K
 // (1: no split).  Few rows give few tiles: up to 128 rows of GPT-2 XL's projections are 13 to 50 tiles
 // for 256 CUs, and a tile's walk through K takes the same time whether 50 or
 // 500 of them run.  Measured at those sizes (65 to 640 rows), the best number
@@ -485,12 +484,10 @@ static bool small_tiles(int M, int N) { return (long)((M + 127) / 128) * ((N + 1
 // k-blocks or more; from 150 tiles on the partial sums ([parts][M][N] floats,
 // written and read once) cost more than the idle CUs.
 // `force` > 0 asks for that many parts wherever K has them (for tests of small sizes).
-extern "C" int gemm_bf16_wide(int N) { return (N + 127) / 128 >= WIDE_TILES; }
-
 extern "C" int gemm_bf16_splits(int M, int N, int K, int force) {
   if (M < TILE_MIN_ROWS) return 1;
   const long cols = (N + 127) / 128;
-  const long tiles = small_tiles(M, N) ? (long)((M + 63) / 64) * cols : (long)((M + 127) / 128) * cols;
+  const long tiles = M <= 32 ? cols : small_tiles(M, N) ? (long)((M + 63) / 64) * cols : (long)((M + 127) / 128) * cols;
   const int n_blocks = (K + BK - 1) / BK;
   int want = (int)((220 + tiles / 2) / tiles);
   if (want > n_blocks / 3) want = n_blocks / 3;
@@ -502,8 +499,8 @@ extern "C" int gemm_bf16_splits(int M, int N, int K, int force) {
 }
 
 // variant: 0 = choose, 1 = 128 x 128 tiles, 2 = skinny kernel, 3 = 256 x 256 tiles, 4 = 256 x 192
-// tiles, 5 = 64 x 128 tiles.  n_splits > 1 (tiles of 128 x 128 and 64 x 128 only): no epilogue, the
-// partial sums go to ws.
+// tiles, 5 = 64 x 128 tiles, 6 = 32 x 128 tiles.  n_splits > 1 (variants 1, 5 and 6 only): no
+// epilogue, the partial sums go to ws.
 extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* bias, int M, int N,
                          int K, int lda, int ldw, int ldo, int flags, int variant, int n_splits,
                          float* ws, size_t ws_floats, hipStream_t stream) {
@@ -521,15 +518,17 @@ extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* b
   if (n_splits < 1 || n_splits > n_blocks) FAIL("gemm_bf16: %d splits of K=%d", n_splits, K);
   p.ws = ws, p.n_splits = n_splits, p.blocks_per_split = (n_blocks + n_splits - 1) / n_splits;
   if (n_splits > 1) {
-    if (variant == 0) variant = small_tiles(M, N) ? 5 : 1;
-    if (variant != 1 && variant != 5) FAIL("gemm_bf16: only the 128 x 128 and 64 x 128 kernels split K");
+    if (variant == 0) variant = M <= 32 ? 6 : small_tiles(M, N) ? 5 : 1;
+    if (variant != 1 && variant != 5 && variant != 6) FAIL("gemm_bf16: only the tiles of 128, 64 and 32 rows by 128 split K");
     if (p.blocks_per_split * (n_splits - 1) >= n_blocks) FAIL("gemm_bf16: %d splits of K=%d leave one empty", n_splits, K);
     if (!ws || ((uintptr_t)ws & 15) || ws_floats < (size_t)n_splits * M * N)
       FAIL("gemm_bf16: %d splits of %d x %d need an aligned workspace of that many floats", n_splits, M, N);
   }
   if (variant == 0) {
-    if (M < TILE_MIN_ROWS && (N + 127) / 128 < WIDE_TILES)
+    if (M < TILE_MIN_ROWS)
       variant = 2;
+    else if (M <= 32)
+      variant = 6;
     else if (M <= 64 || small_tiles(M, N))
       variant = 5;
     else {
@@ -549,15 +548,17 @@ extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* b
       hipLaunchKernelGGL(gemm_bf16_skinny_kernel<3>, grid, block, 0, stream, p);
     else
       hipLaunchKernelGGL(gemm_bf16_skinny_kernel<4>, grid, block, 0, stream, p);
-  } else if (variant == 1 || variant == 3 || variant == 4 || variant == 5) {
+  } else if (variant == 1 || variant == 3 || variant == 4 || variant == 5 || variant == 6) {
     if (variant == 1)
       launch_tiles<Tile128>(p, stream);
     else if (variant == 3)
       launch_tiles<Tile256>(p, stream);
     else if (variant == 4)
       launch_tiles<Tile256x192>(p, stream);
-    else
+    else if (variant == 5)
       launch_tiles<Tile64x128>(p, stream);
+    else
+      launch_tiles<Tile32x128>(p, stream);
   } else {
     FAIL("gemm_bf16: unknown variant %d", variant);
   }

@@ -1,4 +1,4 @@
-// Linear layer for decode steps: at most 64 rows of activations against a
+// Linear layer for decode steps: at most 16 rows of activations against a
 // bfloat16 weight matrix that streams from HBM exactly once.
 //   out[m, n] = epilogue( sum_k A[m, k] * W[n, k] + bias[n] )
 // with fusions that save launches and round trips through memory:
@@ -16,7 +16,7 @@
 // of consecutive bytes; packed weights stream about twice as fast, because a
 // row-major tile is sixteen 64-byte pieces per load.
 //
-// Up to 16 rows: a block of eight waves owns 16 output features.  The
+// A block of eight waves owns 16 output features.  The
 // activations (normed or copied) sit in LDS whole as the MFMA B-operand; each
 // wave takes every eighth 64-wide k-block of the 16 weight rows as the
 // A-operand of two v_mfma_f32_16x16x32_bf16 (lane l reads 32 contiguous bytes
@@ -24,10 +24,8 @@
 // of the MFMAs; the eight partial tiles are summed in a fixed order.  Where
 // the matrix has few features and K is not split, a block owns only eight of
 // them (lanes 8..15 of a group repeat the eighth): twice as many blocks.
-//
-// 17 to 64 rows: every block re-reading all activations would cost more than
-// the weights, so a block takes 64 or 128 features (16 a wave) and a slice of
-// K; the slice of the activations passes through LDS once for all its waves.
+// (More than 16 rows are the tile kernels' of gemm_bf16.hip, which leave their
+// partial sums to the second kernels of this file in the same way.)
 //
 // A CU keeps only so many loads in flight, so a launch that does not occupy
 // every CU cannot reach the memory's bandwidth.  Where the feature blocks alone
@@ -141,29 +139,6 @@ __device__ __forceinline__ void finish4(const DecodeGemmArgs& p, int m, int n, f
     } else {
       *(uint2*)((uint16_t*)p.out + idx) = packed;
     }
-  }
-}
-
-// Four outputs of a row from an MFMA tile: to the workspace when K is split, else through the epilogue.
-__device__ __forceinline__ void emit4(const DecodeGemmArgs& p, int split, int m, int n, float4 v) {
-  if (m >= p.M || n >= p.N) return;
-  if (p.n_splits > 1) {
-    float* dst = p.ws + ((size_t)split * p.M + m) * p.N + n;
-    if (p.vec4) {
-      *(float4*)dst = v;
-    } else {
-      dst[0] = v.x;
-      if (n + 1 < p.N) dst[1] = v.y;
-      if (n + 2 < p.N) dst[2] = v.z;
-      if (n + 3 < p.N) dst[3] = v.w;
-    }
-  } else if (p.vec4) {
-    finish4(p, m, n, v);
-  } else {
-    finish(p, m, n, v.x);
-    if (n + 1 < p.N) finish(p, m, n + 1, v.y);
-    if (n + 2 < p.N) finish(p, m, n + 2, v.z);
-    if (n + 3 < p.N) finish(p, m, n + 3, v.w);
   }
 }
 
@@ -357,101 +332,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArg
 }
 
 // ---------------------------------------------------------------------------
-// 17 to 64 rows of activations (MT groups of 16).  Wave w of block (x, y) owns
-// features 16 * (NWV * x + w) .. + 15 and the k-blocks of split y; the rows'
-// columns of that split pass through LDS in stretches of MID_KB k-blocks, read
-// by all waves.  Weights: packed or row-major as above, a stretch at a time in
-// registers.
-#define MID_KB 8
-#define MID_COLS (MID_KB * 64)
-#define MID_STRIDE (MID_COLS + 8)  // LDS row stride: 16-byte reads of 16 rows on distinct banks
-
-template <int MT, int NWV>
-__global__ __launch_bounds__(NWV * 64) void gemm_bf16_mid_kernel(DecodeGemmArgs p) {
-  extern __shared__ __attribute__((aligned(16))) uint16_t As[];  // [MT * 16][MID_STRIDE]
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int koff = (lane >> 4) * 16;
-  const int n_chunks_all = (p.K + 63) / 64;
-  const int c_begin = blockIdx.y * p.chunks_per_split;
-  const int n_chunks = min(n_chunks_all, c_begin + p.chunks_per_split) - c_begin;
-  const int k_end = min(p.K, (c_begin + n_chunks) * 64);
-  const bool packed = p.ldw == 0;
-  // a wave beyond the matrix repeats the last tile; its results are dropped
-  const int tile = min((int)blockIdx.x * NWV + wave, (p.N + 15) / 16 - 1);
-  const int n0 = ((int)blockIdx.x * NWV + wave) * 16;
-  const uint16_t* wrow = p.W + (size_t)min(tile * 16 + (lane & 15), p.N - 1) * p.ldw;
-  const uint16_t* wtile = p.W + (size_t)tile * n_chunks_all * 1024 + lane * 8;
-
-  f32x4_t acc[MT];
-#pragma unroll
-  for (int g = 0; g < MT; ++g) acc[g] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-
-  const uint16_t* arow[MT];
-#pragma unroll
-  for (int g = 0; g < MT; ++g) arow[g] = As + min(g * 16 + (lane & 15), p.M - 1) * MID_STRIDE + koff;
-
-  for (int c0 = 0; c0 < n_chunks; c0 += MID_KB) {  // uniform over the block
-    Frag w[MID_KB][2];
-#pragma unroll
-    for (int u = 0; u < MID_KB; ++u) {
-      const int c = c_begin + min(c0 + u, n_chunks - 1);
-      if (packed) {
-        w[u][0].u = *(const uint4*)(wtile + (size_t)c * 1024);
-        w[u][1].u = *(const uint4*)(wtile + (size_t)c * 1024 + 512);
-      } else {
-        const int k = c * 64 + koff;
-        w[u][0].u = *(const uint4*)(wrow + min(k, p.K - 8));
-        w[u][1].u = *(const uint4*)(wrow + min(k + 8, p.K - 8));
-      }
-    }
-    __syncthreads();  // the stretch before is no longer read
-    const int k0 = (c_begin + c0) * 64;
-    const int width = min(MID_COLS, k_end - k0);  // a multiple of 8
-    const int per_row = width / 8, total = p.M * per_row;
-    for (int i0 = tid; i0 < total; i0 += 4 * NWV * 64) {
-      uint4 t[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int i = min(i0 + j * NWV * 64, total - 1);
-        const int r = i / per_row, k = (i - r * per_row) * 8;
-        t[j] = *(const uint4*)(p.A + (size_t)r * p.lda + k0 + k);
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int i = i0 + j * NWV * 64;
-        const int r = i / per_row, k = (i - r * per_row) * 8;
-        if (i < total) *(uint4*)(As + r * MID_STRIDE + k) = t[j];
-      }
-    }
-    __syncthreads();
-#pragma unroll
-    for (int u = 0; u < MID_KB; ++u) {
-      if (c0 + u < n_chunks) {  // uniform
-        const int kl = u * 64 + koff;  // this lane's columns within the stretch
-#pragma unroll
-        for (int g = 0; g < MT; ++g) {
-          const bool live = g * 16 + (lane & 15) < p.M;
-          Frag a0, a1;
-          // (columns from `width` on are stale LDS: read, then dropped)
-          const uint4 t0 = *(const uint4*)(arow[g] + u * 64);
-          const uint4 t1 = *(const uint4*)(arow[g] + u * 64 + 8);
-          a0.u = (live && kl < width) ? t0 : ZERO4;
-          a1.u = (live && kl + 8 < width) ? t1 : ZERO4;
-          acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][0].v, a0.v, acc[g], 0, 0, 0);
-          acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][1].v, a1.v, acc[g], 0, 0, 0);
-        }
-      }
-    }
-  }
-  // accumulator r of tile g: feature 4 * (lane / 16) + r, row 16 g + lane % 16
-#pragma unroll
-  for (int g = 0; g < MT; ++g)
-    emit4(p, blockIdx.y, g * 16 + (lane & 15), n0 + 4 * (lane >> 4),
-          make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]));
-}
-
-// ---------------------------------------------------------------------------
 // The second step of a split product: out = epilogue(sum over splits, in their order).
 __global__ __launch_bounds__(256) void sum_partials_kernel(DecodeGemmArgs p) {
   const int n4 = (p.N + 3) / 4;
@@ -571,7 +451,6 @@ __global__ __launch_bounds__(256) void sum_partials_norm_kernel(SumNormArgs q) {
 DEFINE_LAST_ERROR(mlxlm_last_error)
 
 #define MAX_LDS_BYTES (120 * 1024)
-#define MID_WAVES 4
 #define FEW_BLOCKS 150  // fewer blocks of 16 features than this leave many CUs idle
 
 // LDS row stride: rows of 16-byte reads from 16 lanes must fall on distinct
@@ -582,8 +461,7 @@ static int chunks_per_split(int K, int n_splits) { return ((K + 63) / 64 + n_spl
 
 // 1 if gemm_bf16_decode takes these sizes (the caller falls back otherwise)
 extern "C" int gemm_bf16_decode_takes(int M, int K, int with_norm, int n_splits) {
-  if (M < 1 || M > 64 || K < 8 || K % 8 != 0 || n_splits < 1 || n_splits > (K + 63) / 64) return 0;
-  if (M > 16) return !with_norm;
+  if (M < 1 || M > 16 || K < 8 || K % 8 != 0 || n_splits < 1 || n_splits > (K + 63) / 64) return 0;
   if (with_norm && (n_splits != 1 || K > LN_MAX_V * 256 || K > NW * U * 64 || K % 4 != 0)) return 0;
   const int range = K < chunks_per_split(K, n_splits) * 64 ? K : chunks_per_split(K, n_splits) * 64;
   return (size_t)M * a_stride_for(range) * 2 <= MAX_LDS_BYTES;
@@ -594,11 +472,11 @@ extern "C" int gemm_bf16_decode_takes(int M, int K, int with_norm, int n_splits)
 // that many wherever a split is possible at all (for tests of small sizes).
 extern "C" int gemm_bf16_decode_splits(int M, int N, int K, int with_norm, int force) {
   const int n_chunks = (K + 63) / 64;
-  if (with_norm || M < 1 || M > 64) return 1;
+  if (with_norm || M < 1 || M > 16) return 1;
   int want;
   if (force > 0) {
     want = force;
-  } else if (M <= 16) {
+  } else {
     const int n_blocks = (N + 15) / 16;
     if (n_blocks >= 200 || M < 4) return 1;  // (one to three rows: the next projection's norm prologue is cheaper than a second kernel)
     // a small matrix streams in less time than the second kernel costs (measured at N = 1600:
@@ -606,11 +484,6 @@ extern "C" int gemm_bf16_decode_splits(int M, int N, int K, int with_norm, int f
     if ((long)N * K < 5000000L) return 1;
     want = (512 + n_blocks - 1) / n_blocks;  // two blocks a CU (measured at N = 1600: K = 6400 is best in 5, K = 1600 in 2 to 6)
     if (want > n_chunks / 4) want = n_chunks / 4;  // at least four k-blocks a split
-  } else {
-    const int n_blocks = (N + 16 * MID_WAVES - 1) / (16 * MID_WAVES);
-    want = (512 + n_blocks - 1) / n_blocks;
-    if (want > n_chunks / 2) want = n_chunks / 2;
-    if (want > 16) want = 16;
   }
   if (want < 1) want = 1;
   if (want > n_chunks) want = n_chunks;
@@ -683,7 +556,7 @@ extern "C" int gemm_bf16_decode(
   p.K = K, p.lda = lda, p.ldx = ldx, p.ldw = ldw;
   // Few features and no split of K: blocks of eight features (half of each MFMA
   // tile is idle, which costs nothing here) put twice as many CUs to work.
-  p.rows = (M <= 16 && n_splits == 1 && (N + 15) / 16 < FEW_BLOCKS) ? 8 : 16;
+  p.rows = (n_splits == 1 && (N + 15) / 16 < FEW_BLOCKS) ? 8 : 16;
   p.n_splits = n_splits, p.chunks_per_split = chunks_per_split(K, n_splits);
   p.ws = ws;
   if (n_splits > 1) {
@@ -693,25 +566,6 @@ extern "C" int gemm_bf16_decode(
            n_splits, M, N);
     if ((p.chunks_per_split * (n_splits - 1)) >= (K + 63) / 64)
       FAIL("gemm_bf16_decode: %d splits of K=%d leave one empty", n_splits, K);
-    p.vec4 = N % 4 == 0;  // of the workspace's rows, here
-  }
-  if (M > 16) {
-    p.a_stride = MID_STRIDE;
-    const int mt = (M + 15) / 16;
-    const size_t lds = (size_t)mt * 16 * MID_STRIDE * 2;
-    void (*mid[3])(DecodeGemmArgs) = {gemm_bf16_mid_kernel<2, MID_WAVES>, gemm_bf16_mid_kernel<3, MID_WAVES>,
-                                      gemm_bf16_mid_kernel<4, MID_WAVES>};
-    static size_t granted_mid[3] = {0, 0, 0};
-    if (lds > 64 * 1024 && granted_mid[mt - 2] < lds) {
-      hipError_t e = hipFuncSetAttribute((const void*)mid[mt - 2], hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)lds);
-      if (e != hipSuccess) FAIL("gemm_bf16_decode: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-      granted_mid[mt - 2] = lds;
-    }
-    const int n_blocks = (N + 16 * MID_WAVES - 1) / (16 * MID_WAVES);
-    hipLaunchKernelGGL(mid[mt - 2], dim3(n_blocks, n_splits), dim3(MID_WAVES * 64), lds, stream, p);
-    CHECK_LAUNCH("gemm_bf16_decode");
-    return 0;
   }
   const int n_blocks = (N + p.rows - 1) / p.rows;
   const int range = K < p.chunks_per_split * 64 ? K : p.chunks_per_split * 64;

@@ -24,11 +24,9 @@ GEMM_ACCUMULATE = 2
 GEMM_OUT_F32 = 4
 GEMM_KV = 8
 
-# Up to 16 rows a bfloat16 product goes to the decode kernels, which fuse the norm; up to 32 rows
-# too, unless the matrix is very wide.  From 33 rows on the tile kernels are faster (the decode
-# kernels take up to 64 rows and are what explicit `splits` of that many rows exercise).
-DECODE_MAX_ROWS = 64
-TILE_SPLIT_MIN_ROWS = 33
+# Up to this many rows a bfloat16 product goes to the decode kernels, which stream the weights
+# once and fuse the norm and the cache scatter; more rows go to the tile kernels.
+DECODE_MAX_ROWS = 16
 
 
 # torch's current stream as a raw handle.  torch.cuda.current_stream() builds a Stream object
@@ -316,9 +314,9 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
     float32 or both bfloat16; ``bias`` float32.  ``accumulate`` adds into a
     float32 ``out`` (the residual stream); otherwise ``out`` is float32 or the
     operands' dtype.  With ``scatter`` (a ``KVScatter``) the columns from
-    ``scatter.q_width`` on are also written to the key/value pages.  Up to 32
-    bfloat16 rows go to the decode kernels, which fuse the norm (up to 16
-    rows) and the scatter; more go to the tile kernels.  Where the launch
+    ``scatter.q_width`` on are also written to the key/value pages.  Up to 16
+    bfloat16 rows go to the decode kernels, which fuse the norm and the
+    scatter; more go to the tile kernels.  Where the launch
     would not fill the GPU, both split K over ``splits`` blocks and add the
     partial sums in a second kernel; with ``accumulate`` and a ``pending``
     that allows it, that second step is left to the next reader of ``out``.
@@ -356,14 +354,8 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
     else:
         _need(out.dtype == torch.bfloat16, "linear: out must be float32 or bfloat16")
 
-    to_decode = w.dtype == torch.bfloat16 and variant == 0 and 0 < M <= DECODE_MAX_ROWS
-    if to_decode and M > 16 and splits is None:
-        # 33 to 64 rows, and from 17 on a matrix as wide as the vocabulary's head: tiles of 64 x 128
-        to_decode = M < TILE_SPLIT_MIN_ROWS and not build.load("gemm_bf16").gemm_bf16_wide(_c_int(N))
-    if to_decode:
+    if w.dtype == torch.bfloat16 and variant == 0 and 0 < M <= DECODE_MAX_ROWS:
         lib = build.load("gemm_bf16_decode")
-        if M > 16 and lazy:
-            a, lazy = lazy.materialize(), None  # only the 16-row kernel norms its rows itself
         with_norm = _c_int(1 if lazy else 0)
         if splits is None:
             n_splits = lib.gemm_bf16_decode_splits(_c_int(M), _c_int(N), _c_int(K), with_norm, _c_int(force_splits))
@@ -415,7 +407,7 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
         # and the same second kernels add the parts and run the epilogue.
         lib = build.load("gemm_bf16")
         n_splits, ws = 1, None
-        if variant in (0, 1, 5) and M > 0:
+        if variant in (0, 1, 5, 6) and M > DECODE_MAX_ROWS:
             n_blocks = (K + 63) // 64
             if splits is None:
                 n_splits = lib.gemm_bf16_splits(_c_int(M), _c_int(N), _c_int(K), _c_int(force_splits))

@@ -111,7 +111,7 @@ def test_gemm_bf16(M, N, K, mode):
     w = _rand((N, K), torch.bfloat16, 11, 0.1)
     bias = _rand((N,), torch.float32, 12)
     ref = plain.linear(a.double().cpu(), w.double().cpu(), bias.double().cpu())
-    variants = (1, 2, 3, 4, 5) if M <= 64 else (1, 3, 4, 5)  # 128 x 128 tiles, skinny, 256 x 256, 256 x 192, 64 x 128
+    variants = (1, 2, 3, 4, 5, 6) if M <= 64 else (1, 3, 4, 5, 6)  # tiles of 128 x 128, skinny, 256 x 256, 256 x 192, 64 x 128, 32 x 128
     for variant in variants:
         if mode == "accumulate":
             out = _rand((M, N), torch.float32, 13)
@@ -641,8 +641,9 @@ def test_gemm_bf16_decode(M, N, K, mode, normed, packed):
                                    (48, 80, 200), (20, 100, 520)])
 @pytest.mark.parametrize("mode", ["plain", "gelu", "accumulate", "f32out"])
 @pytest.mark.parametrize("packed", [False, True])
-def test_gemm_bf16_decode_mid(M, N, K, mode, packed):
-    """17 to 64 rows: a block takes 64 features, the activations pass through LDS in stretches of 512 columns."""
+def test_gemm_bf16_17_to_64_rows(M, N, K, mode, packed):
+    """17 to 64 rows: tiles of 32 x 128 and 64 x 128, K split over blocks where tiles are few (the
+    library's own choice of parts)."""
     k = _k()
     a = _rand((M, K), torch.bfloat16, 10)
     w = _rand((N, K), torch.bfloat16, 11, 0.1)
@@ -675,7 +676,7 @@ def test_gemm_bf16_decode_mid(M, N, K, mode, packed):
                                    (65, 257, 1608), (130, 300, 200), (300, 1600, 1600), (72, 96, 128)])
 @pytest.mark.parametrize("mode", ["plain", "accumulate", "gelu"])
 def test_gemm_bf16_decode_split_k(M, N, K, mode):
-    """K split over blocks (the decode kernels up to 64 rows, the tile kernel beyond): partial sums
+    """K split over blocks (the decode kernels up to 16 rows, the tile kernels beyond): partial sums
     in the workspace, added in the order of the splits by a second kernel, so a number of splits
     gives the same bits run after run."""
     k = _k()
@@ -798,15 +799,16 @@ def test_default_splits_fill_the_gpu():
     assert lib.gemm_bf16_decode_splits(8, 1600, 6400, 0, 0) > 1
     assert lib.gemm_bf16_decode_splits(1, 1600, 6400, 0, 0) == 1  # a row or two: the norm prologue is cheaper
     assert lib.gemm_bf16_decode_splits(8, 1600, 1600, 1, 0) == 1  # the norm prologue needs whole rows
-    assert lib.gemm_bf16_decode_splits(64, 1600, 6400, 0, 0) > 1
-    assert lib.gemm_bf16_decode_splits(64, 50257, 1600, 0, 0) == 1
+    assert lib.gemm_bf16_decode_splits(16, 1600, 6400, 0, 0) > 1
+    assert lib.gemm_bf16_decode_splits(16, 50257, 1600, 0, 0) == 1
+    assert lib.gemm_bf16_decode_splits(17, 1600, 6400, 0, 0) == 1  # (not this library's rows)
     assert lib.gemm_bf16_decode_splits(8, 64, 64, 0, 0) == 1
     assert lib.gemm_bf16_decode_splits(8, 64, 64, 0, 2) == 1  # one k-block cannot be split
     assert lib.gemm_bf16_decode_splits(8, 64, 200, 0, 2) == 2
     tiles = k.build.load("gemm_bf16")
-    assert tiles.gemm_bf16_splits(32, 1600, 6400, 0) == 1  # (the decode kernels' rows)
+    assert tiles.gemm_bf16_splits(16, 1600, 6400, 0) == 1  # (the decode kernels' rows)
+    assert tiles.gemm_bf16_splits(17, 1600, 6400, 0) > 8
     assert tiles.gemm_bf16_splits(64, 50257, 1600, 0) == 1  # (many tiles fill the GPU as they are)
-    assert tiles.gemm_bf16_wide(50257) == 1 and tiles.gemm_bf16_wide(6400) == 0
     assert tiles.gemm_bf16_splits(64, 1600, 6400, 0) > 8
     assert tiles.gemm_bf16_splits(72, 1600, 6400, 0) >= 8
     assert 3 <= tiles.gemm_bf16_splits(128, 4800, 1600, 0) <= 8
