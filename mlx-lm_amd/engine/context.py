@@ -91,8 +91,10 @@ class AttentionPlan:
         without the second kernel that joining splits needs.  Many rows: few
         waves a block, each with several tiles, so that a block's fixed cost
         (its way to the first key, joining its waves) is spread over more keys.
-        Splits only where sixteen waves would still take several tiles each and
-        blocks are few.
+        Splits only where sixteen waves would take three tiles or more each and
+        the splits' blocks still find a compute unit each at once: measured, a
+        split that has to wait for a compute unit costs more than the longer
+        loop that it saves.
         """
         ctx = self.max_row_context if window <= 0 else min(self.max_row_context, window + 63)
         tiles = max(1, (ctx + 63) // 64)
@@ -103,8 +105,8 @@ class AttentionPlan:
             n_waves *= 2
         rounds = (tiles + n_waves - 1) // n_waves
         n_splits = 1
-        if rounds > 1 and blocks < 2 * self.n_compute_units:
-            n_splits = min(rounds, (2 * self.n_compute_units + blocks - 1) // blocks, 64)
+        if rounds >= 3:
+            n_splits = max(1, min(rounds, self.n_compute_units // blocks, 64))
         return n_splits, n_waves
 
 

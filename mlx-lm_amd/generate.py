@@ -554,11 +554,15 @@ def setup_arg_parser():
                         help="The path to the local model directory.")
     parser.add_argument("--extra-eos-token", type=str, default=(), nargs="+",
                         help="Add tokens in the list of eos tokens that stop generation.")
+    parser.add_argument("--system-prompt", default=None,
+                        help="System prompt to be used for the chat template")
     parser.add_argument("--prompt", "-p", default=DEFAULT_PROMPT,
                         help="Message to be processed by the model ('-' reads from stdin)")
     parser.add_argument("--prompt-ids", type=str, default=None,
                         help="The prompt as token ids separated by commas or spaces "
                         "(for model folders without a tokenizer)")
+    parser.add_argument("--prefill-response", default=None,
+                        help="Prefill response to be used for the chat template")
     parser.add_argument("--max-tokens", "-m", type=int, default=DEFAULT_MAX_TOKENS,
                         help="Maximum number of tokens to generate")
     parser.add_argument("--temp", type=float, default=DEFAULT_TEMP, help="Sampling temperature")
@@ -573,7 +577,10 @@ def setup_arg_parser():
                         help="Minimum tokens to keep for min-p sampling.")
     parser.add_argument("--seed", type=int, default=DEFAULT_SEED, help="PRNG seed")
     parser.add_argument("--ignore-chat-template", action="store_true",
-                        help="Use the raw prompt without a chat template (always so here).")
+                        help="Use the raw prompt without the tokenizer's chat template.")
+    parser.add_argument("--chat-template-config", default=None,
+                        help="Additional config for `apply_chat_template`. Should be a dictionary of "
+                        "string keys to values represented as a JSON decodable string.")
     parser.add_argument("--verbose", type=str2bool, default=True,
                         help="Log verbose output when 'True' or 'T' or only print the response "
                         "when 'False' or 'F'")
@@ -582,6 +589,25 @@ def setup_arg_parser():
     parser.add_argument("--prefill-step-size", type=int, default=2048,
                         help="Most prompt tokens read in one step")
     return parser
+
+
+def chat_prompt(tokenizer, prompt, args):
+    """The prompt inside the tokenizer's chat template, as token ids (mlx_lm/generate.py:2115-2152).
+
+    A tokenizer without a template, or ``--ignore-chat-template``, leaves the text as it is.
+    """
+    if args.ignore_chat_template or not getattr(tokenizer, "has_chat_template", False):
+        return prompt
+    template_kwargs = json.loads(args.chat_template_config) if args.chat_template_config else {}
+    messages = []
+    if args.system_prompt is not None:
+        messages.append({"role": "system", "content": args.system_prompt})
+    messages.append({"role": "user", "content": prompt})
+    has_prefill = args.prefill_response is not None
+    if has_prefill:
+        messages.append({"role": "assistant", "content": args.prefill_response})
+    return tokenizer.apply_chat_template(messages, tokenize=True, continue_final_message=has_prefill,
+                                         add_generation_prompt=not has_prefill, **template_kwargs)
 
 
 def main(argv=None):
@@ -601,9 +627,13 @@ def main(argv=None):
     else:
         prompt = args.prompt.replace("\\n", "\n").replace("\\t", "\t")
         prompt = sys.stdin.read() if prompt == "-" else prompt
+        prompt = chat_prompt(tokenizer, prompt, args)
+    special = []
+    if args.xtc_probability > 0:  # tokens that XTC never removes (mlx_lm/generate.py:2168)
+        special = list(tokenizer.encode("\n", add_special_tokens=False)) + sorted(tokenizer.eos_token_ids)
     sampler = make_sampler(args.temp, args.top_p, args.min_p, args.min_tokens_to_keep,
                            top_k=args.top_k, xtc_probability=args.xtc_probability,
-                           xtc_threshold=args.xtc_threshold)
+                           xtc_threshold=args.xtc_threshold, xtc_special_tokens=special)
     response = generate(model, tokenizer, prompt, max_tokens=args.max_tokens, verbose=args.verbose,
                         sampler=sampler, prefill_step_size=args.prefill_step_size)
     if not args.verbose:

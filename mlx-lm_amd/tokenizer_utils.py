@@ -63,11 +63,48 @@ class TokenizerWrapper:
     over a ``tokenizers.Tokenizer`` read from the folder's ``tokenizer.json``.
     """
 
-    def __init__(self, tokenizer, eos_token_ids=None, bos_token=None):
+    def __init__(self, tokenizer, eos_token_ids=None, bos_token=None, eos_token=None, chat_template=None):
         self._tokenizer = tokenizer
         self.eos_token_ids = set(eos_token_ids or [])
         self.bos_token = bos_token
-        self.chat_template = None
+        self.eos_token = eos_token
+        self.chat_template = chat_template
+
+    @property
+    def has_chat_template(self):
+        return self.chat_template is not None
+
+    def apply_chat_template(self, messages, tokenize=True, add_generation_prompt=False,
+                            continue_final_message=False, **template_kwargs):
+        """Render ``messages`` (dicts with ``role`` and ``content``) with the folder's Jinja template.
+
+        The template sees ``messages``, ``bos_token``, ``eos_token``,
+        ``add_generation_prompt`` and whatever else is passed by keyword, as in
+        mlx_lm/tokenizer_utils.py:332-343.  With ``continue_final_message`` the
+        text ends where the last message's content ends, so that the model
+        goes on writing that message.
+        """
+        if self.chat_template is None:
+            raise ValueError("this tokenizer has no chat template")
+        if continue_final_message and add_generation_prompt:
+            raise ValueError("continue_final_message and add_generation_prompt exclude each other")
+        from jinja2.sandbox import ImmutableSandboxedEnvironment
+
+        def raise_exception(message):
+            raise ValueError(message)
+
+        env = ImmutableSandboxedEnvironment(trim_blocks=True, lstrip_blocks=True)
+        env.globals["raise_exception"] = raise_exception
+        text = env.from_string(self.chat_template).render(
+            messages=messages, bos_token=self.bos_token or "", eos_token=self.eos_token or "",
+            add_generation_prompt=add_generation_prompt, **template_kwargs)
+        if continue_final_message:
+            last = str(messages[-1]["content"]).strip()
+            at = text.rfind(last)
+            if at < 0:
+                raise ValueError("the template does not show the last message's content")
+            text = text[: at + len(last)]
+        return self.encode(text, add_special_tokens=False) if tokenize else text
 
     def encode(self, text, add_special_tokens=True):
         return self._tokenizer.encode(text, add_special_tokens=add_special_tokens).ids
@@ -109,7 +146,7 @@ def load_tokenizer(model_path, eos_token_ids=None):
     if isinstance(eos_token_ids, int):
         eos_token_ids = [eos_token_ids]
     eos = set(eos_token_ids or [])
-    bos = None
+    bos = eos_text = template = None
     cfg_path = os.path.join(model_path, "tokenizer_config.json")
     if os.path.exists(cfg_path):
         with open(cfg_path) as fh:
@@ -119,8 +156,14 @@ def load_tokenizer(model_path, eos_token_ids=None):
             return v.get("content") if isinstance(v, dict) else v
 
         bos = as_text(cfg.get("bos_token"))
-        if not eos and cfg.get("eos_token") is not None:
-            tid = tok.token_to_id(as_text(cfg["eos_token"]))
+        eos_text = as_text(cfg.get("eos_token"))
+        template = cfg.get("chat_template")
+        if not eos and eos_text is not None:
+            tid = tok.token_to_id(eos_text)
             if tid is not None:
                 eos.add(tid)
-    return TokenizerWrapper(tok, eos, bos)
+    jinja = os.path.join(model_path, "chat_template.jinja")
+    if os.path.exists(jinja):
+        with open(jinja) as fh:
+            template = fh.read()
+    return TokenizerWrapper(tok, eos, bos, eos_text, template if isinstance(template, str) else None)

@@ -16,7 +16,11 @@ TINY_B = dict(model_type="gpt2", n_layer=3, n_embd=96, n_head=3, n_inner=384, vo
 TINY_C = dict(model_type="gpt2", n_layer=2, n_embd=240, n_head=5, n_inner=200, vocab_size=333,
               n_positions=448, layer_norm_epsilon=3e-4, activation_function="gelu_pytorch_tanh")
 
-TINY = {"A": (TINY_A, 0, "a"), "B": (TINY_B, 1, "b"), "C": (TINY_C, 5, "b")}
+# Small layers and thousands of positions: a decoded row's keys are split over blocks.
+TINY_LONG = dict(model_type="gpt2", n_layer=2, n_embd=64, n_head=2, n_inner=96, vocab_size=300,
+                 n_positions=3400, layer_norm_epsilon=1e-5, activation_function="gelu_new")
+
+TINY = {"A": (TINY_A, 0, "a"), "B": (TINY_B, 1, "b"), "C": (TINY_C, 5, "b"), "LONG": (TINY_LONG, 9, "a")}
 
 
 def sharpen(tensors, config, score_std):

@@ -118,6 +118,39 @@ def test_first_tokens_and_long_decode(folders, dtype):
         eng.step([StepEntry("full", [1], [0])])
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("use_graphs", [False, True])
+def test_thousands_of_keys_split_over_blocks(tmp_path, monkeypatch, dtype, use_graphs):
+    """A prompt of 3,300 tokens in two portions, then 40 decoded tokens whose keys several blocks share."""
+    from mlx_lm_amd.engine import Engine, StepEntry
+    from mlx_lm_amd.ops import kernels
+    from mlx_lm_amd.utils import load_model
+
+    config, weights = helpers.make_folder(str(tmp_path), "LONG", 8.0)
+    n, n_prompt = 3340, 3300
+    tokens = helpers.random_tokens(n, config["vocab_size"], seed=31)
+    want = _plain_logits(weights, config, tokens, dtype)
+    seen = []
+    for name in ("attn_decode", "attn_row"):
+        inner = getattr(kernels, name)
+
+        def counted(*a, _inner=inner, **kw):
+            seen.append(a[11] if len(a) > 11 else kw.get("n_splits", 1))
+            return _inner(*a, **kw)
+
+        monkeypatch.setattr(kernels, name, counted)
+    model, _ = load_model(str(tmp_path), dtype=dtype)
+    eng = Engine(model, dtype=dtype, page_size=16, n_pages=(n + 63) // 64 * 4, max_requests=2, use_graphs=use_graphs)
+    eng.add_request("r")
+    first = eng.step([StepEntry("r", tokens[:2000], [1999])])
+    _close(first, want[1999:2000], dtype, "the first portion's last row")
+    rows = [eng.step([StepEntry("r", tokens[2000:n_prompt], [n_prompt - 2001])]).clone()]
+    for i in range(n_prompt, n):
+        rows.append(eng.step([StepEntry("r", tokens[i : i + 1], [0])]).clone())
+    assert seen and max(seen) > 1, "no step split a row's keys"
+    _close(torch.cat(rows), want[n_prompt - 1 :], dtype, "decoded after 3,300 tokens")
+
+
 def _mixed_trace(config, seed, lengths, n_live=4):
     """Steps that mix portions of some requests with decoded tokens of others.
 
