@@ -153,8 +153,8 @@ def main():
             engine.add_request(("pre", i))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        out = engine.step([StepEntry(("pre", i), prompts[i], [seq_len - 1]) for i in range(n_seqs)])
-        out.sum().item()
+        engine.step([StepEntry(("pre", i), prompts[i], [seq_len - 1]) for i in range(n_seqs)])
+        torch.cuda.synchronize()
         pre_ms.append((time.perf_counter() - t0) * 1e3)
         for i in range(n_seqs):
             engine.end_request(("pre", i))

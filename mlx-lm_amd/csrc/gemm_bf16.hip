@@ -18,6 +18,7 @@
 #include "common.h"
 
 #include <algorithm>
+#include <type_traits>
 
 #define FLAG_GELU 1
 #define FLAG_ACCUMULATE 2
@@ -121,8 +122,10 @@ using Tile32x128 = TileShape<1, 4, 1, 1, 8, 2>;
 template <typename S, bool SPLIT>
 __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_kernel(GemmArgs p) {
   constexpr int BM = S::BM, BN = S::BN, TM = S::TM, TN = S::TN, PA = S::PA, PB = S::PB;
-  __shared__ __attribute__((aligned(16))) uint16_t As[2][BM * LDS_STRIDE];
-  __shared__ __attribute__((aligned(16))) uint16_t Bs[2][BN * LDS_STRIDE];
+  // (one buffer: the epilogue uses it again for the output tiles)
+  __shared__ __attribute__((aligned(16))) uint16_t smem[2 * (BM + BN) * LDS_STRIDE];
+  uint16_t* const As[2] = {smem, smem + BM * LDS_STRIDE};
+  uint16_t* const Bs[2] = {smem + 2 * BM * LDS_STRIDE, smem + (2 * BM + BN) * LDS_STRIDE};
 
   int tm, tn;
   if (!tile_of_block<S::PANEL>((p.M + BM - 1) / BM, (p.N + BN - 1) / BN, tm, tn)) return;
@@ -194,6 +197,14 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
   const uint16_t* a_frag = As[0] + (wm * TM * 32 + frag_row) * LDS_STRIDE + frag_k;
   const uint16_t* b_frag = Bs[0] + (wn * TN * 32 + frag_row) * LDS_STRIDE + frag_k;
 
+  // Without a split the tiles are accumulated transposed (the weights' rows as the MFMA's rows):
+  // a lane then holds four neighbouring columns of one output row, which the epilogue wants.
+  auto mfma_tile = [](const bf16x8_t& a, const bf16x8_t& b, const f32x16_t& c) __attribute__((always_inline)) {
+    if constexpr (SPLIT)
+      return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    else
+      return __builtin_amdgcn_mfma_f32_32x32x16_bf16(b, a, c, 0, 0, 0);
+  };
   auto multiply = [&](int stage) {
     const uint16_t* af = a_frag + stage * (BM * LDS_STRIDE);
     const uint16_t* bf = b_frag + stage * (BN * LDS_STRIDE);
@@ -208,7 +219,7 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = mfma_tile(a[i], b[j], acc[i][j]);
     }
   };
 
@@ -245,7 +256,7 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = mfma_tile(a[i], b[j], acc[i][j]);
     }
   };
   int kb = 0;
@@ -292,49 +303,125 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
     return;
   }
 
-  // Epilogue.  Accumulator r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4,
-  // column lane%32, so a store covers 32 neighbouring columns of two rows.
-  // (With the operands swapped a lane would hold four neighbouring columns and
-  // store them as one piece, but every lane in another row: measured slower.)
-  // What is read (bias, the residual stream to add to) is read for a whole
-  // 32x32 tile before anything is stored: a load that comes after a store to
-  // memory it might alias waits for it, sixteen times over.
+  // Epilogue.  Accumulator r of a transposed 32x32 tile: output row lane % 32, column
+  // 8*(r/4) + 4*(lane/32) + r%4.  Stored like that, every lane of a store would be in
+  // another row (and with the tiles not transposed, a store would be 64 bytes of 2-byte
+  // pieces): the epilogue took 13 to 24 us of a product's 43 to 62 at 2,048 rows.  So each
+  // wave passes its tile through LDS, 32 rows at a time, and takes it out again with eight
+  // neighbouring columns a lane: stores of 16 or 32 bytes a lane that cover whole rows of
+  // the wave's tile.  The region of a wave is its own; a wave's LDS accesses keep their order.
+  constexpr int NW = S::THREADS / 64;
+  constexpr int WCOLS = TN * 32;   // columns of a wave's tile
+  constexpr int EST = WCOLS + 4;   // floats a row in LDS: sixteen-byte pieces of neighbouring rows on other banks
+  static_assert(NW * 32 * EST * 4 <= (int)sizeof(smem), "the waves' output tiles fit the k-blocks' LDS");
+  __syncthreads();  // nobody reads a k-block any more
+  float* const tile = (float*)smem + wave * 32 * EST;
+  // (read and written through two names: an element is read and then written by the same lane,
+  // and no load has to wait for stores to other elements)
+  const float* __restrict__ res = (const float*)p.out;
+  float* __restrict__ out_f = (float*)p.out;
+  uint16_t* __restrict__ out_h = (uint16_t*)p.out;
+  const bool f32_out = p.flags & (FLAG_ACCUMULATE | FLAG_OUT_F32);
+  // CPL columns a lane on the way out, 16 bytes of the output: eight bfloat16 or four floats, so
+  // that a store covers whole 128-byte lines of a few rows
+  auto emit = [&](auto cpl) __attribute__((always_inline)) {
+    constexpr int CPL = decltype(cpl)::value;
+    constexpr int LPR = WCOLS / CPL;  // lanes a row
+    constexpr int RPP = 64 / LPR;     // rows a pass
+    constexpr int PASSES = (32 + RPP - 1) / RPP;
+    constexpr int GROUP = PASSES < 32 / CPL ? PASSES : 32 / CPL;  // passes whose values are in registers at a time
+    const int erow = lane / LPR, ecol = (lane % LPR) * CPL;
+    const bool elane = erow < RPP;
+    const int n = n0 + wn * WCOLS + ecol;  // this lane's columns, in every row it takes out
+    float bias[CPL];
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int n = n0 + wn * TN * 32 + j * 32 + (lane & 31);
-    const int nc = min(n, p.N - 1);
-    const float bias = p.bias ? p.bias[nc] : 0.f;
+    for (int c = 0; c < CPL; ++c) bias[c] = p.bias ? p.bias[min(n + c, p.N - 1)] : 0.f;
+    // whole pieces of 16 bytes: the row stride and the base keep them aligned, and all the columns exist
+    const bool vec = n + CPL <= p.N && p.ldo % CPL == 0 && ((uintptr_t)p.out & 15) == 0;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-      const int mb = m0 + wm * TM * 32 + i * 32 + 4 * (lane >> 5);
-      float v[16];
-      if (p.flags & FLAG_ACCUMULATE) {
-        const float* o = (const float*)p.out;
+      const int mt = m0 + wm * TM * 32 + i * 32;  // first row of this 32-row tile
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();  // every lane has read the tile before
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          v[r] = o[(size_t)min(mb + 8 * (r >> 2) + (r & 3), p.M - 1) * p.ldo + nc];
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) v[r] += acc[i][j][r] + bias;
-      } else {
+        for (int g = 0; g < 4; ++g)
+          *(float4*)(tile + (lane & 31) * EST + j * 32 + 8 * g + 4 * (lane >> 5)) =
+              make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          v[r] = acc[i][j][r] + bias;
-          if (p.flags & FLAG_GELU) v[r] = gelu_tanh_fast(v[r]);
+      for (int s0 = 0; s0 < PASSES; s0 += GROUP) {
+        // what is added to goes out first, all of the group's at once (left to itself the
+        // compiler puts each load next to its use: one trip after another)
+        float o[GROUP][CPL];
+        if (p.flags & FLAG_ACCUMULATE) {
+#pragma unroll
+          for (int s = 0; s < GROUP; ++s) {
+            const float* orow = res + (size_t)min(mt + (s0 + s) * RPP + erow, p.M - 1) * p.ldo;
+            if (vec) {
+              const float4 t = *(const float4*)(orow + n);  // (CPL is 4 with 32-bit outputs)
+              o[s][0] = t.x, o[s][1] = t.y, o[s][2] = t.z, o[s][3] = t.w;
+            } else {
+#pragma unroll
+              for (int c = 0; c < CPL; ++c) o[s][c] = orow[min(n + c, p.N - 1)];
+            }
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        float v[GROUP][CPL];
+#pragma unroll
+        for (int s = 0; s < GROUP; ++s) {
+          const int row = min((s0 + s) * RPP + erow, 31);
+#pragma unroll
+          for (int c = 0; c < CPL; c += 4) {
+            const float4 t = *(const float4*)(tile + row * EST + ecol + c);
+            v[s][c] = t.x + bias[c], v[s][c + 1] = t.y + bias[c + 1], v[s][c + 2] = t.z + bias[c + 2], v[s][c + 3] = t.w + bias[c + 3];
+          }
+        }
+        if (p.flags & FLAG_ACCUMULATE) {
+#pragma unroll
+          for (int s = 0; s < GROUP; ++s)
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) v[s][c] += o[s][c];
+        } else if (p.flags & FLAG_GELU) {
+#pragma unroll
+          for (int s = 0; s < GROUP; ++s)
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) v[s][c] = gelu_tanh_fast(v[s][c]);
+        }
+#pragma unroll
+        for (int s = 0; s < GROUP; ++s) {
+          const int row = (s0 + s) * RPP + erow, m = mt + row;
+          if (!elane || row >= 32 || m >= p.M || n >= p.N) continue;
+          const size_t at = (size_t)m * p.ldo + n;
+          if (vec) {
+            if constexpr (CPL == 4)
+              *(float4*)(out_f + at) = make_float4(v[s][0], v[s][1], v[s][2], v[s][3]);
+            else
+              *(uint4*)(out_h + at) = make_uint4(pack_bf16x2(v[s][0], v[s][1]), pack_bf16x2(v[s][2], v[s][3]),
+                                                 pack_bf16x2(v[s][4], v[s][5]), pack_bf16x2(v[s][6], v[s][7]));
+          } else {
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) {
+              if (n + c >= p.N) break;
+              if constexpr (CPL == 4)
+                out_f[at + c] = v[s][c];
+              else
+                out_h[at + c] = f32_to_bf16_bits(v[s][c]);
+            }
+          }
         }
       }
-      if (n >= p.N) continue;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = mb + 8 * (r >> 2) + (r & 3);
-        if (m >= p.M) continue;
-        const size_t idx = (size_t)m * p.ldo + n;
-        if (p.flags & (FLAG_ACCUMULATE | FLAG_OUT_F32))
-          ((float*)p.out)[idx] = v[r];
-        else
-          ((uint16_t*)p.out)[idx] = f32_to_bf16_bits(v[r]);
-      }
     }
-  }
+  };
+  if (f32_out)
+    emit(std::integral_constant<int, 4>{});
+  else
+    emit(std::integral_constant<int, 8>{});
 }
 
 // ---------------------------------------------------------------------------
