@@ -53,11 +53,9 @@ class ModelArgs(BaseModelArgs):
                 raise ValueError(f"{key} must be a positive integer, got {getattr(self, key)!r}")
         if self.n_embd % self.n_head:
             raise ValueError("n_embd must be divisible by n_head")  # mlx_lm/models/gpt2.py:33
-        if self.num_key_value_heads != self.n_head:
-            raise ValueError(
-                "GPT-2's fused c_attn holds as many key heads as query heads; "
-                f"num_key_value_heads={self.num_key_value_heads} with n_head={self.n_head} is not that"
-            )
+        # num_key_value_heads is read and not used, as in the reference: keys and values are
+        # reshaped with n_head (mlx_lm/models/gpt2.py:57-58), and the fused c_attn of
+        # [3 n_embd, n_embd] leaves no room for fewer key heads.
         if not self.tie_word_embeddings:
             raise ValueError("an untied output head is not implemented for gpt2")
         if not self.scale_attn_weights or self.scale_attn_by_inverse_layer_idx:
@@ -106,7 +104,7 @@ class Model:
                         {
                             "width": D,
                             "n_heads": args.n_head,
-                            "n_kv_heads": args.num_key_value_heads,
+                            "n_kv_heads": args.n_head,  # mlx_lm/models/gpt2.py:57-58
                             "head_dim": args.head_dim,
                             "scale": args.head_dim**-0.5,  # mlx_lm/models/gpt2.py:39
                             "bias": True,

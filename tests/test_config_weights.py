@@ -27,7 +27,6 @@ def test_from_dict_keeps_known_keys_and_fills_defaults():
 
 @pytest.mark.parametrize("change,match", [
     (dict(n_head=5), "divisible"),
-    (dict(num_key_value_heads=1), "key heads"),
     (dict(activation_function="relu"), "not implemented"),
     (dict(tie_word_embeddings=False), "untied"),
     (dict(scale_attn_by_inverse_layer_idx=True), "scale_attn"),
@@ -38,6 +37,14 @@ def test_what_the_engine_cannot_run_is_refused(change, match):
     cfg = dict(helpers.TINY_A, **change)
     with pytest.raises(ValueError, match=match):
         Model(ModelArgs.from_dict(cfg))
+
+
+def test_num_key_value_heads_is_read_and_not_used():
+    # mlx_lm/models/gpt2.py:24-26,57-58: the key is kept, keys and values are shaped with n_head
+    args = ModelArgs.from_dict(dict(helpers.TINY_A, num_key_value_heads=1))
+    assert args.num_key_value_heads == 1
+    mixer = Model.plan(args).layers[0].mixer
+    assert mixer.params["n_kv_heads"] == mixer.params["n_heads"] == args.n_head
 
 
 def test_missing_required_key_is_an_error():
