@@ -1,5 +1,7 @@
 """Feed-forward parts."""
 
+import torch
+
 from ..ops import kernels
 from .base import FeedForward, TensorSpec, register_feed_forward
 
@@ -22,9 +24,14 @@ class GeluMLP(FeedForward):
             raise ValueError(
                 f"activation '{activation}' is not implemented (only the tanh GELU: {_TANH_GELU})"
             )
-        if width % 8 or inner % 8:
-            raise ValueError(f"feed-forward sizes must be multiples of 8, got {width} and {inner}")
+        if width % 8:
+            raise ValueError(f"the feed-forward's width must be a multiple of 8, got {width}")
+        if inner <= 0:
+            raise ValueError(f"the feed-forward's inner size must be positive, got {inner}")
         self.width, self.inner = width, inner
+        # The products want a multiple of 8 along K.  Inner features beyond ``inner`` get zero
+        # weights and a zero bias: gelu(0) = 0 meets zero columns, so the sum is unchanged.
+        self.inner_padded = (inner + 7) // 8 * 8
         self.fc_w = self.fc_b = self.proj_w = self.proj_b = None
 
     def tensors(self):
@@ -40,10 +47,15 @@ class GeluMLP(FeedForward):
         n = self._name
         self.fc_w, self.fc_b = tensors[n("c_fc.weight")], tensors[n("c_fc.bias")]
         self.proj_w, self.proj_b = tensors[n("c_proj.weight")], tensors[n("c_proj.bias")]
+        pad = self.inner_padded - self.inner
+        if pad:
+            self.fc_w = torch.cat([self.fc_w, self.fc_w.new_zeros(pad, self.width)]).contiguous()
+            self.fc_b = torch.cat([self.fc_b, self.fc_b.new_zeros(pad)]).contiguous()
+            self.proj_w = torch.cat([self.proj_w, self.proj_w.new_zeros(self.width, pad)], dim=1).contiguous()
         self.fc_w, self.proj_w = kernels.for_decode(self.fc_w), kernels.for_decode(self.proj_w)
 
     def forward(self, ctx, x, residual):
-        act = ctx.scratch((x.shape[0], self.inner), ctx.dtype)
+        act = ctx.scratch((x.shape[0], self.inner_padded), ctx.dtype)
         kernels.linear(act, x, self.fc_w, self.fc_b, gelu=True)
         kernels.linear(residual, act, self.proj_w, self.proj_b, accumulate=True, pending=ctx.pending)
 

@@ -20,7 +20,7 @@ def _draw(seed):
     H, hd = rng.choice([1, 2, 3, 5, 8]), rng.choice([16, 32, 48, 64, 80, 128])
     P = rng.choice([64, 130, 256, 400])
     config = dict(model_type="gpt2", n_layer=rng.randint(1, 3), n_embd=H * hd, n_head=H,
-                  n_inner=8 * rng.randint(2, 70), vocab_size=rng.randint(40, 2500), n_positions=P,
+                  n_inner=rng.randint(16, 560), vocab_size=rng.randint(40, 2500), n_positions=P,
                   layer_norm_epsilon=rng.choice([1e-5, 1e-6, 1e-3]), activation_function="gelu_new")
     page_size = rng.choice([16, 32, 64])
     lengths = [min(P, rng.randint(2, P)) for _ in range(rng.randint(2, 5))]
@@ -28,7 +28,7 @@ def _draw(seed):
 
 
 # (seeds chosen to cover widths below a k-block of the tile kernels: n_embd 16, 32, 48)
-@pytest.mark.parametrize("seed", [2, 6, 15, 18, 23, 101, 103, 110])
+@pytest.mark.parametrize("seed", [2, 42, 15, 57, 7, 9, 10, 16, 101, 103])
 def test_random_configuration(tmp_path, seed):
     from safetensors.torch import load_file, save_file
 
