@@ -42,9 +42,13 @@ from typing import Any, Callable, List, Optional, Sequence
 from .step import StepEntry
 
 
-@dataclass
+@dataclass(eq=False)
 class Request:
-    """One generation request and its progress."""
+    """One generation request and its progress.
+
+    Two requests are the same only if they are the same object: looking one up
+    in the scheduler's lists compares identities, not prompts.
+    """
 
     request_id: Any
     prompt: List[int]
@@ -62,6 +66,7 @@ class Request:
     order: int = 0
     # row of the sampling call in flight that holds this request's newest token (not yet in ``generated``)
     inflight_row: Optional[int] = None
+    live: bool = False  # the scheduler holds it (waiting or running)
 
     @property
     def tokens(self):
@@ -161,6 +166,7 @@ class Scheduler:
             raise ValueError(f"request id {request.request_id!r} is in use")
         request.order = self._order
         self._order += 1
+        request.live = True
         self.waiting.append(request)
         return request
 
@@ -169,6 +175,7 @@ class Scheduler:
         for r in list(self.waiting):
             if r.request_id == request_id:
                 self.waiting.remove(r)
+                r.live = False
                 return r
         for r in self.running:
             if r.request_id == request_id:
@@ -181,6 +188,7 @@ class Scheduler:
         return bool(self.waiting or self.running or self._inflight is not None)
 
     def _drop(self, r):
+        r.live = False
         if r in self.running:
             self.running.remove(r)
         elif r in self.waiting:  # pre-empted, and finished by the token that was in flight
@@ -198,6 +206,7 @@ class Scheduler:
         r.num_computed = 0
         r.preemptions += 1
         self.stats.preemptions += 1
+        r.live = True
         self.waiting.appendleft(r)
 
     # -- decisions ---------------------------------------------------------------
@@ -333,7 +342,7 @@ class Scheduler:
         outputs = []
         for r, (token, logprob, logprobs) in zip(job.requests, results):
             r.inflight_row = None
-            if r.finish_reason is not None or not (r in self.running or r in self.waiting):
+            if r.finish_reason is not None or not r.live:
                 continue  # finished a step ago (this token is one too many), or taken out meanwhile
             outputs.append(self._take(r, token, logprob, logprobs))
         return outputs

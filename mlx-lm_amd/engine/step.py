@@ -134,21 +134,24 @@ class Engine:
                 raise ValueError(f"request {e.request_id!r} brings no tokens")
             if e.fed_row >= 0 and n != 1:
                 raise ValueError(f"request {e.request_id!r}: a token fed on the device is one token")
-            toks = np.asarray(e.tokens, dtype=np.int64)
-            if toks.ndim != 1 or int(toks.min()) < 0 or int(toks.max()) >= V:
-                bad = [int(t) for t in np.ravel(toks) if not 0 <= int(t) < V][:1]
-                raise ValueError(f"token id {bad[0] if bad else '?'} of request {e.request_id!r} is outside [0, {V})")
+            if n == 1:  # (the common case, without an array)
+                t = e.tokens[0]
+                if not 0 <= t < V:
+                    raise ValueError(f"token id {int(t)} of request {e.request_id!r} is outside [0, {V})")
+            else:
+                toks = np.asarray(e.tokens, dtype=np.int64)
+                if toks.ndim != 1 or int(toks.min()) < 0 or int(toks.max()) >= V:
+                    bad = [int(t) for t in np.ravel(toks) if not 0 <= int(t) < V][:1]
+                    raise ValueError(f"token id {bad[0] if bad else '?'} of request {e.request_id!r} is outside [0, {V})")
             length = self.cache.requests[e.request_id].length
             if length + n > P:
                 raise ValueError(
                     f"request {e.request_id!r} would reach {length + n} tokens, the model "
                     f"has {P} positions"
                 )
-            if len(e.want):
-                want = np.asarray(e.want, dtype=np.int64)
-                if int(want.min()) < 0 or int(want.max()) >= n:
-                    w = next(int(w) for w in want if not 0 <= int(w) < n)
-                    raise ValueError(f"wanted place {w} of request {e.request_id!r} is outside its {n} tokens")
+            for w in e.want:
+                if not 0 <= w < n:
+                    raise ValueError(f"wanted place {int(w)} of request {e.request_id!r} is outside its {n} tokens")
 
     def step(self, entries: List[StepEntry], fed=None):
         """Run one batch; returns float32 logits ``[n_wanted, vocab]`` (``None`` if nothing is wanted).
