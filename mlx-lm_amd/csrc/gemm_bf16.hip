@@ -558,30 +558,55 @@ static double cost_256(int M, int N) { return (double)((busiest_die<Tile256>(M, 
 // (256 x 192: three quarters of the arithmetic, seven eighths of the bytes; its tiles fit N = 4800)
 static double cost_256x192(int M, int N) { return (double)((busiest_die<Tile256x192>(M, N) + 31) / 32) * 1.6; }
 
-// Tiles of 64 x 128 instead of 128 x 128 where the latter would be few (up to some 160): twice
-// the blocks, each with half the arithmetic.  Measured at GPT-2 XL's projections they are some
-// 10 % ahead up to 384 rows and level at 512; the narrow ones (N = 1600) gain up to 1,024 rows.
-static bool small_tiles(int M, int N) { return (long)((M + 127) / 128) * ((N + 127) / 128) <= 160; }
+// Tiles of 64 x 128 instead of 128 x 128 where the latter would be few (up to 128): twice the
+// blocks, each with half the arithmetic and three quarters of the bytes.  Measured at widths
+// from 768 to 2,048: ahead by up to a quarter while the 128 x 128 tiles leave half the CUs idle,
+// level at 144 tiles, behind from 160 on (2,048 rows of a projection to 1,280 features with
+// K = 5,120: 59 us against 51), where what the tiles fetch from the L2s counts for more.
+static bool small_tiles(int M, int N) { return (long)((M + 127) / 128) * ((N + 127) / 128) <= 128; }
 
-// Into how many parts the kernels with tiles 128 wide should split K
-// (1: no split).  Few rows give few tiles: up to 128 rows of GPT-2 XL's projections are 13 to 50 tiles
-// for 256 CUs, and a tile's walk through K takes the same time whether 50 or
-// 500 of them run.  Measured at those sizes (65 to 640 rows), the best number
-// of parts brings the blocks to some 220, as long as a part keeps three
-// k-blocks or more; from 150 tiles on the partial sums ([parts][M][N] floats,
-// written and read once) cost more than the idle CUs.
+// Microseconds a CU takes per k-block when it holds `n` blocks of tiles `rows` x 128 (measured at
+// widths 768 to 2,048): a block alone waits for its fetches most of the time, so a second block
+// on the CU costs little; from the third on they take turns.
+static double kblock_us(int rows, int n) {
+  const double alone = rows <= 32 ? 0.37 : rows <= 64 ? 0.52 : 0.62;
+  const double pair = rows <= 32 ? 0.56 : rows <= 64 ? 0.80 : 1.14;
+  return (n / 2) * pair + (n % 2) * alone;
+}
+
+// Into how many parts the kernels with tiles 128 wide should split K (1: no split).  Few rows
+// give few tiles (up to 128 rows of GPT-2 XL's projections are 13 to 50 tiles for 256 CUs), and a
+// tile's walk through K takes the same time whether 50 or 500 of them run; a split shortens the
+// walk and costs a second kernel that reads the partial sums ([parts][M][N] floats).  Both sides
+// are priced from what was measured (65 to 768 rows, widths 768 to 2,048, K up to 8,192): the walk
+// as k-blocks times the time per k-block of the busiest CU, the second kernel as a launch plus
+// its bytes at 3 TB/s.  `fused`: the second kernel stands in for one that would run anyway (the
+// norm that follows a sum into the residual stream, the write of keys and values into their
+// pages), so it costs only the extra bytes.  A part keeps three k-blocks or more.
 // `force` > 0 asks for that many parts wherever K has them (for tests of small sizes).
-extern "C" int gemm_bf16_splits(int M, int N, int K, int force) {
+extern "C" int gemm_bf16_splits(int M, int N, int K, int fused, int force) {
   if (M < TILE_MIN_ROWS) return 1;
   const long cols = (N + 127) / 128;
-  const long tiles = M <= 32 ? cols : small_tiles(M, N) ? (long)((M + 63) / 64) * cols : (long)((M + 127) / 128) * cols;
+  const int rows = M <= 32 ? 32 : small_tiles(M, N) ? 64 : 128;
+  const long tiles = (long)((M + rows - 1) / rows) * cols;
   const int n_blocks = (K + BK - 1) / BK;
-  int want = (int)((220 + tiles / 2) / tiles);
-  if (want > n_blocks / 3) want = n_blocks / 3;
-  if (want > 16) want = 16;
-  if (force > 0) want = force < n_blocks ? force : n_blocks;
-  if (want <= 1) return 1;
-  const int per = (n_blocks + want - 1) / want;
+  int best = 1;
+  if (force > 0) {
+    best = force < n_blocks ? force : n_blocks;
+  } else {
+    double best_us = 0.0, whole_us = 0.0;
+    for (int s = 1; s <= 16 && s <= (n_blocks >= 3 ? n_blocks / 3 : 1); ++s) {
+      const int per = (n_blocks + s - 1) / s;
+      const int on_cu = (int)((tiles * s + 255) / 256);
+      double us = kblock_us(rows, on_cu) * per;
+      if (s > 1) us += (fused ? 1.0 : 2.5) + 8.0 * (fused ? s - 1 : s) * (double)M * N / 3e6;
+      if (s == 1) whole_us = us;
+      if (s == 1 || us < best_us) best = s, best_us = us;
+    }
+    if (best_us > 0.9 * whole_us) best = 1;  // (the prices are good to a tenth)
+  }
+  if (best <= 1) return 1;
+  const int per = (n_blocks + best - 1) / best;
   return (n_blocks + per - 1) / per;  // no empty part
 }
 

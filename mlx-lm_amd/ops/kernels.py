@@ -410,7 +410,10 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
         if variant in (0, 1, 5, 6) and M > DECODE_MAX_ROWS:
             n_blocks = (K + 63) // 64
             if splits is None:
-                n_splits = lib.gemm_bf16_splits(_c_int(M), _c_int(N), _c_int(K), _c_int(force_splits))
+                # (the second kernel stands in for one that would run anyway: the next norm, or the cache write)
+                fused = (accumulate and pending is not None and pending.allowed) or scatter is not None
+                n_splits = lib.gemm_bf16_splits(_c_int(M), _c_int(N), _c_int(K), _c_int(1 if fused else 0),
+                                                _c_int(force_splits))
             else:
                 per_split = -(-n_blocks // max(1, min(splits, n_blocks)))
                 n_splits = -(-n_blocks // per_split)

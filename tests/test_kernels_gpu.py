@@ -806,16 +806,21 @@ def test_default_splits_fill_the_gpu():
     assert lib.gemm_bf16_decode_splits(8, 64, 64, 0, 2) == 1  # one k-block cannot be split
     assert lib.gemm_bf16_decode_splits(8, 64, 200, 0, 2) == 2
     tiles = k.build.load("gemm_bf16")
-    assert tiles.gemm_bf16_splits(16, 1600, 6400, 0) == 1  # (the decode kernels' rows)
-    assert tiles.gemm_bf16_splits(17, 1600, 6400, 0) > 8
-    assert tiles.gemm_bf16_splits(64, 50257, 1600, 0) == 1  # (many tiles fill the GPU as they are)
-    assert tiles.gemm_bf16_splits(64, 1600, 6400, 0) > 8
-    assert tiles.gemm_bf16_splits(72, 1600, 6400, 0) >= 8
-    assert 3 <= tiles.gemm_bf16_splits(128, 4800, 1600, 0) <= 8
-    assert tiles.gemm_bf16_splits(512, 4800, 1600, 0) == 1
-    assert tiles.gemm_bf16_splits(2048, 4800, 1600, 0) == 1
-    assert tiles.gemm_bf16_splits(100, 96, 128, 0) == 1  # too few k-blocks to share out
-    assert tiles.gemm_bf16_splits(100, 96, 128, 3) == 2
+    # (rows, features, K, the sum is left to the next norm, forced parts)
+    assert tiles.gemm_bf16_splits(16, 1600, 6400, 1, 0) == 1  # (the decode kernels' rows)
+    assert tiles.gemm_bf16_splits(17, 1600, 6400, 1, 0) > 8
+    assert tiles.gemm_bf16_splits(64, 50257, 1600, 0, 0) == 1  # (many tiles fill the GPU as they are)
+    assert tiles.gemm_bf16_splits(64, 1600, 6400, 1, 0) > 8
+    assert tiles.gemm_bf16_splits(72, 1600, 6400, 1, 0) >= 8
+    assert 3 <= tiles.gemm_bf16_splits(64, 4800, 1600, 0, 0) <= 8
+    assert tiles.gemm_bf16_splits(128, 2304, 768, 0, 0) == 1  # a short K: the second kernel costs more than the walk
+    assert tiles.gemm_bf16_splits(512, 2304, 768, 0, 0) == 1
+    assert tiles.gemm_bf16_splits(512, 4800, 1600, 0, 0) == 1
+    assert tiles.gemm_bf16_splits(2048, 4800, 1600, 0, 0) == 1
+    assert 2 <= tiles.gemm_bf16_splits(768, 1600, 6400, 1, 0) <= 4  # a long K pays for a split at more rows
+    assert tiles.gemm_bf16_splits(2048, 1600, 6400, 1, 0) == 1
+    assert tiles.gemm_bf16_splits(100, 96, 128, 0, 0) == 1  # too few k-blocks to share out
+    assert tiles.gemm_bf16_splits(100, 96, 128, 0, 3) == 2
 
 
 @pytest.mark.parametrize("M", [1, 5, 16, 40, 80])
