@@ -60,12 +60,26 @@ __device__ __forceinline__ unsigned long long mix64(unsigned long long x) {
   x ^= x >> 31;
   return x;
 }
-// uniform in (0, 1), 24 bits, from (seed, counter, index)
-__device__ __forceinline__ float uniform01(unsigned long long seed, unsigned int counter,
-                                           unsigned int index) {
-  unsigned long long x = mix64(seed + 0x9E3779B97F4A7C15ull * (unsigned long long)(counter + 1u));
-  x = mix64(x ^ (0xD1B54A32D192ED03ull * (unsigned long long)(index + 1u)));
-  return ((float)(unsigned int)(x >> 40) + 0.5f) * (1.0f / 16777216.0f);
+// The key of a row's draws: 64 bits mixed from (seed, counter), once per thread.
+__device__ __forceinline__ unsigned long long draw_key(unsigned long long seed, unsigned int counter) {
+  return mix64(seed + 0x9E3779B97F4A7C15ull * (unsigned long long)(counter + 1u));
+}
+// uniform in (0, 1), 24 bits, from a key and an index: two rounds of a 32-bit finalizer
+// (multiply, shift, xor), each keyed with half the key.  32-bit multiplies only: 64-bit
+// ones are several instructions each at a quarter of the rate, and this runs once per
+// vocabulary entry on the one CU that has the row.
+__device__ __forceinline__ unsigned int fmix32(unsigned int x) {
+  x ^= x >> 16;
+  x *= 0x85EBCA6Bu;
+  x ^= x >> 13;
+  x *= 0xC2B2AE35u;
+  x ^= x >> 16;
+  return x;
+}
+__device__ __forceinline__ float uniform01(unsigned long long key, unsigned int index) {
+  unsigned int x = fmix32((index + 1u) * 0x9E3779B1u ^ (unsigned int)key);
+  x = fmix32(x + (unsigned int)(key >> 32));
+  return ((float)(x >> 8) + 0.5f) * (1.0f / 16777216.0f);
 }
 
 struct Kept {
@@ -249,7 +263,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(SampleArgs 
   // the special tokens
   const float xtc_prob = a.xtc_prob[r];
   if (xtc_prob > 0.f) {
-    const float u = uniform01(a.seed[r], (unsigned int)a.counter[r], 0xfffffffeu);
+    const float u = uniform01(draw_key(a.seed[r], (unsigned int)a.counter[r]), 0xfffffffeu);
     if (!(u > xtc_prob)) {
       float z = 0.f;
       for (int i = tid; i < V; i += nt) {
@@ -274,14 +288,15 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(SampleArgs 
 
   // Gumbel-max draw from softmax(lp / temp) over the kept tokens
   const float inv_temp = 1.f / temp;
-  const unsigned long long seed = a.seed[r];
-  const unsigned int counter = (unsigned int)a.counter[r];
+  const unsigned long long key = draw_key(a.seed[r], (unsigned int)a.counter[r]);
   bv = -INFINITY, bi = 0x7fffffff;
   for_row(x, V, tid, nt, [&](int i, float xi) {
     const float lp = xi - lse;
     if (!kept(i, lp)) return;
-    const float u = uniform01(seed, counter, (unsigned int)i);
-    const float g = -logf(-logf(u));
+    // Gumbel noise -log(-log u) through the hardware's log2 (u has 24 bits; v_log_f32 is good to
+    // an ulp of its result)
+    const float u = uniform01(key, (unsigned int)i);
+    const float g = -0.69314718f * __log2f(-0.69314718f * __log2f(u));
     const float v = lp * inv_temp + g;
     if (v > bv) bv = v, bi = i;
   });
