@@ -23,6 +23,7 @@
 #include "common.h"
 
 #define SAMPLE_THREADS 1024
+#define CAND_CAP 4608  // tokens in the list of candidates: three arrays of 18 KB in LDS
 
 struct SampleArgs {
   int* tokens;            // [R]
@@ -201,32 +202,164 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(SampleArgs 
   kept.lo = -INFINITY, kept.hi = INFINITY;
   kept.special = a.xtc_special, kept.n_special = 0;
   const float lp_max = mx - lse;
+  const float top_p = a.top_p[r], min_p = a.min_p[r], xtc_prob = a.xtc_prob[r];
+  const int top_k = a.top_k[r], min_keep = a.min_keep[r];
+  const int lane = tid & 63, wave = tid >> 6;
+
+  // ---- candidates ------------------------------------------------------------
+  // The thresholds of top_p, top_k and min_tokens_to_keep lie among the most likely tokens.
+  // Where some filter needs a bisection (32 probes, each a pass over the row: 170 us a filter at
+  // GPT-2's vocabulary), the tokens nearest the maximum are first put into a list in LDS, as
+  // many as fit: the bins of a histogram over lp_max - lp in quarters of a nat say how far down
+  // the list can go.  One wave then bisects over the list (a fraction of a microsecond a probe),
+  // and the draw runs over the list as well if every kept token is in it.  The list's order is
+  // fixed (by thread, then by index), so sums over it are repeatable.  Whatever the list cannot
+  // decide (a flat row, a nucleus of thousands of tokens, xtc) takes the passes over the row.
+  __shared__ float c_lp[CAND_CAP], c_p[CAND_CAP];
+  __shared__ int c_idx[CAND_CAP];
+  __shared__ int hist[64];
+  __shared__ int wave_tot[SAMPLE_THREADS / 64];
+  __shared__ float bcast[2];
+  auto bin_of = [&](float lp) {
+    const float d = (lp_max - lp) * 4.f;
+    return d < 63.f ? (int)d : 63;  // (lp = -inf: the last bin)
+  };
+  const bool bisects = (top_p > 0.f && top_p < 1.f) || top_k > 0 || (min_p != 0.f && min_keep > 1);
+  bool cand = false;
+  int n_cand = 0;
+  float m_low = 0.f, noncand_max = -INFINITY;
+  if (bisects && !(xtc_prob > 0.f) && V < (1 << 24)) {
+    if (tid < 64) hist[tid] = 0;
+    __syncthreads();
+    // (the first and the last bin are counted in registers: on a flat row, or on a peaked one,
+    // nearly every token falls into one of them, and adds to one LDS word take turns)
+    float in_first = 0.f;
+    for_row(x, V, tid, nt, [&](int, float v) {
+      const int b = bin_of(v - lse);
+      if (b == 0)
+        in_first += 1.f;
+      else if (b < 63)
+        atomicAdd(&hist[b], 1);
+    });
+    in_first = block_sum(in_first, red);  // (exact: at most V < 2^24)
+    int cum = 0, b_last = -1;
+    for (int b = 0; b < 64; ++b) {
+      cum = b == 63 ? V : cum + (b == 0 ? (int)in_first : hist[b]);
+      if (cum <= CAND_CAP) b_last = b, n_cand = cum;
+    }
+    if (b_last >= 0) {
+      cand = true;
+      int cnt = 0;
+      float low = 0.f, ncmax = -INFINITY;
+      for_row(x, V, tid, nt, [&](int, float v) {
+        const float lp = v - lse;
+        if (bin_of(lp) <= b_last) {
+          ++cnt;
+        } else {
+          low += expf(lp);
+          ncmax = fmaxf(ncmax, lp);
+        }
+      });
+      m_low = block_sum(low, red);
+      noncand_max = block_max(ncmax, red);
+      // where this thread's candidates start: the counts of the threads before it
+      int incl = cnt;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(incl, o, WAVE);
+        if (lane >= o) incl += up;
+      }
+      __syncthreads();
+      if (lane == 63) wave_tot[wave] = incl;
+      __syncthreads();
+      int pos = incl - cnt;
+      for (int w = 0; w < wave; ++w) pos += wave_tot[w];
+      for_row(x, V, tid, nt, [&](int i, float v) {
+        const float lp = v - lse;
+        if (bin_of(lp) <= b_last) {
+          c_lp[pos] = lp, c_p[pos] = expf(lp), c_idx[pos] = i;
+          ++pos;
+        }
+      });
+      __syncthreads();
+    }
+  }
 
   // top_p: keep lp >= v*, v* the smallest value whose ascending cumulative
   // probability H(v) = sum_{lp_j <= v} p_j exceeds 1 - top_p.
-  const float top_p = a.top_p[r];
   if (top_p > 0.f && top_p < 1.f) {
     const float need = 1.f - top_p;
-    unsigned int lo = 0u, hi = ordered_key(lp_max);  // H(hi) = 1 > need
-    while (lo < hi) {
-      const unsigned int mid = lo + ((hi - lo) >> 1);
-      const float c = key_to_float(mid);
-      float s = 0.f;
-      for_row(x, V, tid, nt, [&](int, float v) {
-        const float lp = v - lse;
-        if (lp <= c) s += expf(lp);
-      });
-      s = block_sum(s, red);
-      if (s > need)
-        hi = mid;
-      else
-        lo = mid + 1u;
+    if (cand && m_low <= need) {
+      // v* is in the list: H(v) = what lies below the list + the list's part
+      if (wave == 0) {
+        unsigned int lo = 0u, hi = ordered_key(lp_max);
+        while (lo < hi) {
+          const unsigned int mid = lo + ((hi - lo) >> 1);
+          const float c = key_to_float(mid);
+          float s = 0.f;
+          for (int j = lane; j < n_cand; j += 64)
+            if (c_lp[j] <= c) s += c_p[j];
+          s = m_low + wave_sum(s);
+          if (s > need)
+            hi = mid;
+          else
+            lo = mid + 1u;
+        }
+        if (lane == 0) bcast[0] = key_to_float(lo);
+      }
+      __syncthreads();
+      kept.lo = fmaxf(kept.lo, bcast[0]);
+      __syncthreads();
+    } else {
+      unsigned int lo = 0u, hi = ordered_key(lp_max);  // H(hi) = 1 > need
+      while (lo < hi) {
+        const unsigned int mid = lo + ((hi - lo) >> 1);
+        const float c = key_to_float(mid);
+        float s = 0.f;
+        for_row(x, V, tid, nt, [&](int, float v) {
+          const float lp = v - lse;
+          if (lp <= c) s += expf(lp);
+        });
+        s = block_sum(s, red);
+        if (s > need)
+          hi = mid;
+        else
+          lo = mid + 1u;
+      }
+      kept.lo = fmaxf(kept.lo, key_to_float(lo));
     }
-    kept.lo = fmaxf(kept.lo, key_to_float(lo));
   }
 
   // k-th largest value among the kept tokens, -inf if fewer than k are kept
   auto kth_largest = [&](int k) -> float {
+    if (cand) {  // (no xtc here: kept is lp >= kept.lo)
+      if (wave == 0) {
+        float n = 0.f;
+        for (int j = lane; j < n_cand; j += 64) n += c_lp[j] >= kept.lo ? 1.f : 0.f;
+        n = wave_sum(n);
+        float found = NAN;  // the list holds fewer than k kept tokens: the row decides
+        if (n >= (float)k) {
+          unsigned int lo = 0u, hi = ordered_key(lp_max);  // largest c with count(lp >= c) >= k
+          while (lo < hi) {
+            const unsigned int mid = lo + ((hi - lo + 1u) >> 1);
+            const float c = key_to_float(mid);
+            float cnt = 0.f;
+            for (int j = lane; j < n_cand; j += 64) cnt += (c_lp[j] >= c && c_lp[j] >= kept.lo) ? 1.f : 0.f;
+            cnt = wave_sum(cnt);
+            if (cnt >= (float)k)
+              lo = mid;
+            else
+              hi = mid - 1u;
+          }
+          found = key_to_float(lo);
+        }
+        if (lane == 0) bcast[1] = found;
+      }
+      __syncthreads();
+      const float found = bcast[1];
+      __syncthreads();
+      if (found == found) return found;
+    }
     float cnt_all = 0.f;
     for_row(x, V, tid, nt, [&](int i, float v) { cnt_all += kept(i, v - lse) ? 1.f : 0.f; });
     cnt_all = block_sum(cnt_all, red);
@@ -250,10 +383,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(SampleArgs 
   };
 
   // min_p: drop lp < max + log(min_p), but never one of the min_keep best
-  const float min_p = a.min_p[r];
   if (min_p != 0.f) {
     float floor_lp = lp_max + logf(min_p);
-    const int mk = a.min_keep[r];
+    const int mk = min_keep;
     if (mk > 1) floor_lp = fminf(floor_lp, kth_largest(mk));
     kept.lo = fmaxf(kept.lo, floor_lp);
   }
@@ -261,7 +393,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(SampleArgs 
   // xtc: with probability xtc_prob drop every token whose (renormalised)
   // probability is above the threshold, except the least likely of them and
   // the special tokens
-  const float xtc_prob = a.xtc_prob[r];
   if (xtc_prob > 0.f) {
     const float u = uniform01(draw_key(a.seed[r], (unsigned int)a.counter[r]), 0xfffffffeu);
     if (!(u > xtc_prob)) {
@@ -283,23 +414,30 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(SampleArgs 
     }
   }
 
-  const int top_k = a.top_k[r];
   if (top_k > 0) kept.lo = fmaxf(kept.lo, kth_largest(top_k));
 
   // Gumbel-max draw from softmax(lp / temp) over the kept tokens
   const float inv_temp = 1.f / temp;
   const unsigned long long key = draw_key(a.seed[r], (unsigned int)a.counter[r]);
   bv = -INFINITY, bi = 0x7fffffff;
-  for_row(x, V, tid, nt, [&](int i, float xi) {
-    const float lp = xi - lse;
-    if (!kept(i, lp)) return;
+  auto consider = [&](int i, float lp) {
     // Gumbel noise -log(-log u) through the hardware's log2 (u has 24 bits; v_log_f32 is good to
     // an ulp of its result)
     const float u = uniform01(key, (unsigned int)i);
     const float g = -0.69314718f * __log2f(-0.69314718f * __log2f(u));
     const float v = lp * inv_temp + g;
-    if (v > bv) bv = v, bi = i;
-  });
+    if (v > bv || (v == bv && i < bi)) bv = v, bi = i;
+  };
+  if (cand && (n_cand == V || kept.lo > noncand_max)) {
+    // every kept token is in the list (xtc is off: kept is lp >= kept.lo)
+    for (int j = tid; j < n_cand; j += nt)
+      if (c_lp[j] >= kept.lo) consider(c_idx[j], c_lp[j]);
+  } else {
+    for_row(x, V, tid, nt, [&](int i, float xi) {
+      const float lp = xi - lse;
+      if (kept(i, lp)) consider(i, lp);
+    });
+  }
   block_argmax(bv, bi, red, redi);
   if (tid == 0) {
     a.tokens[r] = bi;

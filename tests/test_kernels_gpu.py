@@ -534,6 +534,39 @@ def test_sample_filters_against_plain_on_random_rows():
         assert torch.equal((seen & allowed)[small], allowed[small]), kw
 
 
+@pytest.mark.parametrize("shape", ["peaked", "flat"])
+def test_sample_filters_at_large_vocabularies(shape):
+    """The filters' thresholds at vocabularies beyond the kernel's list of candidates: a peaked row
+    (the thresholds come from the list) and a flat one (no list: passes over the row).  A high
+    temperature makes the draw nearly uniform over what is kept, so the kept set shows."""
+    g = torch.Generator().manual_seed(3)
+    if shape == "peaked":
+        V, n = 50257, 1200
+        logits = -0.35 * torch.arange(V).double() ** 0.75 + 0.3 * torch.randn(V, generator=g).double()
+        logits = logits[torch.randperm(V, generator=g)]
+        cases = [dict(top_p=0.8), dict(top_k=13), dict(min_p=0.3, min_keep=9), dict(top_p=0.95, top_k=25)]
+    else:
+        V, n = 20000, 1200
+        logits = 0.01 * torch.randn(V, generator=g).double()
+        cases = [dict(top_p=0.00045), dict(top_k=7), dict(min_p=0.999, min_keep=6), dict(top_p=0.002, top_k=11)]
+    lp = plain.log_softmax(logits.float().double()[None])[0]
+    probs = lp.exp()
+    for kw in cases:
+        x = lp.clone()[None]
+        if "top_p" in kw:
+            x = plain.top_p_filter(x, kw["top_p"])
+        if "min_p" in kw:
+            x = plain.min_p_filter(x, kw["min_p"], kw.get("min_keep", 1))
+        if "top_k" in kw:
+            x = plain.top_k_filter(x, kw["top_k"])
+        allowed = torch.isfinite(x[0])
+        assert 1 <= int(allowed.sum()) <= 60, (kw, int(allowed.sum()))
+        rows = logits.float().to(DEV)[None].repeat(n, 1).contiguous()
+        tok, _, _ = _sample(rows, temp=200.0, seed=21, counter=list(range(n)), **kw)
+        seen = torch.bincount(tok.long(), minlength=V) > 0
+        assert torch.equal(seen, allowed), (shape, kw, int(seen.sum()), int(allowed.sum()))
+
+
 def test_sample_seed_and_batch_independence():
     logits = _rand((5, 300), torch.float32, 30, 2.0)
     a, _, _ = _sample(logits, temp=0.9, seed=[1, 2, 3, 4, 5], counter=[0, 1, 2, 3, 4])
