@@ -21,7 +21,7 @@ cut into pages of ``page_size`` tokens instead:
 """
 
 from dataclasses import dataclass, field
-from typing import Dict, List, Optional
+from typing import Dict, List
 
 from ..config.plan import CacheNeed, StateNeed
 from .pages import PagePool

@@ -7,7 +7,6 @@ batched sampling kernel, and they can also be called directly on device
 tensors, as the reference's closures are.
 """
 
-import math
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional
 

@@ -3,7 +3,6 @@
 import json
 import os
 
-import torch
 
 from ..config.registry import get_model_classes
 

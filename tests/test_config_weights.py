@@ -7,7 +7,6 @@ import pytest
 import torch
 
 import helpers
-import plain_gpt2 as plain
 from mlx_lm_amd.config import BaseModelArgs, get_model_classes, register_model
 from mlx_lm_amd.models.gpt2 import Model, ModelArgs
 from mlx_lm_amd.utils import load_config

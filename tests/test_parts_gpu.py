@@ -2,7 +2,6 @@
 that are registered, built and stepped without touching the framework's files."""
 
 import json
-import math
 import os
 from dataclasses import dataclass
 

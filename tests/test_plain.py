@@ -2,7 +2,6 @@
 library routines it must reduce to, invariants, and the vectors of the
 reference's own tests."""
 
-import math
 
 import pytest
 import torch
