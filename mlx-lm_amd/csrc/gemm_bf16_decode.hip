@@ -373,12 +373,37 @@ struct SumNormArgs {
   void* out;
   float eps;
   int M, N, ldh, n_splits, out_dtype;
+  // Blocks beyond the M rows read `ahead` (16-byte pieces) and drop it: the weights of the
+  // product that comes next, which then finds them in the caches.  A row a block leaves nearly
+  // every CU idle, and so does the memory.
+  const uint4* ahead;
+  size_t ahead_pieces;  // in a chunk
+  int ahead_chunks;
 };
 
 template <int NV4>
 __global__ __launch_bounds__(256) void sum_partials_norm_kernel(SumNormArgs q) {
   __shared__ float red[32];
   const int m = blockIdx.x, tid = threadIdx.x;
+  if (m >= q.M) {  // (uniform over the block)
+    // Block b of a launch runs on die b % 8, and so will block j of the product that comes next,
+    // which reads chunk j of `ahead` (`ahead_pieces` pieces each): this block reads chunks of its
+    // own die, so that they lie in the L2 where they will be asked for.
+    const int die = blockIdx.x & 7, rank = (m - q.M) >> 3, per_die = max(1, (int)(gridDim.x - q.M) >> 3);
+    unsigned int seen = 0u;
+    for (int j = die + 8 * rank; j < q.ahead_chunks; j += 8 * per_die) {
+      const uint4* src = q.ahead + (size_t)j * q.ahead_pieces;
+      for (size_t i0 = tid; i0 < q.ahead_pieces; i0 += 8 * 256) {
+        uint4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = src[min(i0 + u * 256, q.ahead_pieces - 1)];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) seen |= v[u].x;
+      }
+    }
+    asm volatile("" ::"v"(seen));  // the loads stay although nobody wants the values
+    return;
+  }
   float* hrow = q.h + (size_t)m * q.ldh;
   const size_t step = (size_t)q.M * q.N;
   const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f), one = make_float4(1.f, 1.f, 1.f, 1.f);
@@ -615,8 +640,11 @@ extern "C" int sum_partials_norm_takes(int N, int ldh) { return N > 0 && N % 4 =
 // h[m] += bias + sum of the partial products;  out[m] = LayerNorm(h[m]) (float32 or bfloat16, [M][N])
 extern "C" int sum_partials_norm(float* h, int ldh, const float* ws, int n_splits, const float* bias,
                                  const float* gamma, const float* beta, float eps, void* out,
-                                 int out_dtype, int M, int N, hipStream_t stream) {
+                                 int out_dtype, int M, int N, const void* ahead, size_t ahead_chunk_bytes,
+                                 int ahead_chunks, hipStream_t stream) {
   if (M == 0) return 0;
+  if (ahead && (!aligned16(ahead) || ahead_chunk_bytes % 16 != 0 || ahead_chunks < 0))
+    FAIL("sum_partials_norm: what is read ahead must be chunks of 16-byte pieces");
   if (M < 0 || n_splits < 1 || !ws || !h || !out) FAIL("sum_partials_norm: bad M=%d, splits=%d or null pointer", M, n_splits);
   if (!sum_partials_norm_takes(N, ldh) || ldh < N)
     FAIL("sum_partials_norm: width %d (row stride %d) must be a multiple of 4, at most 8192", N, ldh);
@@ -626,10 +654,15 @@ extern "C" int sum_partials_norm(float* h, int ldh, const float* ws, int n_split
   SumNormArgs q;
   q.h = h, q.ws = ws, q.bias = bias, q.gamma = gamma, q.beta = beta, q.out = out, q.eps = eps;
   q.M = M, q.N = N, q.ldh = ldh, q.n_splits = n_splits, q.out_dtype = out_dtype;
+  q.ahead = (const uint4*)ahead, q.ahead_pieces = ahead ? ahead_chunk_bytes / 16 : 0;
+  q.ahead_chunks = ahead ? ahead_chunks : 0;
+  // as many reading blocks as leave a CU each to the rows' blocks (few rows only: with many, the
+  // CUs are busy and the memory too)
+  const int readers = q.ahead_pieces > 0 && q.ahead_chunks > 0 && M <= 16 ? (256 - M) / 8 * 8 : 0;
   if (N <= 2048)
-    hipLaunchKernelGGL(sum_partials_norm_kernel<2>, dim3(M), dim3(256), 0, stream, q);
+    hipLaunchKernelGGL(sum_partials_norm_kernel<2>, dim3(M + readers), dim3(256), 0, stream, q);
   else
-    hipLaunchKernelGGL(sum_partials_norm_kernel<8>, dim3(M), dim3(256), 0, stream, q);
+    hipLaunchKernelGGL(sum_partials_norm_kernel<8>, dim3(M + readers), dim3(256), 0, stream, q);
   CHECK_LAUNCH("sum_partials_norm");
   return 0;
 }

@@ -181,6 +181,20 @@ class PackedWeight:
         # (block, feature, k-block, k group, half, 8) -> (block, k-block, half, k group, feature, 8)
         t = padded.view(Np // 16, 16, Kp // 64, 4, 2, 8).permute(0, 2, 4, 3, 1, 5)
         self.packed = t.contiguous().view(-1)
+        # what one block of the decode kernel reads (16 features, all of K) and how many there are
+        self.chunk_bytes, self.n_chunks = Kp * 16 * 2, Np // 16
+
+
+def read_ahead_pays(w, n_rows):
+    """Whether the rows' next product should have ``w`` read ahead by the kernel before it: a
+    ``PackedWeight`` that the decode kernel takes whole, 16 features a block (then block ``j``
+    reads chunk ``j``, on die ``j % 8``), for few enough rows that most CUs have none."""
+    if not isinstance(w, PackedWeight) or not 0 < n_rows <= DECODE_MAX_ROWS:
+        return False
+    N, K = w.shape
+    lib = build.load("gemm_bf16_decode")
+    return (w.n_chunks >= 150 and bool(lib.gemm_bf16_decode_takes(_c_int(n_rows), _c_int(K), _c_int(0), _c_int(1)))
+            and lib.gemm_bf16_decode_splits(_c_int(n_rows), _c_int(N), _c_int(K), _c_int(0), _c_int(force_splits)) == 1)
 
 
 def for_decode(w):
@@ -240,11 +254,13 @@ class PendingSum:
         target, self.target = self.target, None
         sum_partials(target, self.ws, self.n_splits, self.bias, accumulate=True)
 
-    def settle_normed(self, out, gamma, beta, eps):
-        """Add what is pending into its target and write the LayerNorm of the new rows to ``out``."""
+    def settle_normed(self, out, gamma, beta, eps, ahead=None):
+        """Add what is pending into its target and write the LayerNorm of the new rows to ``out``.
+
+        ``ahead``: the weights of the product that reads ``out`` (see ``sum_partials_norm``)."""
         target, self.target = self.target, None
         _need(target is not None, "settle_normed: nothing is pending")
-        sum_partials_norm(target, self.ws, self.n_splits, self.bias, gamma, beta, eps, out)
+        sum_partials_norm(target, self.ws, self.n_splits, self.bias, gamma, beta, eps, out, ahead=ahead)
 
     def can_norm(self, x):
         lib = build.load("gemm_bf16_decode")
@@ -285,8 +301,11 @@ def sum_partials(out, ws, n_splits, bias=None, gelu=False, accumulate=False, sca
     return out
 
 
-def sum_partials_norm(h, ws, n_splits, bias, gamma, beta, eps, out):
-    """``h += bias + sum of the partial products``; ``out = LayerNorm(h)`` (rows of ``h``, all of them)."""
+def sum_partials_norm(h, ws, n_splits, bias, gamma, beta, eps, out, ahead=None):
+    """``h += bias + sum of the partial products``; ``out = LayerNorm(h)`` (rows of ``h``, all of them).
+
+    ``ahead``: the ``PackedWeight`` of the product that comes next; CUs that have no row read it
+    meanwhile, each the chunks that a block on its own die will ask for."""
     lib = build.load("gemm_bf16_decode")
     M, N = h.shape
     _dev(h, "h", torch.float32)
@@ -300,7 +319,9 @@ def sum_partials_norm(h, ws, n_splits, bias, gamma, beta, eps, out):
             v.numel() == N or _fail(f"sum_partials_norm: {name} has {v.numel()} elements, width is {N}")
     rc = lib.sum_partials_norm(_ptr(h), _c_int(_rows2d(h, "h")), _ptr(ws), _c_int(n_splits), _ptr(bias),
                                _ptr(gamma), _ptr(beta), _c_float(eps), _ptr(out), _c_int(DT[out.dtype]),
-                               _c_int(M), _c_int(N), _stream())
+                               _c_int(M), _c_int(N), _ptr(ahead.packed if ahead is not None else None),
+                               _c_size_t(ahead.chunk_bytes if ahead is not None else 0),
+                               _c_int(ahead.n_chunks if ahead is not None else 0), _stream())
     build.check(lib, rc, "sum_partials_norm")
     return out
 

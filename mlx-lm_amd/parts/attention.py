@@ -71,6 +71,7 @@ class CausalSelfAttention(Mixer):
             self.qkv_b = tensors[n(self.qkv_name + ".bias")]
             self.out_b = tensors[n(self.out_name + ".bias")]
         self.qkv_w, self.out_w = kernels.for_decode(self.qkv_w), kernels.for_decode(self.out_w)
+        self.first_weight = self.qkv_w  # what the mixer's first product reads
         if self.position is not None:
             self.position.load(tensors)
 

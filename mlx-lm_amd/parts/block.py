@@ -24,7 +24,10 @@ class PreNormBlock(Block):
     def _normed(self, ctx, norm, h, consumer):
         if not getattr(norm, "settles_pending", False):
             ctx.pending.settle()
-        return norm.forward(ctx, h, lazy=getattr(consumer, "accepts_lazy_input", False))
+        lazy = getattr(consumer, "accepts_lazy_input", False)
+        if getattr(norm, "reads_ahead", False):  # it takes the weights its result meets first
+            return norm.forward(ctx, h, lazy=lazy, ahead=getattr(consumer, "first_weight", None))
+        return norm.forward(ctx, h, lazy=lazy)
 
     def forward(self, ctx, h, cache, writes_cache=True):
         mark = ctx.scratch_mark()

@@ -53,6 +53,7 @@ class GeluMLP(FeedForward):
             self.fc_b = torch.cat([self.fc_b, self.fc_b.new_zeros(pad)]).contiguous()
             self.proj_w = torch.cat([self.proj_w, self.proj_w.new_zeros(self.width, pad)], dim=1).contiguous()
         self.fc_w, self.proj_w = kernels.for_decode(self.fc_w), kernels.for_decode(self.proj_w)
+        self.first_weight = self.fc_w  # what the first product reads
 
     def forward(self, ctx, x, residual):
         act = ctx.scratch((x.shape[0], self.inner_padded), ctx.dtype)

@@ -30,14 +30,19 @@ class LayerNorm(Norm):
         self.bias = tensors[self._name("bias")] if self.has_bias else None
 
     settles_pending = True  # adds a sum that is pending on ``x`` before (or while) it norms the rows
+    reads_ahead = True  # ``forward`` takes ``ahead``, the weights that its result meets first
 
-    def forward(self, ctx, x, rows=None, n_rows=None, lazy=False):
+    def forward(self, ctx, x, rows=None, n_rows=None, lazy=False, ahead=None):
+        """``ahead``: the weights of the product that reads the result first, if its caller knows
+        them: a kernel here that leaves most of the GPU idle reads them into the caches meanwhile."""
         pending = ctx.pending
         if pending.waits_on(x):
             if rows is None and pending.can_norm(x):
                 # the last projection split its sum: add the parts and norm the new rows in one kernel
                 out = ctx.scratch((x.shape[0], self.width), ctx.dtype)
-                pending.settle_normed(out, self.weight, self.bias, self.eps)
+                if ahead is not None and not kernels.read_ahead_pays(ahead, x.shape[0]):
+                    ahead = None
+                pending.settle_normed(out, self.weight, self.bias, self.eps, ahead=ahead)
                 return out
             pending.settle()
         if lazy and rows is None:

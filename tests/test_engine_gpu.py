@@ -243,9 +243,9 @@ def test_split_sums_in_the_engine(folders, monkeypatch, name, sharp, use_graphs)
     calls = {"normed": 0, "plain": 0}
     settle_normed, settle = kernels.PendingSum.settle_normed, kernels.PendingSum.settle
 
-    def count_normed(self, *a):
+    def count_normed(self, *a, **kw):
         calls["normed"] += 1
-        return settle_normed(self, *a)
+        return settle_normed(self, *a, **kw)
 
     def count_plain(self):
         calls["plain"] += self.target is not None
