@@ -36,6 +36,12 @@ struct DecodeArgs {
   int ldq, ldo, max_blocks;
   int n_heads, n_kv_heads, page_size, window, n_splits;
   float scale;
+  // Blocks with blockIdx.y >= n_heads have no row: they read `ahead` (chunks of `ahead_pieces`
+  // 16-byte pieces: the weights of a product that comes soon) and drop it, each the chunks that
+  // a block on its own die will ask for.  Few rows leave most CUs idle, and the memory with them.
+  const uint4* ahead;
+  size_t ahead_pieces;
+  int ahead_chunks;
 };
 
 #define MAX_WAVES 16
@@ -59,6 +65,28 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n_waves = blockDim.x >> 6;
+  if (blockIdx.y >= p.n_heads) {  // a reading block (uniform)
+    if (blockIdx.z != 0) return;
+    // blocks go to the dies in turn, in the order x, y, z: this one is on die `lin % 8`, and
+    // block j of the product to come, which reads chunk j, on die j % 8
+    const int r = blockIdx.x + gridDim.x * (blockIdx.y - p.n_heads);
+    const int readers = gridDim.x * (gridDim.y - p.n_heads);
+    const int lin = gridDim.x * p.n_heads + r;
+    const int die = lin & 7, rank = r >> 3, per_die = (readers + 7) >> 3;
+    unsigned int seen = 0u;
+    for (int j = die + 8 * rank; j < p.ahead_chunks; j += 8 * per_die) {
+      const uint4* src = p.ahead + (size_t)j * p.ahead_pieces;
+      for (size_t i0 = tid; i0 < p.ahead_pieces; i0 += 4 * blockDim.x) {
+        uint4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = src[min(i0 + u * blockDim.x, p.ahead_pieces - 1)];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) seen |= v[u].x;
+      }
+    }
+    asm volatile("" ::"v"(seen));  // the loads stay although nobody wants the values
+    return;
+  }
   const int item = blockIdx.x, h = blockIdx.y, split = blockIdx.z;
   const int row = p.rows[item];
   const int kv_head = h / (p.n_heads / p.n_kv_heads);
@@ -201,7 +229,13 @@ DEFINE_LAST_ERROR(mlxlm_last_error)
 
 template <int CPK>
 static void launch(const DecodeArgs& p, int n_rows, int n_waves, hipStream_t stream) {
-  hipLaunchKernelGGL(attn_decode_kernel<CPK>, dim3(n_rows, p.n_heads, p.n_splits), dim3(64 * n_waves), 0, stream, p);
+  // reading blocks for the CUs that the rows leave idle (256 CUs), if there are eight or more
+  int extra_y = 0;
+  if (p.ahead && p.ahead_chunks > 0) {
+    extra_y = (256 - n_rows * p.n_heads * p.n_splits) / n_rows;
+    if (extra_y * n_rows < 8) extra_y = 0;
+  }
+  hipLaunchKernelGGL(attn_decode_kernel<CPK>, dim3(n_rows, p.n_heads + extra_y, p.n_splits), dim3(64 * n_waves), 0, stream, p);
   if (p.n_splits > 1)
     hipLaunchKernelGGL(attn_decode_merge_kernel<CPK>, dim3(n_rows, p.n_heads), dim3(8 * CPK), 0, stream, p);
 }
@@ -213,7 +247,8 @@ extern "C" int attn_decode(void* out, const void* q, int ldq, int ldo, const voi
                            int max_blocks, const int* token_req, const int* positions,
                            const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
                            int page_size, int window, float scale, int n_splits, float* part_o,
-                           float* part_ml, int n_waves, hipStream_t stream) {
+                           float* part_ml, int n_waves, const void* ahead, size_t ahead_chunk_bytes,
+                           int ahead_chunks, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (n_waves < 1 || n_waves > MAX_WAVES) FAIL("attn_decode: %d waves a block, must be 1 to %d", n_waves, MAX_WAVES);
   if (head_dim > 64 * n_waves) FAIL("attn_decode: head_dim %d needs at least %d waves", head_dim, (head_dim + 63) / 64);
@@ -241,6 +276,10 @@ extern "C" int attn_decode(void* out, const void* q, int ldq, int ldo, const voi
   p.ldq = ldq, p.ldo = ldo, p.max_blocks = max_blocks;
   p.n_heads = n_heads, p.n_kv_heads = n_kv_heads, p.page_size = page_size;
   p.window = window, p.n_splits = n_splits, p.scale = scale;
+  if (ahead && (((uintptr_t)ahead & 15) || ahead_chunk_bytes % 16 != 0 || ahead_chunks < 0))
+    FAIL("attn_decode: what is read ahead must be chunks of 16-byte pieces");
+  p.ahead = (const uint4*)ahead, p.ahead_pieces = ahead ? ahead_chunk_bytes / 16 : 0;
+  p.ahead_chunks = ahead ? ahead_chunks : 0;
   if (head_dim == 32)
     launch<4>(p, n_rows, n_waves, stream);
   else if (head_dim == 64)

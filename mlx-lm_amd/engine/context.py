@@ -138,6 +138,7 @@ class StepContext:
 
         self.pending = PendingSum()
         self.wants_every_row = False  # wanted_rows is 0 .. n_tokens - 1
+        self.read_ahead = None  # weights (a PackedWeight) that a kernel with idle CUs may read ahead
 
     def scratch(self, shape, dtype):
         return self._scratch.take(shape, dtype)

@@ -185,7 +185,7 @@ class PackedWeight:
         self.chunk_bytes, self.n_chunks = Kp * 16 * 2, Np // 16
 
 
-def read_ahead_pays(w, n_rows):
+def read_ahead_pays(w, n_rows, with_norm=False):
     """Whether the rows' next product should have ``w`` read ahead by the kernel before it: a
     ``PackedWeight`` that the decode kernel takes whole, 16 features a block (then block ``j``
     reads chunk ``j``, on die ``j % 8``), for few enough rows that most CUs have none."""
@@ -193,8 +193,9 @@ def read_ahead_pays(w, n_rows):
         return False
     N, K = w.shape
     lib = build.load("gemm_bf16_decode")
-    return (w.n_chunks >= 150 and bool(lib.gemm_bf16_decode_takes(_c_int(n_rows), _c_int(K), _c_int(0), _c_int(1)))
-            and lib.gemm_bf16_decode_splits(_c_int(n_rows), _c_int(N), _c_int(K), _c_int(0), _c_int(force_splits)) == 1)
+    norm = _c_int(1 if with_norm else 0)
+    return (w.n_chunks >= 150 and bool(lib.gemm_bf16_decode_takes(_c_int(n_rows), _c_int(K), norm, _c_int(1)))
+            and lib.gemm_bf16_decode_splits(_c_int(n_rows), _c_int(N), _c_int(K), norm, _c_int(force_splits)) == 1)
 
 
 def for_decode(w):
@@ -604,8 +605,11 @@ def attn_decode_takes(q_dtype, kv):
 
 
 def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_heads, scale,
-                window=0, n_splits=1, part_o=None, part_ml=None, n_waves=4):
-    """``attn_row`` for bfloat16 caches with head_dim 32, 64 or 128: keys stream into registers."""
+                window=0, n_splits=1, part_o=None, part_ml=None, n_waves=4, ahead=None, ahead_chunks=0):
+    """``attn_row`` for bfloat16 caches with head_dim 32, 64 or 128: keys stream into registers.
+
+    ``ahead``: a ``PackedWeight`` whose first ``ahead_chunks`` chunks the CUs without a row read
+    meanwhile, each the chunks that a block on its own die will ask for (``sum_partials_norm``)."""
     lib = build.load("attention_decode")
     ldq, ldo = _rows2d(q, "q"), _rows2d(out, "out")
     _need(q.dtype == torch.bfloat16, "attn_decode: bfloat16 only")
@@ -624,7 +628,10 @@ def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_h
         _c_size_t(kv.page_stride), _ptr(block_table), _c_int(block_table.shape[1]),
         _ptr(token_req), _ptr(positions), _ptr(rows), _c_int(n_rows), _c_int(n_heads),
         _c_int(kv.n_kv_heads), _c_int(kv.head_dim), _c_int(kv.page_size), _c_int(window),
-        _c_float(scale), _c_int(n_splits), _ptr(part_o), _ptr(part_ml), _c_int(n_waves), _stream(),
+        _c_float(scale), _c_int(n_splits), _ptr(part_o), _ptr(part_ml), _c_int(n_waves),
+        _ptr(ahead.packed if ahead is not None else None),
+        _c_size_t(ahead.chunk_bytes if ahead is not None else 0),
+        _c_int(min(ahead_chunks, ahead.n_chunks) if ahead is not None else 0), _stream(),
     )
     build.check(lib, rc, "attn_decode")
     return out

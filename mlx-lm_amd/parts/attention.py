@@ -5,6 +5,9 @@ from ..ops import kernels
 from .base import POSITION_ENCODINGS, Mixer, TensorSpec, build_part, register_mixer
 
 
+READ_AHEAD_BYTES_PER_CU = 160 * 1024  # what an idle CU reads while decode attention runs (some 5 us)
+
+
 class CausalSelfAttention(Mixer):
     """Fused q/k/v projection, cache write, attention, output projection.
 
@@ -121,8 +124,18 @@ class CausalSelfAttention(Mixer):
                 part_o = ctx.scratch((n * self.head_dim,), "float32")
                 part_ml = ctx.scratch((n * 2,), "float32")
             if fast:
+                # CUs without a row read the weights that come after this mixer's own (the block
+                # says which), as many chunks as they manage while the rows' blocks run
+                ahead, chunks = getattr(ctx, "read_ahead", None), 0
+                idle = 256 - plan.n_rows * self.n_heads * n_splits
+                if (ahead is not None and idle >= 8 and plan.n_tiles == 0 and plan.n_rows == q.shape[0]
+                        and kernels.read_ahead_pays(ahead, plan.n_rows, with_norm=True)):
+                    chunks = idle * READ_AHEAD_BYTES_PER_CU // ahead.chunk_bytes
+                else:
+                    ahead = None
                 kernels.attn_decode(out, q, *args, plan.rows, plan.n_rows, self.n_heads, self.scale,
-                                    self.window, n_splits, part_o, part_ml, n_waves)
+                                    self.window, n_splits, part_o, part_ml, n_waves, ahead=ahead,
+                                    ahead_chunks=chunks)
             else:
                 kernels.attn_row(out, q, *args, plan.rows, plan.n_rows, self.n_heads, self.scale,
                                  self.window, n_splits, part_o, part_ml)

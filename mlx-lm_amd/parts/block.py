@@ -31,7 +31,11 @@ class PreNormBlock(Block):
 
     def forward(self, ctx, h, cache, writes_cache=True):
         mark = ctx.scratch_mark()
-        self.mixer.forward(ctx, self._normed(ctx, self.mixer_norm, h, self.mixer), h, cache, writes_cache)
+        x = self._normed(ctx, self.mixer_norm, h, self.mixer)
+        # (a mixer whose kernels leave CUs idle may have them read the weights that come after its own)
+        ctx.read_ahead = getattr(self.ffn, "first_weight", None)
+        self.mixer.forward(ctx, x, h, cache, writes_cache)
+        ctx.read_ahead = None
         self.ffn.forward(ctx, self._normed(ctx, self.ffn_norm, h, self.ffn), h)
         ctx.scratch_release(mark)
         return h

@@ -824,6 +824,45 @@ def test_pending_sum_is_added_by_the_norm(M, N, K, out_dtype):
         assert not pending.waits_on(h4) and torch.equal(h4, h3)
 
 
+def test_reading_weights_ahead_changes_nothing():
+    """The blocks that read the next product's weights ahead (in the fused sum-and-norm and in decode
+    attention) only read: results are what they are without them, for weights whose last chunk is
+    short of nothing (padded) and counts of chunks that are no multiple of eight."""
+    k = _k()
+    for n_feat, K in ((2400 + 16 * 3, 192), (16 * 151, 64)):
+        w = k.for_decode(_rand((n_feat, K), torch.bfloat16, 3, 0.1))
+        assert k.read_ahead_pays(w, 8) and w.n_chunks * w.chunk_bytes == w.packed.numel() * 2
+        assert not k.read_ahead_pays(k.for_decode(_rand((1600, 64), torch.bfloat16, 3)), 8)  # 8 features a block
+        assert not k.read_ahead_pays(w, 17)
+        # the fused sum-and-norm
+        M, N = 8, 96
+        ws = _rand((3, M, N), torch.float32, 4)
+        bias, gamma, beta = _rand((N,), torch.float32, 5), 1 + _rand((N,), torch.float32, 6, 0.1), _rand((N,), torch.float32, 7)
+        h0 = _rand((M, N), torch.float32, 8)
+        outs = []
+        for ahead in (None, w):
+            h, y = h0.clone(), torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+            k.sum_partials_norm(h, ws, 3, bias, gamma, beta, 1e-5, y, ahead=ahead)
+            outs.append((h, y))
+        assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+        # decode attention: one row and eight, with and without split keys
+        for ctx, n_splits in (([300], 1), ([40, 7, 90, 3, 200, 64, 65, 1], 1), ([500, 20], 2)):
+            H, hd = 3, 64
+            c = PagedCase(torch.bfloat16, H, H, hd, 16, ctx, [1] * len(ctx), seed=len(ctx))
+            k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
+            rows = torch.arange(c.T, dtype=torch.int32, device=DEV)
+            po = torch.empty(c.T * H * n_splits * hd, dtype=torch.float32, device=DEV)
+            pm = torch.empty(c.T * H * n_splits * 2, dtype=torch.float32, device=DEV)
+            res = []
+            for ahead in (None, w):
+                out = torch.full((c.T, H * hd), float("nan")).to(torch.bfloat16).to(DEV)
+                k.attn_decode(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, c.T,
+                              H, c.scale, 0, n_splits, po, pm, 4, ahead=ahead, ahead_chunks=10**6)
+                res.append(out)
+            assert torch.equal(res[0], res[1])
+            assert (res[1].double().cpu() - c.reference()).abs().max().item() < _attn_tol(torch.bfloat16)
+
+
 def test_default_splits_fill_the_gpu():
     """The library's own choice: no split where feature blocks alone fill the GPU, some where they do not."""
     k = _k()
