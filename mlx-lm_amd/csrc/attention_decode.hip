@@ -73,16 +73,21 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
     const int readers = gridDim.x * (gridDim.y - p.n_heads);
     const int lin = gridDim.x * p.n_heads + r;
     const int die = lin & 7, rank = r >> 3, per_die = (readers + 7) >> 3;
+    // the die's chunks (die, die + 8, ...) laid end to end and cut into equal shares, one a block
+    const size_t mine = die < p.ahead_chunks ? (size_t)((p.ahead_chunks - die + 7) / 8) * p.ahead_pieces : 0;
+    const size_t share = (mine + per_die - 1) / per_die;
+    const size_t lo = (size_t)rank * share, hi = min(lo + share, mine);
     unsigned int seen = 0u;
-    for (int j = die + 8 * rank; j < p.ahead_chunks; j += 8 * per_die) {
-      const uint4* src = p.ahead + (size_t)j * p.ahead_pieces;
-      for (size_t i0 = tid; i0 < p.ahead_pieces; i0 += 4 * blockDim.x) {
-        uint4 v[4];
+    for (size_t i0 = lo + tid; i0 < hi; i0 += 8 * (size_t)blockDim.x) {
+      uint4 v[8];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) v[u] = src[min(i0 + u * blockDim.x, p.ahead_pieces - 1)];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) seen |= v[u].x;
+      for (int u = 0; u < 8; ++u) {
+        const size_t t = min(i0 + u * (size_t)blockDim.x, hi - 1);
+        const size_t c = t / p.ahead_pieces;
+        v[u] = p.ahead[((size_t)die + 8 * c) * p.ahead_pieces + (t - c * p.ahead_pieces)];
       }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) seen |= v[u].x;
     }
     asm volatile("" ::"v"(seen));  // the loads stay although nobody wants the values
     return;

@@ -390,16 +390,22 @@ __global__ __launch_bounds__(256) void sum_partials_norm_kernel(SumNormArgs q) {
     // which reads chunk j of `ahead` (`ahead_pieces` pieces each): this block reads chunks of its
     // own die, so that they lie in the L2 where they will be asked for.
     const int die = blockIdx.x & 7, rank = (m - q.M) >> 3, per_die = max(1, (int)(gridDim.x - q.M) >> 3);
+    // the die's chunks (die, die + 8, ...) laid end to end and cut into equal shares, one a block
+    const size_t mine = die < q.ahead_chunks ? (size_t)((q.ahead_chunks - die + 7) / 8) * q.ahead_pieces : 0;
+    const size_t share = (mine + per_die - 1) / per_die;
+    const size_t lo = (size_t)rank * share, hi = min(lo + share, mine);
     unsigned int seen = 0u;
-    for (int j = die + 8 * rank; j < q.ahead_chunks; j += 8 * per_die) {
-      const uint4* src = q.ahead + (size_t)j * q.ahead_pieces;
-      for (size_t i0 = tid; i0 < q.ahead_pieces; i0 += 8 * 256) {
-        uint4 v[8];
+    // (sixteen loads a thread in flight: a share of some 60 KB in one trip)
+    for (size_t i0 = lo + tid; i0 < hi; i0 += 16 * 256) {
+      uint4 v[16];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = src[min(i0 + u * 256, q.ahead_pieces - 1)];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) seen |= v[u].x;
+      for (int u = 0; u < 16; ++u) {
+        const size_t t = min(i0 + u * 256, hi - 1);
+        const size_t c = t / q.ahead_pieces;
+        v[u] = q.ahead[((size_t)die + 8 * c) * q.ahead_pieces + (t - c * q.ahead_pieces)];
       }
+#pragma unroll
+      for (int u = 0; u < 16; ++u) seen |= v[u].x;
     }
     asm volatile("" ::"v"(seen));  // the loads stay although nobody wants the values
     return;
