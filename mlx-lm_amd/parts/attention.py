@@ -125,10 +125,11 @@ class CausalSelfAttention(Mixer):
                 part_ml = ctx.scratch((n * 2,), "float32")
             if fast:
                 # CUs without a row read the weights that come after this mixer's own (the block
-                # says which), as many chunks as they manage while the rows' blocks run
+                # says which), as many chunks as they manage while the rows' blocks run; where fewer
+                # than half the CUs are idle the reading slows the rows' blocks by more than it gains
                 ahead, chunks = getattr(ctx, "read_ahead", None), 0
                 idle = 256 - plan.n_rows * self.n_heads * n_splits
-                if (ahead is not None and idle >= 8 and plan.n_tiles == 0 and plan.n_rows == q.shape[0]
+                if (ahead is not None and idle >= 128 and plan.n_tiles == 0 and plan.n_rows == q.shape[0]
                         and kernels.read_ahead_pays(ahead, plan.n_rows, with_norm=True)):
                     chunks = idle * READ_AHEAD_BYTES_PER_CU // ahead.chunk_bytes
                 else:
