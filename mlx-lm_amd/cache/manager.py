@@ -43,6 +43,7 @@ class RequestCache:
     reserved: int = 0  # tokens that have pages (>= length)
     blocks: List[List[int]] = field(default_factory=list)  # per group: page of each block or -1
     serial: int = 0  # unique over the manager's life, unlike the id
+    version: int = 0  # counts the edits of ``blocks``: who keeps a copy of a table compares it
 
 
 class _Group:
@@ -164,8 +165,29 @@ class CacheManager:
                 )
             taken.append((gi, pages))
         for gi, pages in taken:
-            rc.blocks[gi].extend(pages)
+            if pages:
+                rc.blocks[gi].extend(pages)
+                rc.version += 1
         rc.reserved = max(rc.reserved, rc.length + n_new)
+        return rc
+
+    def mark(self, request_id):
+        """What ``rollback`` needs to undo the reservations that follow."""
+        rc = self.requests[request_id]
+        return (rc.reserved, [len(b) for b in rc.blocks])
+
+    def rollback(self, request_id, mark):
+        """Give back the pages taken since ``mark`` (a step that could not get all its pages):
+        what the request held before, filled or only reserved, stays its own."""
+        rc = self.requests[request_id]
+        reserved, n_blocks = mark
+        for gi, g in enumerate(self.groups):
+            extra = [p for p in rc.blocks[gi][n_blocks[gi]:] if p >= 0]
+            if len(rc.blocks[gi]) > n_blocks[gi]:
+                g.pool.give_back(extra)
+                del rc.blocks[gi][n_blocks[gi]:]
+                rc.version += 1
+        rc.reserved = reserved
         return rc
 
     def commit(self, request_id, n_new):
@@ -184,6 +206,7 @@ class CacheManager:
                 if rc.blocks[gi][b] >= 0:
                     g.pool.give_back([rc.blocks[gi][b]])
                     rc.blocks[gi][b] = -1
+                    rc.version += 1
         return rc
 
     def truncate(self, request_id, new_length):
@@ -210,6 +233,7 @@ class CacheManager:
             tail = [p for p in rc.blocks[gi][keep:] if p >= 0]
             g.pool.give_back(tail)
             del rc.blocks[gi][keep:]
+        rc.version += 1
         rc.length = new_length
         rc.reserved = min(rc.reserved, keep * self.page_size)
         rc.reserved = max(rc.reserved, rc.length)

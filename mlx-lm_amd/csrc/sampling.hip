@@ -473,7 +473,7 @@ __global__ __launch_bounds__(256) void penalties_kernel(float* logits, int ld, c
                                                         const int* hist, const float* rep,
                                                         const int* rep_ctx, const float* pres,
                                                         const int* pres_ctx, const float* freq,
-                                                        const int* freq_ctx) {
+                                                        const int* freq_ctx, int vocab) {
   const int r = blockIdx.x;
   float* x = logits + (size_t)r * ld;
   const int b = offsets[r], e = offsets[r + 1];
@@ -482,6 +482,7 @@ __global__ __launch_bounds__(256) void penalties_kernel(float* logits, int ld, c
   const int freq_b = max(b, e - freq_ctx[r]);
   for (int j = b + threadIdx.x; j < e; j += blockDim.x) {
     const int t = hist[j];
+    if (t < 0 || t >= vocab) continue;  // (the host refuses such a history; this keeps the write inside the row)
     bool first = true;
     for (int k = b; k < j; ++k)
       if (hist[k] == t) first = false;
@@ -542,12 +543,13 @@ extern "C" int apply_logit_bias(float* logits, int ld, int n_rows, const int* of
 extern "C" int apply_penalties(float* logits, int ld, int n_rows, const int* offsets,
                                const int* hist, const float* rep, const int* rep_ctx,
                                const float* pres, const int* pres_ctx, const float* freq,
-                               const int* freq_ctx, hipStream_t stream) {
+                               const int* freq_ctx, int vocab, hipStream_t stream) {
   if (n_rows <= 0) return 0;
+  if (vocab <= 0) FAIL("apply_penalties: vocabulary of %d", vocab);
   if (!logits || !offsets || !hist || !rep || !rep_ctx || !pres || !pres_ctx || !freq || !freq_ctx)
     FAIL("apply_penalties: null pointer");
   hipLaunchKernelGGL(penalties_kernel, dim3(n_rows), dim3(256), 0, stream, logits, ld, offsets, hist,
-                     rep, rep_ctx, pres, pres_ctx, freq, freq_ctx);
+                     rep, rep_ctx, pres, pres_ctx, freq, freq_ctx, vocab);
   CHECK_LAUNCH("apply_penalties");
   return 0;
 }

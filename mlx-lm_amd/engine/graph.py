@@ -119,7 +119,7 @@ class DecodeGraph:
             h[off[4] + r] = rc.state_slot
             for gi in range(len(cm.groups)):
                 blocks = rc.blocks[gi]
-                key = (rc.serial, len(blocks))
+                key = (rc.serial, rc.version)  # (every edit of a table counts its version up)
                 if self._row_keys[gi][r] != key:
                     base = off[7 + gi] + r * self.max_blocks
                     # pages a window has let go (-1) are never read; page 0 keeps the entry valid
@@ -150,6 +150,10 @@ class DecodeGraph:
             self.graph = graph
             self._keep = (eng.scratch.buffer, eng._logits, eng.fed_src)
             self._copied = torch.cuda.Event()
+            # The step has run (eagerly, above) and recording runs nothing: replaying now would run
+            # it a second time, and a mixer that keeps state would take the step's tokens twice.
+            self._copied.record()
+            return self.logits
         self.graph.replay()
         self._copied.record()
         return self.logits
@@ -192,5 +196,6 @@ class StepGraph:
                 return eng.decoder.forward(ctx)
             self.graph = graph
             self._keep = (eng.scratch.buffer, eng._logits)
+            return self.logits  # (the eager run above was the step; a replay would run it again)
         self.graph.replay()
         return self.logits

@@ -166,6 +166,11 @@ class Scheduler:
             raise ValueError(f"request id {request.request_id!r} is in use")
         request.order = self._order
         self._order += 1
+        if request.max_tokens == 0:
+            # nothing to generate: finished as it comes, with no step run and no token sampled
+            # (``generate_step`` yields nothing for it, mlx_lm/generate.py:448-461)
+            request.finish_reason = "length"
+            return request
         request.live = True
         self.waiting.append(request)
         return request

@@ -118,6 +118,24 @@ class Engine:
     def context_len(self, request_id):
         return self.cache.requests[request_id].length
 
+    def truncate(self, request_id, new_length):
+        """Forget a request's tokens from ``new_length`` on; the next step goes on from there.
+
+        ``trim_prompt_cache`` of the reference (mlx_lm/models/cache.py:91-107,378-381) counts
+        the tokens to drop; see ``trim``.  Pages beyond the new end are given back at once.  A
+        mixer that keeps state of fixed size cannot go back (mlx_lm/models/cache.py:146-147):
+        a model with one refuses.
+        """
+        if self.cache.state_needs:
+            raise ValueError("a model whose mixers keep per-request state cannot be trimmed")
+        return self.cache.truncate(request_id, new_length).length
+
+    def trim(self, request_id, n_tokens):
+        """Drop the last ``n_tokens`` tokens of a request (at most all); returns how many went."""
+        n = max(0, min(int(n_tokens), self.context_len(request_id)))
+        self.truncate(request_id, self.context_len(request_id) - n)
+        return n
+
     # -- the step --------------------------------------------------------------
 
     def _check(self, entries):
@@ -172,15 +190,16 @@ class Engine:
             self.fed_src[: fed.numel()].copy_(fed.reshape(-1), non_blocking=True)
         cm = self.cache
         # pages first: all or nothing for the whole step
-        done = []
+        marks = []
         try:
             for e in entries:
+                marks.append((e.request_id, cm.mark(e.request_id)))
                 cm.reserve(e.request_id, len(e.tokens))
-                done.append(e)
         except Exception:
-            for e in done:
-                rc = cm.requests[e.request_id]
-                cm.truncate(e.request_id, rc.length)  # gives back pages beyond what is stored
+            # only what this step took goes back: pages that a request held before (its whole
+            # prompt's, taken at admission) stay its own
+            for rid, mark in marks:
+                cm.rollback(rid, mark)
             raise
 
         if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):

@@ -20,7 +20,7 @@ from . import sample_utils
 from .engine.scheduler import Request, Scheduler
 from .engine.step import Engine
 from .sample_utils import Sampler, make_logits_processors, make_sampler
-from .sampling import PendingRead, apply_processors, sample_batch
+from .sampling import PendingRead, SamplerBuffers, apply_processors, sample_batch
 
 DEFAULT_PROMPT = "hello"
 DEFAULT_MAX_TOKENS = 100
@@ -86,8 +86,13 @@ class _SampleFn:
     ``logits processors -> logprobs = logits - logsumexp -> sampler`` as in
     mlx_lm/generate.py:400-412,1417-1445, for all rows in one launch each.
     ``launch`` queues the work and returns at once; ``finish`` waits for the
-    tokens; calling the object does both.
+    tokens; calling the object does both.  The arrays that tokens pass through
+    are this object's own: other generators' sampling calls, however many come
+    in between, leave a call's tokens alone until its scheduler has fed them on.
     """
+
+    def __init__(self):
+        self.buffers = SamplerBuffers()
 
     def launch(self, logits, requests):
         if any(r.logits_processors for r in requests):
@@ -97,8 +102,9 @@ class _SampleFn:
         custom = [r for r in requests if r.sampler is not None and not isinstance(r.sampler, Sampler)]
         want = bool(custom) or any(r.want_logprobs for r in requests)
         out = sample_batch(logits, samplers, [r.seed for r in requests],
-                           [len(r.generated) for r in requests], want_logprobs=want)
-        return SampleJob(list(requests), out[0], PendingRead(out[0], out[1]), out[2] if want else None, custom)
+                           [len(r.generated) for r in requests], want_logprobs=want, buffers=self.buffers)
+        read = PendingRead(out[0], out[1], buffers=self.buffers)
+        return SampleJob(list(requests), out[0], read, out[2] if want else None, custom)
 
     def finish(self, job):
         tokens, token_lp = job.read.wait()
@@ -444,7 +450,8 @@ class BatchGenerator:
                 seed=(seeds[i] if seeds else self.seed + uid),
                 want_logprobs=self.want_logprobs)
             self.scheduler.add(req)
-            self._requests[uid] = req
+            if req.finish_reason is None:  # (a request for no tokens at all is over already)
+                self._requests[uid] = req
             uids.append(uid)
         return uids
 

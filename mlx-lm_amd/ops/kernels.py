@@ -703,5 +703,5 @@ def apply_penalties(logits, offsets, hist, rep, rep_ctx, pres, pres_ctx, freq, f
         t.numel() >= n or _fail(f"apply_penalties: {name} shorter than the rows")
     rc = lib.apply_penalties(_ptr(logits), _c_int(ld), _c_int(n), _ptr(offsets), _ptr(hist),
                              _ptr(rep), _ptr(rep_ctx), _ptr(pres), _ptr(pres_ctx), _ptr(freq),
-                             _ptr(freq_ctx), _stream())
+                             _ptr(freq_ctx), _c_int(logits.shape[1]), _stream())
     build.check(lib, rc, "apply_penalties")

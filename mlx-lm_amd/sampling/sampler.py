@@ -54,8 +54,11 @@ def apply_processors(logits, processors, histories):
                 custom.append((r, p))
         bias_off.append(len(bias_idx))
         if span > 0:
-            tail = list(histories[r])[-span:]
-            hist.extend(int(t) for t in tail)
+            tail = [int(t) for t in list(histories[r])[-span:]]
+            for t in tail:
+                if not (0 <= t < logits.shape[1]):
+                    raise ValueError(f"a penalty's token history names token {t}, the vocabulary has {logits.shape[1]}")
+            hist.extend(tail)
             any_pen = any_pen or bool(tail)
         hist_off.append(len(hist))
     if any_bias:
@@ -100,10 +103,21 @@ class _ParamRing:
         return slot
 
 
-_RING = _ParamRing()
+class SamplerBuffers:
+    """The arrays that sampling calls and the reads of their tokens go through, reused in turn.
+
+    Whoever keeps a call's tokens on the device until its *next* call (a scheduler feeds them
+    into the step it launches meanwhile) owns one of these: with at most two calls in flight and
+    four arrays in turn, nothing is written again while it is still wanted.  Callers that share
+    no owner get arrays of their own for every call.
+    """
+
+    def __init__(self, depth=4):
+        self.params = _ParamRing(depth)
+        self.reads = _ReadRing(depth)
 
 
-def sample_batch(logits, samplers, seeds, counters, want_logprobs=False):
+def sample_batch(logits, samplers, seeds, counters, want_logprobs=False, buffers=None):
     """One token for each row of float32 ``logits [R, V]``.
 
     ``samplers[r]`` is the row's ``Sampler``; ``seeds[r]`` and ``counters[r]``
@@ -111,7 +125,9 @@ def sample_batch(logits, samplers, seeds, counters, want_logprobs=False):
     it.  Returns ``(tokens, token_logprobs)`` as device tensors and, with
     ``want_logprobs``, the normalised log-probabilities ``[R, V]`` as a third.
     ``logits - logsumexp(logits)`` then the sampler, as in
-    mlx_lm/generate.py:411-412.  Nothing here waits for the GPU.
+    mlx_lm/generate.py:411-412.  Nothing here waits for the GPU.  The returned tokens lie in
+    an array of ``buffers`` (a ``SamplerBuffers``) that its fourth call from now writes again;
+    without ``buffers`` they lie in arrays made for this call.
     """
     import numpy as np
 
@@ -124,7 +140,7 @@ def sample_batch(logits, samplers, seeds, counters, want_logprobs=False):
             if special and special != list(s.xtc_special_tokens):
                 raise ValueError("rows of one batch must share their xtc_special_tokens")
             special = list(s.xtc_special_tokens)
-    slot = _RING.get(R, dev)
+    slot = (buffers.params if buffers is not None else _ParamRing(1)).get(R, dev)
     host, device_buf = slot[0], slot[1]
     h = host.numpy()
     n = R * _ParamRing.FIELDS
@@ -184,24 +200,22 @@ class _ReadRing:
         return b
 
 
-_READ_RING = _ReadRing()
-
-
 class PendingRead:
     """Tokens and log-probabilities on their way to the host.
 
     ``start`` queues the copy behind the sampling kernel and returns at once;
     ``wait`` blocks until that copy (and nothing queued after it) is done, so a
-    step launched in between keeps the GPU busy while the host reads.  Up to
-    four reads may be pending.
+    step launched in between keeps the GPU busy while the host reads.  With
+    ``buffers`` (a ``SamplerBuffers``) the host array is one of its four, taken in
+    turn; without, one made for this read.
     """
 
-    def __init__(self, tokens, token_logprob):
+    def __init__(self, tokens, token_logprob, buffers=None):
         R = tokens.numel()
         self.rows = R
         adjacent = (token_logprob.data_ptr() == tokens.data_ptr() + 4 * R and tokens.dtype == torch.int32
                     and tokens.is_contiguous() and token_logprob.is_contiguous())
-        self.host = _READ_RING.get(2 * R)
+        self.host = (buffers.reads if buffers is not None else _ReadRing(1)).get(2 * R)
         if adjacent:
             self.host[: 2 * R].copy_(torch.as_strided(tokens, (2 * R,), (1,)), non_blocking=True)
         else:

@@ -71,3 +71,60 @@ def write_trace(path, steps):
     with open(path, "w") as fh:
         for s in steps:
             fh.write(json.dumps(s) + "\n")
+
+
+def cuts_changing(n):
+    sizes, out, i = [7, 2, 64, 3, 16, 2, 33, 5], [], 0
+    while n > 0:
+        s = min(sizes[i % len(sizes)], n)
+        if n - s == 1:  # never leave a single token for the end: portions go down to two
+            s += 1
+        out.append(s)
+        n -= s
+        i += 1
+    return out
+
+
+def mixed_trace(config, seed, lengths, n_live=4):
+    """Steps that mix portions of some requests with decoded tokens of others.
+
+    Requests start when a place is free, run a few portions of changing size,
+    then go on token by token; ends of requests give pages back for the next.
+    """
+    g = torch.Generator().manual_seed(seed)
+    tokens = {f"r{i}": random_tokens(n, config["vocab_size"], seed * 100 + i) for i, n in enumerate(lengths)}
+    waiting = list(tokens)
+    live, fed, steps, step_no = [], {}, [], 0
+    while waiting or live:
+        while waiting and len(live) < n_live:
+            rid = waiting.pop(0)
+            live.append(rid)
+            fed[rid] = 0
+        entries, ended = [], []
+        for rid in list(live):
+            left = len(tokens[rid]) - fed[rid]
+            if torch.rand((), generator=g).item() < 0.15 and len(live) > 1:
+                continue  # left out of this step, goes on later
+            prompt_part = int(len(tokens[rid]) * 0.6)
+            if fed[rid] < prompt_part:
+                n = int(torch.randint(2, 40, (), generator=g))
+                n = min(n, prompt_part - fed[rid])
+                if prompt_part - fed[rid] - n == 1:
+                    n += 1
+            else:
+                n = 1
+            n = min(n, left)
+            part = tokens[rid][fed[rid] : fed[rid] + n]
+            entries.append({"id": rid, "tokens": part, "want": list(range(n))})
+            fed[rid] += n
+            if fed[rid] == len(tokens[rid]):
+                ended.append(rid)
+                live.remove(rid)
+        if entries:
+            steps.append({"step": step_no, "entries": entries, "end": ended})
+            step_no += 1
+    return tokens, steps
+
+
+def held(lengths, n_live):
+    return sum(sorted(((n + 63) // 64 * 64 for n in lengths), reverse=True)[:n_live])

@@ -157,3 +157,48 @@ def test_random_orders_keep_every_page_accounted(seed, window):
     cm.release_all()
     assert all(g.pool.n_free == 12 for g in cm.groups)
     cm.check()
+
+
+def test_every_edit_of_a_table_counts_its_version_up():
+    """Whoever keeps a copy of a request's block table compares versions: a table that was cut
+    and has grown back to its old number of pages is not the table it was."""
+    cm = _manager()
+    rc = cm.add("a")
+    cm.reserve("a", 50)
+    cm.commit("a", 50)
+    v0, pages0 = rc.version, list(rc.blocks[0])
+    cm.reserve("a", 1)  # no new page: the table is the same
+    assert rc.version == v0
+    cm.truncate("a", 30)
+    v1 = rc.version
+    assert v1 > v0
+    other = cm.add("b")
+    cm.reserve("b", 16)  # takes the page that "a" gave back last (the pool is a stack)
+    cm.reserve("a", 34)
+    assert len(rc.blocks[0]) == len(pages0) and rc.blocks[0] != pages0 and rc.version > v1
+    assert set(other.blocks[0]) & set(pages0)
+    cm.check()
+
+
+def test_a_window_passing_a_page_counts_the_version_up():
+    cm = _manager(window=24)
+    rc = cm.add("a")
+    cm.reserve("a", 40)
+    v = rc.version
+    cm.commit("a", 40)  # the first page is out of every later query's reach
+    assert rc.blocks[1][0] == -1 and rc.blocks[0][0] >= 0 and rc.version > v
+
+
+def test_rollback_gives_back_what_was_taken_since_the_mark_and_nothing_else():
+    cm = _manager()
+    rc = cm.add("a")
+    cm.reserve("a", 60)  # a whole prompt's pages, taken at admission
+    cm.commit("a", 10)
+    mark = cm.mark("a")
+    held = list(rc.blocks[0])
+    cm.reserve("a", 70)  # one page more
+    assert len(rc.blocks[0]) == len(held) + 1
+    cm.rollback("a", mark)
+    assert rc.blocks[0] == held and rc.reserved == 60 and rc.length == 10
+    assert cm.free_pages() == 8 - len(held)
+    cm.check()

@@ -66,18 +66,6 @@ def _run(engine, rid, tokens, cuts, want_all=True):
     return torch.cat(rows)
 
 
-def _cuts_changing(n):
-    sizes, out, i = [7, 2, 64, 3, 16, 2, 33, 5], [], 0
-    while n > 0:
-        s = min(sizes[i % len(sizes)], n)
-        if n - s == 1:  # never leave a single token for the end: portions go down to two
-            s += 1
-        out.append(s)
-        n -= s
-        i += 1
-    return out
-
-
 CASES = [("A", 0.0, 100), ("B", 0.0, 200), ("B", 8.0, 250), ("C", 8.0, 300), ("A", 8.0, 128)]
 
 
@@ -92,7 +80,7 @@ def test_whole_decoded_and_portions(folders, dtype, name, sharp, n):
     _close(whole, want, dtype, "whole")
     decoded = _run(eng, "decoded", tokens, [n - 32] + [1] * 32)
     _close(decoded, want, dtype, "last 32 one by one")
-    portions = _run(eng, "portions", tokens, _cuts_changing(n))
+    portions = _run(eng, "portions", tokens, helpers.cuts_changing(n))
     _close(portions, want, dtype, "portions of changing size")
     eng.cache.check()
     assert eng.cache.free_pages() == eng.cache.n_pages
@@ -151,51 +139,6 @@ def test_thousands_of_keys_split_over_blocks(tmp_path, monkeypatch, dtype, use_g
     _close(torch.cat(rows), want[n_prompt - 1 :], dtype, "decoded after 3,300 tokens")
 
 
-def _mixed_trace(config, seed, lengths, n_live=4):
-    """Steps that mix portions of some requests with decoded tokens of others.
-
-    Requests start when a place is free, run a few portions of changing size,
-    then go on token by token; ends of requests give pages back for the next.
-    """
-    g = torch.Generator().manual_seed(seed)
-    tokens = {f"r{i}": helpers.random_tokens(n, config["vocab_size"], seed * 100 + i) for i, n in enumerate(lengths)}
-    waiting = list(tokens)
-    live, fed, steps, step_no = [], {}, [], 0
-    while waiting or live:
-        while waiting and len(live) < n_live:
-            rid = waiting.pop(0)
-            live.append(rid)
-            fed[rid] = 0
-        entries, ended = [], []
-        for rid in list(live):
-            left = len(tokens[rid]) - fed[rid]
-            if torch.rand((), generator=g).item() < 0.15 and len(live) > 1:
-                continue  # left out of this step, goes on later
-            prompt_part = int(len(tokens[rid]) * 0.6)
-            if fed[rid] < prompt_part:
-                n = int(torch.randint(2, 40, (), generator=g))
-                n = min(n, prompt_part - fed[rid])
-                if prompt_part - fed[rid] - n == 1:
-                    n += 1
-            else:
-                n = 1
-            n = min(n, left)
-            part = tokens[rid][fed[rid] : fed[rid] + n]
-            entries.append({"id": rid, "tokens": part, "want": list(range(n))})
-            fed[rid] += n
-            if fed[rid] == len(tokens[rid]):
-                ended.append(rid)
-                live.remove(rid)
-        if entries:
-            steps.append({"step": step_no, "entries": entries, "end": ended})
-            step_no += 1
-    return tokens, steps
-
-
-def _held(lengths, n_live):
-    return sum(sorted(((n + 63) // 64 * 64 for n in lengths), reverse=True)[:n_live])
-
-
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name,sharp", [("A", 8.0), ("B", 8.0), ("C", 0.0)])
 def test_mixed_batches_with_few_pages(folders, dtype, name, sharp):
@@ -204,8 +147,8 @@ def test_mixed_batches_with_few_pages(folders, dtype, name, sharp):
     folder, config, weights = folders[(name, sharp)]
     P = config["n_positions"]
     lengths = [min(P, n) for n in (100, 37, 128, 64, 90, 17, 120, 75)]
-    tokens, steps = _mixed_trace(config, seed=3, lengths=lengths)
-    max_tokens = _held(lengths, 4)
+    tokens, steps = helpers.mixed_trace(config, seed=3, lengths=lengths)
+    max_tokens = helpers.held(lengths, 4)
     eng = _engine(folder, dtype, n_pages=max_tokens // 16)
     got = {rid: [] for rid in tokens}
     used_pages = set()
@@ -257,9 +200,9 @@ def test_split_sums_in_the_engine(folders, monkeypatch, name, sharp, use_graphs)
     folder, config, weights = folders[(name, sharp)]
     P = config["n_positions"]
     lengths = [min(P, n) for n in (100, 37, 128, 64, 90, 17)]
-    tokens, steps = _mixed_trace(config, seed=5, lengths=lengths)
+    tokens, steps = helpers.mixed_trace(config, seed=5, lengths=lengths)
     model, _ = load_model(folder, dtype="bfloat16")
-    eng = Engine(model, dtype="bfloat16", page_size=16, n_pages=_held(lengths, 4) // 16, max_requests=8,
+    eng = Engine(model, dtype="bfloat16", page_size=16, n_pages=helpers.held(lengths, 4) // 16, max_requests=8,
                  use_graphs=use_graphs)
     got = {rid: [] for rid in tokens}
     for s in steps:
@@ -321,7 +264,7 @@ def test_trace_run_program(folders, tmp_path, dtype):
     """bin/trace_run as a user calls it: whole, decoded and mixed, from files."""
     folder, config, weights = folders[("B", 8.0)]
     lengths = [90, 40, 130, 64, 70]
-    tokens, steps = _mixed_trace(config, seed=11, lengths=lengths, n_live=3)
+    tokens, steps = helpers.mixed_trace(config, seed=11, lengths=lengths, n_live=3)
     # a request whole, and the same one with its last 32 tokens one by one
     whole = helpers.random_tokens(120, config["vocab_size"], seed=5)
     base = len(steps)
@@ -336,7 +279,7 @@ def test_trace_run_program(folders, tmp_path, dtype):
     with open(trace) as fh:
         proc = subprocess.run(
             [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
-             "--out", str(out), "--max-tokens", str(_held(lengths + [128], 3))],
+             "--out", str(out), "--max-tokens", str(helpers.held(lengths + [128], 3))],
             stdin=fh, capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert [l for l in proc.stdout.split("\n") if l.startswith("done")] == [f"done {s['step']}" for s in steps]
@@ -540,3 +483,52 @@ def test_tokens_fed_on_the_device(folders, dtype, use_graphs):
     want = plain.greedy_generate(helpers.round_matrices_to_bf16(weights) if dtype == "bfloat16" else weights,
                                  config, prompts["c"], 6)
     assert tokens_host[:6, 2].tolist() == want
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("use_graphs", [True, False])
+def test_trim_and_regenerate_across_a_page_edge(folders, dtype, use_graphs):
+    """Decode, trim three tokens back over a page's edge, let another request take the page that
+    went back, decode the same tokens again: same logits as before and as the plain implementation's
+    (the reference's test of trimming, tests/test_prompt_cache.py:266-294, through this engine).
+    Under recorded decode steps the request's row of the block table must be copied again: the
+    table has its old length but another page, and the old page is the other request's now."""
+    from mlx_lm_amd.engine import Engine, StepEntry
+    from mlx_lm_amd.utils import load_model
+
+    folder, config, weights = folders[("B", 8.0)]
+    V = config["vocab_size"]
+    model, _ = load_model(folder, dtype=dtype)
+    eng = Engine(model, dtype=dtype, page_size=16, n_pages=8, max_requests=4, use_graphs=use_graphs)
+    a = helpers.random_tokens(56, V, seed=301)
+    b = helpers.random_tokens(40, V, seed=302)
+    want_a, want_b = (_plain_logits(weights, config, t, dtype) for t in (a, b))
+
+    eng.add_request("a")
+    eng.step([StepEntry("a", a[:44], [])])
+    first = [eng.step([StepEntry("a", [a[i]], [0])]).clone() for i in range(44, 50)]  # crosses 48
+    _close(torch.cat(first), want_a[44:50], dtype, "before the trim")
+    page_beyond_edge = eng.cache.requests["a"].blocks[0][3]
+    assert eng.trim("a", 3) == 3 and eng.context_len("a") == 47
+    assert len(eng.cache.requests["a"].blocks[0]) == 3
+    # another request takes the page that went back (the pool hands out the last one returned)
+    eng.add_request("b")
+    got_b = [eng.step([StepEntry("b", b[:10], list(range(10)))]).clone()]
+    assert eng.cache.requests["b"].blocks[0] == [page_beyond_edge]
+    # the same tokens again, decoded one by one: position 48 needs a page, and gets another one
+    again = [eng.step([StepEntry("a", [a[i]], [0])]).clone() for i in range(47, 56)]
+    assert eng.cache.requests["a"].blocks[0][3] != page_beyond_edge
+    _close(torch.cat(again), want_a[47:56], dtype, "after the trim")
+    for x, y in zip(first[3:], again):  # positions 47, 48, 49 were computed before the trim too
+        assert torch.equal(x, y)
+    # and the other request's page was left alone
+    got_b += [eng.step([StepEntry("b", [b[i]], [0])]).clone() for i in range(10, 40)]
+    _close(torch.cat(got_b), want_b, dtype, "the request that took the page")
+    if use_graphs:
+        assert eng._graphs[1].graph is not None
+    # trimming more than there is drops everything (tests/test_prompt_cache.py:259-264)
+    assert eng.trim("a", 1000) == 56 and eng.context_len("a") == 0
+    eng.end_request("a")
+    eng.end_request("b")
+    eng.cache.check()
+    assert eng.cache.free_pages() == 8

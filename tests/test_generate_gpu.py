@@ -212,3 +212,49 @@ def test_command_line(tiny):
         capture_output=True, text=True, env=env, timeout=300)
     assert out.returncode == 0, out.stderr[-2000:]
     assert "Prompt: 5 tokens" in out.stdout and "Generation: 6 tokens" in out.stdout and "Peak memory" in out.stdout
+
+
+def test_many_interleaved_generators_keep_their_own_tokens(model_b, tiny):
+    """Seven generators taken in turn, a token from each: every one's tokens (which stay on
+    the device from its sampling call to its next step) equal those of the same request alone,
+    however many other generators' sampling calls come in between."""
+    from mlx_lm_amd import generate_step
+    from mlx_lm_amd.sample_utils import make_sampler
+
+    V = tiny["B"][1]["vocab_size"]
+    sampler = make_sampler(temp=0.9)
+    prompts = [helpers.random_tokens(5 + 3 * i, V, seed=400 + i) for i in range(7)]
+    alone = [[t for t, _ in generate_step(p, model_b, max_tokens=10, sampler=sampler, seed=50 + i)]
+             for i, p in enumerate(prompts)]
+    assert len({tuple(a) for a in alone}) == 7  # the requests do differ
+    gens = [generate_step(p, model_b, max_tokens=10, sampler=sampler, seed=50 + i) for i, p in enumerate(prompts)]
+    together = [[] for _ in gens]
+    for _ in range(10):
+        for i, g in enumerate(gens):
+            together[i].append(next(g)[0])
+    for g in gens:
+        g.close()
+    assert together == alone
+
+
+def test_no_tokens_asked_for_none_made(model_b, tiny):
+    """``max_tokens=0`` (mlx_lm/generate.py:448-461): nothing is yielded, and in a batch the
+    request ends at once beside the others."""
+    from mlx_lm_amd import batch_generate, generate_step
+
+    V = tiny["B"][1]["vocab_size"]
+    p = helpers.random_tokens(9, V, seed=3)
+    assert list(generate_step(p, model_b, max_tokens=0)) == []
+    out = batch_generate(model_b, None, [p, p], max_tokens=[0, 3], return_token_ids=True)
+    assert out.token_ids[0] == [] and len(out.token_ids[1]) == 3
+
+
+def test_penalty_histories_are_checked_against_the_vocabulary(model_b, tiny):
+    from mlx_lm_amd.sample_utils import make_logits_processors
+
+    V = tiny["B"][1]["vocab_size"]
+    logits = torch.zeros(1, V, device="cuda")
+    (proc,) = make_logits_processors(repetition_penalty=1.3)
+    with pytest.raises(ValueError, match="vocabulary"):
+        proc(torch.tensor([1, V + 5]), logits)
+    proc(torch.tensor([1, V - 1]), logits)

@@ -444,3 +444,116 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path, dtype):
     eng.end_request("a")
     eng.end_request("b")
     assert eng.cache.free_pages() == 14
+
+
+# ---------------------------------------------------------------------------
+# a mixer that keeps state and launches kernels only: its steps are recorded and replayed
+
+
+def _register_running_sum():
+    from mlx_lm_amd.config import BaseModelArgs, LayerSpec, ModelPlan, PartSpec, RunEntry, StateNeed, register_model
+    from mlx_lm_amd.parts import DecoderModel, Mixer, register_mixer
+
+    class RunningSum(Mixer):
+        """``s += sum of the portion's rows``; every row of the portion adds the new ``s`` to the
+        residual.  Device-side indexing only (no value comes to the host), so a step with it can
+        be recorded; a step that ran twice would add its rows to the state twice."""
+
+        graph_safe = True
+
+        def __init__(self, width, prefix=""):
+            super().__init__(prefix)
+            self.width = width
+
+        def cache_need(self):
+            return StateNeed((self.width,), "float32")
+
+        def forward(self, ctx, x, residual, cache, writes_cache=True):
+            slots = ctx.slot_ids.long()[ctx.token_req.long()]
+            cache.state.index_add_(0, slots, x.float())
+            residual += cache.state[slots]
+
+    register_mixer("toy_running_sum", RunningSum)
+
+    @dataclass
+    class SumArgs(BaseModelArgs):
+        model_type: str
+        width: int
+        vocab: int
+        max_len: int
+        inner: int
+
+    class SumModel:
+        def __init__(self, args):
+            self.args, self.model_type = args, args.model_type
+            self.decoder = DecoderModel(self.plan(args))
+
+        @property
+        def layers(self):
+            return self.decoder.layers
+
+        @staticmethod
+        def plan(a):
+            def norm(p):
+                return PartSpec("layernorm", {"width": a.width, "eps": 1e-5}, p)
+
+            layers = [
+                LayerSpec("pre_norm", norm("l0.n1."), PartSpec("toy_running_sum", {"width": a.width}, "l0.mix."),
+                          norm("l0.n2."), PartSpec("gelu_mlp", {"width": a.width, "inner": a.inner}, "l0.ff.")),
+                LayerSpec("pre_norm", norm("l1.n1."),
+                          PartSpec("attention", {"width": a.width, "n_heads": 2, "head_dim": a.width // 2}, "l1.mix."),
+                          norm("l1.n2."), PartSpec("gelu_mlp", {"width": a.width, "inner": a.inner}, "l1.ff.")),
+            ]
+            return ModelPlan(
+                width=a.width, vocab_size=a.vocab, max_positions=a.max_len,
+                embedding=PartSpec("token", {"vocab_size": a.vocab, "width": a.width}, "emb."),
+                embedding_positions=None, layers=layers, schedule=[RunEntry(0, 0), RunEntry(1, 1)],
+                final_norm=norm("nf."), head=PartSpec("linear", {"vocab_size": a.vocab, "width": a.width,
+                                                                  "weight_name": "emb.weight"}))
+
+    register_model("toy_sum", SumModel, SumArgs)
+    return SumModel, SumArgs
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_recorded_step_takes_its_tokens_once(tmp_path, dtype):
+    """Steps of a model whose mixer keeps state, replayed from graphs, against the same steps
+    run eagerly, bit for bit: the step that records a graph counts once, like any other."""
+    from safetensors.torch import save_file
+
+    from mlx_lm_amd.engine import Engine, StepEntry
+    from mlx_lm_amd.utils import load_model
+
+    cfg = dict(model_type="toy_sum", width=64, vocab=97, max_len=96, inner=80)
+    SumModel, SumArgs = _register_running_sum()
+    g = torch.Generator().manual_seed(3)
+    tensors = {}
+    for name, spec in SumModel(SumArgs.from_dict(cfg)).decoder.expected_tensors().items():
+        if spec.role == "vector":
+            tensors[name] = (1.0 if name.endswith("weight") else 0.0) + 0.05 * torch.randn(spec.shape, generator=g)
+        else:
+            tensors[name] = 0.1 * torch.randn(spec.shape, generator=g)
+    json.dump(cfg, open(os.path.join(tmp_path, "config.json"), "w"))
+    save_file(tensors, os.path.join(tmp_path, "model.safetensors"))
+    model, _ = load_model(str(tmp_path), dtype=dtype)
+    seqs = {"a": helpers.random_tokens(40, 97, 11), "b": helpers.random_tokens(33, 97, 12)}
+    results, states = {}, {}
+    for use_graphs in (True, False):
+        eng = Engine(model, dtype=dtype, page_size=16, n_pages=8, max_requests=3, use_graphs=use_graphs,
+                     record_prompt_steps=use_graphs)
+        assert eng.use_graphs == use_graphs  # every part launches kernels only
+        out = []
+        for r in seqs:
+            eng.add_request(r)
+        out.append(eng.step([StepEntry("a", seqs["a"][:9], [8]), StepEntry("b", seqs["b"][:2], [1])]).clone())
+        for i in range(24):  # decode steps of both (recorded at the first), then portions of one shape
+            out.append(eng.step([StepEntry("a", [seqs["a"][9 + i]], [0]), StepEntry("b", [seqs["b"][2 + i]], [0])]).clone())
+        for i in range(3):  # (recorded at the third sighting of the shape)
+            out.append(eng.step([StepEntry("a", seqs["a"][33 + 2 * i : 35 + 2 * i], [0, 1])]).clone())
+        if use_graphs:
+            assert eng._graphs[2].graph is not None
+            assert any(sg.graph is not None for sg in eng._step_graphs.values())
+        results[use_graphs] = torch.cat(out)
+        states[use_graphs] = eng.cache.state(0)[[eng.cache.requests[r].state_slot for r in seqs]].clone()
+    assert torch.equal(states[True], states[False])
+    assert torch.equal(results[True], results[False])

@@ -10,7 +10,7 @@ import torch
 
 import helpers
 import plain_gpt2 as plain
-from test_engine_gpu import TOL, _mixed_trace, _plain_logits
+from test_engine_gpu import TOL, _plain_logits
 
 pytestmark = pytest.mark.gpu
 
@@ -43,7 +43,7 @@ def test_random_configuration(tmp_path, seed):
     tensors = helpers.sharpen({k: v.clone() for k, v in load_file(path).items()}, config, 3.0)
     save_file(tensors, path)
     weights = plain.from_checkpoint_layout({k: v.float() for k, v in tensors.items()}, config["n_layer"])
-    tokens, steps = _mixed_trace(config, seed=seed, lengths=lengths)
+    tokens, steps = helpers.mixed_trace(config, seed=seed, lengths=lengths)
     held = sum(sorted(((n + 63) // 64 * 64 for n in lengths), reverse=True)[:4])
     for dtype in ("float32", "bfloat16"):
         model, _ = load_model(folder, dtype=dtype)

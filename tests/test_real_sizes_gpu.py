@@ -1,0 +1,236 @@
+"""The engine at the layer sizes of the published GPT-2 models (random weights): logits against
+the plain implementation and against the same request run whole, the replay program in portions
+of fixed sizes, and continuous batching under load.
+
+Widths, heads, inner sizes, vocabulary and positions are the real ones.  Where a test runs
+fewer layers than the model has, it says so: ``n_layer`` is what runs, ``N_LAYER_FULL`` what
+the model of that name has.  Every test takes seconds on the GPU.
+"""
+
+import json
+import os
+import random
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import plain_gpt2 as plain
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+TOL = {"float32": 2e-5, "bfloat16": 2.5e-2}
+
+
+def _gpt2(n_layer, n_embd, n_head):
+    return dict(model_type="gpt2", n_layer=n_layer, n_embd=n_embd, n_head=n_head, n_inner=4 * n_embd,
+                vocab_size=50257, n_positions=1024, n_ctx=1024, layer_norm_epsilon=1e-5,
+                activation_function="gelu_new")
+
+
+# name: (what the tests run, layers of the full model, seed of the weights)
+N_LAYER_FULL = {"xl": 48, "large": 36, "small": 12}
+SIZES = {
+    "xl": (_gpt2(12, 1600, 25), 2),      # 12 of 48 layers
+    "large": (_gpt2(36, 1280, 20), 4),   # all 36
+    "small": (_gpt2(12, 768, 12), 3),    # all 12
+}
+
+
+@pytest.fixture(scope="module")
+def folder_for(tmp_path_factory):
+    made = {}
+
+    def get(name):
+        if name not in made:
+            from mlx_lm_amd.weights import write_model_folder
+
+            config, seed = SIZES[name]
+            assert config["n_layer"] <= N_LAYER_FULL[name]
+            d = str(tmp_path_factory.mktemp(name))
+            write_model_folder(d, dict(config), seed, "b", dtype="float32")
+            made[name] = d
+        return made[name], SIZES[name][0]
+
+    return get
+
+
+def _plain_weights(folder, config, dtype):
+    from safetensors.torch import load_file
+
+    w = plain.from_checkpoint_layout(
+        {k: v.float() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}, config["n_layer"])
+    return helpers.round_matrices_to_bf16(w) if dtype == "bfloat16" else w
+
+
+def _err(got, want):
+    return (got.double().cpu() - want.double().cpu()).abs().max().item()
+
+
+def _run(engine, rid, tokens, cuts):
+    from mlx_lm_amd.engine import StepEntry
+
+    engine.add_request(rid)
+    rows, i = [], 0
+    for n in cuts:
+        rows.append(engine.step([StepEntry(rid, tokens[i : i + n], list(range(n)))]).cpu())
+        i += n
+    assert i == len(tokens)
+    engine.end_request(rid)
+    return torch.cat(rows)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gpt2_xl_sizes_whole_decoded_portions_and_mixed(folder_for, dtype):
+    """Width 1600, 25 heads of 64, inner 6400, 50,257 tokens, 1,024 positions (12 of 48 layers):
+    one request of 1,024 tokens whole, with its last 32 tokens one by one, and in portions of
+    changing size, against the plain implementation on the first 128 positions and against the
+    whole run everywhere; then four requests mixed with so few pages that they are used again."""
+    from mlx_lm_amd.engine import Engine, StepEntry
+    from mlx_lm_amd.utils import load_model
+
+    folder, config = folder_for("xl")
+    V, n = config["vocab_size"], 1024
+    tokens = helpers.random_tokens(n, V, seed=2)
+    weights = _plain_weights(folder, config, dtype)
+    want = plain.forward(weights, config, tokens[:128])
+    scale = want.abs().max().item()
+    model, _ = load_model(folder, dtype=dtype)
+    eng = Engine(model, dtype=dtype, page_size=16, n_pages=n // 16 + 4, max_requests=4)
+    whole = _run(eng, "whole", tokens, [n])
+    assert _err(whole[:128], want) <= TOL[dtype] * scale, "whole against the plain implementation"
+    scale = whole.abs().max().item()
+    decoded = _run(eng, "decoded", tokens, [n - 32] + [1] * 32)
+    assert _err(decoded, whole) <= TOL[dtype] * scale, "last 32 one by one"
+    portions = _run(eng, "portions", tokens, helpers.cuts_changing(n))
+    assert _err(portions, whole) <= TOL[dtype] * scale, "portions of changing size"
+    assert _err(portions[:128], want) <= TOL[dtype] * want.abs().max().item()
+    eng.cache.check()
+    assert eng.cache.free_pages() == eng.cache.n_pages
+    del eng
+
+    lengths = [300, 130, 210, 64, 170, 90]
+    seqs, steps = helpers.mixed_trace(config, seed=21, lengths=lengths)
+    eng = Engine(model, dtype=dtype, page_size=16, n_pages=helpers.held(lengths, 4) // 16, max_requests=4)
+    assert sum((m + 15) // 16 for m in lengths) > eng.cache.n_pages  # pages are used again
+    got = {rid: [] for rid in seqs}
+    for s in steps:
+        for e in s["entries"]:
+            if not eng.has_request(e["id"]):
+                eng.add_request(e["id"])
+        eng.cache.poison_free_pages()
+        logits = eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]]).cpu()
+        i = 0
+        for e in s["entries"]:
+            got[e["id"]].append(logits[i : i + len(e["want"])])
+            i += len(e["want"])
+        for rid in s["end"]:
+            eng.end_request(rid)
+    eng.cache.check()
+    assert any(len(s["entries"]) == 4 for s in steps)
+    alone = Engine(model, dtype=dtype, page_size=16, n_pages=20, max_requests=2)
+    for rid, toks in seqs.items():
+        ref = _run(alone, rid, toks, [len(toks)])
+        assert _err(torch.cat(got[rid]), ref) <= TOL[dtype] * ref.abs().max().item(), f"mixed, request {rid}"
+        if rid == "r1":
+            w = plain.forward(weights, config, toks)
+            assert _err(ref, w) <= TOL[dtype] * w.abs().max().item(), "a mixed request against the plain implementation"
+
+
+def _replay(folder, dtype, out, steps, max_tokens):
+    text = "".join(json.dumps(s) + "\n" for s in steps)
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+         "--out", str(out), "--max-tokens", str(max_tokens)],
+        input=text, capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.split("\n") if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+    rows = [np.fromfile(os.path.join(out, f"{s['step']}.f32"), dtype="<f4").reshape(-1, 50257) for s in steps]
+    return torch.from_numpy(np.concatenate(rows))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gpt2_large_sizes_replayed_in_portions_of_1_7_64_and_1024(folder_for, tmp_path, dtype):
+    """Width 1280, 20 heads, inner 5120, all 36 layers: a sequence of 1,024 tokens through
+    ``bin/trace_run`` whole and in portions of 64, 7 and 1, logits at every position; all four
+    runs in one call of the program, one request after the other, in a pool of 1,024 tokens."""
+    folder, config = folder_for("large")
+    n = 1024
+    tokens = helpers.random_tokens(n, config["vocab_size"], seed=5)
+    steps = []
+    for chunk in (1024, 64, 7, 1):
+        for i in range(0, n, chunk):
+            c = min(chunk, n - i)
+            steps.append({"step": len(steps), "entries": [{"id": f"c{chunk}", "tokens": tokens[i : i + c],
+                                                           "want": list(range(c))}],
+                          "end": [f"c{chunk}"] if i + c == n else []})
+    rows = _replay(folder, dtype, tmp_path, steps, n)
+    whole = rows[:n]
+    scale = whole.abs().max().item()
+    for k, chunk in enumerate((64, 7, 1), 1):
+        assert _err(rows[k * n : (k + 1) * n], whole) <= TOL[dtype] * scale, f"portions of {chunk}"
+    want = plain.forward(_plain_weights(folder, config, dtype), config, tokens[:96])
+    assert _err(whole[:96], want) <= TOL[dtype] * want.abs().max().item(), "whole against the plain implementation"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gpt2_small_sizes_256_requests_under_load(folder_for, dtype):
+    """Width 768, 12 heads, all 12 layers: 256 requests, prompts of 1 to 1,023 tokens, 1 to 255
+    new tokens, temperature 0.8 with a seed per request, pages of 16 tokens, a pool of 24
+    contexts for up to 48 running requests (so requests are pre-empted).  Every request
+    finishes with ``min(max_new, positions - prompt)`` tokens; fourteen of them, run alone with
+    room to spare, give the same tokens: all of them in float32.  In bfloat16 the logits of a
+    row differ by rounding with the batch around it, and a draw that falls near the edge
+    between two tokens may go the other way (from there on the two runs are different
+    requests): all but three at most have to agree to the end, and the tokens before the first
+    difference have to be nine tenths of all."""
+    from mlx_lm_amd.generate import BatchGenerator, engine_for
+    from mlx_lm_amd.sample_utils import make_sampler
+    from mlx_lm_amd.utils import load_model
+
+    folder, config = folder_for("small")
+    P, V, n_req = config["n_positions"], config["vocab_size"], 256
+    model, _ = load_model(folder, dtype=dtype)
+    rng = random.Random(0)
+    prompts = [[rng.randrange(V) for _ in range(rng.randrange(1, P))] for _ in range(n_req)]
+    max_new = [rng.randrange(1, 256) for _ in range(n_req)]
+    sampler = make_sampler(temp=0.8)
+
+    def run(idx, cache_tokens, batch):
+        eng = engine_for(model, max_requests=64, max_cache_tokens=cache_tokens)
+        gen = BatchGenerator(model, sampler=sampler, completion_batch_size=batch, prefill_batch_size=4,
+                             prefill_step_size=512, want_logprobs=False, engine=eng)
+        uids = gen.insert([prompts[i] for i in idx], [max_new[i] for i in idx], seeds=[1000 + i for i in idx])
+        out, reasons = {u: [] for u in uids}, {}
+        while responses := gen.next_generated():
+            for r in responses:
+                out[r.uid].append(r.token)
+                if r.finish_reason:
+                    reasons[r.uid] = r.finish_reason
+        eng.cache.check()
+        assert eng.cache.free_pages() == eng.cache.n_pages
+        return [out[u] for u in uids], [reasons.get(u) for u in uids], gen.scheduler.stats
+
+    idx = list(range(n_req))
+    crowd, reasons, stats = run(idx, 24 * P, 48)
+    assert stats.preemptions > 0
+    for i in idx:
+        assert len(crowd[i]) == min(max_new[i], P - len(prompts[i])) and reasons[i] == "length", i
+    sample = idx[::19]
+    assert len(sample) >= 12
+    same = agreeing = total = 0
+    for i in sample:
+        alone, _, _ = run([i], 2 * P, 1)
+        assert len(alone[0]) == len(crowd[i])
+        first = next((k for k, (x, y) in enumerate(zip(alone[0], crowd[i])) if x != y), len(crowd[i]))
+        if first < len(crowd[i]):
+            print(f"{dtype}: request {i} alone differs from token {first} of {len(crowd[i])} on")
+        same += first == len(crowd[i])
+        agreeing += first
+        total += len(crowd[i])
+        if dtype == "float32":
+            assert alone[0] == crowd[i], f"request {i}"
+    assert same >= len(sample) - 3 and agreeing >= 0.9 * total, (same, agreeing, total)

@@ -272,3 +272,16 @@ def test_overlapped_steps_abort_and_preemption_with_a_token_in_flight():
     for rid in ("old", "new"):
         assert [o.token for o in done[rid]] == [token_for(rid, i) for i in range(40)]
     assert eng.cache.free_pages() == 5
+
+
+@pytest.mark.parametrize("mode", list(SAMPLERS))
+def test_a_request_for_no_tokens_is_over_at_once(mode):
+    """``max_tokens=0``: no step, no sampled token (mlx_lm/generate.py:448-461 yields nothing)."""
+    eng = FakeEngine(n_pages=16)
+    sched = Scheduler(eng, SAMPLERS[mode](), max_num_seqs=4)
+    r = sched.add(Request("none", [1, 2, 3], 0))
+    assert r.finish_reason == "length" and not sched.has_work and not r.live
+    sched.add(Request("one", [4, 5], 1))
+    done = run_all(sched)
+    assert list(done) == ["one"] and r.generated == [] and not eng.has_request("none")
+    assert all(rid != "none" for step in eng.log for rid, _, _ in step)
