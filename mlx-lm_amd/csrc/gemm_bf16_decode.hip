@@ -40,6 +40,9 @@
 // needs writes back and invalidates an L2 per block on this multi-die GPU and
 // took 120 us where the whole product takes 8.)
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
 
 #define FLAG_GELU 1
 #define FLAG_ACCUMULATE 2
@@ -671,4 +674,65 @@ extern "C" int sum_partials_norm(float* h, int ldh, const float* ws, int n_split
     hipLaunchKernelGGL(sum_partials_norm_kernel<8>, dim3(M + readers), dim3(256), 0, stream, q);
   CHECK_LAUNCH("sum_partials_norm");
   return 0;
+}
+
+// ---------------------------------------------------------------------------
+// The split product for callers that cannot allocate (no_alloc.h).  The partial sums lie in
+// an array of the library's own, one copy on every GPU.  In host code the array's name is only
+// a handle for hipGetSymbolAddress: what kernels, copies and fills get is the address looked
+// up there, once per device, with that device current.
+
+static __device__ __align__(256) float scratch[GEMM_BF16_DECODE_STATIC_FLOATS];
+
+#define STATIC_MAX_DEVICES 64
+static float* g_scratch_ptr[STATIC_MAX_DEVICES];  // per device: where its copy of `scratch` lies
+static std::mutex g_scratch_lock;
+
+// The current device's copy of the array (looked up at the first call on that device).
+static int scratch_of_current_device(float** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) FAIL("gemm_bf16_decode_split_static: no current device: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= STATIC_MAX_DEVICES)
+    FAIL("gemm_bf16_decode_split_static: device %d is beyond the %d this library keeps an array for", dev,
+         STATIC_MAX_DEVICES);
+  std::lock_guard<std::mutex> guard(g_scratch_lock);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      FAIL("gemm_bf16_decode_split_static: the array's address on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = (float*)p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return 0;
+}
+
+extern "C" int gemm_bf16_decode_static_init(void) {
+  float* ptr = nullptr;
+  return scratch_of_current_device(&ptr);
+}
+
+extern "C" int gemm_bf16_decode_split_static(void* out, const void* A, int lda, const void* W,
+                                             const float* bias, int M, int N, int K, int ldw, int ldo,
+                                             int flags, int n_splits, hipStream_t stream) {
+  if (M == 0) return 0;
+  if (flags & ~(FLAG_GELU | FLAG_ACCUMULATE | FLAG_OUT_F32))
+    FAIL("gemm_bf16_decode_split_static: flags %d: only GELU (1), accumulate (2) and float32 out (4)", flags);
+  if (M < 0 || N <= 0 || n_splits < 1) FAIL("gemm_bf16_decode_split_static: bad M=%d, N=%d or splits=%d", M, N, n_splits);
+  if ((size_t)n_splits * (size_t)M * (size_t)N > (size_t)GEMM_BF16_DECODE_STATIC_FLOATS)
+    FAIL("gemm_bf16_decode_split_static: %d splits of %d x %d are %zu partial sums, the library's array holds %u",
+         n_splits, M, N, (size_t)n_splits * M * N, GEMM_BF16_DECODE_STATIC_FLOATS);
+  float* ws = nullptr;
+  if (scratch_of_current_device(&ws)) return 1;
+  // (with one part the product's own kernel runs the epilogue and the array is not touched)
+  int rc = gemm_bf16_decode(out, A, lda, nullptr, 0, nullptr, nullptr, 0.f, W, bias, M, N, K, ldw, ldo, flags,
+                            nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr, 0, 0, 0, 0, n_splits, ws,
+                            GEMM_BF16_DECODE_STATIC_FLOATS, stream);
+  if (rc != 0 || n_splits == 1) return rc != 0;
+  // Every partial sum read below was written by the launch above: each of the n_splits parts
+  // holds k-blocks (an empty part is refused) and its blocks write all M x N sums of the part.
+  rc = sum_partials(out, ws, n_splits, bias, M, N, ldo, flags, nullptr, nullptr, 0, nullptr, 0, nullptr,
+                    nullptr, 0, 0, 0, 0, stream);
+  return rc != 0;
 }

@@ -71,7 +71,8 @@ def _readonly_lib_dir():
 
 def _digest(name):
     h = hashlib.sha256()
-    for f in (os.path.join(CSRC, name + ".hip"), os.path.join(CSRC, "common.h")):
+    headers = sorted(f for f in os.listdir(CSRC) if f.endswith(".h"))
+    for f in [os.path.join(CSRC, name + ".hip")] + [os.path.join(CSRC, h) for h in headers]:
         with open(f, "rb") as fh:
             h.update(fh.read())
     h.update(" ".join(HIPCC_FLAGS).encode())
