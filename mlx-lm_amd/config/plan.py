@@ -22,13 +22,12 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer: an arrangement (block kind) of two norms, a mixer and a feed-forward."""
+    """One layer: an arrangement (block kind) and the parts it arranges, by the names
+    that the arrangement gives them (``pre_norm``: ``mixer_norm``, ``mixer``, ``ffn_norm``,
+    ``ffn``).  Which parts there are, and how many, is the arrangement's business."""
 
     arrangement: str
-    mixer_norm: PartSpec
-    mixer: PartSpec
-    ffn_norm: PartSpec
-    ffn: PartSpec
+    parts: Dict[str, PartSpec]
 
 
 @dataclass(frozen=True)

@@ -9,7 +9,9 @@ import torch
 
 from ..cache import CacheManager
 from ..weights.loader import resolve_dtype
-from .context import BIG_TILE_Q, ROW_KERNEL_MAX_Q, TILE_Q, AttentionPlan, Scratch, StepContext
+from ..ops import native
+from .context import Scratch
+from .pack import EagerStore, pack
 
 
 @dataclass
@@ -23,36 +25,6 @@ class StepEntry:
     # Row of the step's ``fed`` tokens (sampled tokens still on the device) that is
     # this request's one token; ``tokens`` then holds a placeholder.  -1: ``tokens`` are the tokens.
     fed_row: int = -1
-
-
-class _HostRing:
-    """Pinned host buffers for the step's integer arrays, reused in turn.
-
-    A buffer is written again only after the copy that read it has finished.
-    """
-
-    def __init__(self, n=4):
-        self.bufs = [None] * n
-        self.events = [None] * n
-        self.i = 0
-
-    def get(self, n_ints):
-        self.i = (self.i + 1) % len(self.bufs)
-        if self.events[self.i] is not None:
-            self.events[self.i].synchronize()
-        b = self.bufs[self.i]
-        if b is None or b.numel() < n_ints:
-            b = torch.empty(max(n_ints, 4096), dtype=torch.int32, pin_memory=True)
-            self.bufs[self.i] = b
-        return b
-
-    def current(self):
-        return self.bufs[self.i]
-
-    def mark(self):
-        ev = self.events[self.i] or torch.cuda.Event()
-        ev.record()
-        self.events[self.i] = ev
 
 
 class Engine:
@@ -82,10 +54,18 @@ class Engine:
         self.cache = CacheManager(self.decoder.cache_needs(), page_size, n_pages, max_requests,
                                   dtype=self.dtype, device=self.device)
         self.scratch = Scratch(self.device)
-        self._ring = _HostRing()
-        self._meta_dev = None
+        self._eager = EagerStore(self.device)
         self._logits = None
         self.steps = 0
+        # what the native parts need of the device and the cache, made once
+        from ..ops import kernels
+
+        native.lib()
+        self.n_compute_units = kernels.n_compute_units()
+        self.split_ws = kernels.split_workspace(self.device)
+        self.stats = native.EngStats()
+        self.slot_table = self._slot_table()
+        self.array_providers = self.decoder.array_providers()
         # sampled tokens that go into the next step without passing through the host
         self.fed_src = torch.zeros(max(64, max_requests), dtype=torch.int32, device=self.device)
         # decode steps are recorded as graphs where every part launches kernels only
@@ -96,6 +76,24 @@ class Engine:
         self.record_prompt_steps = bool(record_prompt_steps) and self.use_graphs
         self._step_graphs = OrderedDict()
         self._shape_seen = {}
+
+    def _slot_table(self):
+        """One ``EngSlot`` per cache slot: where its pages lie and which block table is its group's."""
+        cm = self.cache
+        n = max([-1, *cm.slot_group, *cm.state_needs]) + 1
+        n = max(n, len(self.decoder.cache_needs()))
+        table = (native.EngSlot * max(n, 1))()
+        for slot in range(n):
+            s = table[slot]
+            s.group = -1
+            if slot in cm.slot_group:
+                g, _ = cm.slot_group[slot]
+                k, v = cm.kv(slot)
+                need = cm.groups[g].need
+                s.k, s.v, s.page_stride = k.data_ptr(), v.data_ptr(), k.stride(0)
+                s.n_kv_heads, s.head_dim, s.page_size = need.n_kv_heads, need.head_dim, cm.page_size
+                s.dtype, s.group = native.DT[k.dtype], g
+        return table
 
     # -- buffers ---------------------------------------------------------------
 
@@ -202,14 +200,8 @@ class Engine:
                 cm.rollback(rid, mark)
             raise
 
-        if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
-            graph = self._graphs.get(len(entries))
-            if graph is None:
-                from .graph import DecodeGraph
-
-                graph = self._graphs[len(entries)] = DecodeGraph(self, len(entries))
-            logits = graph.run(entries)
-        elif self.record_prompt_steps and (graph := self._recorded_step(entries)) is not None:
+        graph = self._recorded_step(entries) if self.use_graphs else None
+        if graph is not None:
             logits = graph.run(entries)
         else:
             ctx = self._build_context(entries)
@@ -224,10 +216,24 @@ class Engine:
     MAX_RECORDED = 24
 
     def _recorded_step(self, entries):
-        """The recorded step for this batch's shape, if it has one (or is due one)."""
+        """The recorded step for this batch's shape, if it has one (or is due one).
+
+        A step in which every request brings one token and wants its logits (a decode step) is
+        recorded at its first sighting; steps of other shapes after ``RECORD_AFTER`` sightings,
+        and only where ``record_prompt_steps`` asks for it."""
         q_lens = tuple(len(e.tokens) for e in entries)
         n_wanted = sum(len(e.want) for e in entries)
         every = n_wanted == sum(q_lens) and all(list(e.want) == list(range(len(e.tokens))) for e in entries)
+        decode = every and n_wanted == len(entries)
+        if decode:
+            graph = self._graphs.get(len(entries))
+            if graph is None:
+                from .graph import StepGraph
+
+                graph = self._graphs[len(entries)] = StepGraph(self)
+            return None if graph.failed else graph
+        if not self.record_prompt_steps:
+            return None
         key = (q_lens, n_wanted, every)
         graph = self._step_graphs.get(key)
         if graph is not None:
@@ -247,102 +253,17 @@ class Engine:
             self._step_graphs.popitem(last=False)
         return graph
 
-    def _build_context(self, entries, static=None):
-        """The step's context.  ``static`` (a ``StepGraph``): the integer arrays go to that graph's own
-        device buffer, at offsets that depend on the step's shape only."""
-        cm = self.cache
-        R = len(entries)
-        T = sum(len(e.tokens) for e in entries)
-        ctx = StepContext(self)
-        q_start = 0
-        token_ids, positions, token_req, wanted, slot_ids, fed_index = [], [], [], [], [], []
-        tiles, rows, all_tiles, big = [], [], [], []
-        plan = AttentionPlan()
-        for r, e in enumerate(entries):
-            rc = cm.requests[e.request_id]
-            n = len(e.tokens)
-            ctx.q_starts.append(q_start)
-            ctx.q_lens.append(n)
-            ctx.context_lens.append(rc.length)
-            token_ids.append(np.asarray(e.tokens, dtype=np.int32))
-            fed_index.append(np.full(n, e.fed_row if e.fed_row >= 0 else -1, dtype=np.int32))
-            positions.append(np.arange(rc.length, rc.length + n, dtype=np.int32))
-            token_req.append(np.full(n, r, dtype=np.int32))
-            wanted.append(q_start + np.asarray(e.want, dtype=np.int32))
-            slot_ids.append(rc.state_slot)
-            ctx.state_slots.append(rc.state_slot)
-            for s in range(0, n, TILE_Q):
-                all_tiles.extend((q_start + s, min(TILE_Q, n - s)))
-            if n <= ROW_KERNEL_MAX_Q:
-                rows.extend(range(q_start, q_start + n))
-                plan.max_row_context = max(plan.max_row_context, rc.length + n)
-            else:
-                for s in range(0, n, TILE_Q):
-                    tiles.extend((q_start + s, min(TILE_Q, n - s)))
-                for s in range(0, n, BIG_TILE_Q):
-                    big.append((rc.length + s + min(BIG_TILE_Q, n - s), q_start + s, min(BIG_TILE_Q, n - s)))
-            q_start += n
-        plan.n_tiles, plan.n_rows, plan.n_all_tiles = len(tiles) // 2, len(rows), len(all_tiles) // 2
-        if static is not None and rows:
-            plan.max_row_context = self.decoder.max_positions  # how keys are split must not depend on lengths
-        big.sort(reverse=True)  # tiles with the most keys start first
-        big_tiles = [v for _, r0, nr in big for v in (r0, nr)]
-        plan.n_big_tiles = len(big)
+    def _build_context(self, entries):
+        """The context of an eager step: its arrays packed and on their way to the device, tokens
+        that are still on the device fed into their places."""
+        ctx = pack(self, entries, self._eager)
+        self._eager.send()
+        self.feed(ctx)
+        return ctx
 
-        # block tables, one per group, padded to the longest of the step
-        tables = []
-        for gi in range(len(cm.groups)):
-            width = max(1, max(len(cm.requests[e.request_id].blocks[gi]) for e in entries))
-            if static is not None:
-                width = cm.blocks_for(self.decoder.max_positions)
-            flat = []
-            for e in entries:
-                b = cm.requests[e.request_id].blocks[gi]
-                flat.extend(b)
-                flat.extend([-1] * (width - len(b)))
-            tables.append((width, flat))
-
-        # everything in one pinned buffer and one copy; pieces start on 4-int boundaries
-        token_ids, positions, token_req = (np.concatenate(x) for x in (token_ids, positions, token_req))
-        wanted, fed_index = np.concatenate(wanted), np.concatenate(fed_index)
-        pieces = [token_ids, positions, token_req, wanted, slot_ids, tiles, rows, all_tiles, big_tiles]
-        pieces += [flat for _, flat in tables]
-        pieces.append(fed_index)  # (last: the pieces before it keep their numbers)
-        offsets, total = [], 0
-        for p in pieces:
-            offsets.append(total)
-            total += (len(p) + 3) // 4 * 4
-        host = self._ring.get(total).numpy()
-        for off, p in zip(offsets, pieces):
-            if len(p):
-                host[off : off + len(p)] = p
-        if static is not None:
-            if static.dev is None:
-                static.dev = torch.empty(total, dtype=torch.int32, device=self.device)
-            if static.dev.numel() != total:
-                raise RuntimeError("a recorded step's arrays changed size")
-            dev = static.dev
-        else:
-            if self._meta_dev is None or self._meta_dev.numel() < total:
-                self._meta_dev = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
-            dev = self._meta_dev
-        dev[:total].copy_(self._ring.current()[:total], non_blocking=True)
-        self._ring.mark()
-
-        def piece(i, n):
-            return dev[offsets[i] : offsets[i] + n]
-
-        ctx.n_tokens, ctx.n_requests, ctx.n_wanted = T, R, len(wanted)
-        ctx.wants_every_row = len(wanted) == T and bool((wanted == np.arange(T, dtype=np.int32)).all())
-        ctx.token_ids, ctx.positions, ctx.token_req = piece(0, T), piece(1, T), piece(2, T)
-        ctx.wanted_rows, ctx.slot_ids = piece(3, len(wanted)), piece(4, R)
-        plan.tiles, plan.rows, plan.all_tiles = piece(5, len(tiles)), piece(6, len(rows)), piece(7, len(all_tiles))
-        plan.big_tiles = piece(8, len(big_tiles))
-        ctx.attention_plan = plan
-        for gi, (width, flat) in enumerate(tables):
-            ctx.block_tables.append(piece(9 + gi, len(flat)).view(R, width))
-        if bool((fed_index >= 0).any()):
+    def feed(self, ctx):
+        """Tokens fed on the device replace the placeholders of their entries."""
+        if ctx.any_fed:
             from ..ops import kernels
 
-            kernels.feed_tokens(ctx.token_ids, self.fed_src, piece(9 + len(tables), T), self.decoder.vocab_size)
-        return ctx
+            kernels.feed_tokens(ctx.token_ids, self.fed_src, ctx.fed_index, self.decoder.vocab_size)

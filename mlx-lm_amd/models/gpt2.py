@@ -98,6 +98,7 @@ class Model:
             layers.append(
                 LayerSpec(
                     arrangement="pre_norm",  # mlx_lm/models/gpt2.py:98-108
+                    parts=dict(
                     mixer_norm=norm(p + "ln_1."),
                     mixer=PartSpec(
                         "attention",
@@ -118,6 +119,7 @@ class Model:
                         "gelu_mlp",
                         {"width": D, "inner": args.n_inner, "activation": args.activation_function},
                         p + "mlp.",
+                    ),
                     ),
                 )
             )

@@ -21,7 +21,7 @@ import time
 _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(_PKG, "csrc")
 
-SOURCES = ("embed", "norm", "gemm_f32", "gemm_bf16", "gemm_bf16_decode", "attention", "attention_decode", "attention_prefill", "sampling")
+SOURCES = ("embed", "norm", "gemm_f32", "gemm_bf16", "gemm_bf16_decode", "attention", "attention_decode", "attention_prefill", "sampling", "engine")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -3,14 +3,19 @@
 Each function takes torch tensors that live on the GPU, checks on the host
 what the kernel assumes about them (shape, dtype, contiguity) and launches on
 torch's current stream.  Nothing here computes on the CPU or through a torch
-operator; a missing library raises.
+operator; a missing library raises.  A model's step does not come through
+here: the native host (``csrc/engine.hip``) issues its launches itself.  These
+faces are for a kernel alone (tests), for parts written in Python, and for
+sampling; ``linear`` and ``PendingSum`` call the native host's own product
+routine, so there is one place that chooses among the product kernels.
 """
 
 import ctypes
+import weakref
 
 import torch
 
-from . import build
+from . import build, native
 
 _c_int = ctypes.c_int
 _c_float = ctypes.c_float
@@ -36,10 +41,38 @@ _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 _current_device = getattr(torch._C, "_cuda_getDevice", None)
 
 
-def _stream():
+def raw_stream():
+    """The handle of the stream that torch launches on now, as an integer."""
     if _raw_stream is not None and _current_device is not None:
-        return _vp(_raw_stream(_current_device()))
-    return _vp(torch.cuda.current_stream().cuda_stream)
+        return _raw_stream(_current_device())
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _stream():
+    return _vp(raw_stream())
+
+
+def n_compute_units():
+    """Compute units of the current device (asked of the device once)."""
+    return native.lib().eng_compute_units()
+
+
+_BARE = {}
+
+
+def bare_context():
+    """A native context outside any step: the stream, the split workspace, no scratch memory."""
+    dev = torch.cuda.current_device()
+    c = _BARE.get(dev)
+    if c is None:
+        c = _BARE[dev] = native.EngCtx()
+        ws = split_workspace(torch.device("cuda", dev))
+        c.split_ws, c.split_ws_floats = ws.data_ptr(), ws.numel()
+        c.n_compute_units = n_compute_units()
+        c.dtype = 1
+    c.stream = raw_stream()
+    c.force_splits = force_splits
+    return c
 
 
 def _ptr(t):
@@ -183,19 +216,27 @@ class PackedWeight:
         self.packed = t.contiguous().view(-1)
         # what one block of the decode kernel reads (16 features, all of K) and how many there are
         self.chunk_bytes, self.n_chunks = Kp * 16 * 2, Np // 16
+        self.c = native.EngWeight(w.data_ptr(), self.packed.data_ptr(), N, K, w.stride(0), DT[w.dtype],
+                                  self.chunk_bytes, self.n_chunks, 0)
+
+
+def weight_struct(w):
+    """The native description of a weight matrix (a ``PackedWeight`` or a 2-D tensor ``[N, K]``)."""
+    if isinstance(w, PackedWeight):
+        return w.c
+    ld = _rows2d(w, "w")
+    w.dtype in DT or _fail(f"weight dtype {w.dtype} not supported")
+    return native.EngWeight(w.data_ptr(), None, w.shape[0], w.shape[1], ld, DT[w.dtype], 0, 0, 0)
 
 
 def read_ahead_pays(w, n_rows, with_norm=False):
     """Whether the rows' next product should have ``w`` read ahead by the kernel before it: a
     ``PackedWeight`` that the decode kernel takes whole, 16 features a block (then block ``j``
     reads chunk ``j``, on die ``j % 8``), for few enough rows that most CUs have none."""
-    if not isinstance(w, PackedWeight) or not 0 < n_rows <= DECODE_MAX_ROWS:
+    if not isinstance(w, PackedWeight):
         return False
-    N, K = w.shape
-    lib = build.load("gemm_bf16_decode")
-    norm = _c_int(1 if with_norm else 0)
-    return (w.n_chunks >= 150 and bool(lib.gemm_bf16_decode_takes(_c_int(n_rows), _c_int(K), norm, _c_int(1)))
-            and lib.gemm_bf16_decode_splits(_c_int(n_rows), _c_int(N), _c_int(K), norm, _c_int(force_splits)) == 1)
+    return bool(native.lib().eng_read_ahead_pays(ctypes.byref(bare_context()), ctypes.byref(w.c), int(n_rows),
+                                                 1 if with_norm else 0))
 
 
 def for_decode(w):
@@ -236,37 +277,49 @@ class PendingSum:
     workspace; with a ``PendingSum`` given, ``linear(accumulate=True)`` may
     stop there.  Whoever reads the stream next either adds them and norms the
     rows in one kernel (``settle_normed``) or just adds them (``settle``).
-    ``allowed`` is set by a caller that promises to do so.
+    ``allowed`` is set by a caller that promises to do so.  The state is a
+    struct of the native host's (a step's own lies in its context).
     """
 
-    def __init__(self):
-        self.allowed = False
-        self.target = None
-        self.ws = self.bias = None
-        self.n_splits = 0
+    def __init__(self, c=None, ctx=None):
+        self.c = c if c is not None else native.EngPending()
+        # the step whose pending sum this is, if any (weakly: the step holds this object)
+        self._ctx = weakref.proxy(ctx) if ctx is not None else None
+
+    allowed = property(lambda self: bool(self.c.allowed),
+                       lambda self, v: setattr(self.c, "allowed", 1 if v else 0))
+    target = property(lambda self: self.c.target)  # the address that the sum goes to, or None
+    n_splits = property(lambda self: self.c.n_splits)
+
+    def _native(self):
+        if self._ctx is None:
+            return bare_context()
+        self._ctx.c.stream = raw_stream()
+        return self._ctx.c
 
     def waits_on(self, x):
-        return self.target is not None and self.target.data_ptr() == x.data_ptr() and self.target.shape == x.shape
+        c = self.c
+        return bool(c.target) and c.target == x.data_ptr() and (c.rows, c.cols) == tuple(x.shape)
 
     def settle(self):
         """Add what is pending (if anything) into its target."""
-        if self.target is None:
-            return
-        target, self.target = self.target, None
-        sum_partials(target, self.ws, self.n_splits, self.bias, accumulate=True)
+        native.check(native.lib().eng_pending_settle(ctypes.byref(self._native()), ctypes.byref(self.c)))
 
     def settle_normed(self, out, gamma, beta, eps, ahead=None):
         """Add what is pending into its target and write the LayerNorm of the new rows to ``out``.
 
         ``ahead``: the weights of the product that reads ``out`` (see ``sum_partials_norm``)."""
-        target, self.target = self.target, None
-        _need(target is not None, "settle_normed: nothing is pending")
-        sum_partials_norm(target, self.ws, self.n_splits, self.bias, gamma, beta, eps, out, ahead=ahead)
+        _need(out.is_contiguous(), "settle_normed: out must be contiguous")
+        m = native.mat(out)
+        native.check(native.lib().eng_pending_settle_normed(
+            ctypes.byref(self._native()), ctypes.byref(self.c), ctypes.byref(m), native.ptr(gamma),
+            native.ptr(beta), float(eps), ctypes.byref(ahead.c) if ahead is not None else None))
 
     def can_norm(self, x):
-        lib = build.load("gemm_bf16_decode")
-        return (self.waits_on(x) and x.stride(1) == 1
-                and bool(lib.sum_partials_norm_takes(_c_int(x.shape[1]), _c_int(x.stride(0)))))
+        if not self.waits_on(x) or x.stride(1) != 1:
+            return False
+        m = native.mat(x)
+        return bool(native.lib().eng_pending_can_norm(ctypes.byref(self.c), ctypes.byref(m)))
 
 
 def _scatter_args(sc):
@@ -342,128 +395,43 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
     would not fill the GPU, both split K over ``splits`` blocks and add the
     partial sums in a second kernel; with ``accumulate`` and a ``pending``
     that allows it, that second step is left to the next reader of ``out``.
-    Everything else is composed from the general kernels.
+    The choices are the native host's (``linear`` in csrc/engine.hip), which
+    a model's step uses too.
     """
-    lazy = a if isinstance(a, NormedInput) else None
-    packed = w if isinstance(w, PackedWeight) else None
-    if packed is not None:
-        w = packed.w
-    M, K = a.shape
-    N = w.shape[0]
-    ldw, ldo = _rows2d(w, "w"), _rows2d(out, "out")
-    w.shape[1] == K or _fail(f"linear: a is [{M},{K}] but w is {list(w.shape)}")
-    tuple(out.shape) == (M, N) or _fail(f"linear: out is {list(out.shape)}, want [{M},{N}]")
-    _need(a.dtype == w.dtype and w.dtype in DT, "linear: a and w must share float32 or bfloat16")
+    L = native.lib()
+    ctx = pending._native() if pending is not None else bare_context()
+    call = native.EngLinear()
+    call.w = weight_struct(w)
+    N, K = call.w.N, call.w.K
+    if isinstance(a, NormedInput):
+        M = a.shape[0]
+        fused = variant == 0 and L.eng_linear_norms_itself(ctypes.byref(ctx), M, N, K, DT[a.dtype], splits or 0)
+        if not fused:
+            a = a.materialize()
+    if isinstance(a, NormedInput):
+        _dev(a.x, "x", torch.float32)
+        call.a.lazy, call.a.ldx = 1, a.x.stride(0)
+        call.a.m = native.EngMat(None, a.shape[0], a.shape[1], a.shape[1], DT[a.dtype])
+        call.a.x, call.a.gamma, call.a.beta, call.a.eps = a.x.data_ptr(), native.ptr(a.gamma), native.ptr(a.beta), a.eps
+    else:
+        call.a.m = native.mat(a)
+    call.out = native.mat(out)
     if bias is not None:
         _dev(bias, "bias", torch.float32)
         _need(bias.numel() == N, "linear: bias length")
-    flags = 0
-    if gelu:
-        flags |= GEMM_GELU
-    if accumulate:
-        _need(out.dtype == torch.float32, "linear: accumulate needs a float32 out")
-        flags |= GEMM_ACCUMULATE
-        if pending is not None and pending.waits_on(out):
-            pending.settle()  # an earlier sum into the same rows goes first
+        call.bias = bias.data_ptr()
+    sc = None
     if scatter is not None:
-        _need(not accumulate and not gelu and out.dtype == w.dtype, "linear: scatter goes with a plain epilogue")
-        _need(scatter.q_width + 2 * scatter.kv_width == N, "linear: scatter widths do not add up to N")
-        _need(scatter.kv.k.dtype == w.dtype, "linear: cache dtype differs from the projection's")
-    if w.dtype == torch.float32:
-        _need(out.dtype == torch.float32, "linear: float32 operands give a float32 out")
-    elif out.dtype == torch.float32:
-        flags |= GEMM_OUT_F32
-    else:
-        _need(out.dtype == torch.bfloat16, "linear: out must be float32 or bfloat16")
-
-    if w.dtype == torch.bfloat16 and variant == 0 and 0 < M <= DECODE_MAX_ROWS:
-        lib = build.load("gemm_bf16_decode")
-        with_norm = _c_int(1 if lazy else 0)
-        if splits is None:
-            n_splits = lib.gemm_bf16_decode_splits(_c_int(M), _c_int(N), _c_int(K), with_norm, _c_int(force_splits))
-        else:
-            n_chunks = (K + 63) // 64
-            per_split = -(-n_chunks // max(1, min(splits, n_chunks)))
-            n_splits = -(-n_chunks // per_split)  # no split without k-blocks
-        ws = None
-        if n_splits > 1:
-            ws = split_workspace(w.device)
-            n_splits = max(1, min(n_splits, ws.numel() // (M * N)))
-        if lib.gemm_bf16_decode_takes(_c_int(M), _c_int(K), with_norm, _c_int(n_splits)):
-            if lazy:
-                _dev(lazy.x, "x", torch.float32)
-                A, lda, X, ldx = None, 0, lazy.x, lazy.x.stride(0)
-                gamma, beta, eps = lazy.gamma, lazy.beta, lazy.eps
-            else:
-                A, lda, X, ldx, gamma, beta, eps = a, _rows2d(a, "a"), None, 0, None, None, 0.0
-            if n_splits > 1 and pending is not None:
-                pending.settle()  # the workspace is about to be written again
-            rc = lib.gemm_bf16_decode(
-                _ptr(out), _ptr(A), _c_int(lda), _ptr(X), _c_int(ldx), _ptr(gamma), _ptr(beta),
-                _c_float(eps), _ptr(packed.packed if packed else w), _ptr(bias), _c_int(M), _c_int(N),
-                _c_int(K), _c_int(0 if packed else ldw),
-                _c_int(ldo), _c_int(flags | (GEMM_KV if scatter else 0)), *_scatter_args(scatter),
-                _c_int(n_splits), _ptr(ws if n_splits > 1 else None),
-                _c_size_t(ws.numel() if n_splits > 1 else 0), _stream(),
-            )
-            build.check(lib, rc, "linear")
-            if n_splits > 1:
-                if accumulate and pending is not None and pending.allowed:
-                    pending.target, pending.ws, pending.n_splits, pending.bias = out, ws, n_splits, bias
-                else:
-                    sum_partials(out, ws, n_splits, bias, gelu=gelu, accumulate=accumulate, scatter=scatter)
-            return out
-
-    if lazy:
-        a = lazy.materialize()
-    lda = _rows2d(a, "a")
-    if w.dtype == torch.float32:
-        lib = build.load("gemm_f32")
-        rc = lib.gemm_f32(
-            _ptr(out), _ptr(a), _ptr(w), _ptr(bias), _c_int(M), _c_int(N), _c_int(K),
-            _c_int(lda), _c_int(ldw), _c_int(ldo), _c_int(flags), _c_int(variant), _stream(),
-        )
-        build.check(lib, rc, "linear")
-    else:
-        # Few rows give the tile kernel few tiles: K is split then as for the decode kernels,
-        # and the same second kernels add the parts and run the epilogue.
-        lib = build.load("gemm_bf16")
-        n_splits, ws = 1, None
-        if variant in (0, 1, 5, 6) and M > DECODE_MAX_ROWS:
-            n_blocks = (K + 63) // 64
-            if splits is None:
-                # (the second kernel stands in for one that would run anyway: the next norm, or the cache write)
-                fused = (accumulate and pending is not None and pending.allowed) or scatter is not None
-                n_splits = lib.gemm_bf16_splits(_c_int(M), _c_int(N), _c_int(K), _c_int(1 if fused else 0),
-                                                _c_int(force_splits))
-            else:
-                per_split = -(-n_blocks // max(1, min(splits, n_blocks)))
-                n_splits = -(-n_blocks // per_split)
-            if n_splits > 1:
-                ws = split_workspace(w.device)
-                n_splits = min(n_splits, ws.numel() // (M * N))
-                if n_splits > 1:  # (again without an empty part)
-                    per_split = -(-n_blocks // n_splits)
-                    n_splits = -(-n_blocks // per_split)
-            if n_splits > 1 and pending is not None:
-                pending.settle()  # the workspace is about to be written again
-        rc = lib.gemm_bf16(
-            _ptr(out), _ptr(a), _ptr(w), _ptr(bias), _c_int(M), _c_int(N), _c_int(K),
-            _c_int(lda), _c_int(ldw), _c_int(ldo), _c_int(flags), _c_int(variant),
-            _c_int(max(1, n_splits)), _ptr(ws if n_splits > 1 else None),
-            _c_size_t(ws.numel() if n_splits > 1 else 0), _stream(),
-        )
-        build.check(lib, rc, "linear")
-        if n_splits > 1:
-            if accumulate and pending is not None and pending.allowed:
-                pending.target, pending.ws, pending.n_splits, pending.bias = out, ws, n_splits, bias
-            else:
-                sum_partials(out, ws, n_splits, bias, gelu=gelu, accumulate=accumulate, scatter=scatter)
-            return out
-    if scatter is not None:
-        q, kw = scatter.q_width, scatter.kv_width
-        kv_write(out[:, q : q + kw], out[:, q + kw :], scatter.kv, scatter.block_table,
-                 scatter.token_req, scatter.positions)
+        kv = scatter.kv
+        _attn_common(out, kv, scatter.block_table, scatter.token_req, scatter.positions)
+        sc = native.EngScatter(kv.k.data_ptr(), kv.v.data_ptr(), kv.page_stride, kv.n_kv_heads, kv.head_dim,
+                               kv.page_size, DT[kv.k.dtype], scatter.block_table.data_ptr(),
+                               scatter.token_req.data_ptr(), scatter.positions.data_ptr(),
+                               scatter.block_table.shape[1], scatter.q_width, scatter.kv_width, 0)
+        call.scatter = ctypes.pointer(sc)
+    call.gelu, call.accumulate, call.variant, call.splits = int(gelu), int(accumulate), int(variant), int(splits or 0)
+    rc = L.eng_linear(ctypes.byref(ctx), ctypes.byref(call), ctypes.byref(pending.c) if pending is not None else None)
+    native.check(rc, "linear")
     return out
 
 

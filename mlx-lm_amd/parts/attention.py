@@ -1,11 +1,14 @@
 """Causal self-attention over the paged cache."""
 
+import ctypes
+
 from ..config.plan import CacheNeed
-from ..ops import kernels
-from .base import POSITION_ENCODINGS, Mixer, TensorSpec, build_part, register_mixer
+from ..ops import kernels, native
+from .base import POSITION_ENCODINGS, Mixer, TensorSpec, build_part, register_mixer, value_of
 
-
-READ_AHEAD_BYTES_PER_CU = 160 * 1024  # what an idle CU reads while decode attention runs (some 5 us)
+ROW_KERNEL_MAX_Q = 4  # requests with at most this many tokens in a step take the row kernels
+TILE_Q = 16  # queries per tile of the general tile kernel
+BIG_TILE_Q = 128  # queries per tile of the matrix-core prefill kernel
 
 
 class CausalSelfAttention(Mixer):
@@ -78,68 +81,63 @@ class CausalSelfAttention(Mixer):
         if self.position is not None:
             self.position.load(tensors)
 
-    def forward(self, ctx, x, residual, cache, writes_cache=True):
-        T = x.shape[0]
-        qkv = ctx.scratch((T, self.q_width + 2 * self.kv_width), ctx.dtype)
-        q = qkv[:, : self.q_width]
-        if self.position is None:
-            # keys and values go to their pages from the projection's epilogue
-            scatter = kernels.KVScatter(cache.kv, cache.block_table, ctx.token_req, ctx.positions,
-                                        self.q_width) if writes_cache else None
-            kernels.linear(qkv, x, self.qkv_w, self.qkv_b, scatter=scatter)
-        else:
-            kernels.linear(qkv, x, self.qkv_w, self.qkv_b)
-            k = qkv[:, self.q_width : self.q_width + self.kv_width]
-            v = qkv[:, self.q_width + self.kv_width :]
-            self.position.rotate(ctx, q, k)
-            if writes_cache:
-                kernels.kv_write(k, v, cache.kv, cache.block_table, ctx.token_req, ctx.positions)
-        out = ctx.scratch((T, self.q_width), ctx.dtype)
-        self.attend(ctx, out, q, cache)
-        kernels.linear(residual, out, self.out_w, self.out_b, accumulate=True, pending=ctx.pending)
+    # -- the step arrays this part asks the packer for ---------------------------
 
-    def attend(self, ctx, out, q, cache):
-        plan = ctx.attention_plan
-        args = (cache.kv, cache.block_table, ctx.token_req, ctx.positions)
-        if self.head_dim > kernels.ATTN_ROW_MAX_HEAD_DIM:
-            kernels.attn_tile(out, q, *args, plan.all_tiles, plan.n_all_tiles, self.n_heads,
-                              self.scale, self.window)
-            return
-        if plan.n_tiles:
-            if kernels.attn_prefill_takes(q.dtype, cache.kv):
-                kernels.attn_prefill(out, q, *args, plan.big_tiles, plan.n_big_tiles, self.n_heads,
-                                     self.scale, self.window)
+    step_arrays_key = "attention"
+    step_array_names = ("tiles", "rows", "all_tiles", "big_tiles", "max_row_context")
+
+    @staticmethod
+    def step_arrays(batch):
+        """Which of the step's rows go to which attention kernel.
+
+        Requests that bring at most ``ROW_KERNEL_MAX_Q`` tokens are handled row by row (``rows``;
+        keys split over blocks); longer portions in tiles of ``TILE_Q`` consecutive queries
+        (``tiles``: first flat row and number of rows each), and the same portions in tiles of
+        ``BIG_TILE_Q`` for the matrix-core kernel (``big_tiles``, the tile with the most keys
+        first).  ``all_tiles`` covers every row with tiles, for head sizes the row kernels do
+        not take.  ``max_row_context``: the most keys that a row of ``rows`` sees, which decides
+        how its keys are split; in a step that is recorded, the model's positions."""
+        tiles, rows, all_tiles, big = [], [], [], []
+        longest = 0
+        for q0, n, length in zip(batch.q_starts, batch.q_lens, batch.context_lens):
+            for s in range(0, n, TILE_Q):
+                all_tiles += (q0 + s, min(TILE_Q, n - s))
+            if n <= ROW_KERNEL_MAX_Q:
+                rows += range(q0, q0 + n)
+                longest = max(longest, length + n)
             else:
-                kernels.attn_tile(out, q, *args, plan.tiles, plan.n_tiles, self.n_heads, self.scale,
-                                  self.window)
-        if plan.n_rows:
-            fast = kernels.attn_decode_takes(q.dtype, cache.kv)
-            if fast:
-                n_splits, n_waves = plan.row_work(self.n_heads, self.window)
-            else:
-                n_splits, n_waves = plan.row_splits(self.n_heads, self.window), 4
-            part_o = part_ml = None
-            if n_splits > 1:
-                n = plan.n_rows * self.n_heads * n_splits
-                part_o = ctx.scratch((n * self.head_dim,), "float32")
-                part_ml = ctx.scratch((n * 2,), "float32")
-            if fast:
-                # CUs without a row read the weights that come after this mixer's own (the block
-                # says which), as many chunks as they manage while the rows' blocks run; where fewer
-                # than half the CUs are idle the reading slows the rows' blocks by more than it gains
-                ahead, chunks = getattr(ctx, "read_ahead", None), 0
-                idle = 256 - plan.n_rows * self.n_heads * n_splits
-                if (ahead is not None and idle >= 128 and plan.n_tiles == 0 and plan.n_rows == q.shape[0]
-                        and kernels.read_ahead_pays(ahead, plan.n_rows, with_norm=True)):
-                    chunks = idle * READ_AHEAD_BYTES_PER_CU // ahead.chunk_bytes
-                else:
-                    ahead = None
-                kernels.attn_decode(out, q, *args, plan.rows, plan.n_rows, self.n_heads, self.scale,
-                                    self.window, n_splits, part_o, part_ml, n_waves, ahead=ahead,
-                                    ahead_chunks=chunks)
-            else:
-                kernels.attn_row(out, q, *args, plan.rows, plan.n_rows, self.n_heads, self.scale,
-                                 self.window, n_splits, part_o, part_ml)
+                for s in range(0, n, TILE_Q):
+                    tiles += (q0 + s, min(TILE_Q, n - s))
+                for s in range(0, n, BIG_TILE_Q):
+                    m = min(BIG_TILE_Q, n - s)
+                    big.append((length + s + m, q0 + s, m))
+        if batch.static and rows:
+            longest = batch.max_positions  # how keys are split must not depend on lengths
+        big.sort(reverse=True)  # tiles with the most keys start first
+        return {"tiles": tiles, "rows": rows, "all_tiles": all_tiles,
+                "big_tiles": [v for _, r0, m in big for v in (r0, m)], "max_row_context": longest}
+
+    # -- the native twin ---------------------------------------------------------
+
+    def make_native(self):
+        L = native.lib()
+        base = native.array_ids(self.step_arrays_key, self.step_array_names)
+        qkv_w, out_w = kernels.weight_struct(self.qkv_w), kernels.weight_struct(self.out_w)
+        pos = self.position.native() if self.position is not None else None
+        return native.made(L.eng_make_attention(
+            self.width, self.n_heads, self.n_kv_heads, self.head_dim, self.scale, self.window,
+            ctypes.byref(qkv_w), native.ptr(self.qkv_b), ctypes.byref(out_w), native.ptr(self.out_b), pos, base),
+            "attention")
+
+    def forward(self, ctx, x, residual, cache, writes_cache=True):
+        """Fused q/k/v projection (keys and values go to their pages from its epilogue, or after
+        the position hook has rotated them), attention through the block table, output projection
+        added into ``residual``: done by the native twin."""
+        v, r = value_of(x), native.mat(residual)
+        with ctx.enter():
+            rc = native.lib().eng_mixer_forward(self.native(), ctypes.byref(ctx.c), ctypes.byref(v),
+                                                ctypes.byref(r), cache.slot, int(bool(writes_cache)))
+        native.check(rc, "attention")
 
 
 register_mixer("attention", CausalSelfAttention)

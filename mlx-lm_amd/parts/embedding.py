@@ -1,6 +1,6 @@
 """Token embedding: a row of the table for each token, written to the residual stream."""
 
-from ..ops import kernels
+from ..ops import kernels, native
 from .base import Part, TensorSpec, register_embedding
 
 
@@ -25,6 +25,12 @@ class TokenEmbedding(Part):
 
     def load(self, tensors):
         self.table = tensors[self.weight_name]
+
+    native_kind = native.EMBEDDING
+
+    def make_native(self):
+        return native.made(native.lib().eng_make_token_embedding(
+            self.table.data_ptr(), self.vocab_size, self.width, native.DT[self.table.dtype]), "token embedding")
 
     def forward(self, ctx, out, add=None):
         """Fill float32 ``out [tokens, width]``; ``add`` is ``(table, index)`` or ``None``."""

@@ -1,9 +1,11 @@
 """Feed-forward parts."""
 
+import ctypes
+
 import torch
 
-from ..ops import kernels
-from .base import FeedForward, TensorSpec, register_feed_forward
+from ..ops import kernels, native
+from .base import FeedForward, TensorSpec, register_feed_forward, value_of
 
 _TANH_GELU = ("gelu_new", "gelu_pytorch_tanh", "gelu_tanh", "gelu_approx")
 
@@ -55,10 +57,17 @@ class GeluMLP(FeedForward):
         self.fc_w, self.proj_w = kernels.for_decode(self.fc_w), kernels.for_decode(self.proj_w)
         self.first_weight = self.fc_w  # what the first product reads
 
+    def make_native(self):
+        fc_w, proj_w = kernels.weight_struct(self.fc_w), kernels.weight_struct(self.proj_w)
+        return native.made(native.lib().eng_make_gelu_mlp(
+            self.width, self.inner_padded, ctypes.byref(fc_w), native.ptr(self.fc_b), ctypes.byref(proj_w),
+            native.ptr(self.proj_b)), "gelu_mlp")
+
     def forward(self, ctx, x, residual):
-        act = ctx.scratch((x.shape[0], self.inner_padded), ctx.dtype)
-        kernels.linear(act, x, self.fc_w, self.fc_b, gelu=True)
-        kernels.linear(residual, act, self.proj_w, self.proj_b, accumulate=True, pending=ctx.pending)
+        v, r = value_of(x), native.mat(residual)
+        with ctx.enter():
+            rc = native.lib().eng_ffn_forward(self.native(), ctypes.byref(ctx.c), ctypes.byref(v), ctypes.byref(r))
+        native.check(rc, "gelu_mlp")
 
 
 register_feed_forward("gelu_mlp", GeluMLP)

@@ -1,7 +1,9 @@
 """Output heads: from the final normed rows to float32 logits."""
 
-from ..ops import kernels
-from .base import Part, TensorSpec, register_head
+import ctypes
+
+from ..ops import kernels, native
+from .base import Part, TensorSpec, register_head, value_of
 
 
 class LinearHead(Part):
@@ -26,8 +28,17 @@ class LinearHead(Part):
     def load(self, tensors):
         self.weight = kernels.for_decode(tensors[self.weight_name])
 
+    native_kind = native.HEAD
+
+    def make_native(self):
+        w = kernels.weight_struct(self.weight)
+        return native.made(native.lib().eng_make_linear_head(ctypes.byref(w)), "linear head")
+
     def forward(self, ctx, x, out):
-        kernels.linear(out, x, self.weight)
+        v, o = value_of(x), native.mat(out)
+        with ctx.enter():
+            rc = native.lib().eng_head_forward(self.native(), ctypes.byref(ctx.c), ctypes.byref(v), ctypes.byref(o))
+        native.check(rc, "linear head")
         return out
 
 

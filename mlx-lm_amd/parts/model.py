@@ -1,16 +1,10 @@
 """A decoder-only model built from a plan: embedding, scheduled layers, final norm, head."""
 
+import ctypes
+
 from ..config.plan import CacheNeed, ModelPlan, StateNeed
-from .base import (
-    BLOCKS,
-    EMBEDDINGS,
-    FEED_FORWARDS,
-    HEADS,
-    MIXERS,
-    NORMS,
-    POSITION_ENCODINGS,
-    build_part,
-)
+from ..ops import native
+from .base import BLOCKS, EMBEDDINGS, FAMILIES, HEADS, NORMS, POSITION_ENCODINGS, build_part
 
 
 class DecoderModel:
@@ -21,6 +15,8 @@ class DecoderModel:
     and the head run only on the rows whose logits are wanted, and that the
     order of layers is the plan's schedule.
     """
+
+    _native = None
 
     def __init__(self, plan: ModelPlan):
         self.plan = plan.validate()
@@ -38,17 +34,17 @@ class DecoderModel:
                 raise ValueError(
                     f"unknown block arrangement '{spec.arrangement}' (known: {sorted(BLOCKS)})"
                 )
-            self.layers.append(
-                BLOCKS[spec.arrangement](
-                    build_part(NORMS, "norm", spec.mixer_norm),
-                    build_part(MIXERS, "mixer", spec.mixer),
-                    build_part(NORMS, "norm", spec.ffn_norm),
-                    build_part(FEED_FORWARDS, "feed-forward", spec.ffn),
+            cls = BLOCKS[spec.arrangement]
+            if set(spec.parts) != set(cls.PARTS):
+                raise ValueError(
+                    f"arrangement '{spec.arrangement}' arranges {sorted(cls.PARTS)}, the plan gives {sorted(spec.parts)}"
                 )
-            )
+            built = {name: build_part(*FAMILIES[cls.PARTS[name]], part_spec) for name, part_spec in spec.parts.items()}
+            self.layers.append(cls(**built))
         self.schedule = list(plan.schedule)
         self.final_norm = build_part(NORMS, "norm", plan.final_norm)
         self.head = build_part(HEADS, "output head", plan.head)
+        self._native = None
 
     # -- tensors ------------------------------------------------------------
 
@@ -82,7 +78,7 @@ class DecoderModel:
         """What each cache slot has to hold, from the mixer of the run that writes it."""
         needs = {}
         for run in self.schedule:
-            need = self.layers[run.layer].mixer.cache_need()
+            need = self.layers[run.layer].cache_need()
             if run.writes_cache:
                 needs[run.cache] = need
             elif needs[run.cache] != need:
@@ -96,30 +92,56 @@ class DecoderModel:
                 raise TypeError(f"cache_need() must give a CacheNeed, a StateNeed or None, got {need!r}")
         return out
 
+    # -- the step arrays that parts ask for ------------------------------------
+
+    def array_providers(self):
+        """``[(first array id, key, names, function of a HostBatch)]``: one entry for each kind of
+        part that declared ``step_arrays`` (parts that share a key share the arrays)."""
+        seen, out = set(), []
+        for part in self.parts():
+            key = getattr(part, "step_arrays_key", None)
+            if key is None or key in seen:
+                continue
+            seen.add(key)
+            names = tuple(part.step_array_names)
+            out.append((native.array_ids(key, names), key, names, part.step_arrays))
+        return out
+
     # -- forward -------------------------------------------------------------
 
+    def native(self):
+        """The native model: the tree of the parts' native twins (made at first use, after ``load``)."""
+        if self._native is None:
+            L = native.lib()
+            layers = (ctypes.c_void_p * len(self.layers))(*[b.native() for b in self.layers])
+            n = len(self.schedule)
+            ints = ctypes.c_int * n
+            self._native = native.made(L.eng_make_model(
+                self.width, self.vocab_size, self.embedding.native(),
+                self.embedding_positions.native() if self.embedding_positions is not None else None,
+                len(self.layers), layers, n, ints(*[r.layer for r in self.schedule]),
+                ints(*[r.cache for r in self.schedule]), ints(*[int(r.writes_cache) for r in self.schedule]),
+                self.final_norm.native(), self.head.native()), "model")
+        return self._native
+
+    def __del__(self):
+        handle, self._native = self._native, None
+        if handle:
+            try:
+                native.lib().eng_free(handle)
+            except Exception:  # noqa: BLE001 (the interpreter may be shutting down)
+                pass
+
     def forward(self, ctx):
-        """Run the step's tokens; returns float32 logits ``[n_wanted, vocab]`` or ``None``."""
-        h = ctx.scratch((ctx.n_tokens, self.width), "float32")
-        add = self.embedding_positions.embedding_term(ctx) if self.embedding_positions else None
-        self.embedding.forward(ctx, h, add)
-        pending = ctx.pending
-        for run in self.schedule:
-            block = self.layers[run.layer]
-            # a block that does not know of pending sums gets the stream with everything added
-            pending.allowed = getattr(block, "handles_pending", False)
-            if not pending.allowed:
-                pending.settle()
-            block.forward(ctx, h, ctx.cache_view(run.cache), run.writes_cache)
-        pending.allowed = False
-        if ctx.n_wanted == 0 or not getattr(self.final_norm, "settles_pending", False):
-            pending.settle()
-        if ctx.n_wanted == 0:
-            return None
-        if ctx.wants_every_row:
-            x = self.final_norm.forward(ctx, h)
-        else:
-            x = self.final_norm.forward(ctx, h, rows=ctx.wanted_rows, n_rows=ctx.n_wanted)
-        logits = ctx.logits_out(ctx.n_wanted, self.vocab_size)
-        self.head.forward(ctx, x, logits)
+        """Run the step's tokens; returns float32 logits ``[n_wanted, vocab]`` or ``None``.
+
+        One call into the native host, which walks the parts: embedding (+ position term),
+        the scheduled blocks, the final norm on the wanted rows only, the head."""
+        logits = None
+        if ctx.n_wanted:
+            logits = ctx.logits_out(ctx.n_wanted, self.vocab_size)
+            ctx.c.logits, ctx.c.logits_rows = logits.data_ptr(), logits.shape[0]
+        with ctx.enter():
+            rc = native.lib().eng_model_forward(self.native(), ctypes.byref(ctx.c))
+        native.check(rc, "the model's step")
         return logits

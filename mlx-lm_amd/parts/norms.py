@@ -1,6 +1,8 @@
 """Norms over the width of the residual stream."""
 
-from ..ops import kernels
+import ctypes
+
+from ..ops import kernels, native
 from .base import Norm, TensorSpec, register_norm
 
 
@@ -32,26 +34,26 @@ class LayerNorm(Norm):
     settles_pending = True  # adds a sum that is pending on ``x`` before (or while) it norms the rows
     reads_ahead = True  # ``forward`` takes ``ahead``, the weights that its result meets first
 
+    def make_native(self):
+        return native.made(native.lib().eng_make_layernorm(self.width, self.eps, native.ptr(self.weight),
+                                                           native.ptr(self.bias)), "layernorm")
+
     def forward(self, ctx, x, rows=None, n_rows=None, lazy=False, ahead=None):
         """``ahead``: the weights of the product that reads the result first, if its caller knows
-        them: a kernel here that leaves most of the GPU idle reads them into the caches meanwhile."""
-        pending = ctx.pending
-        if pending.waits_on(x):
-            if rows is None and pending.can_norm(x):
-                # the last projection split its sum: add the parts and norm the new rows in one kernel
-                out = ctx.scratch((x.shape[0], self.width), ctx.dtype)
-                if ahead is not None and not kernels.read_ahead_pays(ahead, x.shape[0]):
-                    ahead = None
-                pending.settle_normed(out, self.weight, self.bias, self.eps, ahead=ahead)
-                return out
-            pending.settle()
-        if lazy and rows is None:
-            # the consumer's first matrix product may norm the rows itself
+        them: a kernel here that leaves most of the GPU idle reads them into the caches meanwhile.
+        (The native twin does the work: a pending sum is added, fused with the norm where the
+        kernel takes it; with ``lazy`` the norm may be left to the consumer's first product.)"""
+        out = native.EngValue()
+        xm = native.mat(x)
+        with ctx.enter():
+            rc = native.lib().eng_norm_forward(
+                self.native(), ctypes.byref(ctx.c), ctypes.byref(xm), native.ptr(rows), int(n_rows or 0),
+                int(bool(lazy)), ctypes.byref(ahead.c) if ahead is not None and hasattr(ahead, "c") else None,
+                ctypes.byref(out))
+        native.check(rc, "layernorm")
+        if out.lazy:
             return kernels.NormedInput(ctx.scratch, x, self.weight, self.bias, self.eps, ctx.dtype)
-        n = x.shape[0] if n_rows is None else n_rows
-        out = ctx.scratch((n, self.width), ctx.dtype)
-        kernels.layernorm(out, x, self.weight, self.bias, self.eps, rows=rows)
-        return out
+        return ctx.tensor(out.m)
 
 
 register_norm("layernorm", LayerNorm)

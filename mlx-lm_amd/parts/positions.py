@@ -1,5 +1,6 @@
 """Position encodings."""
 
+from ..ops import native
 from .base import PositionEncoding, TensorSpec, register_position_encoding
 
 
@@ -10,6 +11,9 @@ class NoPositions(PositionEncoding):
 
     def __init__(self, prefix=""):
         super().__init__(prefix)
+
+    def make_native(self):
+        return None  # no part at all
 
 
 class LearnedPositions(PositionEncoding):
@@ -36,6 +40,10 @@ class LearnedPositions(PositionEncoding):
 
     def load(self, tensors):
         self.table = tensors[self.weight_name]
+
+    def make_native(self):
+        return native.made(native.lib().eng_make_learned_positions(
+            self.table.data_ptr(), self.max_positions, self.width, native.DT[self.table.dtype]), "learned positions")
 
     def embedding_term(self, ctx):
         return self.table, ctx.positions

@@ -42,7 +42,7 @@ def test_num_key_value_heads_is_read_and_not_used():
     # mlx_lm/models/gpt2.py:24-26,57-58: the key is kept, keys and values are shaped with n_head
     args = ModelArgs.from_dict(dict(helpers.TINY_A, num_key_value_heads=1))
     assert args.num_key_value_heads == 1
-    mixer = Model.plan(args).layers[0].mixer
+    mixer = Model.plan(args).layers[0].parts["mixer"]
     assert mixer.params["n_kv_heads"] == mixer.params["n_heads"] == args.n_head
 
 

@@ -118,15 +118,6 @@ def test_thousands_of_keys_split_over_blocks(tmp_path, monkeypatch, dtype, use_g
     n, n_prompt = 3340, 3300
     tokens = helpers.random_tokens(n, config["vocab_size"], seed=31)
     want = _plain_logits(weights, config, tokens, dtype)
-    seen = []
-    for name in ("attn_decode", "attn_row"):
-        inner = getattr(kernels, name)
-
-        def counted(*a, _inner=inner, **kw):
-            seen.append(a[11] if len(a) > 11 else kw.get("n_splits", 1))
-            return _inner(*a, **kw)
-
-        monkeypatch.setattr(kernels, name, counted)
     model, _ = load_model(str(tmp_path), dtype=dtype)
     eng = Engine(model, dtype=dtype, page_size=16, n_pages=(n + 63) // 64 * 4, max_requests=2, use_graphs=use_graphs)
     eng.add_request("r")
@@ -135,7 +126,7 @@ def test_thousands_of_keys_split_over_blocks(tmp_path, monkeypatch, dtype, use_g
     rows = [eng.step([StepEntry("r", tokens[2000:n_prompt], [n_prompt - 2001])]).clone()]
     for i in range(n_prompt, n):
         rows.append(eng.step([StepEntry("r", tokens[i : i + 1], [0])]).clone())
-    assert seen and max(seen) > 1, "no step split a row's keys"
+    assert eng.stats.key_splits_most > 1, "no step split a row's keys"
     _close(torch.cat(rows), want[n_prompt - 1 :], dtype, "decoded after 3,300 tokens")
 
 
@@ -183,20 +174,7 @@ def test_split_sums_in_the_engine(folders, monkeypatch, name, sharp, use_graphs)
     from mlx_lm_amd.ops import kernels
     from mlx_lm_amd.utils import load_model
 
-    calls = {"normed": 0, "plain": 0}
-    settle_normed, settle = kernels.PendingSum.settle_normed, kernels.PendingSum.settle
-
-    def count_normed(self, *a, **kw):
-        calls["normed"] += 1
-        return settle_normed(self, *a, **kw)
-
-    def count_plain(self):
-        calls["plain"] += self.target is not None
-        return settle(self)
-
     monkeypatch.setattr(kernels, "force_splits", 2)
-    monkeypatch.setattr(kernels.PendingSum, "settle_normed", count_normed)
-    monkeypatch.setattr(kernels.PendingSum, "settle", count_plain)
     folder, config, weights = folders[(name, sharp)]
     P = config["n_positions"]
     lengths = [min(P, n) for n in (100, 37, 128, 64, 90, 17)]
@@ -216,14 +194,14 @@ def test_split_sums_in_the_engine(folders, monkeypatch, name, sharp, use_graphs)
             i += len(e["want"])
         for rid in s["end"]:
             eng.end_request(rid)
-    assert calls["normed"] > 2 * len(model.layers)  # the fused kernel ran, in many steps
+    assert eng.stats.settle_normed > 2 * len(model.layers)  # the fused kernel ran, in many steps
     # a few tokens of which only the last is wanted: the last block's sum is added without a norm,
     # since the final norm gathers its rows
     extra = helpers.random_tokens(11, config["vocab_size"], seed=77)
     eng.add_request("extra")
-    before = calls["plain"]
+    before = eng.stats.settle_plain
     got["extra"] = [eng.step([StepEntry("extra", extra, [10])]).clone()]
-    assert calls["plain"] == before + 1
+    assert eng.stats.settle_plain == before + 1
     want = _plain_logits(weights, config, extra, "bfloat16")[10:]
     _close(got.pop("extra")[0], want, "bfloat16", "split sums, gathered rows")
     for rid, toks in tokens.items():

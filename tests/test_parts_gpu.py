@@ -284,7 +284,7 @@ def _register_toys():
             ffns = [ffn("l0.ff."), PartSpec("toy_hashed_experts", {"width": a.width, "inner": a.inner,
                                                                      "n_experts": a.experts}, "l1.ff."),
                     ffn("l2.ff.")]
-            layers = [LayerSpec("pre_norm", norm(f"l{i}.n1."), m, norm(f"l{i}.n2."), f)
+            layers = [LayerSpec("pre_norm", dict(mixer_norm=norm(f"l{i}.n1."), mixer=m, ffn_norm=norm(f"l{i}.n2."), ffn=f))
                       for i, (m, f) in enumerate(zip(mixers, ffns))]
             # layer 0 runs twice (two cache slots); the last run of layer 1 reads the
             # keys and values that its first run wrote
@@ -498,11 +498,13 @@ def _register_running_sum():
                 return PartSpec("layernorm", {"width": a.width, "eps": 1e-5}, p)
 
             layers = [
-                LayerSpec("pre_norm", norm("l0.n1."), PartSpec("toy_running_sum", {"width": a.width}, "l0.mix."),
-                          norm("l0.n2."), PartSpec("gelu_mlp", {"width": a.width, "inner": a.inner}, "l0.ff.")),
-                LayerSpec("pre_norm", norm("l1.n1."),
-                          PartSpec("attention", {"width": a.width, "n_heads": 2, "head_dim": a.width // 2}, "l1.mix."),
-                          norm("l1.n2."), PartSpec("gelu_mlp", {"width": a.width, "inner": a.inner}, "l1.ff.")),
+                LayerSpec("pre_norm", dict(
+                    mixer_norm=norm("l0.n1."), mixer=PartSpec("toy_running_sum", {"width": a.width}, "l0.mix."),
+                    ffn_norm=norm("l0.n2."), ffn=PartSpec("gelu_mlp", {"width": a.width, "inner": a.inner}, "l0.ff."))),
+                LayerSpec("pre_norm", dict(
+                    mixer_norm=norm("l1.n1."),
+                    mixer=PartSpec("attention", {"width": a.width, "n_heads": 2, "head_dim": a.width // 2}, "l1.mix."),
+                    ffn_norm=norm("l1.n2."), ffn=PartSpec("gelu_mlp", {"width": a.width, "inner": a.inner}, "l1.ff."))),
             ]
             return ModelPlan(
                 width=a.width, vocab_size=a.vocab, max_positions=a.max_len,
