@@ -2,15 +2,20 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--dtype bfloat16]
 
-Prints one JSON line.  ``value`` is decoded tokens a second at the given batch
-(default 8): K timed decode steps after W untimed ones, every request starting
-from a 512-token prompt (the reference's benchmark draws uniform random
-prompts and switches end-of-sequence off, mlx_lm/benchmark.py:118-124).
-``prefill`` is one step of 2 x 1,024 prompt tokens (the best of five: a step
-whose shape keeps coming back is replayed from its recorded graph, as in the
-serving path); ``points`` holds decode at
-batch 1 and 64; ``roofline`` the bytes a decode step has to read over its time.
-Weights are random (seeded), data synthetic.
+Prints one JSON line.  ``value`` is decoded tokens a second at the given batch (default 8):
+K timed decode steps, every request starting from a 512-token prompt, so that the first timed
+step runs at context 512 and, with the default K, the last at the model's last position but one (511 steps)
+(the reference's benchmark draws uniform random prompts and switches end-of-sequence off,
+mlx_lm/benchmark.py:118-124; it warms up, then times five trials and reports their mean,
+mlx_lm/benchmark.py:152-176).  The W warm-up steps run before, on requests of their own, so
+that they do not move the timed steps' context.  ``config`` gives the context range as
+``ctx_from``/``ctx_to``.  ``prefill`` is one step of 2 x 1,024 prompt tokens: two untimed
+warm-up trials (a step whose shape keeps coming back is replayed from its recorded graph, as
+in the serving path), then the mean of five timed ones, each listed in ``trials_ms``.
+``points`` holds decode at batch 1 and 64 over the same steps and, for all three batch sizes,
+at context 1,000; ``roofline`` the bytes a decode step has to read (every weight once, the live
+requests' keys and values at each step's context) over its time, ``roofline_points`` the same
+fraction for every point.  Weights are random (seeded), data synthetic.
 """
 
 import argparse
@@ -32,39 +37,14 @@ XL = dict(model_type="gpt2", n_layer=48, n_embd=1600, n_head=25, n_inner=6400, v
 
 
 def build_model(config, dtype, seed):
-    """Random weights straight onto the GPU, through the architecture's own
-    random_weights, sanitize and strict placement (no file in between)."""
+    """Random weights under a checkpoint's names, loaded the way a folder's are."""
     from mlx_lm_amd.config import get_model_classes
-    from mlx_lm_amd.weights.loader import place_tensors, resolve_dtype
+    from mlx_lm_amd.utils import model_from_tensors
 
     model_cls, args_cls = get_model_classes(config)
-    args = args_cls.from_dict(config)
-    model = model_cls(args)
-    tensors = model.sanitize(model_cls.random_weights(args, seed, "a"))
-    model.decoder.load_tensors(place_tensors(model.decoder.expected_tensors(), tensors, dtype, "cuda:0"))
-    model.dtype = resolve_dtype(dtype)
-    model.device = "cuda:0"
-    return model, args
-
-
-def weight_bytes(model):
-    """Bytes of every tensor a decode step uses once (the position table is read row-wise: left out)."""
-    total = 0
-    seen = {}
-    for part in model.decoder.parts():
-        for name, spec in part.tensors().items():
-            seen[name] = spec
-    import torch
-
-    esize = torch.empty((), dtype=model.dtype).element_size()
-    for name, spec in seen.items():
-        if name.endswith("wpe.weight"):
-            continue
-        n = 1
-        for s in spec.shape:
-            n *= s
-        total += n * (esize if spec.role == "matrix" else 4)
-    return total
+    tensors = model_cls.random_weights(args_cls.from_dict(config), seed, "a")
+    model = model_from_tensors(config, tensors, dtype=dtype, device="cuda:0")
+    return model, model.args
 
 
 def prefill_flops(args, n_seqs, seq_len):
@@ -75,52 +55,77 @@ def prefill_flops(args, n_seqs, seq_len):
     return per_token * n_seqs * seq_len + attn + head
 
 
-def run_decode(engine, batch, prompt_len, steps, warmup, vocab, seed):
-    """`batch` requests of `prompt_len` tokens through the scheduler (the loop that generation uses:
-    a step is launched while the host reads the tokens of the one before); times `steps` decode steps."""
+def _scheduler(engine, batch, prompt_len):
+    from mlx_lm_amd.engine.scheduler import Scheduler
+    from mlx_lm_amd.generate import make_sample_fn
+
+    # all prompts go in one step, so that every request decodes from the same context on
+    return Scheduler(engine, make_sample_fn(), max_num_seqs=batch,
+                     max_num_batched_tokens=batch * (prompt_len + 1), prefill_step_size=prompt_len)
+
+
+def _start(engine, sched, batch, prompt_len, vocab, seed, tag):
     import torch
 
-    from mlx_lm_amd.engine.scheduler import Request, Scheduler
-    from mlx_lm_amd.generate import make_sample_fn
+    from mlx_lm_amd.engine.scheduler import Request
 
     g = torch.Generator().manual_seed(seed)
     prompts = torch.randint(0, vocab, (batch, prompt_len), generator=g).tolist()
-    # prompts go in four at a time to bound the step's scratch memory
-    sched = Scheduler(engine, make_sample_fn(), max_num_seqs=batch,
-                      max_num_batched_tokens=4 * prompt_len + batch, prefill_step_size=prompt_len)
-    rids = [("bench", batch, i) for i in range(batch)]
+    rids = [(tag, batch, i) for i in range(batch)]
     for i, rid in enumerate(rids):
-        sched.add(Request(rid, prompts[i], max_tokens=10**6, seed=i))  # greedy; the timed steps end it
+        sched.add(Request(rid, prompts[i], max_tokens=10**6, seed=i))  # greedy; the caller ends it
     while sched.waiting or not all(r.decoding for r in sched.running):
         sched.step()
-    for _ in range(warmup):
-        sched.step()
+    return rids
+
+
+def run_decode(engine, batch, prompt_len, steps, warmup, vocab, seed):
+    """``batch`` requests of ``prompt_len`` tokens through the scheduler (the loop that generation
+    uses: a step is launched while the host reads the tokens of the one before); times ``steps``
+    decode steps.  Returns ``(seconds, contexts)``: the context each timed step ran at."""
+    import torch
+
+    sched = _scheduler(engine, batch, prompt_len)
+    if warmup > 0:  # on requests of their own, so that the timed steps start at the prompt's end
+        rids = _start(engine, sched, batch, prompt_len, vocab, seed + 1000, "warm")
+        for _ in range(warmup):
+            sched.step()
+        torch.cuda.synchronize()
+        for rid in rids:
+            sched.abort(rid)
+        while sched.has_work:
+            sched.step()
+    rids = _start(engine, sched, batch, prompt_len, vocab, seed, "bench")
     torch.cuda.synchronize()
-    ctx0 = sum(engine.context_len(rid) for rid in rids) / batch
+    ctx0 = engine.context_len(rids[0])
     t0 = time.perf_counter()
     n_out = 0
     for _ in range(steps):
         n_out += len(sched.step())  # every step hands out one token per request
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    ctx1 = sum(engine.context_len(rid) for rid in rids) / batch
     if n_out != batch * steps:
         raise RuntimeError(f"{n_out} tokens came out of {steps} steps of {batch} requests")
-    for rid in rids:
-        sched.abort(rid)
-    return dt, (ctx0 + ctx1) / 2
+    for rid in rids:  # (a request that has reached the model's last position is over already)
+        if engine.has_request(rid):
+            sched.abort(rid)
+    while sched.has_work:
+        sched.step()
+    # steps overlap: the first timed call launches the step at the prompt's end, and every call
+    # hands out the tokens of the step before, so `steps` calls ran `steps` steps
+    return dt, list(range(ctx0, ctx0 + steps))
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--steps", type=int, default=512)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--layers", type=int, default=XL["n_layer"], help="run fewer layers than GPT-2 XL has")
     ap.add_argument("--prompt-len", type=int, default=512)
-    ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the points at context 1,000")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU; this engine does not run on several (asked for %d)" % a.gpus)
@@ -136,19 +141,22 @@ def main():
     model, args = build_model(config, a.dtype, seed=2)
     print(f"[bench] model built in {time.perf_counter() - t_build:.1f} s", file=sys.stderr, flush=True)
     P, V = args.n_positions, args.vocab_size
-    steps = min(a.steps, P - a.prompt_len - a.warmup)
+    # the step after a prompt of p tokens runs at context p; the token that takes the last position
+    # (P - 1) is never fed, so the last step runs at context P - 2
+    steps = max(1, min(a.steps, P - 1 - a.prompt_len))
     # (as the serving path makes it, generate.engine_for: steps of a shape that keeps coming back are recorded)
     engine = Engine(model, dtype=a.dtype, page_size=16, max_tokens=64 * P, max_requests=64, record_prompt_steps=True)
     esize = 2 if a.dtype == "bfloat16" else 4
-    kv_bytes_per_token = 2 * args.n_embd * args.n_layer * esize
-    w_bytes = weight_bytes(model)
+    kv_bytes_per_token = engine.cache.bytes_per_token()
+    w_bytes = model.decoder.bytes_read_per_step(esize)
 
     # prefill: 2 x 1,024 tokens in one step
     g = torch.Generator().manual_seed(0)
     n_seqs, seq_len = 2, 1024
     prompts = torch.randint(0, V, (n_seqs, seq_len), generator=g).tolist()
     pre_ms = []
-    for trial in range(5):  # the third records the step, the later ones replay it
+    warm_trials, timed_trials = 3, 5  # (the third sighting of the shape records it; the timed ones replay)
+    for trial in range(warm_trials + timed_trials):
         for i in range(n_seqs):
             engine.add_request(("pre", i))
         torch.cuda.synchronize()
@@ -158,38 +166,54 @@ def main():
         pre_ms.append((time.perf_counter() - t0) * 1e3)
         for i in range(n_seqs):
             engine.end_request(("pre", i))
-    pre = min(pre_ms[1:])
+    timed = pre_ms[warm_trials:]
+    pre = sum(timed) / len(timed)
     flops = prefill_flops(args, n_seqs, seq_len)
     prefill = {"value": round(n_seqs * seq_len / (pre / 1e3), 1), "tokens": n_seqs * seq_len,
-               "ms": round(pre, 3), "frac": round(flops / (pre / 1e3) / PEAK_FLOPS[a.dtype], 4)}
-    print(f"[bench] prefill {prefill} (trials, ms: {[round(t, 2) for t in pre_ms]})", file=sys.stderr, flush=True)
+               "ms": round(pre, 3), "frac": round(flops / (pre / 1e3) / PEAK_FLOPS[a.dtype], 4),
+               "trials_ms": [round(t, 3) for t in timed]}
+    print(f"[bench] prefill {prefill} (warm-up trials, ms: {[round(t, 2) for t in pre_ms[:warm_trials]]})",
+          file=sys.stderr, flush=True)
 
-    results = {}
-    batches = [a.batch] if a.no_points else sorted({1, a.batch, 64})
-    for b in batches:
-        k = steps if b == a.batch else min(steps, 64)
-        dt, mean_ctx = run_decode(engine, b, a.prompt_len, k, a.warmup, V, seed=b)
-        results[b] = (b * k / dt, dt / k * 1e3, mean_ctx, k)
-        print(f"[bench] decode batch {b}: {results[b][0]:.1f} tok/s, {results[b][1]:.3f} ms/step",
-              file=sys.stderr, flush=True)
+    def measure(batch, prompt_len, k):
+        dt, contexts = run_decode(engine, batch, prompt_len, k, a.warmup, V, seed=batch)
+        ms = dt / k * 1e3
+        step_bytes = w_bytes + batch * (sum(contexts) / len(contexts)) * kv_bytes_per_token
+        gbs = step_bytes / (ms / 1e3) / 1e9
+        print(f"[bench] decode batch {batch}, context {contexts[0]} to {contexts[-1]}: {batch * k / dt:.1f} tok/s, "
+              f"{ms:.3f} ms/step, {gbs:.0f} GB/s", file=sys.stderr, flush=True)
+        return {"tps": batch * k / dt, "ms": ms, "gbs": gbs, "ctx": (contexts[0], contexts[-1]), "k": k}
 
-    tps, ms, mean_ctx, k = results[a.batch]
-    step_bytes = w_bytes + a.batch * mean_ctx * kv_bytes_per_token
-    achieved = step_bytes / (ms / 1e3) / 1e9
+    main_point = measure(a.batch, a.prompt_len, steps)
+    points, fracs = {}, {f"decode_b{a.batch}": round(main_point["gbs"] / PEAK_HBM_GBS, 4)}
+    if not a.no_points:
+        for b in (1, 64):
+            r = main_point if b == a.batch else measure(b, a.prompt_len, steps)
+            points[f"decode_b{b}"] = round(r["tps"], 1)
+            fracs[f"decode_b{b}"] = round(r["gbs"] / PEAK_HBM_GBS, 4)
+        late = min(1000, P - 8)
+        for b in sorted({1, a.batch, 64}):
+            r = measure(b, late, min(steps, P - 1 - late))
+            points[f"decode_b{b}_ctx{late}"] = round(r["tps"], 1)
+            fracs[f"decode_b{b}_ctx{late}"] = round(r["gbs"] / PEAK_HBM_GBS, 4)
+
     line = {
         "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens (GPT-2 XL)",
-        "value": round(tps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": k, "warmup": a.warmup,
-        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
+        "value": round(main_point["tps"], 1), "unit": "tokens/s", "n_gpus": 1, "steps": main_point["k"],
+        "warmup": a.warmup, "ms_per_step": round(main_point["ms"], 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if a.dtype == "bfloat16" else "fp32",
         "data": "synthetic uniform random token ids, random weights (seed 2)",
         "config": {"model": "gpt2-xl layer sizes", "n_layer": a.layers, "n_layer_full": XL["n_layer"],
                    "n_embd": args.n_embd, "n_head": args.n_head, "n_inner": args.n_inner,
-                   "vocab_size": V, "n_positions": P, "global_batch": a.batch,
-                   "seq_len": P, "prompt_len": a.prompt_len, "page_size": 16, "parallelism": "none"},
+                   "vocab_size": V, "n_positions": P, "layer_norm_epsilon": args.layer_norm_epsilon,
+                   "global_batch": a.batch, "seq_len": P, "prompt_len": a.prompt_len,
+                   "ctx_from": main_point["ctx"][0], "ctx_to": main_point["ctx"][1], "page_size": 16,
+                   "parallelism": "none"},
         "prefill": prefill,
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
-        "points": {f"decode_b{b}": round(results[b][0], 1) for b in results if b in (1, 64)},
+        "roofline": {"bound": "hbm", "achieved": round(main_point["gbs"], 1), "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": round(main_point["gbs"] / PEAK_HBM_GBS, 4)},
+        "points": points,
+        "roofline_points": fracs,
     }
     print(json.dumps(line))
 

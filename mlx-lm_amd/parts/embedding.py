@@ -26,6 +26,10 @@ class TokenEmbedding(Part):
     def load(self, tensors):
         self.table = tensors[self.weight_name]
 
+    def reads_rows_of(self):
+        """Tensors of which a step reads a row per token, not all."""
+        return (self.weight_name,)
+
     native_kind = native.EMBEDDING
 
     def make_native(self):

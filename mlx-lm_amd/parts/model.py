@@ -72,6 +72,23 @@ class DecoderModel:
         for part in self.parts():
             part.load(tensors)
 
+    def bytes_read_per_step(self, dtype_size):
+        """Bytes of the tensors that a step reads whole, each counted once.  A table that a part
+        reads row by row (``reads_rows_of()`` names it: an embedding, a position table) does not
+        count unless another part reads all of it (a tied head does)."""
+        whole, by_rows = {}, {}
+        for part in self.parts():
+            rows = set(part.reads_rows_of()) if hasattr(part, "reads_rows_of") else set()
+            for name, spec in part.tensors().items():
+                (by_rows if name in rows else whole)[name] = spec
+        total = 0
+        for spec in whole.values():
+            n = 1
+            for s in spec.shape:
+                n *= s
+            total += n * (dtype_size if spec.role == "matrix" else 4)
+        return total
+
     # -- cache ---------------------------------------------------------------
 
     def cache_needs(self):

@@ -41,6 +41,10 @@ class LearnedPositions(PositionEncoding):
     def load(self, tensors):
         self.table = tensors[self.weight_name]
 
+    def reads_rows_of(self):
+        """Tensors of which a step reads a row per token, not all."""
+        return (self.weight_name,)
+
     def make_native(self):
         return native.made(native.lib().eng_make_learned_positions(
             self.table.data_ptr(), self.max_positions, self.width, native.DT[self.table.dtype]), "learned positions")

@@ -43,17 +43,26 @@ def load_model(model_path, dtype="bfloat16", device="cuda:0", model_config=None,
     config = load_config(model_path)
     if model_config:
         config.update(model_config)
+    return model_from_tensors(config, read_safetensors(model_path), dtype, device, get_model_classes), config
+
+
+def model_from_tensors(config, weights, dtype="bfloat16", device="cuda:0",
+                       get_model_classes=_default_model_classes):
+    """The model that ``config`` names, given ``weights`` under a checkpoint's names: look the
+    architecture up, make its typed arguments and the model, ``sanitize``, load strictly (one
+    error that lists every missing, unexpected and misshapen tensor), set dtype and device.
+    What ``load_model`` does after reading the folder; callers that make their weights
+    themselves (a benchmark's random ones) come in here."""
     model_cls, args_cls = get_model_classes(config)
     args = args_cls.from_dict(config)
     model = model_cls(args)
-    weights = read_safetensors(model_path)
     if hasattr(model, "sanitize"):
         weights = model.sanitize(weights)
     placed = place_tensors(model.decoder.expected_tensors(), weights, dtype, device)
     model.decoder.load_tensors(placed)
     model.dtype = resolve_dtype(dtype)
     model.device = device
-    return model, config
+    return model
 
 
 def load_tokenizer(model_path, eos_token_ids=None):
