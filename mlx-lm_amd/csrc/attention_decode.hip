@@ -234,10 +234,10 @@ DEFINE_LAST_ERROR(mlxlm_last_error)
 
 template <int CPK>
 static void launch(const DecodeArgs& p, int n_rows, int n_waves, hipStream_t stream) {
-  // reading blocks for the CUs that the rows leave idle (256 CUs), if there are eight or more
+  // reading blocks for the CUs that the rows leave idle, if there are eight or more
   int extra_y = 0;
   if (p.ahead && p.ahead_chunks > 0) {
-    extra_y = (256 - n_rows * p.n_heads * p.n_splits) / n_rows;
+    extra_y = (n_compute_units() - n_rows * p.n_heads * p.n_splits) / n_rows;
     if (extra_y * n_rows < 8) extra_y = 0;
   }
   hipLaunchKernelGGL(attn_decode_kernel<CPK>, dim3(n_rows, p.n_heads + extra_y, p.n_splits), dim3(64 * n_waves), 0, stream, p);

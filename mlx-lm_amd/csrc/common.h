@@ -142,7 +142,25 @@ __device__ __forceinline__ float block_max(float v, float* red) {
 }
 
 // ---------------------------------------------------------------------------
-// host side: one error string per thread, returned codes are 0 (ok) or 1.
+// host side: the device's size; one error string per thread, returned codes are 0 (ok) or 1.
+
+// Dies (XCDs) of the GPU: consecutive blocks of a launch go to the dies in turn, and each die has
+// an L2 of its own.  (Kernels that deal tiles or chunks to dies index with it too.)
+#define N_DIES 8
+
+// Compute units of the current device, asked of the device once (256 on an MI355X).
+static inline int n_compute_units() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      n = v;
+    else
+      n = 256;
+  }
+  return n;
+}
 
 static thread_local char g_err[512];
 

@@ -38,18 +38,7 @@ extern "C" void eng_set_hooks(eng_resolver_t resolver, eng_callback_t callback) 
   g_callback = callback;
 }
 
-extern "C" int eng_compute_units(void) {
-  static int n = 0;
-  if (n == 0) {
-    int dev = 0, v = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-      n = v;
-    else
-      n = 256;
-  }
-  return n;
-}
+extern "C" int eng_compute_units(void) { return n_compute_units(); }
 
 template <typename F>
 struct Entry {
@@ -293,6 +282,7 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
   if (out.rows != M || out.cols != N) FAIL("linear: out is [%d,%d], want [%d,%d]", out.rows, out.cols, M, N);
   if (a.m.dtype != w.dtype || (w.dtype != DT_F32 && w.dtype != DT_BF16))
     FAIL("linear: a and w must share float32 or bfloat16");
+  if (!w.w && !(w.packed && w.dtype == DT_BF16)) FAIL("linear: the weights have no memory");
   if (M == 0) return 0;
   int flags = gelu ? GEMM_GELU : 0;
   if (accumulate) {
@@ -376,8 +366,9 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
       if (n_splits > 1 && pending) TRY(settle(ctx, pending));  // the workspace is about to be written again
     }
     if (n_splits < 1) n_splits = 1;
-    KERNEL(k_gemm_bf16, ctx, out.p, A.p, w.w, bias, M, N, K, A.ld, w.ldw, out.ld, flags, variant, n_splits,
-           n_splits > 1 ? ws : nullptr, n_splits > 1 ? ws_floats : (size_t)0, ctx->stream);
+    // (weights kept only in the packed order are read in that order: row stride 0 says so)
+    KERNEL(k_gemm_bf16, ctx, out.p, A.p, w.w ? w.w : w.packed, bias, M, N, K, A.ld, w.w ? w.ldw : 0, out.ld, flags,
+           variant, n_splits, n_splits > 1 ? ws : nullptr, n_splits > 1 ? ws_floats : (size_t)0, ctx->stream);
     if (n_splits > 1) {
       if (accumulate && pending && pending->allowed) {
         pending->target = (float*)out.p, pending->rows = M, pending->cols = N, pending->ld = out.ld;

@@ -40,7 +40,16 @@ struct GemmArgs {
   // K split over blockIdx.y (tile kernel, 128 x 128): partial sums [n_splits][M][N] go to ws
   float* ws;
   int n_splits, blocks_per_split;
+  // W in the decode kernels' packed order instead of row-major (ldw == 0 at the entry point):
+  // tiles of 16 features x 64 k (1024 elements), zero padded, w_kblocks of them a feature block;
+  // in a tile the 8 values k = 16 g + 8 h + 0..7 of feature f lie at ((4 h + g) * 16 + f) * 8.
+  int w_packed, w_kblocks;
 };
+
+// Element offset of the 16-byte piece `piece` (k = 8 piece ..) of feature row n in k-block 0.
+__device__ __forceinline__ int packed_piece(int n, int piece, int w_kblocks) {
+  return (n >> 4) * w_kblocks * 1024 + ((((piece & 1) << 2) + (piece >> 1)) * 16 + (n & 15)) * 8;
+}
 
 __device__ __forceinline__ void store_out(const GemmArgs& p, int m, int n, float v) {
   if (p.bias) v += p.bias[n];
@@ -153,8 +162,13 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
   const int lds_off0 = (tid >> 3) * LDS_STRIDE + (tid & 7) * 8;  // piece i lies ROW_STEP rows further down
 #pragma unroll
   for (int i = 0; i < PA; ++i) a_off[i] = row_inside(m0 + (tid >> 3) + ROW_STEP * i, p.M) * p.lda + (tid & 7) * 8;
+  // (packed weights: a k-block further on is 1024 elements further on, not 64)
+  const int wmul = p.w_packed ? 16 : 1;
 #pragma unroll
-  for (int i = 0; i < PB; ++i) b_off[i] = row_inside(n0 + (tid >> 3) + ROW_STEP * i, p.N) * p.ldw + (tid & 7) * 8;
+  for (int i = 0; i < PB; ++i) {
+    const int n = row_inside(n0 + (tid >> 3) + ROW_STEP * i, p.N);
+    b_off[i] = p.w_packed ? packed_piece(n, tid & 7, p.w_kblocks) : n * p.ldw + (tid & 7) * 8;
+  }
   const int kc_mine = (tid & 7) * 8;
   // this split's k-blocks (all of them without a split); the offsets start at its first column
   const int kb_lo = SPLIT ? blockIdx.y * p.blocks_per_split : 0;
@@ -164,7 +178,7 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
 #pragma unroll
     for (int i = 0; i < PA; ++i) a_off[i] += k_lo;
 #pragma unroll
-    for (int i = 0; i < PB; ++i) b_off[i] += k_lo;
+    for (int i = 0; i < PB; ++i) b_off[i] += k_lo * wmul;
   }
 
   uint4 ra[2][PA], rb[2][PB];
@@ -174,10 +188,11 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
     // columns) and zeroed when it goes to LDS: zeroing it here would make the
     // loads wait at once
     const int kk = (k_lo + k0 + kc_mine < p.K) ? k0 : p.K - 8 - kc_mine - k_lo;
+    const int kw = p.w_packed ? k0 * 16 : kk;  // (packed weights are padded with zeros to whole k-blocks)
 #pragma unroll
     for (int i = 0; i < PA; ++i) xa[i] = *(const uint4*)(p.A + a_off[i] + kk);
 #pragma unroll
-    for (int i = 0; i < PB; ++i) xb[i] = *(const uint4*)(p.W + b_off[i] + kk);
+    for (int i = 0; i < PB; ++i) xb[i] = *(const uint4*)(p.W + b_off[i] + kw);
   };
   auto store_lds = [&](int stage, const uint4 (&xa)[PA], const uint4 (&xb)[PB], int k0) {
     const bool in = k_lo + k0 + kc_mine < p.K;
@@ -231,7 +246,7 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
 #pragma unroll
     for (int i = 0; i < PA; ++i) xa[i] = *(const uint4*)(p.A + a_off[i] + k0);
 #pragma unroll
-    for (int i = 0; i < PB; ++i) xb[i] = *(const uint4*)(p.W + b_off[i] + k0);
+    for (int i = 0; i < PB; ++i) xb[i] = *(const uint4*)(p.W + b_off[i] + k0 * wmul);
   };
   // multiply out of `stage` and, a quarter with each 16 columns, move the next k-block (in
   // registers since the iteration before) into the other stage, which nobody reads any more
@@ -451,6 +466,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(GemmArgs p) {
   const int koff = (lane >> 4) * 16;
   const bool wvalid = wrow < p.N;
   const uint16_t* wrow_p = p.W + (size_t)(wvalid ? wrow : 0) * p.ldw;
+  // packed weights: the lane's two pieces of a k-block are pieces 2 g and 2 g + 1 of its feature
+  const uint16_t* wpack0 = p.W + packed_piece(wvalid ? wrow : 0, 2 * (lane >> 4), p.w_kblocks);
+  const uint16_t* wpack1 = p.W + packed_piece(wvalid ? wrow : 0, 2 * (lane >> 4) + 1, p.w_kblocks);
 
   f32x4_t acc[MT];
 #pragma unroll
@@ -464,8 +482,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(GemmArgs p) {
   for (int k0 = wave * 64; k0 < p.K; k0 += SK_WAVES * 64) {
     const int k = k0 + koff;  // this lane covers k .. k+15
     Frag w0, w1;
-    const uint4 t0 = *(const uint4*)(wrow_p + min(k, p.K - 8));
-    const uint4 t1 = *(const uint4*)(wrow_p + min(k + 8, p.K - 8));
+    const uint4 t0 = *(const uint4*)(p.w_packed ? wpack0 + (size_t)k0 * 16 : wrow_p + min(k, p.K - 8));
+    const uint4 t1 = *(const uint4*)(p.w_packed ? wpack1 + (size_t)k0 * 16 : wrow_p + min(k + 8, p.K - 8));
     w0.u = (wvalid && k < p.K) ? t0 : ZERO4;
     w1.u = (wvalid && k + 8 < p.K) ? t1 : ZERO4;
 #pragma unroll
@@ -515,11 +533,12 @@ static int check_args(const GemmArgs& p) {
   if (p.K % 8 != 0) FAIL("gemm_bf16: K=%d must be a multiple of 8", p.K);
   if (p.lda % 8 != 0 || p.ldw % 8 != 0)
     FAIL("gemm_bf16: row strides lda=%d ldw=%d must be multiples of 8", p.lda, p.ldw);
-  if (p.lda < p.K || p.ldw < p.K || p.ldo < p.N)
+  if (p.lda < p.K || (!p.w_packed && p.ldw < p.K) || p.ldo < p.N)
     FAIL("gemm_bf16: row strides smaller than the rows (lda=%d ldw=%d ldo=%d)", p.lda, p.ldw, p.ldo);
   if (!p.A || !p.W || !p.out) FAIL("gemm_bf16: null pointer");
   if (((uintptr_t)p.A | (uintptr_t)p.W) & 15) FAIL("gemm_bf16: A and W must be 16-byte aligned");
-  if ((size_t)p.M * p.lda >= (1u << 31) || (size_t)p.N * p.ldw >= (1u << 31))
+  const size_t w_elements = p.w_packed ? (size_t)((p.N + 15) / 16) * p.w_kblocks * 1024 : (size_t)p.N * p.ldw;
+  if ((size_t)p.M * p.lda >= (1u << 31) || w_elements >= (1u << 31))
     FAIL("gemm_bf16: operands of 2^31 elements or more are not supported");
   if ((p.flags & FLAG_ACCUMULATE) && (p.flags & FLAG_GELU))
     FAIL("gemm_bf16: GELU and accumulate cannot be combined");
@@ -549,14 +568,22 @@ static int busiest_die(int M, int N) {
 // overlap each other's), a 256 x 256 block (four times the work) in 2.0 us.  A
 // die has 32 CUs.
 static double cost_128(int M, int N) {
+  const int per_die = n_compute_units() / N_DIES;  // CUs of a die: two of these blocks fit each
   const int tiles = busiest_die<Tile128>(M, N);
-  const int rest = tiles % 64;
+  const int rest = tiles % (2 * per_die);
   // (a last round of few blocks finds the L2 idle: 1.0)
-  return (double)(tiles / 64) * 1.15 + (rest == 0 ? 0.0 : rest <= 16 ? 1.0 : rest <= 32 ? 1.3 : 1.15);
+  return (double)(tiles / (2 * per_die)) * 1.15 +
+         (rest == 0 ? 0.0 : rest <= per_die / 2 ? 1.0 : rest <= per_die ? 1.3 : 1.15);
 }
-static double cost_256(int M, int N) { return (double)((busiest_die<Tile256>(M, N) + 31) / 32) * 2.0; }
+static double cost_256(int M, int N) {
+  const int per_die = n_compute_units() / N_DIES;
+  return (double)((busiest_die<Tile256>(M, N) + per_die - 1) / per_die) * 2.0;
+}
 // (256 x 192: three quarters of the arithmetic, seven eighths of the bytes; its tiles fit N = 4800)
-static double cost_256x192(int M, int N) { return (double)((busiest_die<Tile256x192>(M, N) + 31) / 32) * 1.6; }
+static double cost_256x192(int M, int N) {
+  const int per_die = n_compute_units() / N_DIES;
+  return (double)((busiest_die<Tile256x192>(M, N) + per_die - 1) / per_die) * 1.6;
+}
 
 // Tiles of 64 x 128 instead of 128 x 128 where the latter would be few (up to 128): twice the
 // blocks, each with half the arithmetic and three quarters of the bytes.  Measured at widths
@@ -597,7 +624,7 @@ extern "C" int gemm_bf16_splits(int M, int N, int K, int fused, int force) {
     double best_us = 0.0, whole_us = 0.0;
     for (int s = 1; s <= 16 && s <= (n_blocks >= 3 ? n_blocks / 3 : 1); ++s) {
       const int per = (n_blocks + s - 1) / s;
-      const int on_cu = (int)((tiles * s + 255) / 256);
+      const int on_cu = (int)((tiles * s + n_compute_units() - 1) / n_compute_units());
       double us = kblock_us(rows, on_cu) * per;
       if (s > 1) us += (fused ? 1.0 : 2.5) + 8.0 * (fused ? s - 1 : s) * (double)M * N / 3e6;
       if (s == 1) whole_us = us;
@@ -612,7 +639,8 @@ extern "C" int gemm_bf16_splits(int M, int N, int K, int fused, int force) {
 
 // variant: 0 = choose, 1 = 128 x 128 tiles, 2 = skinny kernel, 3 = 256 x 256 tiles, 4 = 256 x 192
 // tiles, 5 = 64 x 128 tiles, 6 = 32 x 128 tiles.  n_splits > 1 (variants 1, 5 and 6 only): no
-// epilogue, the partial sums go to ws.
+// epilogue, the partial sums go to ws.  ldw == 0: W is in the decode kernels' packed order
+// (tiles of 16 features x 64 k, zero padded), which all kernels here read as well as rows.
 extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* bias, int M, int N,
                          int K, int lda, int ldw, int ldo, int flags, int variant, int n_splits,
                          float* ws, size_t ws_floats, hipStream_t stream) {
@@ -624,6 +652,7 @@ extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* b
   p.M = M, p.N = N, p.K = K;
   p.lda = lda, p.ldw = ldw, p.ldo = ldo;
   p.flags = flags;
+  p.w_packed = ldw == 0 ? 1 : 0, p.w_kblocks = (K + BK - 1) / BK;
   if (check_args(p)) return 1;
   if (M == 0) return 0;
   const int n_blocks = (K + BK - 1) / BK;

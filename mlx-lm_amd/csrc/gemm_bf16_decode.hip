@@ -516,7 +516,7 @@ extern "C" int gemm_bf16_decode_splits(int M, int N, int K, int with_norm, int f
     // a small matrix streams in less time than the second kernel costs (measured at N = 1600:
     // K = 1600 loses 2 us by the split, K = 6400 gains 4)
     if ((long)N * K < 5000000L) return 1;
-    want = (512 + n_blocks - 1) / n_blocks;  // two blocks a CU (measured at N = 1600: K = 6400 is best in 5, K = 1600 in 2 to 6)
+    want = (2 * n_compute_units() + n_blocks - 1) / n_blocks;  // two blocks a CU (measured at N = 1600: K = 6400 is best in 5, K = 1600 in 2 to 6)
     if (want > n_chunks / 4) want = n_chunks / 4;  // at least four k-blocks a split
   }
   if (want < 1) want = 1;
@@ -667,7 +667,7 @@ extern "C" int sum_partials_norm(float* h, int ldh, const float* ws, int n_split
   q.ahead_chunks = ahead ? ahead_chunks : 0;
   // as many reading blocks as leave a CU each to the rows' blocks (few rows only: with many, the
   // CUs are busy and the memory too)
-  const int readers = q.ahead_pieces > 0 && q.ahead_chunks > 0 && M <= 16 ? (256 - M) / 8 * 8 : 0;
+  const int readers = q.ahead_pieces > 0 && q.ahead_chunks > 0 && M <= 16 ? (n_compute_units() - M) / N_DIES * N_DIES : 0;
   if (N <= 2048)
     hipLaunchKernelGGL(sum_partials_norm_kernel<2>, dim3(M + readers), dim3(256), 0, stream, q);
   else

@@ -35,6 +35,7 @@ taken part in one step too many, whose result is dropped.  What can be known
 (``max_tokens``, the model's positions) is: such a request is left out.
 """
 
+import time
 from collections import deque
 from dataclasses import dataclass, field
 from typing import Any, Callable, List, Optional, Sequence
@@ -104,11 +105,26 @@ class PlannedEntry:
 
 @dataclass
 class SchedulerStats:
+    """Counters and clocks of a scheduler.  A step's wall time counts as prompt time and as
+    generation time in proportion to the prompt tokens it read and the tokens it handed out
+    (the reference keeps the two apart because it runs them as two model calls,
+    mlx_lm/generate.py:1642-1661,1915-1919; here one step holds both)."""
+
     steps: int = 0
     prompt_tokens: int = 0
     generation_tokens: int = 0
     preemptions: int = 0
     pages_high_water: int = 0
+    prompt_time: float = 0.0
+    generation_time: float = 0.0
+
+    @property
+    def prompt_tps(self):
+        return self.prompt_tokens / max(self.prompt_time, 1e-9)
+
+    @property
+    def generation_tps(self):
+        return self.generation_tokens / max(self.generation_time, 1e-9)
 
 
 def stops(tokens, stop_sequences):
@@ -293,6 +309,17 @@ class Scheduler:
     def step(self):
         """Plan, run and sample one step; returns the ``StepOutput`` of every sampled token
         (of this step, or of the step before where steps overlap)."""
+        tic = time.perf_counter()
+        prompt_before = self.stats.prompt_tokens
+        outputs = self._step()
+        elapsed = time.perf_counter() - tic
+        read, made = self.stats.prompt_tokens - prompt_before, len(outputs)
+        if read + made:
+            self.stats.prompt_time += elapsed * read / (read + made)
+            self.stats.generation_time += elapsed * made / (read + made)
+        return outputs
+
+    def _step(self):
         if not self.pipelined:
             return self._step_in_turn()
         prev, self._inflight = self._inflight, None

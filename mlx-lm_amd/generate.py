@@ -8,6 +8,7 @@ All of them run on the continuous-batching scheduler and the step function of
 
 import argparse
 import contextlib
+import dataclasses
 import json
 import sys
 import time
@@ -147,6 +148,56 @@ def _refuse_unsupported(kwargs):
 _uid = [0]
 
 
+class _OneRequest:
+    """One prompt on a scheduler of its own: iterating yields the ``StepOutput`` of every token.
+
+    The prompt is read in portions of ``prefill_step_size`` (under ``max_num_batched_tokens``
+    a step); then one token per step.  ``stop_tokens`` end the request with reason ``"stop"``,
+    ``max_tokens`` or the model's positions with ``"length"``; its pages go back at once.
+    ``page_size``/``num_pages`` choose the cache that the model's engine is made with.
+    """
+
+    def __init__(self, model, prompt, max_tokens, sampler=None, logits_processors=None,
+                 prefill_step_size=2048, prompt_progress_callback=None, seed=None, stop_tokens=(),
+                 want_logprobs=True, page_size=16, num_pages=None, max_num_seqs=1,
+                 max_num_batched_tokens=None):
+        self.prompt = [int(t) for t in (prompt.tolist() if hasattr(prompt, "tolist") else prompt)]
+        if len(self.prompt) == 0:
+            raise ValueError("Either input_embeddings or prompt (or both) must be provided.")
+        self.engine = engine_for(model, page_size=page_size,
+                                 max_cache_tokens=None if num_pages is None else num_pages * page_size)
+        self.scheduler = Scheduler(self.engine, make_sample_fn(), max_num_seqs=max(1, max_num_seqs),
+                                   max_num_batched_tokens=max_num_batched_tokens or prefill_step_size,
+                                   prefill_step_size=prefill_step_size)
+        _uid[0] += 1
+        self.request_id = ("generate_step", _uid[0])
+        if seed is None:
+            seed = getattr(sampler, "seed", None)
+        if seed is None:
+            seed = sample_utils.default_seed()
+        self.request = Request(self.request_id, self.prompt, max_tokens, sampler=sampler,
+                               logits_processors=logits_processors, seed=seed, want_logprobs=want_logprobs,
+                               stop_sequences=[[int(t)] for t in stop_tokens])
+        self.progress = prompt_progress_callback
+        self.scheduler.add(self.request)
+
+    @property
+    def stats(self):
+        return self.scheduler.stats
+
+    def __iter__(self):
+        sched, req = self.scheduler, self.request
+        try:
+            while sched.has_work:
+                outs = sched.step()
+                if self.progress is not None and not req.generated:
+                    self.progress(min(req.num_computed, len(self.prompt)), len(self.prompt))
+                yield from outs
+        finally:
+            if self.engine.has_request(self.request_id):
+                sched.abort(self.request_id)
+
+
 def generate_step(prompt, model, *, max_tokens=256, sampler=None, logits_processors=None,
                   prefill_step_size=2048, prompt_progress_callback=None, seed=None, **kwargs):
     """Yield ``(token, logprobs)`` for one prompt (mlx_lm/generate.py:298-461).
@@ -154,35 +205,22 @@ def generate_step(prompt, model, *, max_tokens=256, sampler=None, logits_process
     The prompt is read in portions of ``prefill_step_size``; then one token
     per step.  ``logprobs`` is a float32 device tensor ``[vocab]``.  Exactly
     ``max_tokens`` tokens are yielded unless the model's positions run out.
+    Beyond the reference's options: ``seed`` keys the draws; ``page_size``,
+    ``num_pages``, ``max_num_seqs`` and ``max_num_batched_tokens`` shape the
+    cache and the scheduler.
     """
     _refuse_unsupported(kwargs)
+    geometry = {k: kwargs.pop(k) for k in _ENGINE_OPTIONS if k in kwargs}
     if kwargs:
         raise TypeError(f"unknown options: {sorted(kwargs)}")
-    prompt = [int(t) for t in (prompt.tolist() if hasattr(prompt, "tolist") else prompt)]
-    if len(prompt) == 0:
-        raise ValueError("Either input_embeddings or prompt (or both) must be provided.")
-    engine = engine_for(model)
-    sched = Scheduler(engine, make_sample_fn(), max_num_seqs=1,
-                      max_num_batched_tokens=prefill_step_size, prefill_step_size=prefill_step_size)
-    _uid[0] += 1
-    rid = ("generate_step", _uid[0])
-    if seed is None:
-        seed = getattr(sampler, "seed", None)
-    if seed is None:
-        seed = sample_utils.default_seed()
-    req = Request(rid, prompt, max_tokens, sampler=sampler, logits_processors=logits_processors,
-                  seed=seed, want_logprobs=True)
-    sched.add(req)
-    try:
-        while sched.has_work:
-            outs = sched.step()
-            if prompt_progress_callback is not None and not req.generated:
-                prompt_progress_callback(min(req.num_computed, len(prompt)), len(prompt))
-            for o in outs:
-                yield o.token, o.logprobs
-    finally:
-        if engine.has_request(rid):
-            sched.abort(rid)
+    run = _OneRequest(model, prompt, max_tokens, sampler=sampler, logits_processors=logits_processors,
+                      prefill_step_size=prefill_step_size, prompt_progress_callback=prompt_progress_callback,
+                      seed=seed, **geometry)
+    for out in run:
+        yield out.token, out.logprobs
+
+
+_ENGINE_OPTIONS = ("page_size", "num_pages", "max_num_seqs", "max_num_batched_tokens")
 
 
 @dataclass
@@ -252,45 +290,41 @@ def stream_generate(model, tokenizer, prompt, max_tokens=256, draft_model=None, 
     """Yield a ``GenerationResponse`` per token (mlx_lm/generate.py:648-744).
 
     Stops at an end-of-sequence token (which is not added to the text) or
-    after ``max_tokens``; the last response carries ``finish_reason``.
+    after ``max_tokens``; the last response carries ``finish_reason``.  The end
+    tokens are the request's stop tokens, so the scheduler ends it (and gives
+    its pages back) with the token that ends it; rates come from the
+    scheduler's clocks: the prompt's up to the first token, the generation's
+    from there.
     """
     if draft_model is not None:
         raise ValueError("speculative decoding is not supported")
-    if tokenizer is None:
-        tokenizer = IdTokenizer()
+    tokenizer = tokenizer if tokenizer is not None else IdTokenizer()
     if isinstance(prompt, str):
-        add_special = tokenizer.bos_token is None or not prompt.startswith(tokenizer.bos_token)
-        prompt = tokenizer.encode(prompt, add_special_tokens=add_special)
-    prompt = [int(t) for t in (prompt.tolist() if hasattr(prompt, "tolist") else prompt)]
+        bos = tokenizer.bos_token
+        prompt = tokenizer.encode(prompt, add_special_tokens=bos is None or not prompt.startswith(bos))
+    _refuse_unsupported(kwargs)
+    run = _OneRequest(model, prompt, max_tokens, stop_tokens=sorted(tokenizer.eos_token_ids), **kwargs)
     detokenizer = tokenizer.detokenizer
-    kwargs["max_tokens"] = max_tokens
-    tic = time.perf_counter()
-    prompt_tps = 0.0
-    n, token, logprobs = -1, None, None
-    for n, (token, logprobs) in enumerate(generate_step(prompt, model, **kwargs)):
-        if n == 0:
-            prompt_time = time.perf_counter() - tic
-            prompt_tps = len(prompt) / prompt_time
-            tic = time.perf_counter()
-        if token in tokenizer.eos_token_ids:
-            break
-        detokenizer.add_token(token)
-        if (n + 1) == max_tokens:
-            break
-        yield GenerationResponse(
-            text=detokenizer.last_segment, token=token, logprobs=logprobs, from_draft=False,
-            prompt_tokens=len(prompt), prompt_tps=prompt_tps, generation_tokens=n + 1,
-            generation_tps=(n + 1) / max(time.perf_counter() - tic, 1e-9),
-            peak_memory=_peak_memory_gb(), finish_reason=None)
-    if n < 0:
-        return
-    detokenizer.finalize()
-    yield GenerationResponse(
-        text=detokenizer.last_segment, token=token, logprobs=logprobs, from_draft=False,
-        prompt_tokens=len(prompt), prompt_tps=prompt_tps, generation_tokens=n + 1,
-        generation_tps=(n + 1) / max(time.perf_counter() - tic, 1e-9),
-        peak_memory=_peak_memory_gb(),
-        finish_reason="stop" if token in tokenizer.eos_token_ids else "length")
+    started = first_token_at = time.perf_counter()
+    made = 0
+
+    def response(out, reason):
+        now = time.perf_counter()
+        return GenerationResponse(
+            text=detokenizer.last_segment, token=out.token, logprobs=out.logprobs, from_draft=False,
+            prompt_tokens=len(run.prompt), prompt_tps=len(run.prompt) / max(first_token_at - started, 1e-9),
+            generation_tokens=made, generation_tps=made / max(now - first_token_at, 1e-9),
+            peak_memory=_peak_memory_gb(), finish_reason=reason)
+
+    for out in run:
+        if made == 0:
+            first_token_at = time.perf_counter()
+        made += 1
+        if out.finish_reason != "stop":  # the token that stops the request is not part of the text
+            detokenizer.add_token(out.token)
+        if out.finish_reason is not None:
+            detokenizer.finalize()
+        yield response(out, out.finish_reason)
 
 
 def generate(model, tokenizer, prompt, verbose=False, **kwargs):
@@ -298,24 +332,25 @@ def generate(model, tokenizer, prompt, verbose=False, **kwargs):
 
     Without a tokenizer the text is the generated token ids in decimal.
     """
+    rule = "=" * 10
+    pieces, last = [], None
     if verbose:
-        print("=" * 10)
-    text = ""
-    response = None
-    for response in stream_generate(model, tokenizer, prompt, **kwargs):
+        print(rule)
+    for last in stream_generate(model, tokenizer, prompt, **kwargs):
+        pieces.append(last.text)
         if verbose:
-            print(response.text, end="", flush=True)
-        text += response.text
-    if verbose:
-        print()
-        print("=" * 10)
-        if len(text) == 0:
-            print("No text generated for this prompt")
-            return
-        print(f"Prompt: {response.prompt_tokens} tokens, {response.prompt_tps:.3f} tokens-per-sec")
-        print(f"Generation: {response.generation_tokens} tokens, "
-              f"{response.generation_tps:.3f} tokens-per-sec")
-        print(f"Peak memory: {response.peak_memory:.3f} GB")
+            print(last.text, end="", flush=True)
+    text = "".join(pieces)
+    if not verbose:
+        return text
+    print()
+    print(rule)
+    if not text:
+        print("No text generated for this prompt")
+        return
+    print(f"Prompt: {last.prompt_tokens} tokens, {last.prompt_tps:.3f} tokens-per-sec")
+    print(f"Generation: {last.generation_tokens} tokens, {last.generation_tps:.3f} tokens-per-sec")
+    print(f"Peak memory: {last.peak_memory:.3f} GB")
     return text
 
 
@@ -397,9 +432,6 @@ class BatchGenerator:
             prefill_step_size=prefill_step_size)
         self._uid_count = 0
         self._requests = {}
-        self._prompt_tokens_counter = 0
-        self._prompt_time_counter = 0.0
-        self._gen_tokens_counter = 0
 
     def close(self):
         for uid in list(self._requests):
@@ -407,21 +439,19 @@ class BatchGenerator:
 
     @contextlib.contextmanager
     def stats(self, stats=None):
+        """Counts and rates of what runs inside the ``with`` (mlx_lm/generate.py:1642-1661), from
+        the scheduler's counters and clocks."""
         stats = stats or BatchStats()
-        self._prompt_tokens_counter = 0
-        self._prompt_time_counter = 0.0
-        self._gen_tokens_counter = 0
-        tic = time.perf_counter()
+        before = dataclasses.replace(self.scheduler.stats)
         try:
             yield stats
         finally:
-            total = time.perf_counter() - tic
-            gen_time = total - self._prompt_time_counter
-            stats.prompt_tokens += self._prompt_tokens_counter
-            stats.prompt_time += self._prompt_time_counter
+            now = self.scheduler.stats
+            stats.prompt_tokens += now.prompt_tokens - before.prompt_tokens
+            stats.prompt_time += now.prompt_time - before.prompt_time
             stats.prompt_tps = stats.prompt_tokens / max(stats.prompt_time, 1e-9)
-            stats.generation_tokens += self._gen_tokens_counter
-            stats.generation_time += gen_time
+            stats.generation_tokens += now.generation_tokens - before.generation_tokens
+            stats.generation_time += now.generation_time - before.generation_time
             stats.generation_tps = stats.generation_tokens / max(stats.generation_time, 1e-9)
             stats.peak_memory = max(stats.peak_memory, _peak_memory_gb())
 
@@ -466,25 +496,14 @@ class BatchGenerator:
         return {} if return_prompt_caches else None
 
     def _next(self):
-        before = {uid: (r.num_computed, bool(r.generated)) for uid, r in self._requests.items()}
-        tic = time.perf_counter()
+        before = {uid: r.num_computed for uid, r in self._requests.items() if not r.generated}
         outs = self.scheduler.step()
-        elapsed = time.perf_counter() - tic
-        prompt_responses, prompt_tokens = [], 0
-        for uid, (done, had_generated) in before.items():
+        prompt_responses = []
+        for uid, done in before.items():
             r = self._requests[uid]
-            if not had_generated and r.num_computed != done:
-                n = min(r.num_computed, len(r.prompt)) - min(done, len(r.prompt))
-                prompt_tokens += n
-                prompt_responses.append(self.PromptResponse(
-                    uid, (min(r.num_computed, len(r.prompt)), len(r.prompt)),
-                    r.num_computed >= len(r.prompt)))
-        # a step's time counts as prompt time in proportion to its prompt tokens
-        total = prompt_tokens + len(outs)
-        if total:
-            self._prompt_time_counter += elapsed * prompt_tokens / total
-        self._prompt_tokens_counter += prompt_tokens
-        self._gen_tokens_counter += len(outs)
+            if r.num_computed != done:
+                n = len(r.prompt)
+                prompt_responses.append(self.PromptResponse(uid, (min(r.num_computed, n), n), r.num_computed >= n))
         responses = []
         for o in outs:
             r = self._requests[o.request_id]
@@ -508,42 +527,49 @@ class BatchGenerator:
 def batch_generate(model, tokenizer, prompts, prompt_caches=None, max_tokens=128, verbose=False,
                    return_prompt_caches=False, return_token_ids=False, return_logprobs=False,
                    **kwargs):
-    """Run a list of prompts to completion (mlx_lm/generate.py:1971-2060)."""
+    """Run a list of prompts to completion (mlx_lm/generate.py:1971-2060).
+
+    The tokenizer's end tokens stop a request; the token that stops it is not part of its
+    result.  ``kwargs`` go to ``BatchGenerator``.
+    """
     if prompt_caches is not None or return_prompt_caches:
         raise ValueError("prompt caches are not supported")
-    if tokenizer is None:
-        tokenizer = IdTokenizer()
+    tokenizer = tokenizer if tokenizer is not None else IdTokenizer()
     gen = BatchGenerator(model, stop_tokens=[[t] for t in tokenizer.eos_token_ids],
                          want_logprobs=False, **kwargs)
-    num_samples, fin = len(prompts), 0
-    if verbose:
-        print(f"[batch_generate] Finished processing 0/{num_samples} ...", end="\r")
-    if isinstance(max_tokens, int):
-        max_tokens = [max_tokens] * len(prompts)
-    uids = gen.insert(prompts, max_tokens)
-    results = {uid: [] for uid in uids}
-    logprob_results = {uid: [] for uid in uids}
+    limits = [max_tokens] * len(prompts) if isinstance(max_tokens, int) else list(max_tokens)
+    total, finished = len(prompts), 0
+
+    def progress(end="\r"):
+        if verbose:
+            print(f"[batch_generate] Finished processing {finished}/{total}" + (" ..." if end == "\r" else ""),
+                  end=end)
+
+    progress()
+    uids = gen.insert(prompts, limits)
+    kept = {uid: ([], []) for uid in uids}  # tokens and their log-probabilities
     with gen.stats() as stats:
-        while responses := gen.next_generated():
+        while True:
+            responses = gen.next_generated()
+            if not responses:
+                break
             for r in responses:
-                if r.finish_reason is not None and verbose:
-                    fin += 1
-                    print(f"[batch_generate] Finished processing {fin}/{num_samples} ...", end="\r")
                 if r.finish_reason != "stop":
-                    results[r.uid].append(r.token)
-                    logprob_results[r.uid].append(r.token_logprob)
+                    kept[r.uid][0].append(r.token)
+                    kept[r.uid][1].append(r.token_logprob)
+                if r.finish_reason is not None:
+                    finished += 1
+                    progress()
     gen.close()
-    if verbose:
-        print(f"[batch_generate] Finished processing {fin}/{num_samples}")
-    texts = [tokenizer.decode(results[uid]) for uid in uids]
-    token_ids = [results[uid] for uid in uids] if return_token_ids else None
-    logprobs = [logprob_results[uid] for uid in uids] if return_logprobs else None
+    progress(end="\n")
     if verbose:
         print(f"[batch_generate] Prompt: {stats.prompt_tokens} tokens, {stats.prompt_tps:.3f} tokens-per-sec")
         print(f"[batch_generate] Generation: {stats.generation_tokens} tokens, "
               f"{stats.generation_tps:.3f} tokens-per-sec")
         print(f"[batch_generate] Peak memory: {stats.peak_memory:.3f} GB")
-    return BatchResponse(texts, stats, None, token_ids, logprobs)
+    return BatchResponse([tokenizer.decode(kept[uid][0]) for uid in uids], stats, None,
+                         [kept[uid][0] for uid in uids] if return_token_ids else None,
+                         [kept[uid][1] for uid in uids] if return_logprobs else None)
 
 
 # ---------------------------------------------------------------------------
@@ -554,47 +580,49 @@ def str2bool(string):
     return string.lower() not in ["false", "f"]
 
 
+# The options of ``mlx_lm.generate`` that this engine has (mlx_lm/generate.py:54-213), with the
+# reference's names, defaults and meanings, then the engine's own.  (flags, type, default, help, more)
+_OPTIONS = [
+    (("--model",), str, None, "A local model folder (config.json, model.safetensors); not needed with --random-weights.", {}),
+    (("--extra-eos-token",), str, (), "More tokens that end the generation.", {"nargs": "+"}),
+    (("--system-prompt",), None, None, "A system message for the tokenizer's chat template.", {}),
+    (("--prompt", "-p"), None, DEFAULT_PROMPT, "The message to answer ('-' reads it from standard input).", {}),
+    (("--prompt-ids",), str, None, "The prompt as token ids, separated by commas or spaces "
+                                   "(for model folders without a tokenizer).", {}),
+    (("--prefill-response",), None, None, "A start of the answer, which the model goes on from.", {}),
+    (("--max-tokens", "-m"), int, DEFAULT_MAX_TOKENS, "The most tokens to generate.", {}),
+    (("--temp",), float, DEFAULT_TEMP, "Sampling temperature (0: the most likely token).", {}),
+    (("--top-p",), float, DEFAULT_TOP_P, "Sample from the most likely tokens that hold this much probability.", {}),
+    (("--min-p",), float, DEFAULT_MIN_P, "Drop tokens less likely than this fraction of the most likely one's probability.", {}),
+    (("--top-k",), int, DEFAULT_TOP_K, "Sample from the k most likely tokens (0: all).", {}),
+    (("--xtc-probability",), float, DEFAULT_XTC_PROBABILITY, "How often XTC sampling drops the top choices.", {}),
+    (("--xtc-threshold",), float, 0.1, "XTC drops all but the least likely of the tokens above this probability.", {}),
+    (("--min-tokens-to-keep",), int, DEFAULT_MIN_TOKENS_TO_KEEP, "What min-p leaves at least.", {}),
+    (("--seed",), int, DEFAULT_SEED, "Seed of the random draws.", {}),
+    (("--ignore-chat-template",), None, False, "Give the model the prompt as it is.", {"action": "store_true"}),
+    (("--chat-template-config",), None, None, "More variables for the chat template, as a JSON object.", {}),
+    (("--verbose",), str2bool, True, "'True'/'T': stream the text, then print token counts, rates and peak "
+                                     "memory; 'False'/'F': print the text only.", {}),
+    # this engine's own
+    (("--dtype",), None, "bfloat16", "Precision of the weights and the arithmetic.", {"choices": ["bfloat16", "float32"]}),
+    (("--prefill-step-size",), int, 2048, "The most tokens of the prompt that one step reads.", {}),
+    (("--block-size",), int, 16, "Tokens per page of the key/value cache (a multiple of 16).", {}),
+    (("--num-pages",), int, None, "Pages of the cache pool (default: room for 64 full contexts, within memory).", {}),
+    (("--max-num-seqs",), int, 1, "The most requests that run at a time.", {}),
+    (("--max-num-batched-tokens",), int, None, "The most tokens of one step (default: --prefill-step-size).", {}),
+    (("--random-weights",), int, None, "Draw the weights with this seed for the configuration given by --config "
+                                      "(or by --model's config.json) instead of reading them.", {"metavar": "SEED"}),
+    (("--config",), str, None, "A config.json for --random-weights.", {}),
+]
+
+
 def setup_arg_parser():
-    """The options of ``mlx_lm.generate`` that this engine has (mlx_lm/generate.py:54-213)."""
     parser = argparse.ArgumentParser(description="LLM inference script")
-    parser.add_argument("--model", type=str, required=True,
-                        help="The path to the local model directory.")
-    parser.add_argument("--extra-eos-token", type=str, default=(), nargs="+",
-                        help="Add tokens in the list of eos tokens that stop generation.")
-    parser.add_argument("--system-prompt", default=None,
-                        help="System prompt to be used for the chat template")
-    parser.add_argument("--prompt", "-p", default=DEFAULT_PROMPT,
-                        help="Message to be processed by the model ('-' reads from stdin)")
-    parser.add_argument("--prompt-ids", type=str, default=None,
-                        help="The prompt as token ids separated by commas or spaces "
-                        "(for model folders without a tokenizer)")
-    parser.add_argument("--prefill-response", default=None,
-                        help="Prefill response to be used for the chat template")
-    parser.add_argument("--max-tokens", "-m", type=int, default=DEFAULT_MAX_TOKENS,
-                        help="Maximum number of tokens to generate")
-    parser.add_argument("--temp", type=float, default=DEFAULT_TEMP, help="Sampling temperature")
-    parser.add_argument("--top-p", type=float, default=DEFAULT_TOP_P, help="Sampling top-p")
-    parser.add_argument("--min-p", type=float, default=DEFAULT_MIN_P, help="Sampling min-p")
-    parser.add_argument("--top-k", type=int, default=DEFAULT_TOP_K, help="Sampling top-k")
-    parser.add_argument("--xtc-probability", type=float, default=DEFAULT_XTC_PROBABILITY,
-                        help="Probability of XTC sampling to happen each next token")
-    parser.add_argument("--xtc-threshold", type=float, default=0.1,
-                        help="Threshold the probs of each next token candidate to be sampled by XTC")
-    parser.add_argument("--min-tokens-to-keep", type=int, default=DEFAULT_MIN_TOKENS_TO_KEEP,
-                        help="Minimum tokens to keep for min-p sampling.")
-    parser.add_argument("--seed", type=int, default=DEFAULT_SEED, help="PRNG seed")
-    parser.add_argument("--ignore-chat-template", action="store_true",
-                        help="Use the raw prompt without the tokenizer's chat template.")
-    parser.add_argument("--chat-template-config", default=None,
-                        help="Additional config for `apply_chat_template`. Should be a dictionary of "
-                        "string keys to values represented as a JSON decodable string.")
-    parser.add_argument("--verbose", type=str2bool, default=True,
-                        help="Log verbose output when 'True' or 'T' or only print the response "
-                        "when 'False' or 'F'")
-    parser.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16",
-                        help="Compute precision")
-    parser.add_argument("--prefill-step-size", type=int, default=2048,
-                        help="Most prompt tokens read in one step")
+    for flags, kind, default, text, more in _OPTIONS:
+        options = dict(default=default, help=text, **more)
+        if kind is not None:
+            options["type"] = kind
+        parser.add_argument(*flags, **options)
     return parser
 
 
@@ -617,34 +645,52 @@ def chat_prompt(tokenizer, prompt, args):
                                          add_generation_prompt=not has_prefill, **template_kwargs)
 
 
+def _model_of(args):
+    """The model and tokenizer that the command line names: a folder's, or random weights for a configuration."""
+    from .utils import load, load_config, model_from_tensors
+
+    if args.random_weights is None:
+        if args.model is None:
+            raise SystemExit("give --model DIR (or --random-weights SEED with --config FILE)")
+        return load(args.model, dtype=args.dtype)
+    if args.config is not None:
+        with open(args.config) as fh:
+            config = json.load(fh)
+    elif args.model is not None:
+        config = load_config(args.model)
+    else:
+        raise SystemExit("--random-weights needs --config FILE or --model DIR for the configuration")
+    from .config import get_model_classes
+
+    model_cls, args_cls = get_model_classes(config)
+    tensors = model_cls.random_weights(args_cls.from_dict(config), args.random_weights, "b")
+    return model_from_tensors(config, tensors, dtype=args.dtype), None
+
+
 def main(argv=None):
-    parser = setup_arg_parser()
-    args = parser.parse_args(argv)
+    args = setup_arg_parser().parse_args(argv)
     if args.seed is not None:
         sample_utils.seed(args.seed)
-    from .utils import load
-
-    model, tokenizer = load(args.model, dtype=args.dtype)
-    if tokenizer is None:
-        tokenizer = IdTokenizer()
-    for tok in args.extra_eos_token:
-        tokenizer.add_eos_token(tok)
+    model, tokenizer = _model_of(args)
+    tokenizer = tokenizer if tokenizer is not None else IdTokenizer()
+    for token in args.extra_eos_token:
+        tokenizer.add_eos_token(token)
     if args.prompt_ids is not None:
         prompt = [int(t) for t in args.prompt_ids.replace(",", " ").split()]
     else:
-        prompt = args.prompt.replace("\\n", "\n").replace("\\t", "\t")
-        prompt = sys.stdin.read() if prompt == "-" else prompt
-        prompt = chat_prompt(tokenizer, prompt, args)
-    special = []
-    if args.xtc_probability > 0:  # tokens that XTC never removes (mlx_lm/generate.py:2168)
-        special = list(tokenizer.encode("\n", add_special_tokens=False)) + sorted(tokenizer.eos_token_ids)
-    sampler = make_sampler(args.temp, args.top_p, args.min_p, args.min_tokens_to_keep,
-                           top_k=args.top_k, xtc_probability=args.xtc_probability,
-                           xtc_threshold=args.xtc_threshold, xtc_special_tokens=special)
-    response = generate(model, tokenizer, prompt, max_tokens=args.max_tokens, verbose=args.verbose,
-                        sampler=sampler, prefill_step_size=args.prefill_step_size)
+        text = args.prompt.replace("\\n", "\n").replace("\\t", "\t")
+        prompt = chat_prompt(tokenizer, sys.stdin.read() if text == "-" else text, args)
+    never_dropped = []  # by XTC: the line break and the end tokens (mlx_lm/generate.py:2168)
+    if args.xtc_probability > 0:
+        never_dropped = list(tokenizer.encode("\n", add_special_tokens=False)) + sorted(tokenizer.eos_token_ids)
+    sampler = make_sampler(args.temp, args.top_p, args.min_p, args.min_tokens_to_keep, top_k=args.top_k,
+                           xtc_probability=args.xtc_probability, xtc_threshold=args.xtc_threshold,
+                           xtc_special_tokens=never_dropped)
+    text = generate(model, tokenizer, prompt, max_tokens=args.max_tokens, verbose=args.verbose, sampler=sampler,
+                    prefill_step_size=args.prefill_step_size, page_size=args.block_size, num_pages=args.num_pages,
+                    max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens)
     if not args.verbose:
-        print(response)
+        print(text)
 
 
 if __name__ == "__main__":

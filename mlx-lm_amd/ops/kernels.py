@@ -199,13 +199,14 @@ class PackedWeight:
     Tiles of 16 features by 64 k, zero padded; tile ``(b, c)`` holds, for lane
     ``l`` (feature ``l % 16``, k group ``l // 16``), first the 8 values
     ``k = 64 c + 16 (l // 16) + 0..7`` of all lanes, then the 8 values ``+ 8..15``.
-    A wave's load is then 1 KB of consecutive bytes.  The matrix is kept
-    row-major as well (``w``) for the kernels that take many rows.
+    A wave's load is then 1 KB of consecutive bytes.  The kernels that take
+    many rows read this order too, so the row-major matrix need not be kept
+    (``keep_rows=False`` lets it go: one copy of the weights on the device).
     """
 
-    def __init__(self, w):
+    def __init__(self, w, keep_rows=True):
         _need(w.dtype == torch.bfloat16 and w.dim() == 2, "PackedWeight: a 2-D bfloat16 matrix")
-        self.w = w
+        self.w = w if keep_rows else None
         self.shape, self.dtype, self.device = tuple(w.shape), w.dtype, w.device
         N, K = w.shape
         Np, Kp = (N + 15) // 16 * 16, (K + 63) // 64 * 64
@@ -216,8 +217,8 @@ class PackedWeight:
         self.packed = t.contiguous().view(-1)
         # what one block of the decode kernel reads (16 features, all of K) and how many there are
         self.chunk_bytes, self.n_chunks = Kp * 16 * 2, Np // 16
-        self.c = native.EngWeight(w.data_ptr(), self.packed.data_ptr(), N, K, w.stride(0), DT[w.dtype],
-                                  self.chunk_bytes, self.n_chunks, 0)
+        self.c = native.EngWeight(w.data_ptr() if keep_rows else None, self.packed.data_ptr(), N, K,
+                                  w.stride(0) if keep_rows else 0, DT[w.dtype], self.chunk_bytes, self.n_chunks, 0)
 
 
 def weight_struct(w):
@@ -239,11 +240,11 @@ def read_ahead_pays(w, n_rows, with_norm=False):
                                                  1 if with_norm else 0))
 
 
-def for_decode(w):
-    """``w`` with a packed copy beside it where the decode kernel can use one
-    (bfloat16 on the GPU); anything else is returned as it is."""
+def for_decode(w, keep_rows=False):
+    """``w`` in the packed order where the product kernels can use it (bfloat16 on the GPU),
+    instead of the row-major matrix unless ``keep_rows``; anything else is returned as it is."""
     if isinstance(w, torch.Tensor) and w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2:
-        return PackedWeight(w)
+        return PackedWeight(w, keep_rows=keep_rows)
     return w
 
 

@@ -4,55 +4,81 @@ import json
 import os
 
 
+def _byte_of_symbol():
+    """Byte-level BPE writes every byte as one printable character: the bytes that print
+    (``!`` to ``~``, ``¡`` to ``¬``, ``®`` to ``ÿ``) as themselves, the other 68 as the
+    characters from U+0100 on, in the order of the bytes.  Returns character -> byte."""
+    keep = [*range(ord("!"), ord("~") + 1), *range(0xA1, 0xAD), *range(0xAE, 0x100)]
+    table, extra = {}, 0
+    for b in range(256):
+        if b in keep:
+            table[chr(b)] = b
+        else:
+            table[chr(256 + extra)] = b
+            extra += 1
+    return table
+
+
 class StreamingDetokenizer:
     """Turns a stream of token ids into text piece by piece.
 
     The contract of the reference's detokenizers (mlx_lm/tokenizer_utils.py:
     11-58): ``reset()``, ``add_token(id)``, ``finalize()``, then ``text`` is
     everything so far, ``last_segment`` what was added since it was last read,
-    ``tokens`` the ids.  This one decodes the tokens since the last line break
-    again for every token (the reference's ``NaiveStreamingDetokenizer``,
-    mlx_lm/tokenizer_utils.py:61-112) and holds back a trailing incomplete
-    character.
+    ``tokens`` the ids.  For a byte-level BPE vocabulary (what the reference's
+    ``BPEStreamingDetokenizer`` serves, mlx_lm/tokenizer_utils.py:157-250) a
+    token is a fixed run of bytes: each token's bytes are looked up once, and
+    an incremental UTF-8 decoder turns the stream of bytes into text, holding
+    back a character whose bytes have not all come.  The cost of a token does
+    not grow with the text.  Other vocabularies decode the tokens since the last
+    line break again for every token.
     """
 
-    def __init__(self, decode):
+    def __init__(self, decode, token_bytes=None):
         self._decode = decode
+        self._token_bytes = token_bytes  # id -> bytes for a byte-level vocabulary, else None
         self.reset()
 
     def reset(self):
+        import codecs
+
         self.offset = 0
         self.tokens = []
         self._text = ""
-        self._current = []
-        self._current_text = ""
+        self._utf8 = codecs.getincrementaldecoder("utf-8")("replace")
+        self._line = []  # (other vocabularies) the tokens since the last line break
+        self._line_text = ""
 
     def add_token(self, token):
-        self._current.append(int(token))
-        self.tokens.append(int(token))
+        token = int(token)
+        self.tokens.append(token)
+        if self._token_bytes is not None:
+            self._text += self._utf8.decode(self._token_bytes(token))
+            return
+        self._line.append(token)
+        shown = self._decode(self._line)
+        if shown.endswith("\ufffd"):  # a character whose tokens have not all come
+            shown = shown[:-1]
+        if shown.endswith("\n"):
+            self._text += shown
+            self._line, shown = [], ""
+        self._line_text = shown
 
     def finalize(self):
-        self._text += self._decode(self._current)
-        self._current = []
-        self._current_text = ""
+        if self._token_bytes is not None:
+            self._text += self._utf8.decode(b"", final=True)
+        elif self._line:
+            self._text += self._decode(self._line)
+            self._line, self._line_text = [], ""
 
     @property
     def text(self):
-        if self._current:
-            self._current_text = self._decode(self._current)
-            if self._current_text.endswith("�"):
-                self._current_text = self._current_text[:-1]
-        if self._current_text.endswith("\n"):
-            self._text += self._current_text
-            self._current = []
-            self._current_text = ""
-        return self._text + self._current_text
+        return self._text + self._line_text
 
     @property
     def last_segment(self):
         text = self.text
-        segment = text[self.offset :]
-        self.offset = len(text)
+        segment, self.offset = text[self.offset :], len(text)
         return segment
 
 
@@ -122,9 +148,35 @@ class TokenizerWrapper:
             raise ValueError(f"'{token}' is not a token for this tokenizer")
         self.eos_token_ids.add(tid)
 
+    def _byte_level_table(self):
+        """``id -> bytes`` if the vocabulary is byte-level BPE (its decoder says so), else ``None``."""
+        if not hasattr(self, "_bytes_of"):
+            self._bytes_of = None
+            spec = json.loads(self._tokenizer.to_str())
+            decoder = spec.get("decoder") or {}
+            kinds = {decoder.get("type")} | {d.get("type") for d in decoder.get("decoders", [])}
+            if "ByteLevel" in kinds and kinds <= {"ByteLevel", None}:
+                byte_of = _byte_of_symbol()
+                added = {t["id"] for t in spec.get("added_tokens", [])}
+                cache = {}
+
+                def bytes_of(token):
+                    b = cache.get(token)
+                    if b is None:
+                        piece = self._tokenizer.id_to_token(token) or ""
+                        if token in added or any(ch not in byte_of for ch in piece):
+                            b = piece.encode("utf-8")  # an added token is its own text
+                        else:
+                            b = bytes(byte_of[ch] for ch in piece)
+                        cache[token] = b
+                    return b
+
+                self._bytes_of = bytes_of
+        return self._bytes_of
+
     @property
     def detokenizer(self):
-        return StreamingDetokenizer(self.decode)
+        return StreamingDetokenizer(self.decode, self._byte_level_table())
 
     @property
     def vocab_size(self):

@@ -239,42 +239,97 @@ def test_out_of_pages_is_an_error_and_takes_nothing(folders):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(folders, tmp_path, dtype):
-    """bin/trace_run as a user calls it: whole, decoded and mixed, from files."""
+    """bin/trace_run as a user calls it: whole, decoded, in portions of changing size and mixed,
+    from files; the three spellings of ``want``; the page statistics it leaves."""
+    import json
+
     folder, config, weights = folders[("B", 8.0)]
     lengths = [90, 40, 130, 64, 70]
     tokens, steps = helpers.mixed_trace(config, seed=11, lengths=lengths, n_live=3)
-    # a request whole, and the same one with its last 32 tokens one by one
+    # a request whole, the same one with its last 32 tokens one by one, and in portions of changing size
     whole = helpers.random_tokens(120, config["vocab_size"], seed=5)
-    base = len(steps)
-    steps.append({"step": base, "entries": [{"id": "w", "tokens": whole, "want": list(range(120))}], "end": ["w"]})
-    steps.append({"step": base + 1, "entries": [{"id": "d", "tokens": whole[:88], "want": list(range(88))}], "end": []})
+
+    def add(rid, toks, want, end=False):
+        steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": toks, "want": want}],
+                      "end": [rid] if end else []})
+
+    add("w", whole, "all", end=True)
+    add("d", whole[:88], list(range(88)))
     for i in range(32):
-        steps.append({"step": base + 2 + i, "entries": [{"id": "d", "tokens": [whole[88 + i]], "want": [0]}],
-                      "end": ["d"] if i == 31 else []})
+        add("d", [whole[88 + i]], [0], end=i == 31)
+    at = 0
+    for n in helpers.cuts_changing(120):
+        add("p", whole[at : at + n], "all", end=at + n == 120)
+        at += n
+    add("l", whole[:50], "none")
+    add("l", whole[50:], "last", end=True)
     trace = tmp_path / "trace.jsonl"
     helpers.write_trace(trace, steps)
     out = tmp_path / "out"
+    max_tokens = helpers.held(lengths + [128], 3)
     with open(trace) as fh:
         proc = subprocess.run(
             [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
-             "--out", str(out), "--max-tokens", str(helpers.held(lengths + [128], 3))],
+             "--out", str(out), "--max-tokens", str(max_tokens), "--page-stats"],
             stdin=fh, capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stderr[-2000:]
-    assert [l for l in proc.stdout.split("\n") if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+    lines = proc.stdout.split("\n")
+    assert [l for l in lines if l.startswith("done")] == [f"done {s['step']}" for s in steps]
     V = config["vocab_size"]
     got = {}
     for s in steps:
-        data = np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(-1, V)
+        f = out / f"{s['step']}.f32"
+        wants = [e["want"] for e in s["entries"]]
+        if wants == ["none"]:
+            assert not f.exists()
+            continue
+        data = np.fromfile(f, dtype="<f4").reshape(-1, V)
         i = 0
         for e in s["entries"]:
-            got.setdefault(e["id"], []).append(torch.from_numpy(data[i : i + len(e["want"])].copy()))
-            i += len(e["want"])
+            n = {"all": len(e["tokens"]), "last": 1}.get(e["want"], len(e["want"])) if isinstance(e["want"], str) else len(e["want"])
+            got.setdefault(e["id"], []).append(torch.from_numpy(data[i : i + n].copy()))
+            i += n
         assert i == data.shape[0]
-    tokens["w"] = whole
-    tokens["d"] = whole
+    last = got.pop("l")
+    for rid in ("w", "d", "p"):
+        tokens[rid] = whole
     for rid, toks in tokens.items():
         want = _plain_logits(weights, config, toks, dtype)
         _close(torch.cat(got[rid]), want, dtype, f"trace_run, request {rid}")
+    _close(last[0], _plain_logits(weights, config, whole, dtype)[119:], dtype, 'want "last"')
+    # page statistics: a line a step, in the file and (asked for) on standard output; nothing is
+    # held at the end, and never more than the pool has
+    stats = [json.loads(l) for l in open(out / "pages.jsonl")]
+    assert [st["step"] for st in stats] == [s["step"] for s in steps]
+    assert [json.loads(l[len("pages "):]) for l in lines if l.startswith("pages ")] == stats
+    n_pages = max_tokens // 16
+    assert all(st["n_pages"] == n_pages and g["held"] + g["free"] == n_pages for st in stats for g in st["groups"])
+    assert stats[-1]["groups"][0]["held"] == 0 and stats[-1]["live_requests"] == 0
+    assert 0 < max(g["high_water"] for g in stats[-1]["groups"]) <= n_pages
+
+
+def test_trace_run_draws_its_own_weights(folders, tmp_path):
+    """``--config FILE --seed N``: the same logits as from the folder that the random-weights
+    mode writes for that configuration and seed."""
+    import json
+
+    from mlx_lm_amd.weights import write_model_folder
+
+    config = dict(helpers.TINY_A)
+    folder = tmp_path / "model"
+    write_model_folder(str(folder), dict(config), 7, "b")
+    (tmp_path / "cfg.json").write_text(json.dumps(config))
+    toks = helpers.random_tokens(40, config["vocab_size"], seed=1)
+    trace = json.dumps({"step": 0, "entries": [{"id": "a", "tokens": toks, "want": "all"}], "end": ["a"]}) + "\n"
+    outs = []
+    for i, source in enumerate((["--model", str(folder)], ["--config", str(tmp_path / "cfg.json"), "--seed", "7"])):
+        out = tmp_path / f"out{i}"
+        proc = subprocess.run(
+            [sys.executable, os.path.join(ROOT, "bin", "trace_run"), *source, "--dtype", "float32", "--out", str(out),
+             "--max-tokens", "64"], input=trace, capture_output=True, text=True, timeout=300)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        outs.append(np.fromfile(out / "0.f32", dtype="<f4"))
+    assert outs[0].shape == (40 * config["vocab_size"],) and np.array_equal(outs[0], outs[1])
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

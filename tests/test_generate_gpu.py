@@ -258,3 +258,36 @@ def test_penalty_histories_are_checked_against_the_vocabulary(model_b, tiny):
     with pytest.raises(ValueError, match="vocabulary"):
         proc(torch.tensor([1, V + 5]), logits)
     proc(torch.tensor([1, V - 1]), logits)
+
+
+def test_command_line_cache_geometry_and_random_weights(tiny, tmp_path):
+    """The engine's own options: pages of 32 tokens in a pool of 8, a scheduler's limits, and
+    weights drawn for a configuration instead of read (``--random-weights SEED --config FILE``:
+    the same tokens as from the folder that the random-weights mode writes with that seed)."""
+    import json
+
+    from mlx_lm_amd.weights import write_model_folder
+
+    d, config, weights = tiny["A"]
+    prompt = [3, 1, 4, 1, 5]
+    want = plain.greedy_generate(weights, config, prompt, 6)
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    base = [sys.executable, "-m", "mlx_lm_amd", "generate", "--prompt-ids", "3,1,4,1,5", "--max-tokens", "6",
+            "--dtype", "float32", "--verbose", "F"]
+    out = subprocess.run(base + ["--model", d, "--block-size", "32", "--num-pages", "8", "--max-num-seqs", "2",
+                                 "--max-num-batched-tokens", "3", "--prefill-step-size", "2"],
+                         capture_output=True, text=True, env=env, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    assert out.stdout.strip() == " ".join(map(str, want))
+    cfg = tmp_path / "config.json"
+    cfg.write_text(json.dumps(helpers.TINY_B))
+    folder = tmp_path / "drawn"
+    write_model_folder(str(folder), dict(helpers.TINY_B), 12, "b")
+    outs = []
+    for source in (["--model", str(folder)], ["--random-weights", "12", "--config", str(cfg)]):
+        out = subprocess.run(base + source, capture_output=True, text=True, env=env, timeout=300)
+        assert out.returncode == 0, out.stderr[-2000:]
+        outs.append(out.stdout.strip())
+    assert outs[0] == outs[1] and len(outs[0].split()) == 6
+    out = subprocess.run(base, capture_output=True, text=True, env=env, timeout=300)
+    assert out.returncode != 0 and "--model" in out.stderr

@@ -670,6 +670,33 @@ def test_gemm_bf16_decode(M, N, K, mode, normed, packed):
         assert (got - want).abs().max().item() < tol, (got - want).abs().max()
 
 
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES + [(2048, 1600, 1600), (260, 200, 6400)])
+def test_gemm_bf16_reads_weights_kept_in_packed_order_only(M, N, K):
+    """Every kernel of the many-row products (all tile shapes, the skinny kernel, the splits of K)
+    reads weights that exist in the decode kernels' packed order only: bit for bit what the same
+    kernel makes of the row-major matrix, at sizes with ragged edges (features that are no
+    multiple of 16, K no multiple of 64 or shorter than a k-block)."""
+    k = _k()
+    a = _rand((M, K), torch.bfloat16, 10)
+    w = _rand((N, K), torch.bfloat16, 11, 0.1)
+    bias = _rand((N,), torch.float32, 12)
+    packed = k.PackedWeight(w.clone(), keep_rows=False)
+    assert packed.w is None and not packed.c.w
+    ref = plain.linear(a.double().cpu(), w.double().cpu(), bias.double().cpu())
+    variants = [(v, None) for v in ((1, 2, 3, 4, 5, 6) if M <= 64 else (1, 3, 4, 5, 6))]
+    if M > 16 and K >= 192:
+        variants += [(1, 3), (5, 2), (6, 3), (0, 2)]  # K in parts
+    variants.append((0, None))  # the library's own choice
+    for variant, splits in variants:
+        outs = []
+        for weights in (w, packed):
+            out = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=DEV)
+            k.linear(out, a, weights, bias, gelu=True, variant=variant, splits=splits)
+            outs.append(out)
+        assert torch.equal(outs[0], outs[1]), (variant, splits)
+        assert torch.allclose(outs[1].double().cpu(), plain.gelu_tanh(ref), rtol=2**-7, atol=1e-3), (variant, splits)
+
+
 @pytest.mark.parametrize("M,N,K", [(17, 48, 64), (33, 257, 384), (64, 4800, 1600), (40, 1600, 6400), (64, 333, 1608),
                                    (48, 80, 200), (20, 100, 520)])
 @pytest.mark.parametrize("mode", ["plain", "gelu", "accumulate", "f32out"])

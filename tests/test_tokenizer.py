@@ -144,3 +144,27 @@ def test_the_command_lines_prompt(folder):
     args = parse(["--model", "x", "--ignore-chat-template"])
     assert chat_prompt(tok, "fox", args) == "fox"
     assert chat_prompt(IdTokenizer(), "1 2 3", parse(["--model", "x"])) == "1 2 3"
+
+
+def test_the_detokenizer_of_a_byte_level_vocabulary_looks_bytes_up(folder, tmp_path):
+    """A byte-level vocabulary's tokens are fixed runs of bytes (the table covers all 256); any
+    other vocabulary is decoded again from the last line break."""
+    from tokenizers import Tokenizer, models, pre_tokenizers, trainers
+
+    from mlx_lm_amd.tokenizer_utils import TokenizerWrapper, _byte_of_symbol, load_tokenizer
+
+    table = _byte_of_symbol()
+    assert sorted(table.values()) == list(range(256)) and table["A"] == 65 and table["Ġ"] == 32
+    tok = load_tokenizer(folder)
+    det = tok.detokenizer
+    assert det._token_bytes is not None
+    assert det._token_bytes(0) == b"<|endoftext|>"  # an added token is its own text
+    words = Tokenizer(models.WordLevel({"[UNK]": 0, "fox": 1, "dog": 2, "\n": 3}, unk_token="[UNK]"))
+    words.pre_tokenizer = pre_tokenizers.Whitespace()
+    plain_tok = TokenizerWrapper(words)
+    det = plain_tok.detokenizer
+    assert det._token_bytes is None
+    for t in (1, 2, 1):
+        det.add_token(t)
+    det.finalize()
+    assert det.text == plain_tok.decode([1, 2, 1]) and det.tokens == [1, 2, 1]
