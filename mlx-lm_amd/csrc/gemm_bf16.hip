@@ -128,7 +128,12 @@ using Tile32x128 = TileShape<1, 4, 1, 1, 8, 2>;
 // MFMA units idle: 8 % slower); one barrier an iteration.
 // SPLIT: K is shared out over blockIdx.y and the partial sums go to the workspace (a kernel of
 // its own, so that the unsplit one carries none of it).
-template <typename S, bool SPLIT>
+// PACKED: W lies in the decode kernels' packed order.  A wave's load is then half a tile of 16
+// features x 64 k, 1 KB of consecutive bytes: lane l gets the 8 values k = 16 (l / 16) + 8 h + 0..7
+// of feature l % 16, and load g of the block's BN / 8 covers feature block g / 2, half h = g % 2.
+// (Reading the packed order with the row-major kernel's lanes, eight pieces of one row to eight
+// neighbouring lanes, touched eight lines with every eight lanes: 14 % slower.)
+template <typename S, bool SPLIT, bool PACKED>
 __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_kernel(GemmArgs p) {
   constexpr int BM = S::BM, BN = S::BN, TM = S::TM, TN = S::TN, PA = S::PA, PB = S::PB;
   // (one buffer: the epilogue uses it again for the output tiles)
@@ -163,11 +168,19 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
 #pragma unroll
   for (int i = 0; i < PA; ++i) a_off[i] = row_inside(m0 + (tid >> 3) + ROW_STEP * i, p.M) * p.lda + (tid & 7) * 8;
   // (packed weights: a k-block further on is 1024 elements further on, not 64)
-  const int wmul = p.w_packed ? 16 : 1;
+  constexpr int wmul = PACKED ? 16 : 1;
+  int lds_b[PB];  // where the thread's pieces of W go in a stage of LDS
 #pragma unroll
   for (int i = 0; i < PB; ++i) {
-    const int n = row_inside(n0 + (tid >> 3) + ROW_STEP * i, p.N);
-    b_off[i] = p.w_packed ? packed_piece(n, tid & 7, p.w_kblocks) : n * p.ldw + (tid & 7) * 8;
+    if constexpr (PACKED) {
+      const int g = wave * PB + i, fb = g >> 1, h = g & 1;
+      const int nb = min(n0 / 16 + fb, (p.N + 15) / 16 - 1);  // (blocks beyond the matrix read its last one)
+      b_off[i] = nb * p.w_kblocks * 1024 + h * 512 + lane * 8;
+      lds_b[i] = (fb * 16 + (lane & 15)) * LDS_STRIDE + (2 * (lane >> 4) + h) * 8;
+    } else {
+      b_off[i] = row_inside(n0 + (tid >> 3) + ROW_STEP * i, p.N) * p.ldw + (tid & 7) * 8;
+      lds_b[i] = lds_off0 + i * ROW_STEP * LDS_STRIDE;
+    }
   }
   const int kc_mine = (tid & 7) * 8;
   // this split's k-blocks (all of them without a split); the offsets start at its first column
@@ -188,7 +201,7 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
     // columns) and zeroed when it goes to LDS: zeroing it here would make the
     // loads wait at once
     const int kk = (k_lo + k0 + kc_mine < p.K) ? k0 : p.K - 8 - kc_mine - k_lo;
-    const int kw = p.w_packed ? k0 * 16 : kk;  // (packed weights are padded with zeros to whole k-blocks)
+    const int kw = PACKED ? k0 * 16 : kk;  // (packed weights are padded with zeros to whole k-blocks)
 #pragma unroll
     for (int i = 0; i < PA; ++i) xa[i] = *(const uint4*)(p.A + a_off[i] + kk);
 #pragma unroll
@@ -199,7 +212,7 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
 #pragma unroll
     for (int i = 0; i < PA; ++i) *(uint4*)(As[stage] + lds_off0 + i * ROW_STEP * LDS_STRIDE) = in ? xa[i] : ZERO4;
 #pragma unroll
-    for (int i = 0; i < PB; ++i) *(uint4*)(Bs[stage] + lds_off0 + i * ROW_STEP * LDS_STRIDE) = in ? xb[i] : ZERO4;
+    for (int i = 0; i < PB; ++i) *(uint4*)(Bs[stage] + lds_b[i]) = (PACKED || in) ? xb[i] : ZERO4;
   };
 
   load_global(ra[0], rb[0], 0);
@@ -254,7 +267,7 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
     const uint16_t* af = a_frag + stage * (BM * LDS_STRIDE);
     const uint16_t* bf = b_frag + stage * (BN * LDS_STRIDE);
     uint16_t* an = As[stage ^ 1] + lds_off0;
-    uint16_t* bn = Bs[stage ^ 1] + lds_off0;
+    uint16_t* bn = Bs[stage ^ 1];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int ks = q * 16;
@@ -266,7 +279,7 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
 #pragma unroll
       for (int i = q * PA / 4; i < (q + 1) * PA / 4; ++i) *(uint4*)(an + i * ROW_STEP * LDS_STRIDE) = xa[i];
 #pragma unroll
-      for (int i = q * PB / 4; i < (q + 1) * PB / 4; ++i) *(uint4*)(bn + i * ROW_STEP * LDS_STRIDE) = xb[i];
+      for (int i = q * PB / 4; i < (q + 1) * PB / 4; ++i) *(uint4*)(bn + lds_b[i]) = xb[i];
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -549,10 +562,17 @@ template <typename S>
 static void launch_tiles(const GemmArgs& p, hipStream_t stream) {
   const long tiles = (long)((p.M + S::BM - 1) / S::BM) * ((p.N + S::BN - 1) / S::BN);
   dim3 grid((unsigned)((tiles + 7) / 8 * 8), p.n_splits), block(S::THREADS);  // a run of tiles for each die
-  if (p.n_splits > 1)
-    hipLaunchKernelGGL((gemm_bf16_tile_kernel<S, true>), grid, block, 0, stream, p);
-  else
-    hipLaunchKernelGGL((gemm_bf16_tile_kernel<S, false>), grid, block, 0, stream, p);
+  if (p.n_splits > 1) {
+    if (p.w_packed)
+      hipLaunchKernelGGL((gemm_bf16_tile_kernel<S, true, true>), grid, block, 0, stream, p);
+    else
+      hipLaunchKernelGGL((gemm_bf16_tile_kernel<S, true, false>), grid, block, 0, stream, p);
+  } else {
+    if (p.w_packed)
+      hipLaunchKernelGGL((gemm_bf16_tile_kernel<S, false, true>), grid, block, 0, stream, p);
+    else
+      hipLaunchKernelGGL((gemm_bf16_tile_kernel<S, false, false>), grid, block, 0, stream, p);
+  }
 }
 
 // How many tiles a die gets (tile_of_block shares them out evenly).
