@@ -84,10 +84,6 @@ typedef struct {
   int dtype;  // compute dtype: 0 float32, 1 bfloat16
   int n_tokens, n_requests, n_wanted, wants_every_row;
   int force_splits;  // tests: split K wherever the kernels can
-  // 1: a product of up to 16 rows that splits K joins its parts in its own kernel even where it
-  // may leave them pending (the next product norms its rows itself at so few rows); 0: it leaves
-  // them pending where it may
-  int join_few_rows, pad_;
   const int* token_ids;
   const int* positions;
   const int* token_req;
@@ -102,8 +98,6 @@ typedef struct {
   EngScratch* scratch;
   float* split_ws;
   size_t split_ws_floats;
-  unsigned* split_counters;  // all zero between launches: a split product's blocks meet at them
-  long n_split_counters;
   float* logits;  // [>= n_wanted, vocab] float32
   long logits_rows;
   EngPending pending;

@@ -62,14 +62,14 @@ typedef int (*fn_layernorm)(void*, const float*, const int*, const float*, const
 typedef int (*fn_gemm_f32)(void*, const void*, const void*, const float*, int, int, int, int, int, int, int,
                            int, hipStream_t);
 typedef int (*fn_gemm_bf16)(void*, const void*, const void*, const float*, int, int, int, int, int, int, int,
-                            int, int, float*, size_t, unsigned*, int, hipStream_t);
+                            int, int, float*, size_t, hipStream_t);
 typedef int (*fn_int5)(int, int, int, int, int);
 typedef int (*fn_int4)(int, int, int, int);
 typedef int (*fn_int2)(int, int);
 typedef int (*fn_gemm_decode)(void*, const void*, int, const float*, int, const float*, const float*, float,
                               const void*, const float*, int, int, int, int, int, int, void*, void*, size_t,
                               const int*, int, const int*, const int*, int, int, int, int, int, float*,
-                              size_t, unsigned*, int, hipStream_t);
+                              size_t, hipStream_t);
 typedef int (*fn_sum_partials)(void*, const float*, int, const float*, int, int, int, int, void*, void*,
                                size_t, const int*, int, const int*, const int*, int, int, int, int,
                                hipStream_t);
@@ -93,10 +93,9 @@ typedef int (*fn_attn_prefill)(void*, const void*, int, int, const void*, const 
 static Entry<fn_embed> k_embed("embed", "embed_gather_add");
 static Entry<fn_layernorm> k_layernorm("norm", "layernorm");
 static Entry<fn_gemm_f32> k_gemm_f32("gemm_f32", "gemm_f32");
-static Entry<fn_gemm_bf16> k_gemm_bf16("gemm_bf16", "gemm_bf16_joined");
-static Entry<fn_int2> k_gemm_bf16_join_counters("gemm_bf16", "gemm_bf16_join_counters");
+static Entry<fn_gemm_bf16> k_gemm_bf16("gemm_bf16", "gemm_bf16");
 static Entry<fn_int5> k_gemm_bf16_splits("gemm_bf16", "gemm_bf16_splits");
-static Entry<fn_gemm_decode> k_gemm_decode("gemm_bf16_decode", "gemm_bf16_decode_joined");
+static Entry<fn_gemm_decode> k_gemm_decode("gemm_bf16_decode", "gemm_bf16_decode");
 static Entry<fn_int4> k_decode_takes("gemm_bf16_decode", "gemm_bf16_decode_takes");
 static Entry<fn_int5> k_decode_splits("gemm_bf16_decode", "gemm_bf16_decode_splits");
 static Entry<fn_sum_partials> k_sum_partials("gemm_bf16_decode", "sum_partials");
@@ -322,11 +321,6 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
     QUERY(k_decode_takes, takes, M, K, with_norm, n_splits);
     if (takes) {
       if (n_splits > 1 && pending) TRY(settle(ctx, pending));  // the workspace is about to be written again
-      // With counters the parts are joined in the product's own kernel (the block that arrives
-      // last adds them and runs the epilogue): no second kernel, and nothing is left pending.
-      const bool may_pend = accumulate && pending && pending->allowed;
-      const bool joined = n_splits > 1 && ctx->split_counters && ctx->n_split_counters >= (N + 7) / 8 &&
-                          (ctx->join_few_rows || !may_pend);
       KERNEL(k_gemm_decode, ctx, out.p, a.lazy ? nullptr : a.m.p, a.lazy ? 0 : a.m.ld, a.lazy ? a.x : nullptr,
              a.lazy ? a.ldx : 0, a.lazy ? a.gamma : nullptr, a.lazy ? a.beta : nullptr, a.lazy ? a.eps : 0.f,
              w.packed ? w.packed : w.w, bias, M, N, K, w.packed ? 0 : w.ldw, out.ld, flags | (sc ? GEMM_KV : 0),
@@ -334,8 +328,8 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
              sc ? sc->block_table : nullptr, sc ? sc->max_blocks : 0, sc ? sc->token_req : nullptr,
              sc ? sc->positions : nullptr, sc ? sc->q_width : 0, sc ? sc->kv_width : 0, sc ? sc->head_dim : 0,
              sc ? sc->page_size : 0, n_splits, n_splits > 1 ? ws : nullptr, n_splits > 1 ? ws_floats : (size_t)0,
-             joined ? ctx->split_counters : nullptr, joined ? (int)ctx->n_split_counters : 0, ctx->stream);
-      if (n_splits > 1 && !joined) {
+             ctx->stream);
+      if (n_splits > 1) {
         if (accumulate && pending && pending->allowed) {
           pending->target = (float*)out.p, pending->rows = M, pending->cols = N, pending->ld = out.ld;
           pending->ws = ws, pending->n_splits = n_splits, pending->bias = bias;
@@ -372,21 +366,9 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
       if (n_splits > 1 && pending) TRY(settle(ctx, pending));  // the workspace is about to be written again
     }
     if (n_splits < 1) n_splits = 1;
-    // The parts are joined in the product's own kernel where no second kernel is wanted for
-    // another reason: not where the sum stays pending for the norm that follows anyway, and not
-    // where the second kernel also writes keys and values into their pages.
-    const bool leave_pending = accumulate && pending && pending->allowed;
-    bool joined = n_splits > 1 && !leave_pending && !sc && ctx->split_counters;
-    if (joined) {
-      int wanted = 0;
-      QUERY(k_gemm_bf16_join_counters, wanted, M, N);
-      joined = wanted <= ctx->n_split_counters;
-    }
     // (weights kept only in the packed order are read in that order: row stride 0 says so)
     KERNEL(k_gemm_bf16, ctx, out.p, A.p, w.w ? w.w : w.packed, bias, M, N, K, A.ld, w.w ? w.ldw : 0, out.ld, flags,
-           variant, n_splits, n_splits > 1 ? ws : nullptr, n_splits > 1 ? ws_floats : (size_t)0,
-           joined ? ctx->split_counters : nullptr, joined ? (int)ctx->n_split_counters : 0, ctx->stream);
-    if (joined) return 0;
+           variant, n_splits, n_splits > 1 ? ws : nullptr, n_splits > 1 ? ws_floats : (size_t)0, ctx->stream);
     if (n_splits > 1) {
       if (accumulate && pending && pending->allowed) {
         pending->target = (float*)out.p, pending->rows = M, pending->cols = N, pending->ld = out.ld;

@@ -40,10 +40,6 @@ struct GemmArgs {
   // K split over blockIdx.y (tile kernel, 128 x 128): partial sums [n_splits][M][N] go to ws
   float* ws;
   int n_splits, blocks_per_split;
-  // With counters (one per output tile, all zero between launches) a split's parts are joined in
-  // the kernel: the block that finds the others' sums written adds them, in the order of the
-  // parts, and runs the epilogue.  Without, sum_partials or sum_partials_norm does it afterwards.
-  unsigned* counters;
   // W in the decode kernels' packed order instead of row-major (ldw == 0 at the entry point):
   // tiles of 16 features x 64 k (1024 elements), zero padded, w_kblocks of them a feature block;
   // in a tile the 8 values k = 16 g + 8 h + 0..7 of feature f lie at ((4 h + g) * 16 + f) * 8.
@@ -328,43 +324,7 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int m = mb + 8 * (r >> 2) + (r & 3);
-          if (m >= p.M) continue;
-          if (p.counters)  // (past the die's L2: the block that joins the parts may run on another die)
-            __hip_atomic_store(ws + (size_t)m * p.N + n, acc[i][j][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          else
-            ws[(size_t)m * p.N + n] = acc[i][j][r];
-        }
-      }
-    }
-    if (!p.counters) return;
-    // the block that arrives last at the tile's counter joins the parts (and leaves the counter at zero)
-    __shared__ int s_last;
-    __builtin_amdgcn_s_waitcnt(0);  // this thread's partial sums have been taken
-    __syncthreads();
-    if (tid == 0) {
-      unsigned* counter = p.counters + (size_t)tm * ((p.N + BN - 1) / BN) + tn;
-      const unsigned before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      s_last = before == (unsigned)p.n_splits - 1;
-      if (s_last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    if (!s_last) return;
-    const size_t part = (size_t)p.M * p.N;
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int n = n0 + wn * TN * 32 + j * 32 + (lane & 31);
-      if (n >= p.N) continue;
-#pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int mb = m0 + wm * TM * 32 + i * 32 + 4 * (lane >> 5);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int m = mb + 8 * (r >> 2) + (r & 3);
-          if (m >= p.M) continue;
-          float sum = 0.f;
-          for (int s2 = 0; s2 < p.n_splits; ++s2)
-            sum += __hip_atomic_load(p.ws + s2 * part + (size_t)m * p.N + n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          store_out(p, m, n, sum);
+          if (m < p.M) ws[(size_t)m * p.N + n] = acc[i][j][r];
         }
       }
     }
@@ -701,29 +661,9 @@ extern "C" int gemm_bf16_splits(int M, int N, int K, int fused, int force) {
 // tiles, 5 = 64 x 128 tiles, 6 = 32 x 128 tiles.  n_splits > 1 (variants 1, 5 and 6 only): no
 // epilogue, the partial sums go to ws.  ldw == 0: W is in the decode kernels' packed order
 // (tiles of 16 features x 64 k, zero padded), which all kernels here read as well as rows.
-extern "C" int gemm_bf16_joined(void* out, const void* A, const void* W, const float* bias, int M, int N,
-                                int K, int lda, int ldw, int ldo, int flags, int variant, int n_splits,
-                                float* ws, size_t ws_floats, unsigned* counters, int n_counters,
-                                hipStream_t stream);
-
 extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* bias, int M, int N,
                          int K, int lda, int ldw, int ldo, int flags, int variant, int n_splits,
                          float* ws, size_t ws_floats, hipStream_t stream) {
-  return gemm_bf16_joined(out, A, W, bias, M, N, K, lda, ldw, ldo, flags, variant, n_splits, ws, ws_floats,
-                          nullptr, 0, stream);
-}
-
-// How many counters gemm_bf16_joined wants for a product of M x N in parts (the most any of the
-// splitting tile shapes would use).
-extern "C" int gemm_bf16_join_counters(int M, int N) { return ((M + 31) / 32) * ((N + 127) / 128); }
-
-// The same with `counters` (all zero, gemm_bf16_join_counters(M, N) of them or more): with K
-// split, the block that arrives last at an output tile joins the parts and runs the epilogue, so
-// no second kernel follows.  Null counters: the partial sums are left in ws.
-extern "C" int gemm_bf16_joined(void* out, const void* A, const void* W, const float* bias, int M, int N,
-                                int K, int lda, int ldw, int ldo, int flags, int variant, int n_splits,
-                                float* ws, size_t ws_floats, unsigned* counters, int n_counters,
-                                hipStream_t stream) {
   GemmArgs p;
   p.A = (const uint16_t*)A;
   p.W = (const uint16_t*)W;
@@ -738,13 +678,6 @@ extern "C" int gemm_bf16_joined(void* out, const void* A, const void* W, const f
   const int n_blocks = (K + BK - 1) / BK;
   if (n_splits < 1 || n_splits > n_blocks) FAIL("gemm_bf16: %d splits of K=%d", n_splits, K);
   p.ws = ws, p.n_splits = n_splits, p.blocks_per_split = (n_blocks + n_splits - 1) / n_splits;
-  p.counters = nullptr;
-  if (n_splits > 1 && counters) {
-    if (n_counters < gemm_bf16_join_counters(M, N))
-      FAIL("gemm_bf16: %d counters, a product of %d x %d in parts needs %d", n_counters, M, N,
-           gemm_bf16_join_counters(M, N));
-    p.counters = counters;
-  }
   if (n_splits > 1) {
     if (variant == 0) variant = M <= 32 ? 6 : small_tiles(M, N) ? 5 : 1;
     if (variant != 1 && variant != 5 && variant != 6) FAIL("gemm_bf16: only the tiles of 128, 64 and 32 rows by 128 split K");

@@ -78,34 +78,7 @@ struct DecodeGemmArgs {
   int rows;            // output features a block of the 16-row kernel owns (16, or 8 where features are few)
   float* ws;           // [n_splits][M][N] partial sums, when n_splits > 1
   int vec4;            // four outputs at a time: N, ldo and the scatter widths are multiples of 4, pointers aligned
-  // With counters (one per feature block, all zero between launches) the parts are joined in this
-  // kernel: the block that finds the others' sums written adds them, in the order of the parts,
-  // and runs the epilogue.  Without, sum_partials or sum_partials_norm does it afterwards.
-  unsigned* counters;
 };
-
-// Partial sums pass between blocks on different dies, whose L2s do not see each other's lines:
-// they are written and read at agent scope (past the die's L2), a counter says when all are there.
-__device__ __forceinline__ void put_partial(float* at, float v) {
-  __hip_atomic_store(at, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ float get_partial(const float* at) {
-  return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-// Called by every thread of the block after its put_partial calls; true in all threads of the
-// block that arrives last at `counter` (which it leaves at zero again for the next launch).
-__device__ __forceinline__ bool last_to_arrive(unsigned* counter, unsigned n_parts) {
-  __shared__ int s_last;
-  __builtin_amdgcn_s_waitcnt(0);  // this thread's partial sums have been taken
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    const unsigned before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    s_last = before == n_parts - 1;
-    if (s_last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  __syncthreads();
-  return s_last != 0;
-}
 
 __device__ __forceinline__ uint32_t pack2(float a, float b) { return pack_bf16x2(a, b); }
 
@@ -352,31 +325,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArg
     const int f = 4 * (L >> 4) + r;
     const int n = n0 + f;
     const int m = L & 15;
-    const bool mine = m < p.M && f < p.rows && n < p.N;
-    if (p.n_splits == 1) {
-      if (mine) finish(p, m, n, v);
-      return;
-    }
-    const size_t at = (size_t)m * p.N + n, part = (size_t)p.M * p.N;
-    if (!p.counters) {
-      if (mine) p.ws[blockIdx.y * part + at] = v;  // summed, and finished, by sum_partials
-      return;
-    }
-    if (mine) put_partial(p.ws + blockIdx.y * part + at, v);
-  }
-  if (p.n_splits > 1 && p.counters) {
-    if (!last_to_arrive(p.counters + blockIdx.x, p.n_splits)) return;
-    if (tid < 256) {
-      const int L = tid >> 2, r = tid & 3;
-      const int f = 4 * (L >> 4) + r;
-      const int n = n0 + f;
-      const int m = L & 15;
-      if (m < p.M && f < p.rows && n < p.N) {
-        const size_t at = (size_t)m * p.N + n, part = (size_t)p.M * p.N;
-        float sum = 0.f;
-        for (int s = 0; s < p.n_splits; ++s) sum += get_partial(p.ws + s * part + at);
-        finish(p, m, n, sum);
-      }
+    if (m < p.M && f < p.rows && n < p.N) {
+      if (p.n_splits > 1)
+        p.ws[((size_t)blockIdx.y * p.M + m) * p.N + n] = v;  // summed, and finished, by sum_partials
+      else
+        finish(p, m, n, v);
     }
   }
 }
@@ -606,14 +559,6 @@ static int fill_epilogue(DecodeGemmArgs& p, const char* who, void* out, const fl
   return 0;
 }
 
-extern "C" int gemm_bf16_decode_joined(
-    void* out, const void* A, int lda, const float* X, int ldx, const float* gamma,
-    const float* beta, float eps, const void* W, const float* bias, int M, int N, int K, int ldw,
-    int ldo, int flags, void* k_pages, void* v_pages, size_t page_stride, const int* block_table,
-    int max_blocks, const int* token_req, const int* positions, int q_width, int kv_width,
-    int head_dim, int page_size, int n_splits, float* ws, size_t ws_floats, unsigned* counters,
-    int n_counters, hipStream_t stream);
-
 // With n_splits > 1 the epilogue does not run: the partial sums go to `ws`
 // ([n_splits][M][N] floats) and sum_partials or sum_partials_norm finishes.
 extern "C" int gemm_bf16_decode(
@@ -622,21 +567,6 @@ extern "C" int gemm_bf16_decode(
     int ldo, int flags, void* k_pages, void* v_pages, size_t page_stride, const int* block_table,
     int max_blocks, const int* token_req, const int* positions, int q_width, int kv_width,
     int head_dim, int page_size, int n_splits, float* ws, size_t ws_floats, hipStream_t stream) {
-  return gemm_bf16_decode_joined(out, A, lda, X, ldx, gamma, beta, eps, W, bias, M, N, K, ldw, ldo, flags, k_pages,
-                                 v_pages, page_stride, block_table, max_blocks, token_req, positions, q_width,
-                                 kv_width, head_dim, page_size, n_splits, ws, ws_floats, nullptr, 0, stream);
-}
-
-// The same with `counters` (n_counters of them, all zero, at least one per block of features):
-// with K split, the block that arrives last joins the parts and runs the epilogue, so no second
-// kernel follows.  Null counters: the partial sums are left in ws as above.
-extern "C" int gemm_bf16_decode_joined(
-    void* out, const void* A, int lda, const float* X, int ldx, const float* gamma,
-    const float* beta, float eps, const void* W, const float* bias, int M, int N, int K, int ldw,
-    int ldo, int flags, void* k_pages, void* v_pages, size_t page_stride, const int* block_table,
-    int max_blocks, const int* token_req, const int* positions, int q_width, int kv_width,
-    int head_dim, int page_size, int n_splits, float* ws, size_t ws_floats, unsigned* counters,
-    int n_counters, hipStream_t stream) {
   if (M == 0) return 0;
   const bool ln = X != nullptr;
   if (!gemm_bf16_decode_takes(M, K, ln, n_splits))
@@ -663,12 +593,6 @@ extern "C" int gemm_bf16_decode_joined(
   p.rows = (n_splits == 1 && (N + 15) / 16 < FEW_BLOCKS) ? 8 : 16;
   p.n_splits = n_splits, p.chunks_per_split = chunks_per_split(K, n_splits);
   p.ws = ws;
-  p.counters = nullptr;
-  if (n_splits > 1 && counters) {
-    if (n_counters < (N + p.rows - 1) / p.rows)
-      FAIL("gemm_bf16_decode: %d counters for %d blocks of features", n_counters, (N + p.rows - 1) / p.rows);
-    p.counters = counters;
-  }
   if (n_splits > 1) {
     if (!ws || !aligned16(ws)) FAIL("gemm_bf16_decode: a split of K needs a 16-byte aligned workspace");
     if (ws_floats < (size_t)n_splits * M * N)

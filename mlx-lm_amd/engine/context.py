@@ -152,7 +152,6 @@ class StepContext:
         c.slots, c.n_slots = engine.slot_table, len(engine.slot_table)
         c.n_compute_units = engine.n_compute_units
         c.split_ws, c.split_ws_floats = engine.split_ws.data_ptr(), engine.split_ws.numel()
-        c.split_counters, c.n_split_counters = engine.split_counters.data_ptr(), engine.split_counters.numel()
         c.stats = ctypes.pointer(engine.stats)
         self.n_tokens = self.n_requests = self.n_wanted = 0
         self.wants_every_row = False  # wanted_rows is 0 .. n_tokens - 1
@@ -224,7 +223,7 @@ class StepContext:
         from ..ops import kernels
 
         self.c.stream = kernels.raw_stream()
-        self.c.force_splits, self.c.join_few_rows = kernels.force_splits, int(kernels.join_few_rows)
+        self.c.force_splits = kernels.force_splits
         return native.running(self)
 
     @property

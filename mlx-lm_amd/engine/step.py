@@ -63,7 +63,6 @@ class Engine:
         native.lib()
         self.n_compute_units = kernels.n_compute_units()
         self.split_ws = kernels.split_workspace(self.device)
-        self.split_counters = kernels.split_counters(self.device)
         self.stats = native.EngStats()
         self.slot_table = self._slot_table()
         self.array_providers = self.decoder.array_providers()

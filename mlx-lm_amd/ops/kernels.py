@@ -68,12 +68,10 @@ def bare_context():
         c = _BARE[dev] = native.EngCtx()
         ws = split_workspace(torch.device("cuda", dev))
         c.split_ws, c.split_ws_floats = ws.data_ptr(), ws.numel()
-        counters = split_counters(torch.device("cuda", dev))
-        c.split_counters, c.n_split_counters = counters.data_ptr(), counters.numel()
         c.n_compute_units = n_compute_units()
         c.dtype = 1
     c.stream = raw_stream()
-    c.force_splits, c.join_few_rows = force_splits, int(join_few_rows)
+    c.force_splits = force_splits
     return c
 
 
@@ -257,12 +255,6 @@ SPLIT_WS_FLOATS = 8 << 20  # 32 MB: sixteen splits of 64 rows by 8192 features
 # launch would fill the GPU without (tiny models): 0 leaves the choice to the library.
 force_splits = 0
 
-# A product of up to 16 rows that splits K joins its parts in its own kernel (the block that
-# arrives last adds them) even where it might leave them pending for the next norm: at so few
-# rows the next product norms its rows itself, and the second kernel is saved.  Tests of the
-# pending sums switch this off.
-join_few_rows = True
-
 
 def split_workspace(device):
     """Float32 room for the partial sums of projections that split K over blocks.
@@ -277,21 +269,6 @@ def split_workspace(device):
         ws = torch.empty(SPLIT_WS_FLOATS, dtype=torch.float32, device=device)
         _SPLIT_WS[key] = ws
     return ws
-
-
-_SPLIT_COUNTERS = {}
-N_SPLIT_COUNTERS = 8192
-
-
-def split_counters(device):
-    """Counters (all zero between launches) at which the blocks of a product that splits K meet:
-    the block that arrives last at its output tile's counter joins the parts.  One array per device."""
-    device = torch.device(device)
-    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
-    c = _SPLIT_COUNTERS.get(key)
-    if c is None:
-        c = _SPLIT_COUNTERS[key] = torch.zeros(N_SPLIT_COUNTERS, dtype=torch.int32, device=device)
-    return c
 
 
 class PendingSum:

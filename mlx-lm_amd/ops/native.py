@@ -67,14 +67,12 @@ class EngCtx(Structure):
     _fields_ = [
         ("stream", c_void_p), ("dtype", c_int), ("n_tokens", c_int), ("n_requests", c_int),
         ("n_wanted", c_int), ("wants_every_row", c_int), ("force_splits", c_int),
-        ("join_few_rows", c_int), ("pad_", c_int),
         ("token_ids", c_void_p), ("positions", c_void_p), ("token_req", c_void_p),
         ("wanted_rows", c_void_p), ("slot_ids", c_void_p),
         ("arrays", c_void_p * MAX_ARRAYS), ("counts", c_long * MAX_ARRAYS),
         ("block_tables", c_void_p * MAX_GROUPS), ("table_width", c_int * MAX_GROUPS),
         ("slots", POINTER(EngSlot)), ("n_slots", c_int), ("n_compute_units", c_int),
         ("scratch", POINTER(EngScratch)), ("split_ws", c_void_p), ("split_ws_floats", c_size_t),
-        ("split_counters", c_void_p), ("n_split_counters", c_long),
         ("logits", c_void_p), ("logits_rows", c_long), ("pending", EngPending),
         ("read_ahead", POINTER(EngWeight)), ("stats", POINTER(EngStats)), ("py", c_void_p),
     ]

@@ -799,12 +799,11 @@ def test_gemm_bf16_small_tiles_split_k(M, N, K, mode):
 @pytest.mark.parametrize("M,N,K", [(1, 64, 256), (8, 1600, 6400), (16, 96, 384), (40, 240, 200), (64, 1600, 1600),
                                    (5, 4100, 512), (100, 1600, 1600), (200, 240, 456)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
-def test_pending_sum_is_added_by_the_norm(M, N, K, out_dtype, monkeypatch):
+def test_pending_sum_is_added_by_the_norm(M, N, K, out_dtype):
     """A split projection into the residual stream may stop at its partial sums; the norm that reads the
     stream next adds them, writes the stream and norms the new rows in one kernel.  A bias of 3 on one
     feature and a stream row far from zero show a sum or a shift left out."""
     k = _k()
-    monkeypatch.setattr(k, "join_few_rows", False)  # (few rows would join their parts themselves)
     a = _rand((M, K), torch.bfloat16, 10)
     w = _rand((N, K), torch.bfloat16, 11, 0.1)
     bias = _rand((N,), torch.float32, 12)
@@ -850,47 +849,6 @@ def test_pending_sum_is_added_by_the_norm(M, N, K, out_dtype, monkeypatch):
         h4 = h0.clone()
         k.linear(h4, a, w, bias, accumulate=True, splits=splits, pending=pending)
         assert not pending.waits_on(h4) and torch.equal(h4, h3)
-
-
-@pytest.mark.parametrize("M,N,K", [(1, 64, 256), (8, 1600, 6400), (16, 96, 384), (11, 333, 1608), (5, 4100, 512),
-                                   (40, 240, 200), (64, 6400, 1600), (33, 257, 1608), (100, 1600, 1600), (300, 520, 456)])
-@pytest.mark.parametrize("mode", ["plain", "gelu", "accumulate", "f32out"])
-def test_split_products_join_their_parts_in_their_own_kernel(M, N, K, mode, monkeypatch):
-    """A product that splits K joins the parts itself: the block that arrives last at its tile's
-    counter adds the partial sums in the order of the parts and runs the epilogue.  Bit for bit what
-    the second kernel makes of the same parts, ten times over (the counters are left at zero)."""
-    k = _k()
-    a = _rand((M, K), torch.bfloat16, 10)
-    w = _rand((N, K), torch.bfloat16, 11, 0.1)
-    bias = _rand((N,), torch.float32, 12)
-    ref = plain.linear(a.double().cpu(), w.double().cpu(), bias.double().cpu())
-    start = _rand((M, N), torch.float32, 13)
-    launches = []
-    lib = k.build.load("gemm_bf16_decode")
-    for splits in (2, 3, 5):
-        if splits > (K + 63) // 64:
-            continue
-
-        def run(counters):
-            dtype = torch.float32 if mode in ("accumulate", "f32out") else torch.bfloat16
-            out = start.clone().to(dtype)
-            ctx = k.bare_context()
-            keep = (ctx.split_counters, ctx.n_split_counters)
-            if not counters:
-                ctx.split_counters, ctx.n_split_counters = None, 0
-            try:
-                k.linear(out, a, w, bias, gelu=(mode == "gelu"), accumulate=(mode == "accumulate"), splits=splits)
-            finally:
-                ctx.split_counters, ctx.n_split_counters = keep
-            return out
-
-        two_kernels = run(False)
-        for _ in range(10):
-            assert torch.equal(run(True), two_kernels), splits
-        assert int(k.split_counters(DEV).abs().sum()) == 0
-        want = plain.gelu_tanh(ref) if mode == "gelu" else ref + start.double().cpu() if mode == "accumulate" else ref
-        tol = 2**-6 if two_kernels.dtype == torch.bfloat16 else 1e-4 * math.sqrt(K)
-        assert torch.allclose(two_kernels.double().cpu(), want, rtol=tol, atol=tol)
 
 
 def test_reading_weights_ahead_changes_nothing():
