@@ -62,7 +62,8 @@ typedef int (*fn_layernorm)(void*, const float*, const int*, const float*, const
 typedef int (*fn_gemm_f32)(void*, const void*, const void*, const float*, int, int, int, int, int, int, int,
                            int, hipStream_t);
 typedef int (*fn_gemm_bf16)(void*, const void*, const void*, const float*, int, int, int, int, int, int, int,
-                            int, int, float*, size_t, hipStream_t);
+                            int, int, float*, size_t, void*, void*, size_t, const int*, int, const int*,
+                            const int*, int, int, int, int, hipStream_t);
 typedef int (*fn_int5)(int, int, int, int, int);
 typedef int (*fn_int4)(int, int, int, int);
 typedef int (*fn_int2)(int, int);
@@ -93,7 +94,7 @@ typedef int (*fn_attn_prefill)(void*, const void*, int, int, const void*, const 
 static Entry<fn_embed> k_embed("embed", "embed_gather_add");
 static Entry<fn_layernorm> k_layernorm("norm", "layernorm");
 static Entry<fn_gemm_f32> k_gemm_f32("gemm_f32", "gemm_f32");
-static Entry<fn_gemm_bf16> k_gemm_bf16("gemm_bf16", "gemm_bf16");
+static Entry<fn_gemm_bf16> k_gemm_bf16("gemm_bf16", "gemm_bf16_scatter");
 static Entry<fn_int5> k_gemm_bf16_splits("gemm_bf16", "gemm_bf16_splits");
 static Entry<fn_gemm_decode> k_gemm_decode("gemm_bf16_decode", "gemm_bf16_decode");
 static Entry<fn_int4> k_decode_takes("gemm_bf16_decode", "gemm_bf16_decode_takes");
@@ -366,9 +367,16 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
       if (n_splits > 1 && pending) TRY(settle(ctx, pending));  // the workspace is about to be written again
     }
     if (n_splits < 1) n_splits = 1;
-    // (weights kept only in the packed order are read in that order: row stride 0 says so)
+    // (weights kept only in the packed order are read in that order: row stride 0 says so; without a
+    // split of K the product's own epilogue puts keys and values into their pages)
+    const EngScatter* own = n_splits == 1 ? sc : nullptr;
     KERNEL(k_gemm_bf16, ctx, out.p, A.p, w.w ? w.w : w.packed, bias, M, N, K, A.ld, w.w ? w.ldw : 0, out.ld, flags,
-           variant, n_splits, n_splits > 1 ? ws : nullptr, n_splits > 1 ? ws_floats : (size_t)0, ctx->stream);
+           variant, n_splits, n_splits > 1 ? ws : nullptr, n_splits > 1 ? ws_floats : (size_t)0,
+           own ? own->k : nullptr, own ? own->v : nullptr, own ? own->page_stride : (size_t)0,
+           own ? own->block_table : nullptr, own ? own->max_blocks : 0, own ? own->token_req : nullptr,
+           own ? own->positions : nullptr, own ? own->q_width : 0, own ? own->kv_width : 0,
+           own ? own->head_dim : 0, own ? own->page_size : 0, ctx->stream);
+    if (own) return 0;
     if (n_splits > 1) {
       if (accumulate && pending && pending->allowed) {
         pending->target = (float*)out.p, pending->rows = M, pending->cols = N, pending->ld = out.ld;

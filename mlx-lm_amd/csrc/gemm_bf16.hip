@@ -23,6 +23,7 @@
 #define FLAG_GELU 1
 #define FLAG_ACCUMULATE 2
 #define FLAG_OUT_F32 4
+#define FLAG_KV 8  // columns from q_width on are keys, then values: they go to their cache pages, not to out
 
 // Out-of-range loads read a clamped address and are zeroed afterwards with this
 // constant: selecting between an address and a zero kept in a variable turns
@@ -40,6 +41,14 @@ struct GemmArgs {
   // K split over blockIdx.y (tile kernel, 128 x 128): partial sums [n_splits][M][N] go to ws
   float* ws;
   int n_splits, blocks_per_split;
+  // key/value scatter (FLAG_KV): row m is token m of the step, at positions[m] of request token_req[m]
+  uint16_t* k_pages;
+  uint16_t* v_pages;
+  size_t page_stride;
+  const int* block_table;
+  const int* token_req;
+  const int* positions;
+  int max_blocks, q_width, kv_width, head_dim, page_size;
   // W in the decode kernels' packed order instead of row-major (ldw == 0 at the entry point):
   // tiles of 16 features x 64 k (1024 elements), zero padded, w_kblocks of them a feature block;
   // in a tile the 8 values k = 16 g + 8 h + 0..7 of feature f lie at ((4 h + g) * 16 + f) * 8.
@@ -51,9 +60,25 @@ __device__ __forceinline__ int packed_piece(int n, int piece, int w_kblocks) {
   return (n >> 4) * w_kblocks * 1024 + ((((piece & 1) << 2) + (piece >> 1)) * 16 + (n & 15)) * 8;
 }
 
+// Where column n (a key's or a value's: n >= q_width) of token m lies in the cache pages.
+__device__ __forceinline__ uint16_t* kv_place(const GemmArgs& p, int m, int n) {
+  const int c = n - p.q_width;
+  const bool is_v = c >= p.kv_width;
+  const int cc = is_v ? c - p.kv_width : c;
+  const int head = cc / p.head_dim, d = cc - head * p.head_dim;
+  const int pos = p.positions[m];
+  const int page = p.block_table[(size_t)p.token_req[m] * p.max_blocks + pos / p.page_size];
+  return (is_v ? p.v_pages : p.k_pages) + (size_t)page * p.page_stride +
+         ((size_t)head * p.page_size + pos % p.page_size) * p.head_dim + d;
+}
+
 __device__ __forceinline__ void store_out(const GemmArgs& p, int m, int n, float v) {
   if (p.bias) v += p.bias[n];
   if (p.flags & FLAG_GELU) v = gelu_tanh_fast(v);
+  if ((p.flags & FLAG_KV) && n >= p.q_width) {
+    *kv_place(p, m, n) = f32_to_bf16_bits(v);
+    return;
+  }
   const size_t idx = (size_t)m * p.ldo + n;
   if (p.flags & FLAG_ACCUMULATE) {
     float* o = (float*)p.out;
@@ -366,6 +391,9 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
     for (int c = 0; c < CPL; ++c) bias[c] = p.bias ? p.bias[min(n + c, p.N - 1)] : 0.f;
     // whole pieces of 16 bytes: the row stride and the base keep them aligned, and all the columns exist
     const bool vec = n + CPL <= p.N && p.ldo % CPL == 0 && ((uintptr_t)p.out & 15) == 0;
+    // this lane's columns are a key's or a value's: its pieces go to the token's place in the
+    // cache pages (the host has seen to it that a piece of eight columns stays inside a head)
+    const bool kv_lane = CPL == 8 && (p.flags & FLAG_KV) && n >= p.q_width;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const int mt = m0 + wm * TM * 32 + i * 32;  // first row of this 32-row tile
@@ -399,6 +427,11 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
             }
           }
         }
+        uint16_t* place[GROUP];
+        if (kv_lane) {
+#pragma unroll
+          for (int s = 0; s < GROUP; ++s) place[s] = kv_place(p, min(mt + (s0 + s) * RPP + erow, p.M - 1), n);
+        }
         __builtin_amdgcn_sched_barrier(0);
         float v[GROUP][CPL];
 #pragma unroll
@@ -430,8 +463,13 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
             if constexpr (CPL == 4)
               *(float4*)(out_f + at) = make_float4(v[s][0], v[s][1], v[s][2], v[s][3]);
             else
-              *(uint4*)(out_h + at) = make_uint4(pack_bf16x2(v[s][0], v[s][1]), pack_bf16x2(v[s][2], v[s][3]),
-                                                 pack_bf16x2(v[s][4], v[s][5]), pack_bf16x2(v[s][6], v[s][7]));
+              *(uint4*)(kv_lane ? place[s] : out_h + at) =
+                  make_uint4(pack_bf16x2(v[s][0], v[s][1]), pack_bf16x2(v[s][2], v[s][3]),
+                             pack_bf16x2(v[s][4], v[s][5]), pack_bf16x2(v[s][6], v[s][7]));
+          } else if (kv_lane) {
+#pragma unroll
+            for (int c = 0; c < CPL; ++c)
+              if (n + c < p.N) place[s][c] = f32_to_bf16_bits(v[s][c]);
           } else {
 #pragma unroll
             for (int c = 0; c < CPL; ++c) {
@@ -661,9 +699,30 @@ extern "C" int gemm_bf16_splits(int M, int N, int K, int fused, int force) {
 // tiles, 5 = 64 x 128 tiles, 6 = 32 x 128 tiles.  n_splits > 1 (variants 1, 5 and 6 only): no
 // epilogue, the partial sums go to ws.  ldw == 0: W is in the decode kernels' packed order
 // (tiles of 16 features x 64 k, zero padded), which all kernels here read as well as rows.
+extern "C" int gemm_bf16_scatter(void* out, const void* A, const void* W, const float* bias, int M, int N,
+                                 int K, int lda, int ldw, int ldo, int flags, int variant, int n_splits,
+                                 float* ws, size_t ws_floats, void* k_pages, void* v_pages, size_t page_stride,
+                                 const int* block_table, int max_blocks, const int* token_req,
+                                 const int* positions, int q_width, int kv_width, int head_dim, int page_size,
+                                 hipStream_t stream);
+
 extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* bias, int M, int N,
                          int K, int lda, int ldw, int ldo, int flags, int variant, int n_splits,
                          float* ws, size_t ws_floats, hipStream_t stream) {
+  return gemm_bf16_scatter(out, A, W, bias, M, N, K, lda, ldw, ldo, flags, variant, n_splits, ws, ws_floats,
+                           nullptr, nullptr, 0, nullptr, 0, nullptr, nullptr, 0, 0, 0, 0, stream);
+}
+
+// The same with the cache scatter of a fused q/k/v projection (k_pages != null, no split of K, a
+// bfloat16 output): the columns from q_width on (kv_width of keys, then kv_width of values) of
+// row m go to position positions[m] of request token_req[m] in the pages, through the block
+// table, and are not written to out.
+extern "C" int gemm_bf16_scatter(void* out, const void* A, const void* W, const float* bias, int M, int N,
+                                 int K, int lda, int ldw, int ldo, int flags, int variant, int n_splits,
+                                 float* ws, size_t ws_floats, void* k_pages, void* v_pages, size_t page_stride,
+                                 const int* block_table, int max_blocks, const int* token_req,
+                                 const int* positions, int q_width, int kv_width, int head_dim, int page_size,
+                                 hipStream_t stream) {
   GemmArgs p;
   p.A = (const uint16_t*)A;
   p.W = (const uint16_t*)W;
@@ -675,6 +734,23 @@ extern "C" int gemm_bf16(void* out, const void* A, const void* W, const float* b
   p.w_packed = ldw == 0 ? 1 : 0, p.w_kblocks = (K + BK - 1) / BK;
   if (check_args(p)) return 1;
   if (M == 0) return 0;
+  p.k_pages = (uint16_t*)k_pages, p.v_pages = (uint16_t*)v_pages, p.page_stride = page_stride;
+  p.block_table = block_table, p.token_req = token_req, p.positions = positions;
+  p.max_blocks = max_blocks, p.q_width = q_width, p.kv_width = kv_width, p.head_dim = head_dim, p.page_size = page_size;
+  if (k_pages) {
+    if (flags & (FLAG_GELU | FLAG_ACCUMULATE | FLAG_OUT_F32)) FAIL("gemm_bf16: the cache scatter goes with a plain bfloat16 output");
+    if (n_splits > 1) FAIL("gemm_bf16: with K split, sum_partials scatters keys and values");
+    if (!v_pages || !block_table || !token_req || !positions)
+      FAIL("gemm_bf16: the cache scatter needs pages, block table, token_req and positions");
+    if (head_dim <= 0 || page_size <= 0 || head_dim % 8 != 0 || q_width % 8 != 0 || kv_width % head_dim != 0 ||
+        q_width + 2 * kv_width != N)
+      FAIL("gemm_bf16: q_width %d + 2 * kv_width %d must be N=%d, widths multiples of 8, kv_width of head_dim %d",
+           q_width, kv_width, N, head_dim);
+    if (page_stride % 8 != 0 || (((uintptr_t)k_pages | (uintptr_t)v_pages) & 15))
+      FAIL("gemm_bf16: cache pages must be 16-byte aligned");
+    if (ldo < q_width) FAIL("gemm_bf16: ldo=%d smaller than q_width=%d", ldo, q_width);
+    p.flags |= FLAG_KV;
+  }
   const int n_blocks = (K + BK - 1) / BK;
   if (n_splits < 1 || n_splits > n_blocks) FAIL("gemm_bf16: %d splits of K=%d", n_splits, K);
   p.ws = ws, p.n_splits = n_splits, p.blocks_per_split = (n_blocks + n_splits - 1) / n_splits;

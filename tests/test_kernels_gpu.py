@@ -948,3 +948,36 @@ def test_projection_scatters_keys_and_values(M, dtype, splits):
         assert torch.allclose(pool[page, 1, :, row].reshape(-1).double(), ref[m, qw + kw :], **tol)
         # and nothing else in the page was touched
         assert torch.isnan(pool[page, 0, :, row + 1 :].float()).all()
+
+
+@pytest.mark.parametrize("variant", [0, 1, 3, 4, 5, 6])
+@pytest.mark.parametrize("packed", [False, True])
+def test_tile_products_scatter_keys_and_values_themselves(variant, packed):
+    """The many-row product writes keys and values into their pages from its own epilogue (every tile
+    shape; head size 64 and 80, requests at different positions, rows that are no multiple of a tile,
+    a tile that straddles the edge between queries and keys): the same pages as the product followed
+    by kv_write, and the key and value columns of the output are left alone."""
+    k = _k()
+    for H, Hkv, hd, M_per in ((5, 5, 64, [70, 1, 130, 33]), (4, 2, 80, [90, 45])):
+        ps, D = 16, 136
+        c = PagedCase(torch.bfloat16, H, Hkv, hd, ps, [7 + 20 * i for i in range(len(M_per))], M_per, seed=variant)
+        M = sum(M_per)
+        qw, kw = H * hd, Hkv * hd
+        w = _rand((qw + 2 * kw, D), torch.bfloat16, 3, 0.2)
+        bias = _rand((qw + 2 * kw,), torch.float32, 4, 0.1)
+        a = _rand((M, D), torch.bfloat16, 5)
+        # the product alone, then kv_write (into pages that hold nothing else)
+        c.pool.fill_(float("nan"))
+        plain_out = torch.empty(M, qw + 2 * kw, dtype=torch.bfloat16, device=DEV)
+        k.linear(plain_out, a, w, bias, variant=variant)
+        k.kv_write(plain_out[:, qw : qw + kw], plain_out[:, qw + kw :], c.kv, c.block_table_dev, c.token_req, c.positions)
+        want_pool = c.pool.clone()
+        c.pool.fill_(float("nan"))
+        out = torch.full((M, qw + 2 * kw), float("nan"), dtype=torch.bfloat16, device=DEV)
+        sc = k.KVScatter(c.kv, c.block_table_dev, c.token_req, c.positions, qw)
+        k.linear(out, a, k.PackedWeight(w, keep_rows=False) if packed else w, bias, scatter=sc, variant=variant)
+        assert torch.equal(out[:, :qw], plain_out[:, :qw])
+        assert torch.isnan(out[:, qw:].float()).all()
+        written = ~torch.isnan(want_pool.float())
+        assert written.any() and torch.equal(c.pool[written], want_pool[written])
+        assert torch.isnan(c.pool[~written].float()).all()
