@@ -559,3 +559,131 @@ def test_a_recorded_step_takes_its_tokens_once(tmp_path, dtype):
         states[use_graphs] = eng.cache.state(0)[[eng.cache.requests[r].state_slot for r in seqs]].clone()
     assert torch.equal(states[True], states[False])
     assert torch.equal(results[True], results[False])
+
+
+# ---------------------------------------------------------------------------
+# windowed attention under recorded steps
+
+
+def _register_windowed():
+    from mlx_lm_amd.config import BaseModelArgs, LayerSpec, ModelPlan, PartSpec, RunEntry, register_model
+    from mlx_lm_amd.parts import DecoderModel
+
+    @dataclass
+    class WinArgs(BaseModelArgs):
+        model_type: str
+        width: int
+        vocab: int
+        max_len: int
+        heads: int
+        kv_heads: int
+        window: int
+        inner: int
+
+    class WinModel:
+        """Built-in parts only (so its steps are recorded): a layer that sees every key and one
+        that sees a window of them, grouped key heads, no position term at all."""
+
+        def __init__(self, args):
+            self.args, self.model_type = args, args.model_type
+            self.decoder = DecoderModel(self.plan(args))
+
+        @property
+        def layers(self):
+            return self.decoder.layers
+
+        @staticmethod
+        def plan(a):
+            def norm(p):
+                return PartSpec("layernorm", {"width": a.width, "eps": 1e-5}, p)
+
+            def layer(i, window):
+                p = f"l{i}."
+                return LayerSpec("pre_norm", dict(
+                    mixer_norm=norm(p + "n1."),
+                    mixer=PartSpec("attention", {"width": a.width, "n_heads": a.heads, "n_kv_heads": a.kv_heads,
+                                                 "head_dim": a.width // a.heads, "window": window, "bias": True}, p + "mix."),
+                    ffn_norm=norm(p + "n2."), ffn=PartSpec("gelu_mlp", {"width": a.width, "inner": a.inner}, p + "ff.")))
+
+            return ModelPlan(
+                width=a.width, vocab_size=a.vocab, max_positions=a.max_len,
+                embedding=PartSpec("token", {"vocab_size": a.vocab, "width": a.width}, "emb."),
+                embedding_positions=None, layers=[layer(0, 0), layer(1, a.window)],
+                schedule=[RunEntry(0, 0), RunEntry(1, 1)], final_norm=norm("nf."),
+                head=PartSpec("linear", {"vocab_size": a.vocab, "width": a.width, "weight_name": "emb.weight"}))
+
+    register_model("toy_windowed", WinModel, WinArgs)
+    return WinModel, WinArgs
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_window_under_recorded_steps(tmp_path, dtype):
+    """Decoding far past a window of 24 keys under recorded steps: the windowed group's pages go
+    back as the window passes them (their table entries turn to -1 and stay in the recorded
+    step's table), pages are used again by a second request, and the logits equal the eager
+    engine's bit for bit and the plain implementation's with the window's mask."""
+    from safetensors.torch import save_file
+
+    from mlx_lm_amd.engine import Engine, StepEntry
+    from mlx_lm_amd.utils import load_model
+
+    cfg = dict(model_type="toy_windowed", width=64, vocab=131, max_len=160, heads=4, kv_heads=2, window=24, inner=96)
+    WinModel, WinArgs = _register_windowed()
+    g = torch.Generator().manual_seed(5)
+    tensors = {}
+    for name, spec in WinModel(WinArgs.from_dict(cfg)).decoder.expected_tensors().items():
+        if spec.role == "vector":
+            tensors[name] = (1.0 if name.endswith("n1.weight") or name.endswith("n2.weight") or name == "nf.weight"
+                             else 0.0) + 0.05 * torch.randn(spec.shape, generator=g)
+        else:
+            tensors[name] = torch.randn(spec.shape, generator=g) * (0.15 if "c_attn" in name else 0.08)
+    json.dump(cfg, open(os.path.join(tmp_path, "config.json"), "w"))
+    save_file(tensors, os.path.join(tmp_path, "model.safetensors"))
+    model, _ = load_model(str(tmp_path), dtype=dtype)
+    ref = helpers.round_matrices_to_bf16(tensors) if dtype == "bfloat16" else tensors
+    w = {k: v.double() for k, v in ref.items()}
+    H, Hkv, hd = cfg["heads"], cfg["kv_heads"], cfg["width"] // cfg["heads"]
+
+    def plain_logits(ids):
+        L = len(ids)
+        h = plain.embed_tokens(w["emb.weight"], torch.tensor(ids))
+        for i, window in ((0, None), (1, cfg["window"])):
+            p = f"l{i}."
+            x = plain.layer_norm(h, w[p + "n1.weight"], w[p + "n1.bias"], 1e-5)
+            qkv = plain.linear(x, w[p + "mix.c_attn.weight"], w[p + "mix.c_attn.bias"])
+            q = qkv[:, : H * hd].reshape(L, H, hd).permute(1, 0, 2)
+            k = qkv[:, H * hd : (H + Hkv) * hd].reshape(L, Hkv, hd).permute(1, 0, 2).repeat_interleave(H // Hkv, 0)
+            v = qkv[:, (H + Hkv) * hd :].reshape(L, Hkv, hd).permute(1, 0, 2).repeat_interleave(H // Hkv, 0)
+            o = plain.attention(q, k, v, hd**-0.5, plain.causal_mask(L, 0, window))
+            h = h + plain.linear(plain.merge_heads(o), w[p + "mix.c_proj.weight"], w[p + "mix.c_proj.bias"])
+            h = h + plain.mlp(plain.layer_norm(h, w[p + "n2.weight"], w[p + "n2.bias"], 1e-5), w, p + "ff.")
+        return plain.tied_head(plain.layer_norm(h, w["nf.weight"], w["nf.bias"], 1e-5), w["emb.weight"])
+
+    seqs = {"a": helpers.random_tokens(150, cfg["vocab"], 21), "b": helpers.random_tokens(90, cfg["vocab"], 22)}
+    results = {}
+    for use_graphs in (True, False):
+        eng = Engine(model, dtype=dtype, page_size=16, n_pages=16, max_requests=3, use_graphs=use_graphs)
+        assert eng.use_graphs == use_graphs and len(eng.cache.groups) == 2
+        got = {r: [] for r in seqs}
+        eng.add_request("a")
+        got["a"].append(eng.step([StepEntry("a", seqs["a"][:20], list(range(20)))]).clone())
+        for i in range(20, 100):  # alone, one by one: the window passes pages of the windowed group
+            got["a"].append(eng.step([StepEntry("a", [seqs["a"][i]], [0])]).clone())
+        windowed = next(g for g in eng.cache.groups if g.need.window)
+        full = next(g for g in eng.cache.groups if not g.need.window)
+        assert windowed.pool.n_held < full.pool.n_held and -1 in eng.cache.requests["a"].blocks[eng.cache.groups.index(windowed)]
+        eng.add_request("b")  # takes pages that the window gave back
+        got["b"].append(eng.step([StepEntry("b", seqs["b"][:30], list(range(30)))]).clone())
+        for i in range(50):
+            out = eng.step([StepEntry("a", [seqs["a"][100 + i]], [0]), StepEntry("b", [seqs["b"][30 + i]], [0])])
+            got["a"].append(out[0:1].clone())
+            got["b"].append(out[1:2].clone())
+            eng.cache.check()
+        for i in range(80, 90):
+            got["b"].append(eng.step([StepEntry("b", [seqs["b"][i]], [0])]).clone())
+        if use_graphs:
+            assert all(eng._graphs[n].graph is not None for n in (1, 2))
+        results[use_graphs] = {r: torch.cat(v) for r, v in got.items()}
+    for r, toks in seqs.items():
+        _close(results[True][r], plain_logits(toks[: results[True][r].shape[0]]), dtype, f"a window under recorded steps, request {r}")
+        assert torch.equal(results[True][r], results[False][r]), r
