@@ -42,6 +42,10 @@ struct DecodeArgs {
   const uint4* ahead;
   size_t ahead_pieces;
   int ahead_chunks;
+  // rows_are_requests: item i of `rows` is row i and belongs to request i (a step in which every
+  // request brings one token), so neither `rows` nor `token_req` has to be read.
+  // table_in_lds: the request's page numbers are copied to LDS once (max_blocks of them fit).
+  int rows_are_requests, table_in_lds;
 };
 
 #define MAX_WAVES 16
@@ -62,6 +66,7 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
   constexpr int NL = TILE / KPL;   // loads per tile (= CPK)
   __shared__ float Ms[MAX_WAVES], Ls[MAX_WAVES];
   __shared__ float Os[MAX_WAVES][HD];
+  extern __shared__ int page_of[];  // [max_blocks] with table_in_lds
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n_waves = blockDim.x >> 6;
@@ -93,10 +98,18 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
     return;
   }
   const int item = blockIdx.x, h = blockIdx.y, split = blockIdx.z;
-  const int row = p.rows[item];
+  // Which row, whose pages, at which position: looked up one after the other these are three
+  // trips to memory before the first key can be asked for, in a kernel that otherwise makes one
+  // or two.  In a decode step item i is row i of request i, and the request's page numbers go to
+  // LDS beside the position and the query: one trip, then the keys.
+  const int row = p.rows_are_requests ? item : p.rows[item];
+  const int req = p.rows_are_requests ? item : p.token_req[row];
   const int kv_head = h / (p.n_heads / p.n_kv_heads);
+  const int* table = p.block_table + (size_t)req * p.max_blocks;
+  if (p.table_in_lds) {
+    for (int i = tid; i < p.max_blocks; i += blockDim.x) page_of[i] = table[i];
+  }
   const int pos = p.positions[row];
-  const int* table = p.block_table + (size_t)p.token_req[row] * p.max_blocks;
   const int sub = lane % CPK;  // which 8 columns of the key
   const int kin = lane / CPK;  // which key of a load
 
@@ -121,6 +134,7 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
   for (int i = 0; i < 8; ++i) o[i] = 0.f;
 
   const size_t head_off = (size_t)kv_head * p.page_size * HD;
+  if (p.table_in_lds) __syncthreads();  // (uniform over the block)
 
   for (int t = t_begin + wave; t < t_end; t += n_waves) {
     const int kt = kt0 + t * TILE;
@@ -131,7 +145,7 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
     for (int j = 0; j < NL; ++j) {
       int key = kt + j * KPL + kin;
       key = min(max(key, k_lo), k_hi - 1);
-      const int page = table[key / p.page_size];
+      const int page = p.table_in_lds ? page_of[key / p.page_size] : table[key / p.page_size];
       const size_t off = (size_t)page * p.page_stride + head_off +
                          (size_t)(key % p.page_size) * HD + sub * 8;
       kv[j] = *(const uint4*)(p.k_pages + off);
@@ -215,7 +229,7 @@ template <int CPK>
 __global__ void attn_decode_merge_kernel(DecodeArgs p) {
   constexpr int HD = 8 * CPK;
   const int item = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
-  const int row = p.rows[item];
+  const int row = p.rows_are_requests ? item : p.rows[item];
   const size_t base = ((size_t)item * p.n_heads + h) * p.n_splits;
   float M = -INFINITY;
   for (int s = 0; s < p.n_splits; ++s) M = fmaxf(M, p.part_ml[(base + s) * 2]);
@@ -240,13 +254,22 @@ static void launch(const DecodeArgs& p, int n_rows, int n_waves, hipStream_t str
     extra_y = (n_compute_units() - n_rows * p.n_heads * p.n_splits) / n_rows;
     if (extra_y * n_rows < 8) extra_y = 0;
   }
-  hipLaunchKernelGGL(attn_decode_kernel<CPK>, dim3(n_rows, p.n_heads + extra_y, p.n_splits), dim3(64 * n_waves), 0, stream, p);
+  const size_t lds = p.table_in_lds ? (size_t)p.max_blocks * sizeof(int) : 0;
+  hipLaunchKernelGGL(attn_decode_kernel<CPK>, dim3(n_rows, p.n_heads + extra_y, p.n_splits), dim3(64 * n_waves), lds, stream, p);
   if (p.n_splits > 1)
     hipLaunchKernelGGL(attn_decode_merge_kernel<CPK>, dim3(n_rows, p.n_heads), dim3(8 * CPK), 0, stream, p);
 }
 
 // Same arguments as attn_row; bfloat16 only, head_dim 32, 64 or 128, and pages
 // that hold whole loads (page_size a multiple of 512 / head_dim keys).
+extern "C" int attn_decode_rows(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                                const void* v_pages, size_t page_stride, const int* block_table,
+                                int max_blocks, const int* token_req, const int* positions,
+                                const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
+                                int page_size, int window, float scale, int n_splits, float* part_o,
+                                float* part_ml, int n_waves, const void* ahead, size_t ahead_chunk_bytes,
+                                int ahead_chunks, int rows_are_requests, hipStream_t stream);
+
 extern "C" int attn_decode(void* out, const void* q, int ldq, int ldo, const void* k_pages,
                            const void* v_pages, size_t page_stride, const int* block_table,
                            int max_blocks, const int* token_req, const int* positions,
@@ -254,6 +277,20 @@ extern "C" int attn_decode(void* out, const void* q, int ldq, int ldo, const voi
                            int page_size, int window, float scale, int n_splits, float* part_o,
                            float* part_ml, int n_waves, const void* ahead, size_t ahead_chunk_bytes,
                            int ahead_chunks, hipStream_t stream) {
+  return attn_decode_rows(out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table, max_blocks, token_req,
+                          positions, rows, n_rows, n_heads, n_kv_heads, head_dim, page_size, window, scale,
+                          n_splits, part_o, part_ml, n_waves, ahead, ahead_chunk_bytes, ahead_chunks, 0, stream);
+}
+
+// The same with rows_are_requests: 1 says that item i of `rows` is row i and belongs to request i
+// (every request of the step brings one token), which saves the kernel two trips to memory.
+extern "C" int attn_decode_rows(void* out, const void* q, int ldq, int ldo, const void* k_pages,
+                                const void* v_pages, size_t page_stride, const int* block_table,
+                                int max_blocks, const int* token_req, const int* positions,
+                                const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
+                                int page_size, int window, float scale, int n_splits, float* part_o,
+                                float* part_ml, int n_waves, const void* ahead, size_t ahead_chunk_bytes,
+                                int ahead_chunks, int rows_are_requests, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (n_waves < 1 || n_waves > MAX_WAVES) FAIL("attn_decode: %d waves a block, must be 1 to %d", n_waves, MAX_WAVES);
   if (head_dim > 64 * n_waves) FAIL("attn_decode: head_dim %d needs at least %d waves", head_dim, (head_dim + 63) / 64);
@@ -285,6 +322,8 @@ extern "C" int attn_decode(void* out, const void* q, int ldq, int ldo, const voi
     FAIL("attn_decode: what is read ahead must be chunks of 16-byte pieces");
   p.ahead = (const uint4*)ahead, p.ahead_pieces = ahead ? ahead_chunk_bytes / 16 : 0;
   p.ahead_chunks = ahead ? ahead_chunks : 0;
+  p.rows_are_requests = rows_are_requests ? 1 : 0;
+  p.table_in_lds = max_blocks > 0 && max_blocks <= 8192;  // (32 KB of LDS at most)
   if (head_dim == 32)
     launch<4>(p, n_rows, n_waves, stream);
   else if (head_dim == 64)

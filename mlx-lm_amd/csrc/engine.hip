@@ -86,7 +86,7 @@ typedef int (*fn_attn_row)(void*, const void*, int, int, const void*, const void
                            float*, float*, int, hipStream_t);
 typedef int (*fn_attn_decode)(void*, const void*, int, int, const void*, const void*, size_t, const int*, int,
                               const int*, const int*, const int*, int, int, int, int, int, int, float, int,
-                              float*, float*, int, const void*, size_t, int, hipStream_t);
+                              float*, float*, int, const void*, size_t, int, int, hipStream_t);
 typedef int (*fn_attn_prefill)(void*, const void*, int, int, const void*, const void*, size_t, const int*,
                                int, const int*, const int*, const int*, int, int, int, int, int, int, float,
                                hipStream_t);
@@ -105,7 +105,7 @@ static Entry<fn_int2> k_sum_partials_norm_takes("gemm_bf16_decode", "sum_partial
 static Entry<fn_kv_write> k_kv_write("attention", "kv_write");
 static Entry<fn_attn_tile> k_attn_tile("attention", "attn_tile");
 static Entry<fn_attn_row> k_attn_row("attention", "attn_row");
-static Entry<fn_attn_decode> k_attn_decode("attention_decode", "attn_decode");
+static Entry<fn_attn_decode> k_attn_decode("attention_decode", "attn_decode_rows");
 static Entry<fn_attn_prefill> k_attn_prefill("attention_prefill", "attn_prefill");
 
 // Launch through an entry: a missing library or a refused call becomes this library's error.
@@ -599,7 +599,7 @@ struct LayerNorm : Norm {
 // -- attention ------------------------------------------------------------------
 
 // ids of the arrays that the attention part asks the packer for, from `array_base` on
-enum { ARR_TILES = 0, ARR_ROWS, ARR_ALL_TILES, ARR_BIG_TILES, ARR_MAX_ROW_CONTEXT };
+enum { ARR_TILES = 0, ARR_ROWS, ARR_ALL_TILES, ARR_BIG_TILES, ARR_MAX_ROW_CONTEXT, ARR_ROWS_ARE_REQUESTS };
 
 struct Attention : Mixer {
   int width, n_heads, n_kv_heads, head_dim, window, q_width, kv_width, array_base;
@@ -670,6 +670,7 @@ struct Attention : Mixer {
     const int n_all_tiles = (int)ctx->counts[array_base + ARR_ALL_TILES] / 2;
     const int n_big_tiles = (int)ctx->counts[array_base + ARR_BIG_TILES] / 2;
     const long max_row_context = ctx->counts[array_base + ARR_MAX_ROW_CONTEXT];
+    const int rows_are_requests = ctx->counts[array_base + ARR_ROWS_ARE_REQUESTS] != 0;
     if (n_tiles == 0 && n_rows == 0 && q.rows > 0)
       FAIL("attention: the step carries no work lists for its %d rows", q.rows);
     const bool bf16 = q.dtype == DT_BF16;
@@ -723,7 +724,8 @@ struct Attention : Mixer {
         KERNEL(k_attn_decode, ctx, out.p, q.p, q.ld, out.ld, kv.k, kv.v, kv.page_stride, kv.block_table,
                kv.max_blocks, kv.token_req, kv.positions, rows, n_rows, n_heads, n_kv_heads, head_dim,
                kv.page_size, window, scale, n_splits, (float*)part_o.p, (float*)part_ml.p, n_waves,
-               ahead ? ahead->packed : nullptr, ahead ? ahead->chunk_bytes : (size_t)0, chunks, ctx->stream);
+               ahead ? ahead->packed : nullptr, ahead ? ahead->chunk_bytes : (size_t)0, chunks, rows_are_requests,
+               ctx->stream);
       } else {
         KERNEL(k_attn_row, ctx, out.p, q.p, q.ld, out.ld, kv.k, kv.v, kv.page_stride, kv.block_table,
                kv.max_blocks, kv.token_req, kv.positions, rows, n_rows, n_heads, n_kv_heads, head_dim,
@@ -923,7 +925,7 @@ extern "C" EngPart* eng_make_attention(int width, int n_heads, int n_kv_heads, i
                                        int array_base) {
   Position* pos = nullptr;
   if (position && !(pos = as<Position>(position, KIND_POSITION, "eng_make_attention"))) return nullptr;
-  if (array_base < 0 || array_base + ARR_MAX_ROW_CONTEXT >= ENG_MAX_ARRAYS) {
+  if (array_base < 0 || array_base + ARR_ROWS_ARE_REQUESTS >= ENG_MAX_ARRAYS) {
     snprintf(g_err, sizeof(g_err), "eng_make_attention: array ids from %d do not fit", array_base);
     return nullptr;
   }

@@ -574,11 +574,13 @@ def attn_decode_takes(q_dtype, kv):
 
 
 def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_heads, scale,
-                window=0, n_splits=1, part_o=None, part_ml=None, n_waves=4, ahead=None, ahead_chunks=0):
+                window=0, n_splits=1, part_o=None, part_ml=None, n_waves=4, ahead=None, ahead_chunks=0,
+                rows_are_requests=False):
     """``attn_row`` for bfloat16 caches with head_dim 32, 64 or 128: keys stream into registers.
 
     ``ahead``: a ``PackedWeight`` whose first ``ahead_chunks`` chunks the CUs without a row read
-    meanwhile, each the chunks that a block on its own die will ask for (``sum_partials_norm``)."""
+    meanwhile, each the chunks that a block on its own die will ask for (``sum_partials_norm``).
+    ``rows_are_requests``: item ``i`` of ``rows`` is row ``i`` of request ``i`` (the caller says so)."""
     lib = build.load("attention_decode")
     ldq, ldo = _rows2d(q, "q"), _rows2d(out, "out")
     _need(q.dtype == torch.bfloat16, "attn_decode: bfloat16 only")
@@ -592,7 +594,9 @@ def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_h
         _dev(part_ml, "part_ml", torch.float32)
         _need(part_o.numel() >= n_rows * n_heads * n_splits * kv.head_dim, "attn_decode: part_o too small")
         _need(part_ml.numel() >= n_rows * n_heads * n_splits * 2, "attn_decode: part_ml too small")
-    rc = lib.attn_decode(
+    if rows_are_requests:
+        _need(n_rows <= block_table.shape[0], "attn_decode: more rows than requests")
+    rc = lib.attn_decode_rows(
         _ptr(out), _ptr(q), _c_int(ldq), _c_int(ldo), _ptr(kv.k), _ptr(kv.v),
         _c_size_t(kv.page_stride), _ptr(block_table), _c_int(block_table.shape[1]),
         _ptr(token_req), _ptr(positions), _ptr(rows), _c_int(n_rows), _c_int(n_heads),
@@ -600,7 +604,8 @@ def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_h
         _c_float(scale), _c_int(n_splits), _ptr(part_o), _ptr(part_ml), _c_int(n_waves),
         _ptr(ahead.packed if ahead is not None else None),
         _c_size_t(ahead.chunk_bytes if ahead is not None else 0),
-        _c_int(min(ahead_chunks, ahead.n_chunks) if ahead is not None else 0), _stream(),
+        _c_int(min(ahead_chunks, ahead.n_chunks) if ahead is not None else 0),
+        _c_int(1 if rows_are_requests else 0), _stream(),
     )
     build.check(lib, rc, "attn_decode")
     return out

@@ -84,7 +84,7 @@ class CausalSelfAttention(Mixer):
     # -- the step arrays this part asks the packer for ---------------------------
 
     step_arrays_key = "attention"
-    step_array_names = ("tiles", "rows", "all_tiles", "big_tiles", "max_row_context")
+    step_array_names = ("tiles", "rows", "all_tiles", "big_tiles", "max_row_context", "rows_are_requests")
 
     @staticmethod
     def step_arrays(batch):
@@ -96,7 +96,9 @@ class CausalSelfAttention(Mixer):
         ``BIG_TILE_Q`` for the matrix-core kernel (``big_tiles``, the tile with the most keys
         first).  ``all_tiles`` covers every row with tiles, for head sizes the row kernels do
         not take.  ``max_row_context``: the most keys that a row of ``rows`` sees, which decides
-        how its keys are split; in a step that is recorded, the model's positions."""
+        how its keys are split; in a step that is recorded, the model's positions.
+        ``rows_are_requests``: 1 if every request brings one token, so that item ``i`` of ``rows``
+        is row ``i`` of request ``i`` (the decode kernel then need not look either up)."""
         tiles, rows, all_tiles, big = [], [], [], []
         longest = 0
         for q0, n, length in zip(batch.q_starts, batch.q_lens, batch.context_lens):
@@ -115,7 +117,8 @@ class CausalSelfAttention(Mixer):
             longest = batch.max_positions  # how keys are split must not depend on lengths
         big.sort(reverse=True)  # tiles with the most keys start first
         return {"tiles": tiles, "rows": rows, "all_tiles": all_tiles,
-                "big_tiles": [v for _, r0, m in big for v in (r0, m)], "max_row_context": longest}
+                "big_tiles": [v for _, r0, m in big for v in (r0, m)], "max_row_context": longest,
+                "rows_are_requests": int(all(n == 1 for n in batch.q_lens))}
 
     # -- the native twin ---------------------------------------------------------
 

@@ -325,6 +325,33 @@ def test_attn_decode(case, n_splits, n_waves):
     assert err < _attn_tol(torch.bfloat16), err
 
 
+@pytest.mark.parametrize("case", [
+    (8, 2, 32, 16, [700, 15, 16, 0], [1, 1, 1, 1], 0),
+    (25, 25, 64, 16, [511, 63, 1022, 64, 300], [1, 1, 1, 1, 1], 0),
+    (4, 4, 128, 32, [63, 64, 1000], [1, 1, 1], 100),
+])
+@pytest.mark.parametrize("n_splits,n_waves", [(1, 2), (1, 16), (3, 4)])
+def test_attn_decode_when_rows_are_requests(case, n_splits, n_waves):
+    """A step in which every request brings one token: the kernel is told that item i is row i of
+    request i and looks neither up (the row list it is handed here is garbage on purpose)."""
+    k = _k()
+    H, Hkv, hd, ps, ctx, ql, window = case
+    c = PagedCase(torch.bfloat16, H, Hkv, hd, ps, ctx, ql, seed=hd + H + 5, window=window)
+    k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
+    garbage = torch.full((c.T,), 10**6, dtype=torch.int32, device=DEV)
+    part_o = torch.empty(c.T * H * n_splits * hd, dtype=torch.float32, device=DEV)
+    part_ml = torch.empty(c.T * H * n_splits * 2, dtype=torch.float32, device=DEV)
+    outs = []
+    for told in (True, False):
+        out = torch.full((c.T, H * hd), float("nan")).to(torch.bfloat16).to(DEV)
+        rows = garbage if told else torch.arange(c.T, dtype=torch.int32, device=DEV)
+        k.attn_decode(out, c.q.to(DEV), c.kv, c.block_table_dev, garbage if told else c.token_req, c.positions,
+                      rows, c.T, H, c.scale, window, n_splits, part_o, part_ml, n_waves, rows_are_requests=told)
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1])
+    assert (outs[0].double().cpu() - c.reference()).abs().max().item() < _attn_tol(torch.bfloat16)
+
+
 PREFILL_CASES = [c for c in ATTN_CASES if c[2] in (32, 64, 128)] + [
     (3, 3, 64, 16, [0, 100, 700], [300, 129, 5], 0),
     (4, 2, 32, 16, [5, 0], [260, 64], 0),
