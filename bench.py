@@ -9,9 +9,10 @@ step runs at context 512 and, with the default K, the last at the model's last p
 mlx_lm/benchmark.py:118-124; it warms up, then times five trials and reports their mean,
 mlx_lm/benchmark.py:152-176).  The W warm-up steps run before, on requests of their own, so
 that they do not move the timed steps' context.  ``config`` gives the context range as
-``ctx_from``/``ctx_to``.  ``prefill`` is one step of 2 x 1,024 prompt tokens: two untimed
-warm-up trials (a step whose shape keeps coming back is replayed from its recorded graph, as
-in the serving path), then the mean of five timed ones, each listed in ``trials_ms``.
+``ctx_from``/``ctx_to``.  ``prefill`` is one step of 2 x 1,024 prompt tokens: W untimed
+warm-up trials, three at least (a step whose shape keeps coming back is replayed from its
+recorded graph, as in the serving path: the third trial records it), then the mean of five
+timed ones, each listed in ``trials_ms``.
 ``points`` holds decode at batch 1 and 64 over the same steps and, for all three batch sizes,
 at context 1,000; ``roofline`` the bytes a decode step has to read (every weight once, the live
 requests' keys and values at each step's context) over its time, ``roofline_points`` the same
@@ -155,7 +156,8 @@ def main():
     n_seqs, seq_len = 2, 1024
     prompts = torch.randint(0, V, (n_seqs, seq_len), generator=g).tolist()
     pre_ms = []
-    warm_trials, timed_trials = 3, 5  # (the third sighting of the shape records it; the timed ones replay)
+    # (the third sighting of the shape records it; the warm-up trials after it and the timed ones replay)
+    warm_trials, timed_trials = max(3, a.warmup), 5
     for trial in range(warm_trials + timed_trials):
         for i in range(n_seqs):
             engine.add_request(("pre", i))

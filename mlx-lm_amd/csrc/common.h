@@ -141,6 +141,31 @@ __device__ __forceinline__ float block_max(float v, float* red) {
   return t;
 }
 
+// Stores that go through to memory as they are issued (system scope: sc0 sc1).  When a kernel
+// ends, what its stores left dirty in the eight L2s is written back before the next kernel may
+// start: 9 us after a product that wrote 26 MB, 3 us when the stores had gone through at once,
+// spread over the kernel's last microseconds.  For outputs of megabytes that the same kernel does
+// not read again.  The compiler takes a cache policy only on buffer stores, so the output is
+// described as a buffer: offsets are 32-bit byte offsets from its base, and the hardware drops a
+// store at or beyond `bytes` (which must be below 4 GB; `fits_through_buffer` on the host).
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+#define BUFFER_WORD3 0x00020000  // untyped 32-bit data, no swizzle
+#define POLICY_THROUGH 0x11      // sc0 | sc1
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t through_buffer(void* base, size_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(base, 0, (int)(uint32_t)bytes, BUFFER_WORD3);
+}
+__device__ __forceinline__ void store_through(__amdgpu_buffer_rsrc_t r, uint32_t byte_offset, u32x4_t v) {
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)byte_offset, 0, POLICY_THROUGH);
+}
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void store_through(__amdgpu_buffer_rsrc_t r, uint32_t byte_offset, u32x2_t v) {
+  __builtin_amdgcn_raw_buffer_store_b64(v, r, (int)byte_offset, 0, POLICY_THROUGH);
+}
+__device__ __forceinline__ void store_through(__amdgpu_buffer_rsrc_t r, uint32_t byte_offset, float v) {
+  __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned int, v), r, (int)byte_offset, 0, POLICY_THROUGH);
+}
+static inline bool fits_through_buffer(size_t bytes) { return bytes < ((size_t)1 << 32); }
+
 // ---------------------------------------------------------------------------
 // host side: the device's size; one error string per thread, returned codes are 0 (ok) or 1.
 

@@ -24,6 +24,7 @@
 #define FLAG_ACCUMULATE 2
 #define FLAG_OUT_F32 4
 #define FLAG_KV 8  // columns from q_width on are keys, then values: they go to their cache pages, not to out
+#define FLAG_THROUGH 16  // (set here) out and ws are below 4 GB: the tile kernels' stores go through to memory
 
 // Out-of-range loads read a clamped address and are zeroed afterwards with this
 // constant: selecting between an address and a zero kept in a variable turns
@@ -339,6 +340,8 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
 
   if constexpr (SPLIT) {  // the partial sums as they are; sum_partials adds them and runs the epilogue
     float* ws = p.ws + (size_t)blockIdx.y * p.M * p.N;
+    const bool through = p.flags & FLAG_THROUGH;
+    const __amdgpu_buffer_rsrc_t ws_buf = through_buffer(ws, (size_t)p.M * p.N * 4);
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int n = n0 + wn * TN * 32 + j * 32 + (lane & 31);
@@ -349,7 +352,11 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int m = mb + 8 * (r >> 2) + (r & 3);
-          if (m < p.M) ws[(size_t)m * p.N + n] = acc[i][j][r];
+          if (m >= p.M) continue;
+          if (through)
+            store_through(ws_buf, (uint32_t)(((size_t)m * p.N + n) * 4), acc[i][j][r]);
+          else
+            ws[(size_t)m * p.N + n] = acc[i][j][r];
         }
       }
     }
@@ -375,6 +382,8 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
   float* __restrict__ out_f = (float*)p.out;
   uint16_t* __restrict__ out_h = (uint16_t*)p.out;
   const bool f32_out = p.flags & (FLAG_ACCUMULATE | FLAG_OUT_F32);
+  const bool through = p.flags & FLAG_THROUGH;
+  const __amdgpu_buffer_rsrc_t out_buf = through_buffer(p.out, ((size_t)(p.M - 1) * p.ldo + p.N) * (f32_out ? 4 : 2));
   // CPL columns a lane on the way out, 16 bytes of the output: eight bfloat16 or four floats, so
   // that a store covers whole 128-byte lines of a few rows
   auto emit = [&](auto cpl) __attribute__((always_inline)) {
@@ -460,12 +469,18 @@ __global__ __launch_bounds__(S::THREADS, S::BLOCKS_PER_CU) void gemm_bf16_tile_k
           if (!elane || row >= 32 || m >= p.M || n >= p.N) continue;
           const size_t at = (size_t)m * p.ldo + n;
           if (vec) {
+            u32x4_t t;
             if constexpr (CPL == 4)
-              *(float4*)(out_f + at) = make_float4(v[s][0], v[s][1], v[s][2], v[s][3]);
+              t = u32x4_t{__float_as_uint(v[s][0]), __float_as_uint(v[s][1]), __float_as_uint(v[s][2]), __float_as_uint(v[s][3])};
             else
-              *(uint4*)(kv_lane ? place[s] : out_h + at) =
-                  make_uint4(pack_bf16x2(v[s][0], v[s][1]), pack_bf16x2(v[s][2], v[s][3]),
-                             pack_bf16x2(v[s][4], v[s][5]), pack_bf16x2(v[s][6], v[s][7]));
+              t = u32x4_t{pack_bf16x2(v[s][0], v[s][1]), pack_bf16x2(v[s][2], v[s][3]),
+                          pack_bf16x2(v[s][4], v[s][5]), pack_bf16x2(v[s][6], v[s][7])};
+            if (kv_lane)
+              *(u32x4_t*)place[s] = t;  // (attention reads it next: it may stay in the L2)
+            else if (through)
+              store_through(out_buf, (uint32_t)(at * (CPL == 4 ? 4 : 2)), t);
+            else
+              *(u32x4_t*)(CPL == 4 ? (void*)(out_f + at) : (void*)(out_h + at)) = t;
           } else if (kv_lane) {
 #pragma unroll
             for (int c = 0; c < CPL; ++c)
@@ -730,7 +745,7 @@ extern "C" int gemm_bf16_scatter(void* out, const void* A, const void* W, const 
   p.out = out;
   p.M = M, p.N = N, p.K = K;
   p.lda = lda, p.ldw = ldw, p.ldo = ldo;
-  p.flags = flags;
+  p.flags = flags & (FLAG_GELU | FLAG_ACCUMULATE | FLAG_OUT_F32);
   p.w_packed = ldw == 0 ? 1 : 0, p.w_kblocks = (K + BK - 1) / BK;
   if (check_args(p)) return 1;
   if (M == 0) return 0;
@@ -754,6 +769,7 @@ extern "C" int gemm_bf16_scatter(void* out, const void* A, const void* W, const 
   const int n_blocks = (K + BK - 1) / BK;
   if (n_splits < 1 || n_splits > n_blocks) FAIL("gemm_bf16: %d splits of K=%d", n_splits, K);
   p.ws = ws, p.n_splits = n_splits, p.blocks_per_split = (n_blocks + n_splits - 1) / n_splits;
+  if (fits_through_buffer((size_t)M * ldo * 4) && fits_through_buffer((size_t)M * N * 4)) p.flags |= FLAG_THROUGH;
   if (n_splits > 1) {
     if (variant == 0) variant = M <= 32 ? 6 : small_tiles(M, N) ? 5 : 1;
     if (variant != 1 && variant != 5 && variant != 6) FAIL("gemm_bf16: only the tiles of 128, 64 and 32 rows by 128 split K");

@@ -47,7 +47,7 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(T* __restrict__ out
                                                              const int* __restrict__ rows,
                                                              const float* __restrict__ gamma,
                                                              const float* __restrict__ beta,
-                                                             float eps, int n_rows, int width) {
+                                                             float eps, int n_rows, int width, bool through) {
   const int lane = threadIdx.x & 63;
   const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (r >= n_rows) return;  // whole waves leave; no barrier follows
@@ -77,6 +77,9 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(T* __restrict__ out
   }
   const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)width + eps);
   T* o = out + (size_t)r * width;
+  // (the next kernel reads the rows, this one does not: the stores go through to memory)
+  const __amdgpu_buffer_rsrc_t out_buf = through_buffer(out, (size_t)n_rows * width * sizeof(T));
+  const uint32_t o_at = (uint32_t)((size_t)r * width * sizeof(T));
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int k = (lane + 64 * i) * 4;
@@ -84,12 +87,17 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(T* __restrict__ out
     const float y[4] = {(v[i].x - mean) * rstd * g[i].x + b[i].x, (v[i].y - mean) * rstd * g[i].y + b[i].y,
                         (v[i].z - mean) * rstd * g[i].z + b[i].z, (v[i].w - mean) * rstd * g[i].w + b[i].w};
     if constexpr (sizeof(T) == 4) {
-      *(float4*)((float*)o + k) = make_float4(y[0], y[1], y[2], y[3]);
+      const u32x4_t t = {__float_as_uint(y[0]), __float_as_uint(y[1]), __float_as_uint(y[2]), __float_as_uint(y[3])};
+      if (through)
+        store_through(out_buf, o_at + k * 4, t);
+      else
+        *(u32x4_t*)((float*)o + k) = t;
     } else {
-      uint2 pk;
-      pk.x = f32_to_bf16_bits(y[0]) | ((uint32_t)f32_to_bf16_bits(y[1]) << 16);
-      pk.y = f32_to_bf16_bits(y[2]) | ((uint32_t)f32_to_bf16_bits(y[3]) << 16);
-      *(uint2*)((uint16_t*)o + k) = pk;
+      const u32x2_t pk = {pack_bf16x2(y[0], y[1]), pack_bf16x2(y[2], y[3])};
+      if (through)
+        store_through(out_buf, o_at + k * 2, pk);
+      else
+        *(u32x2_t*)((uint16_t*)o + k) = pk;
     }
   }
 }
@@ -98,14 +106,15 @@ template <typename T>
 static void launch_wave(int nv, dim3 grid, hipStream_t stream, T* out, const float* x, const int* rows,
                         const float* gamma, const float* beta, float eps, int n_rows, int width) {
   dim3 block(256);
+  const bool through = fits_through_buffer((size_t)n_rows * width * sizeof(T));
   if (nv <= 2)
-    hipLaunchKernelGGL((layernorm_wave_kernel<T, 2>), grid, block, 0, stream, out, x, rows, gamma, beta, eps, n_rows, width);
+    hipLaunchKernelGGL((layernorm_wave_kernel<T, 2>), grid, block, 0, stream, out, x, rows, gamma, beta, eps, n_rows, width, through);
   else if (nv <= 4)
-    hipLaunchKernelGGL((layernorm_wave_kernel<T, 4>), grid, block, 0, stream, out, x, rows, gamma, beta, eps, n_rows, width);
+    hipLaunchKernelGGL((layernorm_wave_kernel<T, 4>), grid, block, 0, stream, out, x, rows, gamma, beta, eps, n_rows, width, through);
   else if (nv <= 8)
-    hipLaunchKernelGGL((layernorm_wave_kernel<T, 8>), grid, block, 0, stream, out, x, rows, gamma, beta, eps, n_rows, width);
+    hipLaunchKernelGGL((layernorm_wave_kernel<T, 8>), grid, block, 0, stream, out, x, rows, gamma, beta, eps, n_rows, width, through);
   else
-    hipLaunchKernelGGL((layernorm_wave_kernel<T, 16>), grid, block, 0, stream, out, x, rows, gamma, beta, eps, n_rows, width);
+    hipLaunchKernelGGL((layernorm_wave_kernel<T, 16>), grid, block, 0, stream, out, x, rows, gamma, beta, eps, n_rows, width, through);
 }
 
 DEFINE_LAST_ERROR(mlxlm_last_error)
