@@ -79,6 +79,7 @@ GEMM_SHAPES = [
     (130, 48, 16),  # K shorter than a k-block of the tile kernels
     (100, 96, 32),
     (70, 100, 48),
+    (2100, 2064, 136),  # 17 x 17 tiles of 128: more blocks than CUs, two to a CU
 ]
 
 
