@@ -24,6 +24,7 @@ DEFINE_LAST_ERROR(mlxlm_last_error)
 #define GEMM_OUT_F32 4
 #define GEMM_KV 8
 #define DECODE_MAX_ROWS 16
+#define ROWS_MAX_ROWS 48  // up to here the kernel for 17 to 48 rows
 #define ATTN_ROW_MAX_HEAD_DIM 144
 #define READ_AHEAD_BYTES_PER_CU (160 * 1024)  // what an idle CU reads while decode attention runs
 
@@ -66,11 +67,15 @@ typedef int (*fn_gemm_bf16)(void*, const void*, const void*, const float*, int, 
                             const int*, int, int, int, int, hipStream_t);
 typedef int (*fn_int5)(int, int, int, int, int);
 typedef int (*fn_int4)(int, int, int, int);
+typedef int (*fn_int3)(int, int, int);
 typedef int (*fn_int2)(int, int);
 typedef int (*fn_gemm_decode)(void*, const void*, int, const float*, int, const float*, const float*, float,
                               const void*, const float*, int, int, int, int, int, int, void*, void*, size_t,
                               const int*, int, const int*, const int*, int, int, int, int, int, float*,
                               size_t, hipStream_t);
+typedef int (*fn_gemm_rows)(void*, const void*, int, const void*, const float*, int, int, int, int, int, void*,
+                            void*, size_t, const int*, int, const int*, const int*, int, int, int, int, int,
+                            float*, size_t, hipStream_t);
 typedef int (*fn_sum_partials)(void*, const float*, int, const float*, int, int, int, int, void*, void*,
                                size_t, const int*, int, const int*, const int*, int, int, int, int,
                                hipStream_t);
@@ -99,6 +104,9 @@ static Entry<fn_int5> k_gemm_bf16_splits("gemm_bf16", "gemm_bf16_splits");
 static Entry<fn_gemm_decode> k_gemm_decode("gemm_bf16_decode", "gemm_bf16_decode");
 static Entry<fn_int4> k_decode_takes("gemm_bf16_decode", "gemm_bf16_decode_takes");
 static Entry<fn_int5> k_decode_splits("gemm_bf16_decode", "gemm_bf16_decode_splits");
+static Entry<fn_gemm_rows> k_gemm_rows("gemm_bf16_decode", "gemm_bf16_rows");
+static Entry<fn_int4> k_rows_splits("gemm_bf16_decode", "gemm_bf16_rows_splits");
+static Entry<fn_int3> k_rows_takes("gemm_bf16_decode", "gemm_bf16_rows_takes");
 static Entry<fn_sum_partials> k_sum_partials("gemm_bf16_decode", "sum_partials");
 static Entry<fn_sum_partials_norm> k_sum_partials_norm("gemm_bf16_decode", "sum_partials_norm");
 static Entry<fn_int2> k_sum_partials_norm_takes("gemm_bf16_decode", "sum_partials_norm_takes");
@@ -344,6 +352,38 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
 
   EngMat A;
   TRY(materialize(ctx, a, &A));
+  if (w.dtype == DT_BF16 && variant == 0 && M > DECODE_MAX_ROWS && M <= ROWS_MAX_ROWS && w.packed) {
+    // 17 to 48 rows: the kernel that holds a block's weights in registers, if the sizes fit it
+    int n_splits = 0;
+    if (splits == 0)
+      QUERY(k_rows_splits, n_splits, M, N, K, ctx->force_splits);
+    else
+      n_splits = split_count((K + 63) / 64, splits);
+    if (n_splits > 1 && (!ws || (size_t)n_splits > ws_floats / ((size_t)M * N))) n_splits = 0;  // (the tiles then)
+    if (n_splits >= 1) {
+      int takes = 0;
+      QUERY(k_rows_takes, takes, M, K, n_splits);
+      if (!takes) n_splits = 0;
+    }
+    if (n_splits >= 1) {
+      if (n_splits > 1 && pending) TRY(settle(ctx, pending));  // the workspace is about to be written again
+      KERNEL(k_gemm_rows, ctx, out.p, A.p, A.ld, w.packed, bias, M, N, K, out.ld, flags | (sc ? GEMM_KV : 0),
+             sc ? sc->k : nullptr, sc ? sc->v : nullptr, sc ? sc->page_stride : (size_t)0,
+             sc ? sc->block_table : nullptr, sc ? sc->max_blocks : 0, sc ? sc->token_req : nullptr,
+             sc ? sc->positions : nullptr, sc ? sc->q_width : 0, sc ? sc->kv_width : 0, sc ? sc->head_dim : 0,
+             sc ? sc->page_size : 0, n_splits, n_splits > 1 ? ws : nullptr, n_splits > 1 ? ws_floats : (size_t)0,
+             ctx->stream);
+      if (n_splits > 1) {
+        if (accumulate && pending && pending->allowed) {
+          pending->target = (float*)out.p, pending->rows = M, pending->cols = N, pending->ld = out.ld;
+          pending->ws = ws, pending->n_splits = n_splits, pending->bias = bias;
+          return 0;
+        }
+        return sum_partials(ctx, out, ws, n_splits, bias, gelu, accumulate, sc);
+      }
+      return 0;
+    }
+  }
   if (w.dtype == DT_F32) {
     KERNEL(k_gemm_f32, ctx, out.p, A.p, w.w, bias, M, N, K, A.ld, w.ldw, out.ld, flags, variant, ctx->stream);
   } else {

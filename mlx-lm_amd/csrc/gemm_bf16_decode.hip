@@ -24,8 +24,9 @@
 // of the MFMAs; the eight partial tiles are summed in a fixed order.  Where
 // the matrix has few features and K is not split, a block owns only eight of
 // them (lanes 8..15 of a group repeat the eighth): twice as many blocks.
-// (More than 16 rows are the tile kernels' of gemm_bf16.hip, which leave their
-// partial sums to the second kernels of this file in the same way.)
+// (17 to 48 rows have a kernel of their own further down, gemm_bf16_rows; more
+// are the tile kernels' of gemm_bf16.hip.  Both leave their partial sums to the
+// second kernels of this file in the same way.)
 //
 // A CU keeps only so many loads in flight, so a launch that does not occupy
 // every CU cannot reach the memory's bandwidth.  Where the feature blocks alone
@@ -335,6 +336,123 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArg
 }
 
 // ---------------------------------------------------------------------------
+// 17 to 48 rows.  The weights still stream exactly once and all of a block's are in flight from
+// its first instruction on: a block of four waves owns 32 output features (two packed chunks)
+// and a slice of K of at most 28 k-blocks; wave w takes the slice's k-blocks w, w + 4, ... and
+// holds their weights in registers (seven k-blocks of two chunks: 112 registers a lane).  The
+// activations are the MFMA's other operand, two or three tiles of 16 rows, read straight from
+// memory (the L2s: every block reads the same rows) a k-block ahead; no LDS on the way.  The four
+// waves' tiles are summed in their order through LDS and finished as in the kernel above.  The
+// tile kernels of gemm_bf16.hip need K split over some 220 blocks at these sizes and a second
+// kernel for the sum; here the wide products are one launch of 150 or 200 blocks, and the narrow
+// ones split K in two or four.  A decode step of GPT-2 XL's sizes at batch 17 / 24 / 32 / 40 / 48:
+// 2.93 / 3.23 / 3.52 / 3.97 / 4.44 ms instead of 3.34 / 3.64 / 3.91 / 4.23 / 4.64 through the
+// tiles.  (With four tiles of rows a block reads twice as many bytes of rows as of weights, and
+// at 56 to 64 rows the tiles are as fast or faster: 5.13 against 5.23 ms at batch 64.  A variant
+// with eight waves that held their k-blocks of rows as well as of weights, one trip to memory
+// for everything, was slower at every size.)
+#define RW 4          // waves a block
+#define R_FEATURES 32 // output features a block
+#define R_HELD 7      // k-blocks whose weights a wave holds
+#define ROWS_MAX_M 48
+#define ROWS_WANT_BLOCKS 100  // a split of K where the features give fewer blocks than this
+template <int R_TILES>  // tiles of 16 rows
+__global__ __launch_bounds__(RW * 64) void gemm_bf16_rows_kernel(DecodeGemmArgs p) {
+  __shared__ float red[RW][R_TILES * 2][256];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n0 = blockIdx.x * R_FEATURES;
+  const int n_chunks_all = (p.K + 63) / 64;
+  const int c_begin = blockIdx.y * p.chunks_per_split;
+  const int n_chunks = min(n_chunks_all, c_begin + p.chunks_per_split) - c_begin;
+  const int n_fb = (p.N + 15) / 16;
+  const int koff = (lane >> 4) * 16;
+
+  // the weights, all at once (k-blocks beyond the slice repeat its last one and are not used)
+  Frag w[R_HELD][2][2];
+#pragma unroll
+  for (int i = 0; i < R_HELD; ++i) {
+    const int c = c_begin + min(wave + RW * i, n_chunks - 1);
+#pragma unroll
+    for (int ft = 0; ft < 2; ++ft) {
+      const int fb = min((n0 >> 4) + ft, n_fb - 1);  // (a second chunk beyond the matrix repeats the first)
+      const uint16_t* t = p.W + ((size_t)fb * n_chunks_all + c) * 1024 + lane * 8;
+      w[i][ft][0].u = *(const uint4*)t;
+      w[i][ft][1].u = *(const uint4*)(t + 512);
+    }
+  }
+  // the activations of a k-block: lane l holds row l % 16 of each tile, 16 columns from
+  // (l / 16) * 16 on (rows beyond M repeat the last; what they give is not stored)
+  const uint16_t* arow[R_TILES];
+#pragma unroll
+  for (int rt = 0; rt < R_TILES; ++rt) arow[rt] = p.A + (size_t)min(rt * 16 + (lane & 15), p.M - 1) * p.lda;
+  auto load_a = [&](Frag (&a)[R_TILES][2], int i) {
+    const int k = (c_begin + min(wave + RW * i, n_chunks - 1)) * 64 + koff;
+#pragma unroll
+    for (int rt = 0; rt < R_TILES; ++rt) {
+      a[rt][0].u = *(const uint4*)(arow[rt] + min(k, p.K - 8));
+      a[rt][1].u = *(const uint4*)(arow[rt] + min(k + 8, p.K - 8));
+    }
+  };
+  f32x4_t acc[R_TILES][2];
+#pragma unroll
+  for (int rt = 0; rt < R_TILES; ++rt)
+#pragma unroll
+    for (int ft = 0; ft < 2; ++ft) acc[rt][ft] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  auto multiply = [&](Frag (&a)[R_TILES][2], int i) {
+    if (wave + RW * i >= n_chunks) return;  // (uniform over the wave)
+    const int k = (c_begin + wave + RW * i) * 64 + koff;
+    // columns beyond K meet zero weights (the packed order pads them), but must not be NaN
+    const bool in0 = k < p.K, in1 = k + 8 < p.K;
+#pragma unroll
+    for (int rt = 0; rt < R_TILES; ++rt) {
+      Frag a0, a1;
+      a0.u = in0 ? a[rt][0].u : ZERO4, a1.u = in1 ? a[rt][1].u : ZERO4;
+#pragma unroll
+      for (int ft = 0; ft < 2; ++ft) {
+        acc[rt][ft] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[i][ft][0].v, a0.v, acc[rt][ft], 0, 0, 0);
+        acc[rt][ft] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[i][ft][1].v, a1.v, acc[rt][ft], 0, 0, 0);
+      }
+    }
+  };
+  Frag a0[R_TILES][2], a1[R_TILES][2];
+  load_a(a0, 0);
+#pragma unroll
+  for (int i = 0; i < R_HELD; i += 2) {
+    if (i + 1 < R_HELD) load_a(a1, i + 1);
+    multiply(a0, i);
+    if (i + 2 < R_HELD) load_a(a0, i + 2);
+    if (i + 1 < R_HELD) multiply(a1, i + 1);
+  }
+
+  // ---- sum the waves' tiles in their order, then the epilogue -----------------
+#pragma unroll
+  for (int rt = 0; rt < R_TILES; ++rt)
+#pragma unroll
+    for (int ft = 0; ft < 2; ++ft)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[wave][rt * 2 + ft][lane * 4 + r] = acc[rt][ft][r];
+  __syncthreads();
+  // element tid = 4 * L + r of a tile: feature 4 * (L / 16) + r, row L % 16
+  const int L = tid >> 2, r = tid & 3;
+#pragma unroll
+  for (int rt = 0; rt < R_TILES; ++rt)
+#pragma unroll
+    for (int ft = 0; ft < 2; ++ft) {
+      float v = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < RW; ++wv) v += red[wv][rt * 2 + ft][tid];
+      const int n = n0 + ft * 16 + 4 * (L >> 4) + r;
+      const int m = rt * 16 + (L & 15);
+      if (m < p.M && n < p.N) {
+        if (p.n_splits > 1)
+          p.ws[((size_t)blockIdx.y * p.M + m) * p.N + n] = v;  // summed, and finished, by sum_partials
+        else
+          finish(p, m, n, v);
+      }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // The second step of a split product: out = epilogue(sum over splits, in their order).
 __global__ __launch_bounds__(256) void sum_partials_kernel(DecodeGemmArgs p) {
   const int n4 = (p.N + 3) / 4;
@@ -620,6 +738,66 @@ extern "C" int gemm_bf16_decode(
   }
   hipLaunchKernelGGL(kernels[which], dim3(n_blocks, n_splits), dim3(NW * 64), lds, stream, p);
   CHECK_LAUNCH("gemm_bf16_decode");
+  return 0;
+}
+
+// 1 if gemm_bf16_rows takes these sizes
+extern "C" int gemm_bf16_rows_takes(int M, int K, int n_splits) {
+  if (M < 17 || M > ROWS_MAX_M || K < 8 || K % 8 != 0 || n_splits < 1 || n_splits > (K + 63) / 64) return 0;
+  const int cps = chunks_per_split(K, n_splits);
+  return cps <= RW * R_HELD && cps * (n_splits - 1) < (K + 63) / 64;
+}
+
+// Into how many parts gemm_bf16_rows splits K: as few as give some ROWS_WANT_BLOCKS blocks of 32 features and
+// slices of at most 28 k-blocks (0: the sizes do not fit, for the workspace's room or otherwise).
+// `force` > 0 asks for that many wherever K has them (for tests of small sizes).
+extern "C" int gemm_bf16_rows_splits(int M, int N, int K, int force) {
+  const int n_chunks = (K + 63) / 64;
+  if (M < 17 || M > ROWS_MAX_M || K % 8 != 0) return 0;
+  const int blocks = (N + R_FEATURES - 1) / R_FEATURES;
+  int want = force > 0 ? force : (ROWS_WANT_BLOCKS + blocks - 1) / blocks;
+  const int least = (n_chunks + RW * R_HELD - 1) / (RW * R_HELD);
+  if (want < least) want = least;
+  if (want > n_chunks) want = n_chunks;
+  if (force <= 0 && want > least && n_chunks / want < 4) want = n_chunks / 4 > least ? n_chunks / 4 : least;  // four k-blocks a part
+  const int cps = (n_chunks + want - 1) / want;
+  const int n = (n_chunks + cps - 1) / cps;  // no empty part
+  return gemm_bf16_rows_takes(M, K, n) ? n : 0;
+}
+
+// The product for 17 to 48 rows (see gemm_bf16_rows_kernel): W in the packed order only.  With
+// n_splits > 1 the partial sums go to `ws` and sum_partials or sum_partials_norm finishes.
+extern "C" int gemm_bf16_rows(void* out, const void* A, int lda, const void* W, const float* bias, int M,
+                              int N, int K, int ldo, int flags, void* k_pages, void* v_pages,
+                              size_t page_stride, const int* block_table, int max_blocks,
+                              const int* token_req, const int* positions, int q_width, int kv_width,
+                              int head_dim, int page_size, int n_splits, float* ws, size_t ws_floats,
+                              hipStream_t stream) {
+  if (M == 0) return 0;
+  if (!gemm_bf16_rows_takes(M, K, n_splits))
+    FAIL("gemm_bf16_rows: M=%d K=%d in %d splits is outside what this kernel takes", M, K, n_splits);
+  if (!A || !W) FAIL("gemm_bf16_rows: null pointer");
+  if (!aligned16(W)) FAIL("gemm_bf16_rows: W must be 16-byte aligned");
+  if (lda % 8 != 0 || lda < K || !aligned16(A)) FAIL("gemm_bf16_rows: A rows must be 16-byte aligned");
+  DecodeGemmArgs p = {};
+  if (fill_epilogue(p, "gemm_bf16_rows", out, bias, M, N, ldo, flags, k_pages, v_pages, page_stride,
+                    block_table, max_blocks, token_req, positions, q_width, kv_width, head_dim, page_size))
+    return -1;
+  p.W = (const uint16_t*)W, p.A = (const uint16_t*)A;
+  p.K = K, p.lda = lda, p.ldw = 0;
+  p.n_splits = n_splits, p.chunks_per_split = chunks_per_split(K, n_splits);
+  p.ws = ws;
+  if (n_splits > 1) {
+    if (!ws || !aligned16(ws)) FAIL("gemm_bf16_rows: a split of K needs a 16-byte aligned workspace");
+    if (ws_floats < (size_t)n_splits * M * N)
+      FAIL("gemm_bf16_rows: workspace of %zu floats is too small for %d splits of %d x %d", ws_floats, n_splits, M, N);
+  }
+  const dim3 grid((N + R_FEATURES - 1) / R_FEATURES, n_splits), block(RW * 64);
+  if (M <= 32)
+    hipLaunchKernelGGL(gemm_bf16_rows_kernel<2>, grid, block, 0, stream, p);
+  else
+    hipLaunchKernelGGL(gemm_bf16_rows_kernel<3>, grid, block, 0, stream, p);
+  CHECK_LAUNCH("gemm_bf16_rows");
   return 0;
 }
 

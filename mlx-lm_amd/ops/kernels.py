@@ -392,7 +392,8 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
     operands' dtype.  With ``scatter`` (a ``KVScatter``) the columns from
     ``scatter.q_width`` on are also written to the key/value pages.  Up to 16
     bfloat16 rows go to the decode kernels, which fuse the norm and the
-    scatter; more go to the tile kernels.  Where the launch
+    scatter; 17 to 48 rows of packed weights to the kernel that holds a
+    block's weights in registers; more go to the tile kernels.  Where the launch
     would not fill the GPU, both split K over ``splits`` blocks and add the
     partial sums in a second kernel; with ``accumulate`` and a ``pending``
     that allows it, that second step is left to the next reader of ``out``.

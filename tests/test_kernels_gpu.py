@@ -721,17 +721,22 @@ def test_gemm_bf16_reads_weights_kept_in_packed_order_only(M, N, K):
             out = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=DEV)
             k.linear(out, a, weights, bias, gelu=True, variant=variant, splits=splits)
             outs.append(out)
-        assert torch.equal(outs[0], outs[1]), (variant, splits)
+        # (left to itself the library takes another kernel for 17 to 64 rows of packed weights,
+        # which adds in another order)
+        if variant != 0 or not 16 < M <= 48:
+            assert torch.equal(outs[0], outs[1]), (variant, splits)
         assert torch.allclose(outs[1].double().cpu(), plain.gelu_tanh(ref), rtol=2**-7, atol=1e-3), (variant, splits)
 
 
 @pytest.mark.parametrize("M,N,K", [(17, 48, 64), (33, 257, 384), (64, 4800, 1600), (40, 1600, 6400), (64, 333, 1608),
-                                   (48, 80, 200), (20, 100, 520)])
+                                   (48, 80, 200), (20, 100, 520), (32, 4800, 1600), (24, 1600, 6400), (30, 333, 1608)])
 @pytest.mark.parametrize("mode", ["plain", "gelu", "accumulate", "f32out"])
 @pytest.mark.parametrize("packed", [False, True])
 def test_gemm_bf16_17_to_64_rows(M, N, K, mode, packed):
-    """17 to 64 rows: tiles of 32 x 128 and 64 x 128, K split over blocks where tiles are few (the
-    library's own choice of parts)."""
+    """17 to 64 rows, the library's own choice of kernel and parts: up to 48 rows of packed weights
+    the kernel that holds a block's weights in registers (32 features a block; K in parts where
+    that gives few blocks or a part would be longer than a block holds), otherwise tiles of
+    32 x 128 and 64 x 128 with K split over blocks."""
     k = _k()
     a = _rand((M, K), torch.bfloat16, 10)
     w = _rand((N, K), torch.bfloat16, 11, 0.1)
@@ -757,6 +762,69 @@ def test_gemm_bf16_17_to_64_rows(M, N, K, mode, packed):
         assert torch.allclose(got, want, rtol=2**-7, atol=1e-3), (got - want).abs().max()
     else:
         assert (got - want).abs().max().item() < tol, (got - want).abs().max()
+
+
+@pytest.mark.parametrize("M,N,K", [(17, 48, 1024), (48, 1600, 6400), (24, 333, 1608), (33, 4800, 1600), (32, 1000, 1792),
+                                   (41, 72, 136), (20, 100, 1856)])
+def test_gemm_bf16_rows_kernel_in_parts_and_with_the_cache_scatter(M, N, K):
+    """The kernel for 17 to 48 rows, asked for directly: whole and with K in 2, 3 and 8 parts (the
+    same bits run after run), at the longest slice it holds (28 k-blocks), refusing a longer one,
+    and with keys and values going to their pages from its epilogue or from the second kernel."""
+    k = _k()
+    from mlx_lm_amd.ops import build
+
+    lib = build.load("gemm_bf16_decode")
+    n_blocks = (K + 63) // 64
+    assert lib.gemm_bf16_rows_takes(M, K, 1) == (1 if n_blocks <= 28 else 0)
+    assert lib.gemm_bf16_rows_takes(16, K, 1) == 0 and lib.gemm_bf16_rows_takes(49, K, 1) == 0
+    auto = lib.gemm_bf16_rows_splits(M, N, K, 0)
+    assert auto >= 1 and (n_blocks + auto - 1) // auto <= 28
+    a = _rand((M, K), torch.bfloat16, 10)
+    w = _rand((N, K), torch.bfloat16, 11, 0.1)
+    bias = _rand((N,), torch.float32, 12)
+    ref = plain.linear(a.double().cpu(), w.double().cpu(), bias.double().cpu())
+    packed = k.PackedWeight(w, keep_rows=False)
+    for splits in (None, 2, 3, 8):
+        if splits is not None and (splits > n_blocks or (n_blocks + splits - 1) // splits > 28):
+            continue
+        if splits is None and n_blocks > 28:
+            continue
+        outs = []
+        for _ in range(2):
+            out = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=DEV)
+            k.linear(out, a, packed, bias, gelu=True, splits=splits or 1)
+            outs.append(out)
+        assert torch.equal(outs[0], outs[1]), splits
+        assert torch.allclose(outs[0].double().cpu(), plain.gelu_tanh(ref), rtol=2**-7, atol=1e-3), splits
+    # the cache scatter: rows of several requests, grouped key heads, a head size that is no power of two
+    for H, Hkv, hd, M_per in ((5, 5, 64, [20, 1, 10]), (4, 2, 80, [17, 30])):
+        ps, D = 16, 264
+        c = PagedCase(torch.bfloat16, H, Hkv, hd, ps, [7 + 20 * i for i in range(len(M_per))], M_per, seed=M)
+        rows, qw, kw = sum(M_per), H * hd, Hkv * hd
+        w2 = _rand((qw + 2 * kw, D), torch.bfloat16, 3, 0.2)
+        b2 = _rand((qw + 2 * kw,), torch.float32, 4, 0.1)
+        a2 = _rand((rows, D), torch.bfloat16, 5)
+        c.pool.fill_(float("nan"))
+        plain_out = torch.empty(rows, qw + 2 * kw, dtype=torch.bfloat16, device=DEV)
+        k.linear(plain_out, a2, k.PackedWeight(w2, keep_rows=False), b2, splits=1)
+        want = plain.linear(a2.double().cpu(), w2.double().cpu(), b2.double().cpu())
+        assert torch.allclose(plain_out.double().cpu(), want, rtol=2**-7, atol=1e-3)
+        k.kv_write(plain_out[:, qw : qw + kw], plain_out[:, qw + kw :], c.kv, c.block_table_dev, c.token_req, c.positions)
+        want_pool = c.pool.clone()
+        written = ~torch.isnan(want_pool.float())
+        for splits in (1, 2):
+            c.pool.fill_(float("nan"))
+            out = torch.full((rows, qw + 2 * kw), float("nan"), dtype=torch.bfloat16, device=DEV)
+            sc = k.KVScatter(c.kv, c.block_table_dev, c.token_req, c.positions, qw)
+            k.linear(out, a2, k.PackedWeight(w2, keep_rows=False), b2, scatter=sc, splits=splits)
+            if splits == 1:  # (parts are added in another order than one walk through K)
+                assert torch.equal(out[:, :qw], plain_out[:, :qw])
+                assert torch.equal(c.pool[written], want_pool[written])
+            else:
+                assert torch.allclose(out[:, :qw].float(), plain_out[:, :qw].float(), rtol=2**-6, atol=2e-3)
+                assert torch.allclose(c.pool[written].float(), want_pool[written].float(), rtol=2**-6, atol=2e-3)
+            assert torch.isnan(out[:, qw:].float()).all()
+            assert written.any() and torch.isnan(c.pool[~written].float()).all()
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 48, 1024), (8, 1600, 6400), (16, 80, 200), (16, 1600, 6400), (11, 333, 1608),
