@@ -13,7 +13,7 @@ that they do not move the timed steps' context.  ``config`` gives the context ra
 warm-up trials, three at least (a step whose shape keeps coming back is replayed from its
 recorded graph, as in the serving path: the third trial records it), then the mean of five
 timed ones, each listed in ``trials_ms``.
-``points`` holds decode at batch 1 and 64 over the same steps and, for all three batch sizes,
+``points`` holds decode at batch 1, 32 and 64 over the same steps and, for batch 1, 8 and 64,
 at context 1,000; ``roofline`` the bytes a decode step has to read (every weight once, the live
 requests' keys and values at each step's context) over its time, ``roofline_points`` the same
 fraction for every point.  Weights are random (seeded), data synthetic.
@@ -126,7 +126,7 @@ def main():
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     ap.add_argument("--layers", type=int, default=XL["n_layer"], help="run fewer layers than GPT-2 XL has")
     ap.add_argument("--prompt-len", type=int, default=512)
-    ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the points at context 1,000")
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1, 32 and 64 and the points at context 1,000")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU; this engine does not run on several (asked for %d)" % a.gpus)
@@ -189,7 +189,7 @@ def main():
     main_point = measure(a.batch, a.prompt_len, steps)
     points, fracs = {}, {f"decode_b{a.batch}": round(main_point["gbs"] / PEAK_HBM_GBS, 4)}
     if not a.no_points:
-        for b in (1, 64):
+        for b in (1, 32, 64):
             r = main_point if b == a.batch else measure(b, a.prompt_len, steps)
             points[f"decode_b{b}"] = round(r["tps"], 1)
             fracs[f"decode_b{b}"] = round(r["gbs"] / PEAK_HBM_GBS, 4)
