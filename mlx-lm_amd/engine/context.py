@@ -257,8 +257,6 @@ class StepContext:
             raw = torch.as_tensor(_DeviceArray(m.p, n_bytes), device=self.device)
         return torch.as_strided(raw.view(dtype), (m.rows, m.cols), (m.ld, 1))
 
-    foreign = tensor
-
     def int_array(self, p, n):
         """The int32 device array of ``n`` entries at address ``p`` (one of the step's own)."""
         if self._meta is not None:

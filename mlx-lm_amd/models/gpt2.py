@@ -95,32 +95,29 @@ class Model:
         layers = []
         for i in range(args.n_layer):
             p = f"model.h.{i}."
+            attention = PartSpec(
+                "attention",
+                {
+                    "width": D,
+                    "n_heads": args.n_head,
+                    "n_kv_heads": args.n_head,  # mlx_lm/models/gpt2.py:57-58
+                    "head_dim": args.head_dim,
+                    "scale": args.head_dim**-0.5,  # mlx_lm/models/gpt2.py:39
+                    "bias": True,
+                    "window": 0,
+                    "position": None,
+                },
+                p + "attn.",
+            )
+            mlp = PartSpec(
+                "gelu_mlp",
+                {"width": D, "inner": args.n_inner, "activation": args.activation_function},
+                p + "mlp.",
+            )
             layers.append(
                 LayerSpec(
                     arrangement="pre_norm",  # mlx_lm/models/gpt2.py:98-108
-                    parts=dict(
-                    mixer_norm=norm(p + "ln_1."),
-                    mixer=PartSpec(
-                        "attention",
-                        {
-                            "width": D,
-                            "n_heads": args.n_head,
-                            "n_kv_heads": args.n_head,  # mlx_lm/models/gpt2.py:57-58
-                            "head_dim": args.head_dim,
-                            "scale": args.head_dim**-0.5,  # mlx_lm/models/gpt2.py:39
-                            "bias": True,
-                            "window": 0,
-                            "position": None,
-                        },
-                        p + "attn.",
-                    ),
-                    ffn_norm=norm(p + "ln_2."),
-                    ffn=PartSpec(
-                        "gelu_mlp",
-                        {"width": D, "inner": args.n_inner, "activation": args.activation_function},
-                        p + "mlp.",
-                    ),
-                    ),
+                    parts=dict(mixer_norm=norm(p + "ln_1."), mixer=attention, ffn_norm=norm(p + "ln_2."), ffn=mlp),
                 )
             )
         return ModelPlan(

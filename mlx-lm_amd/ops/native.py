@@ -303,7 +303,7 @@ def run_python_part(part, method, ctx, call):
     elif method == CB_EMBEDDING:
         add = None
         if call.result.p:
-            add = (ctx.foreign(call.result), ctx.int_array(call.index, call.out.rows))
+            add = (ctx.tensor(call.result), ctx.int_array(call.index, call.out.rows))
         part.forward(ctx, T(call.out), add)
     elif method == CB_HEAD:
         part.forward(ctx, T(call.x), T(call.out))
