@@ -634,7 +634,10 @@ extern "C" int gemm_bf16_decode_splits(int M, int N, int K, int with_norm, int f
     // a small matrix streams in less time than the second kernel costs (measured at N = 1600:
     // K = 1600 loses 2 us by the split, K = 6400 gains 4)
     if ((long)N * K < 5000000L) return 1;
-    want = (2 * n_compute_units() + n_blocks - 1) / n_blocks;  // two blocks a CU (measured at N = 1600: K = 6400 is best in 5, K = 1600 in 2 to 6)
+    // one and a half blocks a CU (N = 1600, K = 6400: four parts; with six, two blocks a CU, a decode step of
+    // GPT-2 XL's sizes at batch 8 took 2.25 ms instead of 2.22, the parts' sum being read by the next kernel;
+    // three parts are more k-blocks than a wave holds at once, 2.41 ms)
+    want = (3 * n_compute_units() / 2 + n_blocks - 1) / n_blocks;
     if (want > n_chunks / 4) want = n_chunks / 4;  // at least four k-blocks a split
   }
   if (want < 1) want = 1;
