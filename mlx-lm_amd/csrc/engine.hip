@@ -283,6 +283,19 @@ extern "C" int eng_linear_norms_itself(const EngCtx* ctx, int M, int N, int K, i
   return takes(M, K, 1, n_splits) != 0;
 }
 
+// What follows a product that left K in parts in the workspace: the sum stays pending where it
+// goes into the residual stream and the caller allows that (the next norm adds it), otherwise
+// the second kernel adds the parts and runs the epilogue.
+static int finish_parts(EngCtx* ctx, const EngMat& out, float* ws, int n_splits, const float* bias, bool gelu,
+                        bool accumulate, const EngScatter* sc, EngPending* pending) {
+  if (accumulate && pending && pending->allowed) {
+    pending->target = (float*)out.p, pending->rows = out.rows, pending->cols = out.cols, pending->ld = out.ld;
+    pending->ws = ws, pending->n_splits = n_splits, pending->bias = bias;
+    return 0;
+  }
+  return sum_partials(ctx, out, ws, n_splits, bias, gelu, accumulate, sc);
+}
+
 static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWeight& w, const float* bias,
                   bool gelu, bool accumulate, int variant, const EngScatter* sc, int splits,
                   EngPending* pending) {
@@ -338,15 +351,7 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
              sc ? sc->positions : nullptr, sc ? sc->q_width : 0, sc ? sc->kv_width : 0, sc ? sc->head_dim : 0,
              sc ? sc->page_size : 0, n_splits, n_splits > 1 ? ws : nullptr, n_splits > 1 ? ws_floats : (size_t)0,
              ctx->stream);
-      if (n_splits > 1) {
-        if (accumulate && pending && pending->allowed) {
-          pending->target = (float*)out.p, pending->rows = M, pending->cols = N, pending->ld = out.ld;
-          pending->ws = ws, pending->n_splits = n_splits, pending->bias = bias;
-        } else {
-          TRY(sum_partials(ctx, out, ws, n_splits, bias, gelu, accumulate, sc));
-        }
-      }
-      return 0;
+      return n_splits > 1 ? finish_parts(ctx, out, ws, n_splits, bias, gelu, accumulate, sc, pending) : 0;
     }
   }
 
@@ -378,15 +383,7 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
              sc ? sc->positions : nullptr, sc ? sc->q_width : 0, sc ? sc->kv_width : 0, sc ? sc->head_dim : 0,
              sc ? sc->page_size : 0, n_splits, n_splits > 1 ? ws : nullptr, n_splits > 1 ? ws_floats : (size_t)0,
              ctx->stream);
-      if (n_splits > 1) {
-        if (accumulate && pending && pending->allowed) {
-          pending->target = (float*)out.p, pending->rows = M, pending->cols = N, pending->ld = out.ld;
-          pending->ws = ws, pending->n_splits = n_splits, pending->bias = bias;
-          return 0;
-        }
-        return sum_partials(ctx, out, ws, n_splits, bias, gelu, accumulate, sc);
-      }
-      return 0;
+      return n_splits > 1 ? finish_parts(ctx, out, ws, n_splits, bias, gelu, accumulate, sc, pending) : 0;
     }
   }
   if (w.dtype == DT_F32) {
@@ -422,14 +419,7 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
            own ? own->positions : nullptr, own ? own->q_width : 0, own ? own->kv_width : 0,
            own ? own->head_dim : 0, own ? own->page_size : 0, ctx->stream);
     if (own) return 0;
-    if (n_splits > 1) {
-      if (accumulate && pending && pending->allowed) {
-        pending->target = (float*)out.p, pending->rows = M, pending->cols = N, pending->ld = out.ld;
-        pending->ws = ws, pending->n_splits = n_splits, pending->bias = bias;
-        return 0;
-      }
-      return sum_partials(ctx, out, ws, n_splits, bias, gelu, accumulate, sc);
-    }
+    if (n_splits > 1) return finish_parts(ctx, out, ws, n_splits, bias, gelu, accumulate, sc, pending);
   }
   if (sc) {
     const EngMat k = columns(out, sc->q_width, sc->kv_width);
