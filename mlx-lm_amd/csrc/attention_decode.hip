@@ -1,8 +1,9 @@
-// Decode attention for bfloat16 caches: one query row per block, keys streamed
-// from the pages straight into registers (no LDS staging), for head sizes 32,
-// 64 and 128.  Same contract as attn_row in attention.hip (same arguments,
-// same partial buffers, same merge); this is the kernel that serving uses,
-// attn_row stays as the general one (any head size, float caches).
+// Decode attention: one query row per block, keys streamed from the pages
+// straight into registers (no LDS staging).  bfloat16 caches with head sizes
+// 32, 64 and 128, float caches with 16, 32 and 64 (a lane holds 16 bytes of a
+// key, and 4 to 16 lanes a key).  Same contract as attn_row in attention.hip
+// (same arguments, same partial buffers, same merge); this is the kernel that
+// serving uses, attn_row stays as the general one (any head size).
 //
 // Replaces scaled_dot_product_attention with one query per sequence
 // (mlx_lm/models/base.py:132-139 with mask=None, mlx_lm/generate.py:1414).
@@ -13,19 +14,20 @@
 // it is the many waves of a block, joined through LDS, that give the GPU
 // enough to do: splits need a second kernel to join them, which at these sizes
 // costs as much as the attention itself.  A wave reads a tile as
-// CPK-lane groups: lane l holds 16 bytes (8 columns) l % CPK of key l / CPK of
-// each load, where CPK = head_dim / 8 lanes cover one key.  One load
-// instruction therefore reads 64 / CPK whole keys that lie back to back in a
-// page.  Scores: 8 products per lane, summed over the CPK lanes of the key by
-// xor shuffles.  The weighted sum keeps, per lane, the 8 columns of *its* keys
-// and is only joined over the lane groups (and then the waves) at the end.
+// CPK-lane groups: lane l holds 16 bytes (EPL = 8 bfloat16 or 4 float columns)
+// l % CPK of key l / CPK of each load, where CPK = head_dim / EPL lanes cover
+// one key.  One load instruction therefore reads 64 / CPK whole keys that lie
+// back to back in a page.  Scores: EPL products per lane, summed over the CPK
+// lanes of the key by xor shuffles.  The weighted sum keeps, per lane, the EPL
+// columns of *its* keys and is only joined over the lane groups (and then the
+// waves) at the end.
 #include "common.h"
 
 struct DecodeArgs {
-  uint16_t* out;
-  const uint16_t* q;
-  const uint16_t* k_pages;
-  const uint16_t* v_pages;
+  void* out;  // out, q and the pages hold the kernel's element type
+  const void* q;
+  const void* k_pages;
+  const void* v_pages;
   const int* block_table;
   const int* token_req;
   const int* positions;
@@ -52,16 +54,25 @@ struct DecodeArgs {
 
 #define TILE 64
 
-__device__ __forceinline__ void unpack8(const uint4& v, float* f) {
+// 16 bytes of a row as floats, and a float back as an element
+__device__ __forceinline__ void unpack(const uint4& v, float (&f)[8], const uint16_t*) {
   f[0] = __uint_as_float(v.x << 16), f[1] = __uint_as_float(v.x & 0xffff0000u);
   f[2] = __uint_as_float(v.y << 16), f[3] = __uint_as_float(v.y & 0xffff0000u);
   f[4] = __uint_as_float(v.z << 16), f[5] = __uint_as_float(v.z & 0xffff0000u);
   f[6] = __uint_as_float(v.w << 16), f[7] = __uint_as_float(v.w & 0xffff0000u);
 }
+__device__ __forceinline__ void unpack(const uint4& v, float (&f)[4], const float*) {
+  f[0] = __uint_as_float(v.x), f[1] = __uint_as_float(v.y);
+  f[2] = __uint_as_float(v.z), f[3] = __uint_as_float(v.w);
+}
+__device__ __forceinline__ void put(uint16_t* at, float v) { *at = f32_to_bf16_bits(v); }
+__device__ __forceinline__ void put(float* at, float v) { *at = v; }
 
-template <int CPK>  // lanes per key: head_dim = 8 * CPK
+// T: uint16_t (bfloat16 bits) or float.  CPK lanes per key: head_dim = EPL * CPK
+template <typename T, int CPK>
 __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void attn_decode_kernel(DecodeArgs p) {
-  constexpr int HD = 8 * CPK;
+  constexpr int EPL = 16 / sizeof(T);  // elements a lane holds of a key
+  constexpr int HD = EPL * CPK;
   constexpr int KPL = 64 / CPK;    // keys per load instruction
   constexpr int NL = TILE / KPL;   // loads per tile (= CPK)
   __shared__ float Ms[MAX_WAVES], Ls[MAX_WAVES];
@@ -110,15 +121,17 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
     for (int i = tid; i < p.max_blocks; i += blockDim.x) page_of[i] = table[i];
   }
   const int pos = p.positions[row];
-  const int sub = lane % CPK;  // which 8 columns of the key
+  const int sub = lane % CPK;  // which EPL columns of the key
   const int kin = lane / CPK;  // which key of a load
+  const T* k_pages = (const T*)p.k_pages;
+  const T* v_pages = (const T*)p.v_pages;
 
-  float qf[8];
+  float qf[EPL];
   {
-    const uint4 qv = *(const uint4*)(p.q + (size_t)row * p.ldq + h * HD + sub * 8);
-    unpack8(qv, qf);
+    const uint4 qv = *(const uint4*)((const T*)p.q + (size_t)row * p.ldq + h * HD + sub * EPL);
+    unpack(qv, qf, (const T*)nullptr);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) qf[i] *= p.scale;
+    for (int i = 0; i < EPL; ++i) qf[i] *= p.scale;
   }
 
   const int k_hi = pos + 1;
@@ -129,9 +142,9 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
   const int t_begin = split * per_split;
   const int t_end = min(n_tiles, t_begin + per_split);
 
-  float m = -INFINITY, l = 0.f, o[8];
+  float m = -INFINITY, l = 0.f, o[EPL];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) o[i] = 0.f;
+  for (int i = 0; i < EPL; ++i) o[i] = 0.f;
 
   const size_t head_off = (size_t)kv_head * p.page_size * HD;
   if (p.table_in_lds) __syncthreads();  // (uniform over the block)
@@ -147,19 +160,19 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
       key = min(max(key, k_lo), k_hi - 1);
       const int page = p.table_in_lds ? page_of[key / p.page_size] : table[key / p.page_size];
       const size_t off = (size_t)page * p.page_stride + head_off +
-                         (size_t)(key % p.page_size) * HD + sub * 8;
-      kv[j] = *(const uint4*)(p.k_pages + off);
-      vv[j] = *(const uint4*)(p.v_pages + off);
+                         (size_t)(key % p.page_size) * HD + sub * EPL;
+      kv[j] = *(const uint4*)(k_pages + off);
+      vv[j] = *(const uint4*)(v_pages + off);
     }
     float s[NL];
     float tmax = -INFINITY;
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
-      float kf[8];
-      unpack8(kv[j], kf);
+      float kf[EPL];
+      unpack(kv[j], kf, (const T*)nullptr);
       float d = 0.f;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) d += qf[i] * kf[i];
+      for (int i = 0; i < EPL; ++i) d += qf[i] * kf[i];
       d = group_sum<CPK>(d);  // over the key's lanes
       const int key = kt + j * KPL + kin;
       s[j] = (key >= k_lo && key < k_hi) ? d : -INFINITY;
@@ -170,15 +183,15 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
     const float alpha = __expf(m - m_new);
     l *= alpha;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) o[i] *= alpha;
+    for (int i = 0; i < EPL; ++i) o[i] *= alpha;
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
       const float pj = __expf(s[j] - m_new);  // exp(-inf) = 0 for masked keys
-      float vf[8];
-      unpack8(vv[j], vf);
+      float vf[EPL];
+      unpack(vv[j], vf, (const T*)nullptr);
       if (sub == 0) l += pj;  // one lane of the key's group counts it
 #pragma unroll
-      for (int i = 0; i < 8; ++i) o[i] += pj * vf[i];
+      for (int i = 0; i < EPL; ++i) o[i] += pj * vf[i];
     }
     m = m_new;
   }
@@ -194,13 +207,13 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
   };
   l = over_groups(l);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) o[i] = over_groups(o[i]);
+  for (int i = 0; i < EPL; ++i) o[i] = over_groups(o[i]);
   l = group_sum<CPK>(l);
 
   if (lane == 0) Ms[wave] = m, Ls[wave] = l;
   if (lane < CPK) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) Os[wave][lane * 8 + i] = o[i];
+    for (int i = 0; i < EPL; ++i) Os[wave][lane * EPL + i] = o[i];
   }
   __syncthreads();
 
@@ -215,7 +228,7 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
   }
   if (tid < HD) {
     if (p.n_splits == 1) {
-      p.out[(size_t)row * p.ldo + h * HD + tid] = f32_to_bf16_bits(acc / L);
+      put((T*)p.out + (size_t)row * p.ldo + h * HD + tid, acc / L);
     } else {
       const size_t base = ((size_t)item * p.n_heads + h) * p.n_splits + split;
       p.part_o[base * HD + tid] = acc;
@@ -225,9 +238,9 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
 }
 
 // grid (rows, heads), HD threads: join the splits
-template <int CPK>
+template <typename T, int CPK>
 __global__ void attn_decode_merge_kernel(DecodeArgs p) {
-  constexpr int HD = 8 * CPK;
+  constexpr int HD = 16 / sizeof(T) * CPK;
   const int item = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
   const int row = p.rows_are_requests ? item : p.rows[item];
   const size_t base = ((size_t)item * p.n_heads + h) * p.n_splits;
@@ -241,12 +254,12 @@ __global__ void attn_decode_merge_kernel(DecodeArgs p) {
     L += p.part_ml[(base + s) * 2 + 1] * w;
     acc += p.part_o[(base + s) * HD + d] * w;
   }
-  p.out[(size_t)row * p.ldo + h * HD + d] = f32_to_bf16_bits(acc / L);
+  put((T*)p.out + (size_t)row * p.ldo + h * HD + d, acc / L);
 }
 
 DEFINE_LAST_ERROR(mlxlm_last_error)
 
-template <int CPK>
+template <typename T, int CPK>
 static void launch(const DecodeArgs& p, int n_rows, int n_waves, hipStream_t stream) {
   // reading blocks for the CUs that the rows leave idle, if there are eight or more
   int extra_y = 0;
@@ -255,64 +268,47 @@ static void launch(const DecodeArgs& p, int n_rows, int n_waves, hipStream_t str
     if (extra_y * n_rows < 8) extra_y = 0;
   }
   const size_t lds = p.table_in_lds ? (size_t)p.max_blocks * sizeof(int) : 0;
-  hipLaunchKernelGGL(attn_decode_kernel<CPK>, dim3(n_rows, p.n_heads + extra_y, p.n_splits), dim3(64 * n_waves), lds, stream, p);
+  hipLaunchKernelGGL((attn_decode_kernel<T, CPK>), dim3(n_rows, p.n_heads + extra_y, p.n_splits), dim3(64 * n_waves), lds, stream, p);
   if (p.n_splits > 1)
-    hipLaunchKernelGGL(attn_decode_merge_kernel<CPK>, dim3(n_rows, p.n_heads), dim3(8 * CPK), 0, stream, p);
+    hipLaunchKernelGGL((attn_decode_merge_kernel<T, CPK>), dim3(n_rows, p.n_heads), dim3(16 / sizeof(T) * CPK), 0, stream, p);
 }
 
-// Same arguments as attn_row; bfloat16 only, head_dim 32, 64 or 128, and pages
-// that hold whole loads (page_size a multiple of 512 / head_dim keys).
+// Same arguments as attn_row, with what is read ahead and rows_are_requests between: 1 says that
+// item i of `rows` is row i and belongs to request i (every request of the step brings one token),
+// which saves the kernel two trips to memory.  dtype DT_BF16 with head_dim 32, 64 or 128, DT_F32
+// with 16, 32 or 64, and pages that hold whole loads (page_size a multiple of the keys in 1 KB).
 extern "C" int attn_decode_rows(void* out, const void* q, int ldq, int ldo, const void* k_pages,
                                 const void* v_pages, size_t page_stride, const int* block_table,
                                 int max_blocks, const int* token_req, const int* positions,
                                 const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
                                 int page_size, int window, float scale, int n_splits, float* part_o,
                                 float* part_ml, int n_waves, const void* ahead, size_t ahead_chunk_bytes,
-                                int ahead_chunks, int rows_are_requests, hipStream_t stream);
-
-extern "C" int attn_decode(void* out, const void* q, int ldq, int ldo, const void* k_pages,
-                           const void* v_pages, size_t page_stride, const int* block_table,
-                           int max_blocks, const int* token_req, const int* positions,
-                           const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
-                           int page_size, int window, float scale, int n_splits, float* part_o,
-                           float* part_ml, int n_waves, const void* ahead, size_t ahead_chunk_bytes,
-                           int ahead_chunks, hipStream_t stream) {
-  return attn_decode_rows(out, q, ldq, ldo, k_pages, v_pages, page_stride, block_table, max_blocks, token_req,
-                          positions, rows, n_rows, n_heads, n_kv_heads, head_dim, page_size, window, scale,
-                          n_splits, part_o, part_ml, n_waves, ahead, ahead_chunk_bytes, ahead_chunks, 0, stream);
-}
-
-// The same with rows_are_requests: 1 says that item i of `rows` is row i and belongs to request i
-// (every request of the step brings one token), which saves the kernel two trips to memory.
-extern "C" int attn_decode_rows(void* out, const void* q, int ldq, int ldo, const void* k_pages,
-                                const void* v_pages, size_t page_stride, const int* block_table,
-                                int max_blocks, const int* token_req, const int* positions,
-                                const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
-                                int page_size, int window, float scale, int n_splits, float* part_o,
-                                float* part_ml, int n_waves, const void* ahead, size_t ahead_chunk_bytes,
-                                int ahead_chunks, int rows_are_requests, hipStream_t stream) {
+                                int ahead_chunks, int rows_are_requests, int dtype, hipStream_t stream) {
   if (n_rows <= 0) return 0;
+  if (dtype != DT_F32 && dtype != DT_BF16) FAIL("attn_decode: unknown dtype code %d", dtype);
+  const int epl = dtype == DT_F32 ? 4 : 8;  // elements in a lane's 16 bytes
   if (n_waves < 1 || n_waves > MAX_WAVES) FAIL("attn_decode: %d waves a block, must be 1 to %d", n_waves, MAX_WAVES);
+  if (head_dim != 4 * epl && head_dim != 8 * epl && head_dim != 16 * epl)
+    FAIL("attn_decode: head_dim %d is not %d, %d or %d (attn_row takes the others)", head_dim, 4 * epl, 8 * epl,
+         16 * epl);
+  const int cpk = head_dim / epl;
   if (head_dim > 64 * n_waves) FAIL("attn_decode: head_dim %d needs at least %d waves", head_dim, (head_dim + 63) / 64);
-  if (head_dim == 128 && n_waves > MAX_WAVES / 2) n_waves = MAX_WAVES / 2;  // (that kernel's registers allow eight)
-  if (head_dim != 32 && head_dim != 64 && head_dim != 128)
-    FAIL("attn_decode: head_dim %d is not 32, 64 or 128 (attn_row takes the others)", head_dim);
-  const int kpl = 512 / head_dim;
+  if (cpk == 16 && n_waves > MAX_WAVES / 2) n_waves = MAX_WAVES / 2;  // (that kernel's registers allow eight)
+  const int kpl = 64 / cpk;
   if (page_size <= 0 || page_size % kpl != 0)
     FAIL("attn_decode: page_size %d must be a multiple of %d for head_dim %d", page_size, kpl, head_dim);
   if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads != 0)
     FAIL("attn_decode: %d query heads cannot be grouped over %d key heads", n_heads, n_kv_heads);
   if (!out || !q || !k_pages || !v_pages || !block_table || !token_req || !positions || !rows)
     FAIL("attn_decode: null pointer");
-  if (ldq % 8 != 0 || ((uintptr_t)q & 15)) FAIL("attn_decode: queries must be 16-byte aligned rows");
-  if (page_stride % 8 != 0 || (((uintptr_t)k_pages | (uintptr_t)v_pages) & 15))
+  if (ldq % epl != 0 || ((uintptr_t)q & 15)) FAIL("attn_decode: queries must be 16-byte aligned rows");
+  if (page_stride % epl != 0 || (((uintptr_t)k_pages | (uintptr_t)v_pages) & 15))
     FAIL("attn_decode: pages must be 16-byte aligned");
   if (window < 0) FAIL("attn_decode: window %d must not be negative", window);
   if (n_splits < 1 || n_splits > 65535) FAIL("attn_decode: n_splits %d out of range", n_splits);
   if (n_splits > 1 && (!part_o || !part_ml)) FAIL("attn_decode: splits need the partial buffers");
   DecodeArgs p;
-  p.out = (uint16_t*)out, p.q = (const uint16_t*)q;
-  p.k_pages = (const uint16_t*)k_pages, p.v_pages = (const uint16_t*)v_pages;
+  p.out = out, p.q = q, p.k_pages = k_pages, p.v_pages = v_pages;
   p.block_table = block_table, p.token_req = token_req, p.positions = positions, p.rows = rows;
   p.part_o = part_o, p.part_ml = part_ml, p.page_stride = page_stride;
   p.ldq = ldq, p.ldo = ldo, p.max_blocks = max_blocks;
@@ -324,12 +320,21 @@ extern "C" int attn_decode_rows(void* out, const void* q, int ldq, int ldo, cons
   p.ahead_chunks = ahead ? ahead_chunks : 0;
   p.rows_are_requests = rows_are_requests ? 1 : 0;
   p.table_in_lds = max_blocks > 0 && max_blocks <= 8192;  // (32 KB of LDS at most)
-  if (head_dim == 32)
-    launch<4>(p, n_rows, n_waves, stream);
-  else if (head_dim == 64)
-    launch<8>(p, n_rows, n_waves, stream);
-  else
-    launch<16>(p, n_rows, n_waves, stream);
+  if (dtype == DT_BF16) {
+    if (cpk == 4)
+      launch<uint16_t, 4>(p, n_rows, n_waves, stream);
+    else if (cpk == 8)
+      launch<uint16_t, 8>(p, n_rows, n_waves, stream);
+    else
+      launch<uint16_t, 16>(p, n_rows, n_waves, stream);
+  } else {
+    if (cpk == 4)
+      launch<float, 4>(p, n_rows, n_waves, stream);
+    else if (cpk == 8)
+      launch<float, 8>(p, n_rows, n_waves, stream);
+    else
+      launch<float, 16>(p, n_rows, n_waves, stream);
+  }
   CHECK_LAUNCH("attn_decode");
   return 0;
 }

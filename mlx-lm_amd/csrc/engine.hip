@@ -61,7 +61,7 @@ typedef int (*fn_embed)(void*, const void*, const int*, const void*, const int*,
 typedef int (*fn_layernorm)(void*, const float*, const int*, const float*, const float*, float, int, int, int,
                             hipStream_t);
 typedef int (*fn_gemm_f32)(void*, const void*, const void*, const float*, int, int, int, int, int, int, int,
-                           int, hipStream_t);
+                           int, int, float*, size_t, hipStream_t);
 typedef int (*fn_gemm_bf16)(void*, const void*, const void*, const float*, int, int, int, int, int, int, int,
                             int, int, float*, size_t, void*, void*, size_t, const int*, int, const int*,
                             const int*, int, int, int, int, hipStream_t);
@@ -91,7 +91,7 @@ typedef int (*fn_attn_row)(void*, const void*, int, int, const void*, const void
                            float*, float*, int, hipStream_t);
 typedef int (*fn_attn_decode)(void*, const void*, int, int, const void*, const void*, size_t, const int*, int,
                               const int*, const int*, const int*, int, int, int, int, int, int, float, int,
-                              float*, float*, int, const void*, size_t, int, int, hipStream_t);
+                              float*, float*, int, const void*, size_t, int, int, int, hipStream_t);
 typedef int (*fn_attn_prefill)(void*, const void*, int, int, const void*, const void*, size_t, const int*,
                                int, const int*, const int*, const int*, int, int, int, int, int, int, float,
                                hipStream_t);
@@ -99,6 +99,7 @@ typedef int (*fn_attn_prefill)(void*, const void*, int, int, const void*, const 
 static Entry<fn_embed> k_embed("embed", "embed_gather_add");
 static Entry<fn_layernorm> k_layernorm("norm", "layernorm");
 static Entry<fn_gemm_f32> k_gemm_f32("gemm_f32", "gemm_f32");
+static Entry<fn_int4> k_gemm_f32_splits("gemm_f32", "gemm_f32_splits");
 static Entry<fn_gemm_bf16> k_gemm_bf16("gemm_bf16", "gemm_bf16_scatter");
 static Entry<fn_int5> k_gemm_bf16_splits("gemm_bf16", "gemm_bf16_splits");
 static Entry<fn_gemm_decode> k_gemm_decode("gemm_bf16_decode", "gemm_bf16_decode");
@@ -387,7 +388,26 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
     }
   }
   if (w.dtype == DT_F32) {
-    KERNEL(k_gemm_f32, ctx, out.p, A.p, w.w, bias, M, N, K, A.ld, w.ldw, out.ld, flags, variant, ctx->stream);
+    // Few rows of a narrow matrix give the kernel for them fewer blocks than there are compute
+    // units: K goes in parts then, and the same second kernels add them up as for bfloat16.
+    int n_splits = 1;
+    if ((variant == 0 || variant == 3) && M <= DECODE_MAX_ROWS) {
+      if (splits == 0)
+        QUERY(k_gemm_f32_splits, n_splits, M, N, K, ctx->force_splits);
+      else
+        n_splits = split_count((K + 63) / 64, splits);
+      if (n_splits > 1) {
+        const size_t most = ws ? ws_floats / ((size_t)M * N) : 0;
+        if ((size_t)n_splits > most) n_splits = (int)most;
+        if (n_splits > 1) n_splits = split_count((K + 63) / 64, n_splits);
+      }
+      if (n_splits < 1) n_splits = 1;
+      if (n_splits > 1 && pending) TRY(settle(ctx, pending));  // the workspace is about to be written again
+    }
+    KERNEL(k_gemm_f32, ctx, out.p, A.p, w.w, bias, M, N, K, A.ld, w.ldw, out.ld, flags, variant, n_splits,
+           n_splits > 1 ? ws : nullptr, n_splits > 1 ? ws_floats : (size_t)0, ctx->stream);
+    // (keys and values go to their pages from the finished rows, below)
+    if (n_splits > 1) TRY(finish_parts(ctx, out, ws, n_splits, bias, gelu, accumulate, nullptr, pending));
   } else {
     // Few rows give the tile kernel few tiles: K is split then as for the decode kernels,
     // and the same second kernels add the parts and run the epilogue.
@@ -727,7 +747,10 @@ struct Attention : Mixer {
                kv.page_size, window, scale, q.dtype, ctx->stream);
     }
     if (n_rows) {
-      const bool fast = mfma_sizes && kv.page_size % (512 / head_dim) == 0;
+      // the kernel that streams keys into registers: a key in 4, 8 or 16 lanes of 16 bytes
+      const int key_bytes = head_dim * (bf16 ? 2 : 4);
+      const bool fast = (key_bytes == 64 || key_bytes == 128 || key_bytes == 256) &&
+                        kv.page_size % (1024 / key_bytes) == 0;
       int n_splits = 1, n_waves = 4;
       if (fast)
         row_work(ctx, n_rows, max_row_context, &n_splits, &n_waves);
@@ -760,7 +783,7 @@ struct Attention : Mixer {
                kv.max_blocks, kv.token_req, kv.positions, rows, n_rows, n_heads, n_kv_heads, head_dim,
                kv.page_size, window, scale, n_splits, (float*)part_o.p, (float*)part_ml.p, n_waves,
                ahead ? ahead->packed : nullptr, ahead ? ahead->chunk_bytes : (size_t)0, chunks, rows_are_requests,
-               ctx->stream);
+               q.dtype, ctx->stream);
       } else {
         KERNEL(k_attn_row, ctx, out.p, q.p, q.ld, out.ld, kv.k, kv.v, kv.page_stride, kv.block_table,
                kv.max_blocks, kv.token_req, kv.positions, rows, n_rows, n_heads, n_kv_heads, head_dim,

@@ -7,11 +7,9 @@
 // (mlx_lm/models/gpt2.py:41-42,52,68,76-80,167).
 //
 // Up to 16 rows (decode steps) take a kernel of their own, which streams W
-// once with plain float FMAs: a 64 x 64 MFMA tile would spend its time on rows
-// that are not there.  A wave owns four features; its lanes stride along k in
-// float4 pieces, the rows sit in LDS in stretches of 512 columns; a lane sums
-// its share in the order of k and the 64 shares are added by a fixed tree, so
-// an output does not depend on the other rows of the step.
+// once through v_mfma_f32_16x16x4_f32, 16 features a block: a 64 x 64 tile
+// would spend its time on rows that are not there and leave most compute units
+// without a block.
 #include "common.h"
 
 #define FLAG_GELU 1
@@ -30,6 +28,10 @@ struct GemmArgs {
   int M, N, K;
   int lda, ldw, ldo;
   int flags;
+  // the kernel for few rows: blockIdx.y takes part y of K's chunks and leaves its sums in
+  // ws[y][M][N], without bias or epilogue
+  int n_splits;
+  float* ws;
 };
 
 #define BK 16
@@ -170,80 +172,129 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs p) {
   }
 }
 
-#define SKF_FW 4     // features a wave
-#define SKF_KC 512   // columns of the rows held in LDS at a time
+#define SKF_WAVES_FEW 8   // waves a block where the blocks are fewer than the compute units
+#define SKF_WAVES_MANY 4  // and where every unit has a block or more (8: 12.1 us instead of 10.6 for 4,800 features of 1,600)
+#define SKF_MAX_WAVES 8
+#define SKF_SPLIT_FROM 5000000L  // elements of a matrix from which a split of K pays
+#define SKF_CHUNK 64                    // columns of a chunk
+#define SKF_STRIDE (SKF_CHUNK + 4)      // floats between a chunk's rows in LDS: no two of a load's lanes share a bank
 
-template <int MR>  // rows, rounded up to a power of two (rows that are not there are zero)
-__global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(GemmArgs p) {
-  __shared__ float4 As[MR][SKF_KC / 4];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n_base = blockIdx.x * (4 * SKF_FW) + wave * SKF_FW;
-  const float* wrow[SKF_FW];
+// Up to 16 rows.  A block owns 16 features and, where K is split over blockIdx.y, a run of
+// chunks of 64 columns; its waves take the run's chunks in turn, each wave on its own (no
+// barrier inside the loop).  A chunk of the weights comes from memory as 256 contiguous bytes a
+// feature, four features a load, goes through the wave's own piece of LDS and comes back in the
+// layout of v_mfma_f32_16x16x4_f32: lane l holds columns 4 * (l / 16) .. + 3 of each 16 of
+// feature l % 16.  The rows are the other operand, read in that layout from the L2, where they
+// stay.  The next chunk is asked for before this one is multiplied; other waves cover the rest
+// of the wait (a deeper queue was slower: 82 us against 72 for the vocabulary's matrix at 8
+// rows).  The same instructions run whatever the number of rows, so a row's result does not
+// depend on it.
+__global__ __launch_bounds__(64 * SKF_MAX_WAVES) void gemm_f32_skinny_kernel(GemmArgs p) {
+  // (native vectors: a struct copied to LDS keeps what was loaded out of registers)
+  __shared__ f32x4_t stage[SKF_MAX_WAVES][16 * SKF_STRIDE / 4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n_waves = blockDim.x >> 6;
+  const int n0 = blockIdx.x * 16;
+  const int l16 = lane & 15, kq = lane >> 4;
+  // features and rows that are not there read the last one that is; nothing of theirs is stored
+  const float* wsrc[4];  // load i: feature 4 * i + l / 16, columns 4 * (l % 16) .. + 3 of the chunk
 #pragma unroll
-  for (int f = 0; f < SKF_FW; ++f) wrow[f] = p.W + (size_t)min(n_base + f, p.N - 1) * p.ldw;
+  for (int i = 0; i < 4; ++i) wsrc[i] = p.W + (size_t)min(n0 + 4 * i + kq, p.N - 1) * p.ldw;
+  const float* arow = p.A + (size_t)min(l16, p.M - 1) * p.lda;
+  f32x4_t* mine = stage[wave];
+  const int n_chunks = (p.K + SKF_CHUNK - 1) / SKF_CHUNK;
+  const int per_split = (n_chunks + p.n_splits - 1) / p.n_splits;
+  const int c_end = min(n_chunks, (blockIdx.y + 1) * per_split);
 
-  float acc[SKF_FW][MR];
+  f32x4_t wv[4], av[4];
+  // columns beyond K (in the last chunk) and chunks beyond the run (asked for ahead by the wave's
+  // last round) are read from inside the matrix; the rows' values beyond K count as zero
+  auto ask = [&](int c) {
 #pragma unroll
-  for (int f = 0; f < SKF_FW; ++f)
+    for (int i = 0; i < 4; ++i) wv[i] = *(const f32x4_t*)(wsrc[i] + min(c * SKF_CHUNK + 4 * l16, p.K - 4));
 #pragma unroll
-    for (int m = 0; m < MR; ++m) acc[f][m] = 0.f;
-
-  for (int k0 = 0; k0 < p.K; k0 += SKF_KC) {
-    const int width = min(SKF_KC, p.K - k0);  // a multiple of 4
-    // the weights first: they are on their way while the rows are copied into LDS
-    // (columns beyond the stretch are read from inside it; they meet zeros in LDS)
-    float4 w[SKF_KC / 256][SKF_FW];
+    for (int t = 0; t < 4; ++t) av[t] = *(const f32x4_t*)(arow + min(c * SKF_CHUNK + 16 * t + 4 * kq, p.K - 4));
+  };
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+  int c = blockIdx.y * per_split + wave;
+  ask(c);
+  for (; c < c_end; c += n_waves) {
+    f32x4_t a[4];
 #pragma unroll
-    for (int j = 0; j < SKF_KC / 256; ++j)
+    for (int i = 0; i < 4; ++i) mine[(4 * i + kq) * (SKF_STRIDE / 4) + l16] = wv[i];
 #pragma unroll
-      for (int f = 0; f < SKF_FW; ++f) w[j][f] = *(const float4*)(wrow[f] + k0 + min((lane + 64 * j) * 4, width - 4));
-    __syncthreads();  // the stretch before is no longer read
-    for (int i = tid; i < MR * (SKF_KC / 4); i += 256) {
-      const int r = i / (SKF_KC / 4), c = i - r * (SKF_KC / 4);
-      const float4 t = *(const float4*)(p.A + (size_t)min(r, p.M - 1) * p.lda + k0 + min(c * 4, width - 4));
-      As[r][c] = (r < p.M && c * 4 < width) ? t : ZERO4;
+    for (int t = 0; t < 4; ++t) {
+      const float live = c * SKF_CHUNK + 16 * t + 4 * kq < p.K ? 1.f : 0.f;
+      a[t] = av[t] * live;
     }
-    __syncthreads();
+    ask(c + n_waves);
+    __builtin_amdgcn_wave_barrier();  // (orders the compiler; a wave's LDS accesses run in order)
 #pragma unroll
-    for (int j = 0; j < SKF_KC / 256; ++j) {
-      const int c = lane + 64 * j;
-#pragma unroll
-      for (int m = 0; m < MR; ++m) {
-        const float4 a = As[m][c];
-#pragma unroll
-        for (int f = 0; f < SKF_FW; ++f) {
-          acc[f][m] = fmaf(w[j][f].x, a.x, acc[f][m]);
-          acc[f][m] = fmaf(w[j][f].y, a.y, acc[f][m]);
-          acc[f][m] = fmaf(w[j][f].z, a.z, acc[f][m]);
-          acc[f][m] = fmaf(w[j][f].w, a.w, acc[f][m]);
-        }
-      }
+    for (int t = 0; t < 4; ++t) {
+      const f32x4_t w = mine[l16 * (SKF_STRIDE / 4) + 4 * t + kq];
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t].x, w.x, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t].y, w.y, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t].z, w.z, acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t].w, w.w, acc, 0, 0, 0);
     }
+    __builtin_amdgcn_wave_barrier();
   }
+  // accumulator r of lane l: row 4 * (l / 16) + r, feature l % 16.  The waves' sums are added
+  // in the order of the waves, one thread an output.
+  __syncthreads();  // the pieces of LDS are no longer read
+  float* parts = (float*)&stage[0][0];
 #pragma unroll
-  for (int f = 0; f < SKF_FW; ++f) {
-    const int n = n_base + f;
-#pragma unroll
-    for (int m = 0; m < MR; ++m) {
-      float v = wave_sum(acc[f][m]);
-      if (lane == 0 && n < p.N && m < p.M) {
-        if (p.bias) v += p.bias[n];
-        const size_t idx = (size_t)m * p.ldo + n;
-        if (p.flags & FLAG_ACCUMULATE)
-          p.out[idx] += v;
-        else
-          p.out[idx] = (p.flags & FLAG_GELU) ? gelu_tanh(v) : v;
+  for (int r = 0; r < 4; ++r) parts[(wave * 16 + 4 * kq + r) * 16 + l16] = acc[r];
+  __syncthreads();
+  if (tid < 256) {
+    const int m = tid >> 4, n = n0 + (tid & 15);
+    if (m < p.M && n < p.N) {
+      float v = parts[tid];
+      for (int w = 1; w < n_waves; ++w) v += parts[w * 256 + tid];
+      if (p.n_splits > 1) {
+        p.ws[((size_t)blockIdx.y * p.M + m) * p.N + n] = v;  // added up, and finished, by the caller's second kernel
+        return;
       }
+      if (p.bias) v += p.bias[n];
+      const size_t idx = (size_t)m * p.ldo + n;
+      if (p.flags & FLAG_ACCUMULATE)
+        p.out[idx] += v;
+      else
+        p.out[idx] = (p.flags & FLAG_GELU) ? gelu_tanh(v) : v;
     }
   }
 }
 
 DEFINE_LAST_ERROR(mlxlm_last_error)
 
-// variant: 0 = choose, 1 = 128x128 block tile, 2 = 64x64 block tile, 3 = the kernel for up to 16 rows
+// In how many parts the kernel for few rows should take K so that its blocks fill the GPU: one
+// and a half blocks a compute unit, eight chunks of 64 columns a part at least.  1 where the
+// matrix gives a block to every unit anyway, or is so small that a second kernel costs more
+// than the split gains.
+extern "C" int gemm_f32_splits(int M, int N, int K, int force) {
+  const int n_chunks = (K + SKF_CHUNK - 1) / SKF_CHUNK;
+  if (M < 1 || M > 16) return 1;
+  int want;
+  if (force > 0) {
+    want = force;
+  } else {
+    const int n_blocks = (N + 15) / 16;
+    if (n_blocks >= n_compute_units() || (long)N * K < SKF_SPLIT_FROM) return 1;
+    want = (3 * n_compute_units() / 2 + n_blocks - 1) / n_blocks;
+    if (want > n_chunks / 8) want = n_chunks / 8;
+  }
+  if (want < 1) want = 1;
+  if (want > n_chunks) want = n_chunks;
+  const int per = (n_chunks + want - 1) / want;
+  return (n_chunks + per - 1) / per;  // no empty part
+}
+
+// variant: 0 = choose, 1 = 128x128 block tile, 2 = 64x64 block tile, 3 = the kernel for up to 16 rows.
+// n_splits > 1 (the kernel for few rows only): K in that many parts, whose sums go to
+// ws[part][M][N] (ws_floats floats at least) for sum_partials of gemm_bf16_decode.hip to add up
+// and finish; out is not written then.
 extern "C" int gemm_f32(void* out, const void* A, const void* W, const float* bias, int M, int N,
-                        int K, int lda, int ldw, int ldo, int flags, int variant,
-                        hipStream_t stream) {
+                        int K, int lda, int ldw, int ldo, int flags, int variant, int n_splits, float* ws,
+                        size_t ws_floats, hipStream_t stream) {
   GemmArgs p;
   p.A = (const float*)A;
   p.W = (const float*)W;
@@ -252,6 +303,7 @@ extern "C" int gemm_f32(void* out, const void* A, const void* W, const float* bi
   p.M = M, p.N = N, p.K = K;
   p.lda = lda, p.ldw = ldw, p.ldo = ldo;
   p.flags = flags;
+  p.n_splits = 1, p.ws = nullptr;
   if (M < 0 || N <= 0 || K <= 0) FAIL("gemm_f32: bad sizes M=%d N=%d K=%d", M, N, K);
   if (K % 4 != 0) FAIL("gemm_f32: K=%d must be a multiple of 4", K);
   if (lda % 4 != 0 || ldw % 4 != 0)
@@ -263,6 +315,14 @@ extern "C" int gemm_f32(void* out, const void* A, const void* W, const float* bi
   if ((flags & FLAG_ACCUMULATE) && (flags & FLAG_GELU))
     FAIL("gemm_f32: GELU and accumulate cannot be combined");
   if (M == 0) return 0;
+  if (n_splits < 1) FAIL("gemm_f32: n_splits=%d", n_splits);
+  if (n_splits > 1) {
+    if (variant == 0 && M <= 16) variant = 3;
+    if (variant != 3) FAIL("gemm_f32: only the kernel for up to 16 rows takes K in parts");
+    if (n_splits > (K + SKF_CHUNK - 1) / SKF_CHUNK) FAIL("gemm_f32: %d parts of K=%d", n_splits, K);
+    if (!ws || ws_floats < (size_t)n_splits * M * N) FAIL("gemm_f32: the parts' workspace is too small");
+    p.n_splits = n_splits, p.ws = ws;
+  }
   if (variant == 0) variant = M <= 16 ? 3 : (M <= 64 || (size_t)M * N < (size_t)128 * 128 * 128) ? 2 : 1;
   if (variant == 1) {
     dim3 grid((N + 127) / 128, (M + 127) / 128), block(256);
@@ -272,17 +332,10 @@ extern "C" int gemm_f32(void* out, const void* A, const void* W, const float* bi
     hipLaunchKernelGGL((gemm_f32_kernel<1, 1>), grid, block, 0, stream, p);
   } else if (variant == 3) {
     if (M > 16) FAIL("gemm_f32: the kernel for few rows takes at most 16, got %d", M);
-    dim3 grid((N + 4 * SKF_FW - 1) / (4 * SKF_FW)), block(256);
-    if (M <= 1)
-      hipLaunchKernelGGL(gemm_f32_skinny_kernel<1>, grid, block, 0, stream, p);
-    else if (M <= 2)
-      hipLaunchKernelGGL(gemm_f32_skinny_kernel<2>, grid, block, 0, stream, p);
-    else if (M <= 4)
-      hipLaunchKernelGGL(gemm_f32_skinny_kernel<4>, grid, block, 0, stream, p);
-    else if (M <= 8)
-      hipLaunchKernelGGL(gemm_f32_skinny_kernel<8>, grid, block, 0, stream, p);
-    else
-      hipLaunchKernelGGL(gemm_f32_skinny_kernel<16>, grid, block, 0, stream, p);
+    // where the blocks are fewer than the compute units, more waves each
+    const int blocks = (N + 15) / 16;
+    const int waves = blocks * p.n_splits < n_compute_units() ? SKF_WAVES_FEW : SKF_WAVES_MANY;
+    hipLaunchKernelGGL(gemm_f32_skinny_kernel, dim3(blocks, p.n_splits), dim3(64 * waves), 0, stream, p);
   } else {
     FAIL("gemm_f32: unknown variant %d", variant);
   }

@@ -570,21 +570,24 @@ def attn_prefill(out, q, kv, block_table, token_req, positions, tiles, n_tiles, 
 
 def attn_decode_takes(q_dtype, kv):
     """Whether the register-streaming decode kernel takes this cache geometry."""
-    return (q_dtype == torch.bfloat16 and kv.head_dim in (32, 64, 128)
-            and kv.page_size % (512 // kv.head_dim) == 0)
+    if q_dtype not in (torch.bfloat16, torch.float32):
+        return False
+    key_bytes = kv.head_dim * q_dtype.itemsize
+    return key_bytes in (64, 128, 256) and kv.page_size % (1024 // key_bytes) == 0
 
 
 def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_heads, scale,
                 window=0, n_splits=1, part_o=None, part_ml=None, n_waves=4, ahead=None, ahead_chunks=0,
                 rows_are_requests=False):
-    """``attn_row`` for bfloat16 caches with head_dim 32, 64 or 128: keys stream into registers.
+    """``attn_row`` for keys of 64, 128 or 256 bytes (bfloat16 with head_dim 32, 64 or 128, float32
+    with 16, 32 or 64): keys stream into registers.
 
     ``ahead``: a ``PackedWeight`` whose first ``ahead_chunks`` chunks the CUs without a row read
     meanwhile, each the chunks that a block on its own die will ask for (``sum_partials_norm``).
     ``rows_are_requests``: item ``i`` of ``rows`` is row ``i`` of request ``i`` (the caller says so)."""
     lib = build.load("attention_decode")
     ldq, ldo = _rows2d(q, "q"), _rows2d(out, "out")
-    _need(q.dtype == torch.bfloat16, "attn_decode: bfloat16 only")
+    _need(q.dtype in (torch.bfloat16, torch.float32), "attn_decode: bfloat16 or float32")
     _need(q.shape[1] == n_heads * kv.head_dim, "attn_decode: q width must be n_heads*head_dim")
     _need(out.shape[1] == n_heads * kv.head_dim and out.dtype == q.dtype, "attn_decode: out shape/dtype")
     _attn_common(q, kv, block_table, token_req, positions)
@@ -606,7 +609,7 @@ def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_h
         _ptr(ahead.packed if ahead is not None else None),
         _c_size_t(ahead.chunk_bytes if ahead is not None else 0),
         _c_int(min(ahead_chunks, ahead.n_chunks) if ahead is not None else 0),
-        _c_int(1 if rows_are_requests else 0), _stream(),
+        _c_int(1 if rows_are_requests else 0), _c_int(DT[q.dtype]), _stream(),
     )
     build.check(lib, rc, "attn_decode")
     return out

@@ -104,6 +104,43 @@ def test_gemm_f32(M, N, K, mode):
         assert err < 1e-5 * math.sqrt(K) * 4, (variant, err)
 
 
+@pytest.mark.parametrize("N,K", [(1, 4), (7, 508), (9, 512), (17, 516), (40, 1024), (33, 1028), (100, 1600),
+                                 (24, 2052), (4100, 520), (4097, 1600)])
+def test_gemm_f32_few_rows(N, K):
+    """The kernel for up to 16 rows at the edges of its chunks of 64 columns and of a block's 16
+    features, with 8 and with 12 waves a block (from 4,096 features on there is a block for every
+    compute unit), with K whole and in parts, and that a row's result does not depend on how many
+    other rows the step holds."""
+    k = _k()
+    w = _rand((N, K), torch.float32, 21, 0.1)
+    bias = _rand((N,), torch.float32, 22)
+    a_all = _rand((16, K + 4), torch.float32, 23)[:, :K]  # rows with a stride of their own
+    alone = torch.empty(1, N, dtype=torch.float32, device=DEV)
+    k.linear(alone, a_all[:1], w, bias, variant=3)
+    for M in (1, 2, 3, 4, 5, 8, 9, 16):
+        a = a_all[:M]
+        wide = torch.full((M, N + 3), float("nan"), dtype=torch.float32, device=DEV)
+        out = wide[:, :N]
+        k.linear(out, a, w, bias, variant=3)
+        ref = plain.linear(a.double().cpu(), w.double().cpu(), bias.double().cpu())
+        err = (out.double().cpu() - ref).abs().max().item()
+        assert err < 1e-5 * math.sqrt(K) * 4, (M, err)
+        assert torch.isnan(wide[:, N:]).all()
+        assert torch.equal(out[:1], alone), M
+        k.linear(out, a, w, None, accumulate=True, variant=3)
+        err = (out.double().cpu() - (2 * ref - bias.double().cpu())).abs().max().item()
+        assert err < 2e-5 * math.sqrt(K) * 4, (M, err)
+        # K in parts over the blocks, added up by the second kernel
+        for splits in (2, 3, 7):
+            for mode in ("plain", "gelu", "accumulate"):
+                got = torch.full((M, N), 0.5, dtype=torch.float32, device=DEV)
+                k.linear(got, a, w, bias, gelu=(mode == "gelu"), accumulate=(mode == "accumulate"), variant=3,
+                         splits=splits)
+                want = {"plain": ref, "gelu": plain.gelu_tanh(ref), "accumulate": ref + 0.5}[mode]
+                err = (got.double().cpu() - want).abs().max().item()
+                assert err < 1e-5 * math.sqrt(K) * 4, (M, splits, mode, err)
+
+
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
 @pytest.mark.parametrize("mode", ["plain", "gelu", "accumulate", "f32out"])
 def test_gemm_bf16(M, N, K, mode):
@@ -326,6 +363,45 @@ def test_attn_decode(case, n_splits, n_waves):
     assert err < _attn_tol(torch.bfloat16), err
 
 
+@pytest.mark.parametrize("case", [c for c in ATTN_CASES if c[2] in (16, 32, 64)] + [
+    (8, 2, 16, 16, [700, 15, 16], [1, 1, 3], 0),
+    (3, 1, 64, 4, [63, 64, 1000], [1, 2, 1], 100),
+    (25, 25, 64, 16, [511, 63, 1022, 64, 300], [1, 1, 1, 1, 1], 0),
+])
+@pytest.mark.parametrize("n_splits,n_waves", [(1, 4), (3, 4), (8, 2), (1, 16), (2, 8), (1, 1)])
+def test_attn_decode_float32(case, n_splits, n_waves):
+    """The same kernel over float caches: a key of 16, 32 or 64 floats in 4, 8 or 16 lanes."""
+    k = _k()
+    H, Hkv, hd, ps, ctx, ql, window = case
+    c = PagedCase(torch.float32, H, Hkv, hd, ps, ctx, ql, seed=hd + H + 3, window=window)
+    assert k.attn_decode_takes(torch.float32, c.kv)
+    k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
+    rows = torch.arange(c.T, dtype=torch.int32, device=DEV)
+    part_o = torch.empty(c.T * H * n_splits * hd, dtype=torch.float32, device=DEV)
+    part_ml = torch.empty(c.T * H * n_splits * 2, dtype=torch.float32, device=DEV)
+    out = torch.full((c.T, H * hd), float("nan"), dtype=torch.float32, device=DEV)
+    k.attn_decode(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, c.T, H,
+                  c.scale, window, n_splits, part_o, part_ml, n_waves)
+    err = (out.double().cpu() - c.reference()).abs().max().item()
+    assert err < _attn_tol(torch.float32), err
+
+
+def test_attn_decode_takes_keys_of_64_to_256_bytes():
+    k = _k()
+    for dtype, hd, ps, takes in [(torch.float32, 128, 16, False), (torch.float32, 48, 16, False),
+                                 (torch.float32, 64, 2, False), (torch.float32, 64, 4, True),
+                                 (torch.float32, 16, 16, True), (torch.bfloat16, 16, 16, False),
+                                 (torch.bfloat16, 128, 4, True), (torch.bfloat16, 32, 8, False)]:
+        c = PagedCase(dtype, 2, 2, hd, ps, [5], [1], seed=1)
+        assert k.attn_decode_takes(dtype, c.kv) == takes, (dtype, hd, ps)
+        if not takes:
+            out = torch.empty(1, 2 * hd, dtype=dtype, device=DEV)
+            rows = torch.zeros(1, dtype=torch.int32, device=DEV)
+            with pytest.raises(RuntimeError, match="attn_decode"):
+                k.attn_decode(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, 1, 2,
+                              c.scale)
+
+
 @pytest.mark.parametrize("case", [
     (8, 2, 32, 16, [700, 15, 16, 0], [1, 1, 1, 1], 0),
     (25, 25, 64, 16, [511, 63, 1022, 64, 300], [1, 1, 1, 1, 1], 0),
@@ -400,25 +476,26 @@ def test_attn_prefill_far_key_stands_out():
     assert (out.double().cpu() - c.reference()).abs().max().item() < 2.5e-2
 
 
-def test_attn_decode_far_key_stands_out():
-    """bfloat16, keys streamed into registers: one key among hundreds carries the answer."""
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_attn_decode_far_key_stands_out(dtype):
+    """Keys streamed into registers: one key among hundreds carries the answer."""
     k = _k()
     H, hd, ps = 2, 64, 16
-    for far in (0, 7, 8, 15, 16, 63, 64, 255, 256, 399, 400):
-        c = PagedCase(torch.bfloat16, H, H, hd, ps, [401], [1], seed=far)
+    for far in (0, 3, 4, 7, 8, 15, 16, 63, 64, 255, 256, 399, 400):
+        c = PagedCase(dtype, H, H, hd, ps, [401], [1], seed=far)
         kf = c.k_full[0][far, 1].float()
-        c.q[0, hd:] = (kf * (30.0 / (c.scale * float(kf.norm() ** 2)))).to(torch.bfloat16)
+        c.q[0, hd:] = (kf * (30.0 / (c.scale * float(kf.norm() ** 2)))).to(dtype)
         k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
         rows = torch.zeros(1, dtype=torch.int32, device=DEV)
         for n_splits, n_waves in ((1, 4), (4, 4), (1, 16)):
-            out = torch.empty(1, H * hd, dtype=torch.bfloat16, device=DEV)
+            out = torch.empty(1, H * hd, dtype=dtype, device=DEV)
             po = torch.empty(H * n_splits * hd, dtype=torch.float32, device=DEV)
             pm = torch.empty(H * n_splits * 2, dtype=torch.float32, device=DEV)
             k.attn_decode(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, 1,
                           H, c.scale, 0, n_splits, po, pm, n_waves)
             v_far = c.v_full[0][far, 1].double()
             assert (out[0, hd:].double().cpu() - v_far).abs().max().item() < 0.1, (far, n_splits)
-            assert (out.double().cpu() - c.reference()).abs().max().item() < _attn_tol(torch.bfloat16)
+            assert (out.double().cpu() - c.reference()).abs().max().item() < _attn_tol(dtype)
 
 
 def test_attn_far_key_stands_out():
