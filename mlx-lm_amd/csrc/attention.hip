@@ -18,6 +18,8 @@
 //  * kv_write: scatter this step's keys and values into their pages.
 //  * attn_tile: 16 consecutive queries of one request per block, key tiles
 //    of 64 staged in LDS; any head_dim that is a multiple of 16 up to 256.
+//    Float caches with head_dim 64 or 128 in pages of whole 16 keys take
+//    attn_tile_mfma instead: a wave a tile, v_mfma_f32_16x16x4_f32, no LDS.
 //  * attn_row: one query per block, its keys split over the block's four
 //    waves and over `n_splits` blocks; attn_merge joins the splits.
 #include "common.h"
@@ -255,6 +257,143 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(AttnArgs p) {
       const int d = lane + 64 * j;
       if (d < hd) out[(size_t)(row0 + qi) * p.ldo + h * hd + d] = from_f32<T>(o[i][j] * inv);
     }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// attn_tile_mfma: float storage, head_dim = 64 * NV, page_size a multiple of 16.  Grid
+// (ceil(n_tiles / 4), n_heads), 256 threads; every wave takes a tile of its own and walks its
+// keys 16 at a time (no LDS, no barrier).  v_mfma_f32_16x16x4_f32 computes D = A B for A 16 x 4
+// and B 4 x 16: lane l brings A[l % 16][l / 16] and B[l / 16][l % 16] and gets
+// D[4 * (l / 16) + r][l % 16] in accumulator r.
+//   scores, transposed: S^T[key][query] = sum_d K[key][d] Q[query][d].  The four floats of one
+//     16-byte load go to four instructions; which d an instruction's four slots stand for is
+//     free as long as both operands agree: lane (x = l % 16, g = l / 16) loads columns
+//     16 * t + 4 * g .. + 3 of key x and of query x.  Accumulator r is key 4 * g + r, query x.
+//   softmax runs per query, which is one lane column: the four keys of a lane, then the four
+//     lane groups by two shuffles.
+//   output, transposed: O^T[column][query] = sum_key V[key][column] P[key][query].  The scores'
+//     accumulator r is the second operand as it stands, with slot g standing for key 4 * g + r;
+//     the first is V[key 4 * g + r][columns 4 * x .. + 3], one 16-byte load of a row that the 16
+//     lanes read whole, its four floats going to four accumulators: accumulator r' of the c-th
+//     is column 16 * g + 4 * r' + c, so a lane ends with 16 consecutive columns of its query.
+// Keys of a tile beyond the last one written are read from that one instead (their scores are
+// masked; a page's unwritten rows may hold anything, and 0 x NaN is NaN).
+
+template <int NV>
+__global__ __launch_bounds__(256) void attn_tile_mfma_kernel(AttnArgs p, int n_tiles) {
+  constexpr int HD = 64 * NV;
+  constexpr int NT = 4 * NV;  // 16-byte loads that cover a row of HD floats, per lane group
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = blockIdx.x * 4 + wave;
+  if (tile >= n_tiles) return;
+  const int x = lane & 15, g = lane >> 4;
+  const int row0 = p.items[2 * tile];
+  const int nq = p.items[2 * tile + 1];
+  const int h = blockIdx.y;
+  const int kv_head = h / (p.n_heads / p.n_kv_heads);
+  const int req = p.token_req[row0];
+  const int pos0 = p.positions[row0];
+  const int* table = p.block_table + (size_t)req * p.max_blocks;
+  const float* k_pages = (const float*)p.k_pages;
+  const float* v_pages = (const float*)p.v_pages;
+
+  f32x4_t qv[NT];
+  {
+    const float* qrow = (const float*)p.q + (size_t)(row0 + min(x, nq - 1)) * p.ldq + h * HD + 4 * g;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) qv[t] = *(const f32x4_t*)(qrow + 16 * t) * p.scale;
+  }
+  const int qpos = pos0 + x;
+  const int k_hi = pos0 + nq;  // one past the last key any query of the tile sees
+  const int k_lo = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
+  const size_t head_off = (size_t)kv_head * p.page_size * HD;
+
+  f32x4_t kf[NT], vf[NV][4];
+  auto ask = [&](int kt) {
+    const size_t base = (size_t)table[kt / p.page_size] * p.page_stride + head_off;
+    const int in_page = kt % p.page_size;
+    const float* krow = k_pages + base + (size_t)(in_page + min(x, k_hi - 1 - kt)) * HD + 4 * g;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) kf[t] = *(const f32x4_t*)(krow + 16 * t);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float* vrow = v_pages + base + (size_t)(in_page + min(4 * g + r, k_hi - 1 - kt)) * HD + 4 * x;
+#pragma unroll
+      for (int v = 0; v < NV; ++v) vf[v][r] = *(const f32x4_t*)(vrow + 64 * v);
+    }
+  };
+
+  float m = -INFINITY, l = 0.f;
+  f32x4_t o[NT];
+#pragma unroll
+  for (int i = 0; i < NT; ++i) o[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  int kt = (k_lo / 16) * 16;
+  ask(kt);
+  for (; kt < k_hi; kt += 16) {
+    f32x4_t s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      s = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[t].x, qv[t].x, s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[t].y, qv[t].y, s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[t].z, qv[t].z, s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[t].w, qv[t].w, s, 0, 0, 0);
+    }
+    f32x4_t vc[NV][4];
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) vc[v][r] = vf[v][r];
+    if (kt + 16 < k_hi) ask(kt + 16);  // (uniform) the next tile is on its way during the softmax
+
+    bool ok[4];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int key = kt + 4 * g + r;
+      ok[r] = x < nq && key <= qpos && key >= k_lo && (p.window == 0 || key > qpos - p.window);
+      tmax = fmaxf(tmax, ok[r] ? s[r] : -INFINITY);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+    const float m_new = fmaxf(m, tmax);
+    float alpha = 1.f, sum = 0.f;
+    f32x4_t pr = {0.f, 0.f, 0.f, 0.f};
+    if (m_new != -INFINITY) {
+      alpha = expf(m - m_new);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        pr[r] = ok[r] ? expf(s[r] - m_new) : 0.f;
+        sum += pr[r];
+      }
+    }
+    sum += __shfl_xor(sum, 16, WAVE);
+    sum += __shfl_xor(sum, 32, WAVE);
+    l = l * alpha + sum;
+    m = m_new;
+#pragma unroll
+    for (int i = 0; i < NT; ++i) o[i] *= alpha;
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        o[4 * v + 0] = __builtin_amdgcn_mfma_f32_16x16x4f32(vc[v][r].x, pr[r], o[4 * v + 0], 0, 0, 0);
+        o[4 * v + 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(vc[v][r].y, pr[r], o[4 * v + 1], 0, 0, 0);
+        o[4 * v + 2] = __builtin_amdgcn_mfma_f32_16x16x4f32(vc[v][r].z, pr[r], o[4 * v + 2], 0, 0, 0);
+        o[4 * v + 3] = __builtin_amdgcn_mfma_f32_16x16x4f32(vc[v][r].w, pr[r], o[4 * v + 3], 0, 0, 0);
+      }
+  }
+
+  if (x < nq) {
+    const float inv = 1.0f / l;
+    float* orow = (float*)p.out + (size_t)(row0 + x) * p.ldo + h * HD + 16 * g;
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        *(f32x4_t*)(orow + 64 * v + 4 * r) =
+            f32x4_t{o[4 * v][r], o[4 * v + 1][r], o[4 * v + 2][r], o[4 * v + 3][r]} * inv;
   }
 }
 
@@ -510,6 +649,16 @@ extern "C" int attn_tile(void* out, const void* q, int ldq, int ldo, const void*
                 max_blocks, token_req, positions, tiles, n_heads, n_kv_heads, head_dim, page_size,
                 window, scale, dtype))
     return 1;
+  if (dtype == DT_F32 && (head_dim == 64 || head_dim == 128) && page_size % 16 == 0 && ldq % 4 == 0 &&
+      ldo % 4 == 0 && (((uintptr_t)q | (uintptr_t)out) & 15) == 0) {
+    dim3 grid((n_tiles + 3) / 4, n_heads), block(256);
+    if (head_dim == 64)
+      hipLaunchKernelGGL(attn_tile_mfma_kernel<1>, grid, block, 0, stream, p, n_tiles);
+    else
+      hipLaunchKernelGGL(attn_tile_mfma_kernel<2>, grid, block, 0, stream, p, n_tiles);
+    CHECK_LAUNCH("attn_tile");
+    return 0;
+  }
   const size_t lds = sizeof(float) * ((size_t)QT * head_dim + (size_t)KT * (head_dim + 1) + QT * KT);
   dim3 grid(n_tiles, n_heads), block(256);
   if (dtype == DT_F32) {

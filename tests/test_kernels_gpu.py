@@ -302,6 +302,48 @@ def test_kv_write_and_attn_tile(dtype, case):
     assert err < _attn_tol(dtype), err
 
 
+@pytest.mark.parametrize("case", [
+    # H, Hkv, hd, page, ctx_lens, q_lens, window
+    (3, 3, 64, 16, [0, 100, 17, 64, 15], [90, 1, 2, 17, 16], 0),
+    (6, 2, 64, 48, [3, 0, 250], [20, 70, 1], 0),
+    (5, 1, 128, 32, [130, 0, 31], [1, 130, 34], 0),
+    (4, 2, 64, 16, [0, 300, 90], [200, 1, 5], 37),
+    (2, 2, 128, 16, [0, 300], [150, 33], 16),
+    (2, 1, 64, 32, [500, 0], [40, 300], 1),
+])
+def test_attn_tile_float32_on_matrix_cores(case):
+    """Float caches with head_dim 64 or 128 in pages of whole 16 keys: a wave a tile of 16 queries
+    and 16 keys at a time; tiles that start and end inside a page, short last tiles, windows that
+    end inside a tile of keys, grouped heads.  Free page slots hold NaN."""
+    k = _k()
+    H, Hkv, hd, ps, ctx, ql, window = case
+    c = PagedCase(torch.float32, H, Hkv, hd, ps, ctx, ql, seed=hd + H + ps, window=window)
+    k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
+    tiles = c.tiles()
+    out = torch.full((c.T, H * hd), float("nan"), dtype=torch.float32, device=DEV)
+    k.attn_tile(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, tiles,
+                tiles.shape[0], H, c.scale, window)
+    err = (out.double().cpu() - c.reference()).abs().max().item()
+    assert err < _attn_tol(torch.float32), err
+
+
+def test_attn_tile_float32_far_key_stands_out():
+    """A prompt's last query points at one key among hundreds: a dropped or doubled tile of keys shows."""
+    k = _k()
+    H, hd, ps = 2, 64, 16
+    for far in (0, 3, 4, 15, 16, 17, 255, 256, 383, 384, 399):
+        c = PagedCase(torch.float32, H, H, hd, ps, [0], [400], seed=far)
+        kf = c.k_full[0][far, 1].clone()
+        c.q[399, hd:] = kf * (30.0 / (c.scale * float(kf.norm() ** 2)))
+        k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
+        tiles = c.tiles()
+        out = torch.full((c.T, H * hd), float("nan"), dtype=torch.float32, device=DEV)
+        k.attn_tile(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, tiles,
+                    tiles.shape[0], H, c.scale, 0)
+        assert (out[399, hd:].double().cpu() - c.v_full[0][far, 1].double()).abs().max().item() < 0.1, far
+        assert (out.double().cpu() - c.reference()).abs().max().item() < _attn_tol(torch.float32), far
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_kv_write_from_rows_that_are_not_aligned(dtype):
     """Sources that start in the middle of a 16-byte piece take the element-wise kernel: same pages."""
