@@ -1,5 +1,5 @@
 // Linear layer in true 32-bit: float operands, float products and sums
-// (v_mfma_f32_32x32x2_f32; no reduced-precision matrix mode, no splitting).
+// (v_mfma_f32_16x16x4_f32; no reduced-precision matrix mode, no splitting).
 //   out[m, n] = epilogue( sum_k A[m, k] * W[n, k] + bias[n] )
 // A is [M, K], W is [N, K], both contiguous along k.  Epilogues: plain,
 // tanh-GELU, or accumulate into the residual stream.  Any M, N; K % 4 == 0.
@@ -15,11 +15,6 @@
 #define FLAG_GELU 1
 #define FLAG_ACCUMULATE 2
 
-// Out-of-range loads read a clamped address and are zeroed afterwards with this
-// constant: selecting between an address and a zero kept in a variable turns
-// the load into a flat load through scratch memory.
-#define ZERO4 make_float4(0.f, 0.f, 0.f, 0.f)
-
 struct GemmArgs {
   const float* A;
   const float* W;
@@ -34,9 +29,6 @@ struct GemmArgs {
   float* ws;
 };
 
-#define BK 16
-#define LDS_STRIDE (BK + 1)
-
 // Rows of a tile beyond the matrix read a row inside it (their products are
 // never stored): the row one tile back where there is one, so that they do not
 // all read the matrix's last row at once, which one cache channel would have
@@ -45,129 +37,114 @@ __device__ __forceinline__ int row_inside(int r, int n, int tile) {
   return r < n ? r : (r - tile >= 0 && r - tile < n ? r - tile : n - 1);
 }
 
-// WM x WN waves of 64x64 (BIG) or 32x32 (small) wave tiles
-template <int TM, int TN>  // 32x32 MFMA tiles per wave along m and n
+// Many rows: 2 x 2 waves a block, each with RT x RT tiles of 16 x 16 outputs (a block tile of
+// 128 x 128 or 64 x 64).  v_mfma_f32_16x16x4_f32 computes D = A B for A 16 x 4 and B 4 x 16: lane
+// l brings A[l % 16][l / 16] and B[l / 16][l % 16] and gets D[4 * (l / 16) + r][l % 16] in
+// accumulator r.  Which column of k an instruction's four slots stand for is free as long as both
+// operands agree, so a lane loads 16 bytes, columns 4 * (l / 16) .. + 3 of each 16, of row l % 16
+// of a tile of A and of feature l % 16 of a tile of W, and the four floats go to four
+// instructions.  The operands come straight from memory (the L2s, mostly) in that layout: no LDS
+// and no barrier; the next 32 columns are asked for before this step's products begin.  At 32-bit
+// speed of the matrix cores (a sixteenth of bfloat16's) the L1 carries that easily.
+template <int RT>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs p) {
-  constexpr int BM_ = 2 * TM * 32;
-  constexpr int BN_ = 2 * TN * 32;
-  __shared__ float As[BM_ * LDS_STRIDE];
-  __shared__ float Bs[BN_ * LDS_STRIDE];
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  const int m0 = blockIdx.y * BM_;
-  const int n0 = blockIdx.x * BN_;
-
-  f32x16_t acc[TM][TN];
+  constexpr int WT = 16 * RT;  // a wave's tile
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int x = lane & 15, g = lane >> 4;
+  const int m0 = blockIdx.y * (2 * WT) + (wave >> 1) * WT;
+  const int n0 = blockIdx.x * (2 * WT) + (wave & 1) * WT;
+  // rows and features beyond the matrix read one inside it; their products are never stored
+  const float* arow[RT];
+  const float* wrow[RT];
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-  // a k-block of a tile is BM_ x 16 floats = BM_*4 pieces of 16 bytes
-  constexpr int PA = (BM_ * 4) / 256;
-  constexpr int PB = (BN_ * 4) / 256;
-  float4 ra[PA], rb[PB];
-
-  auto load_global = [&](int k0) {
-#pragma unroll
-    for (int i = 0; i < PA; ++i) {
-      const int c = tid + 256 * i;
-      const int row = c >> 2, gk = k0 + (c & 3) * 4, gm = m0 + row;
-      const float4 t = *(const float4*)(p.A + (size_t)row_inside(gm, p.M, BM_) * p.lda + min(gk, p.K - 4));
-      ra[i] = (gm < p.M && gk < p.K) ? t : ZERO4;
-    }
-#pragma unroll
-    for (int i = 0; i < PB; ++i) {
-      const int c = tid + 256 * i;
-      const int row = c >> 2, gk = k0 + (c & 3) * 4, gn = n0 + row;
-      const float4 t = *(const float4*)(p.W + (size_t)row_inside(gn, p.N, BN_) * p.ldw + min(gk, p.K - 4));
-      rb[i] = (gn < p.N && gk < p.K) ? t : ZERO4;
-    }
-  };
-  auto store_lds = [&]() {
-#pragma unroll
-    for (int i = 0; i < PA; ++i) {
-      const int c = tid + 256 * i;
-      float* d = As + (c >> 2) * LDS_STRIDE + (c & 3) * 4;
-      d[0] = ra[i].x, d[1] = ra[i].y, d[2] = ra[i].z, d[3] = ra[i].w;
-    }
-#pragma unroll
-    for (int i = 0; i < PB; ++i) {
-      const int c = tid + 256 * i;
-      float* d = Bs + (c >> 2) * LDS_STRIDE + (c & 3) * 4;
-      d[0] = rb[i].x, d[1] = rb[i].y, d[2] = rb[i].z, d[3] = rb[i].w;
-    }
-  };
-
-  load_global(0);
-  store_lds();
-  __syncthreads();
-
-  const int frag_row = lane & 31;
-  const int frag_k = lane >> 5;
-
-  for (int k0 = 0; k0 < p.K; k0 += BK) {
-    const bool more = (k0 + BK) < p.K;
-    if (more) load_global(k0 + BK);
-#pragma unroll
-    for (int ks = 0; ks < BK; ks += 2) {
-      float a[TM], b[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-        a[i] = As[(wm * TM * 32 + i * 32 + frag_row) * LDS_STRIDE + ks + frag_k];
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        b[j] = Bs[(wn * TN * 32 + j * 32 + frag_row) * LDS_STRIDE + ks + frag_k];
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
-    }
-    __syncthreads();
-    if (more) {
-      store_lds();
-      __syncthreads();
-    }
+  for (int i = 0; i < RT; ++i) {
+    arow[i] = p.A + (size_t)row_inside(m0 + 16 * i + x, p.M, 2 * WT) * p.lda + 4 * g;
+    wrow[i] = p.W + (size_t)row_inside(n0 + 16 * i + x, p.N, 2 * WT) * p.ldw + 4 * g;
   }
+  f32x4_t acc[RT][RT];
+#pragma unroll
+  for (int i = 0; i < RT; ++i)
+#pragma unroll
+    for (int j = 0; j < RT; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  // Epilogue.  Accumulator r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4,
-  // column lane%32.  What is read (bias, the residual stream to add to) is
-  // read for a whole 32x32 tile before anything is stored: a load that comes
-  // after a store to memory it might alias waits for it, sixteen times over.
+  // a step: 32 columns, two 16-byte pieces a lane of each row and feature (a whole 128-byte line
+  // of each by the lane's group of four).  The rows' values beyond K count as zero.
+  f32x4_t a0[2][RT], w0[2][RT], a1[2][RT], w1[2][RT];
+  auto ask = [&](int k0, f32x4_t (&ad)[2][RT], f32x4_t (&wd)[2][RT]) {
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int n = n0 + wn * TN * 32 + j * 32 + (lane & 31);
-    const int nc = min(n, p.N - 1);
-    const float bias = p.bias ? p.bias[nc] : 0.f;
+    for (int h = 0; h < 2; ++h) {
+      const int col = min(k0 + 16 * h, p.K - 4 - 4 * g);  // (+ 4 * g is in the pointers)
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int mb = m0 + wm * TM * 32 + i * 32 + 4 * (lane >> 5);
-      float v[16];
-      if (p.flags & FLAG_ACCUMULATE) {
+      for (int i = 0; i < RT; ++i) {
+        ad[h][i] = *(const f32x4_t*)(arow[i] + col);
+        wd[h][i] = *(const f32x4_t*)(wrow[i] + col);
+      }
+    }
+  };
+  auto multiply = [&](int k0, const f32x4_t (&as)[2][RT], const f32x4_t (&ws)[2][RT]) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          v[r] = p.out[(size_t)min(mb + 8 * (r >> 2) + (r & 3), p.M - 1) * p.ldo + nc];
+    for (int h = 0; h < 2; ++h) {
+      const float live = k0 + 16 * h + 4 * g < p.K ? 1.f : 0.f;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) v[r] += acc[i][j][r] + bias;
-      } else {
+      for (int i = 0; i < RT; ++i) {
+        const f32x4_t av = as[h][i] * live;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          v[r] = acc[i][j][r] + bias;
-          if (p.flags & FLAG_GELU) v[r] = gelu_tanh(v[r]);
+        for (int j = 0; j < RT; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, ws[h][j].x, acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, ws[h][j].y, acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, ws[h][j].z, acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, ws[h][j].w, acc[i][j], 0, 0, 0);
         }
       }
+    }
+  };
+  // Two steps a round, their operands in two sets of registers by turns.  A step's loads are
+  // issued on one path whether its columns exist or not (beyond K they read inside the matrix),
+  // and stay ahead of the products before them: the wait is then for the older set only.
+  ask(0, a0, w0);
+  for (int k0 = 0; k0 < p.K; k0 += 64) {
+    ask(k0 + 32, a1, w1);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(k0, a0, w0);
+    __builtin_amdgcn_sched_barrier(0);
+    ask(k0 + 64, a0, w0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (k0 + 32 < p.K) multiply(k0 + 32, a1, w1);  // (uniform)
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  // Epilogue.  Accumulator r of tile (i, j): row 16 * i + 4 * g + r, feature 16 * j + x.  What is
+  // read (bias, the residual stream to add to) is read for a row of tiles before anything of it is
+  // stored: a load that comes after a store to memory it might alias waits for it.
+#pragma unroll
+  for (int i = 0; i < RT; ++i) {
+    const int mb = m0 + 16 * i + 4 * g;
+    f32x4_t v[RT];
+#pragma unroll
+    for (int j = 0; j < RT; ++j) {
+      const int n = n0 + 16 * j + x;
+      const int nc = min(n, p.N - 1);
+      const float bias = p.bias ? p.bias[nc] : 0.f;
+      if (p.flags & FLAG_ACCUMULATE) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[j][r] = p.out[(size_t)min(mb + r, p.M - 1) * p.ldo + nc];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[j][r] += acc[i][j][r] + bias;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          v[j][r] = acc[i][j][r] + bias;
+          if (p.flags & FLAG_GELU) v[j][r] = gelu_tanh(v[j][r]);
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < RT; ++j) {
+      const int n = n0 + 16 * j + x;
       if (n >= p.N) continue;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = mb + 8 * (r >> 2) + (r & 3);
-        if (m < p.M) p.out[(size_t)m * p.ldo + n] = v[r];
-      }
+      for (int r = 0; r < 4; ++r)
+        if (mb + r < p.M) p.out[(size_t)(mb + r) * p.ldo + n] = v[j][r];
     }
   }
 }
@@ -326,10 +303,10 @@ extern "C" int gemm_f32(void* out, const void* A, const void* W, const float* bi
   if (variant == 0) variant = M <= 16 ? 3 : (M <= 64 || (size_t)M * N < (size_t)128 * 128 * 128) ? 2 : 1;
   if (variant == 1) {
     dim3 grid((N + 127) / 128, (M + 127) / 128), block(256);
-    hipLaunchKernelGGL((gemm_f32_kernel<2, 2>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL(gemm_f32_kernel<4>, grid, block, 0, stream, p);
   } else if (variant == 2) {
     dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
-    hipLaunchKernelGGL((gemm_f32_kernel<1, 1>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL(gemm_f32_kernel<2>, grid, block, 0, stream, p);
   } else if (variant == 3) {
     if (M > 16) FAIL("gemm_f32: the kernel for few rows takes at most 16, got %d", M);
     // where the blocks are fewer than the compute units, more waves each
