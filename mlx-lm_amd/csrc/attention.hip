@@ -288,12 +288,13 @@ __global__ __launch_bounds__(256) void attn_tile_mfma_kernel(AttnArgs p, int n_t
   const int tile = blockIdx.x * 4 + wave;
   if (tile >= n_tiles) return;
   const int x = lane & 15, g = lane >> 4;
-  const int row0 = p.items[2 * tile];
-  const int nq = p.items[2 * tile + 1];
+  // (the same in every lane: said so, the page numbers below come through scalar loads)
+  const int row0 = __builtin_amdgcn_readfirstlane(p.items[2 * tile]);
+  const int nq = __builtin_amdgcn_readfirstlane(p.items[2 * tile + 1]);
   const int h = blockIdx.y;
   const int kv_head = h / (p.n_heads / p.n_kv_heads);
-  const int req = p.token_req[row0];
-  const int pos0 = p.positions[row0];
+  const int req = __builtin_amdgcn_readfirstlane(p.token_req[row0]);
+  const int pos0 = __builtin_amdgcn_readfirstlane(p.positions[row0]);
   const int* table = p.block_table + (size_t)req * p.max_blocks;
   const float* k_pages = (const float*)p.k_pages;
   const float* v_pages = (const float*)p.v_pages;
@@ -310,8 +311,8 @@ __global__ __launch_bounds__(256) void attn_tile_mfma_kernel(AttnArgs p, int n_t
   const size_t head_off = (size_t)kv_head * p.page_size * HD;
 
   f32x4_t kf[NT], vf[NV][4];
-  auto ask = [&](int kt) {
-    const size_t base = (size_t)table[kt / p.page_size] * p.page_stride + head_off;
+  auto ask = [&](int kt, int page) {
+    const size_t base = (size_t)page * p.page_stride + head_off;
     const int in_page = kt % p.page_size;
     const float* krow = k_pages + base + (size_t)(in_page + min(x, k_hi - 1 - kt)) * HD + 4 * g;
 #pragma unroll
@@ -329,8 +330,11 @@ __global__ __launch_bounds__(256) void attn_tile_mfma_kernel(AttnArgs p, int n_t
 #pragma unroll
   for (int i = 0; i < NT; ++i) o[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
+  // the page of the tile after next is looked up while the next tile's keys are on their way
   int kt = (k_lo / 16) * 16;
-  ask(kt);
+  const int last_block = (k_hi - 1) / p.page_size;
+  ask(kt, table[kt / p.page_size]);
+  int page_next = table[min((kt + 16) / p.page_size, last_block)];
   for (; kt < k_hi; kt += 16) {
     f32x4_t s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -345,7 +349,9 @@ __global__ __launch_bounds__(256) void attn_tile_mfma_kernel(AttnArgs p, int n_t
     for (int v = 0; v < NV; ++v)
 #pragma unroll
       for (int r = 0; r < 4; ++r) vc[v][r] = vf[v][r];
-    if (kt + 16 < k_hi) ask(kt + 16);  // (uniform) the next tile is on its way during the softmax
+    ask(min(kt + 16, ((k_hi - 1) / 16) * 16), page_next);  // the next tile (after the last: the last again)
+    page_next = table[min((kt + 32) / p.page_size, last_block)];
+    __builtin_amdgcn_sched_barrier(0);  // (the loads stay here, ahead of the softmax and the second products)
 
     bool ok[4];
     float tmax = -INFINITY;
