@@ -145,6 +145,7 @@ using Tile256 = TileShape<2, 4, 4, 2, 4, 1>;
 using Tile256x192 = TileShape<4, 2, 2, 3, 4, 1>;
 using Tile64x128 = TileShape<1, 4, 2, 1, 8, 2>;
 using Tile32x128 = TileShape<1, 4, 1, 1, 8, 2>;
+using Tile128x8 = TileShape<2, 4, 2, 1, 8, 1>;  // the same tile with eight waves, for a block that has its CU alone
 
 // Pipeline: LDS holds two k-blocks; registers hold two more on their way.  In
 // iteration i the loads of k-block i+2 are issued and k-block i is multiplied
@@ -787,6 +788,10 @@ extern "C" int gemm_bf16_scatter(void* out, const void* A, const void* W, const 
     else {
       const double c1 = cost_128(M, N), c3 = cost_256(M, N), c4 = cost_256x192(M, N);
       variant = c4 < c3 && c4 < c1 ? 4 : c3 < c1 ? 3 : 1;
+      // No more tiles of 128 x 128 than CUs: a block alone on its CU hides more of its waits with eight
+      // waves of 64 x 32 than with four of 64 x 64 (2,048 rows to 1,600 features: 24.0 us against 26.4 at
+      // K = 1,600, 65.1 against 67.6 at 6,400; with two blocks a CU the four waves are level or ahead).
+      if (variant == 1 && n_splits == 1 && busiest_die<Tile128>(M, N) <= n_compute_units() / N_DIES) variant = 7;
     }
   }
   if (variant == 2) {
@@ -801,6 +806,8 @@ extern "C" int gemm_bf16_scatter(void* out, const void* A, const void* W, const 
       hipLaunchKernelGGL(gemm_bf16_skinny_kernel<3>, grid, block, 0, stream, p);
     else
       hipLaunchKernelGGL(gemm_bf16_skinny_kernel<4>, grid, block, 0, stream, p);
+  } else if (variant == 7) {
+    launch_tiles<Tile128x8>(p, stream);
   } else if (variant == 1 || variant == 3 || variant == 4 || variant == 5 || variant == 6) {
     if (variant == 1)
       launch_tiles<Tile128>(p, stream);

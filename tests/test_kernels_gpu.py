@@ -149,7 +149,7 @@ def test_gemm_bf16(M, N, K, mode):
     w = _rand((N, K), torch.bfloat16, 11, 0.1)
     bias = _rand((N,), torch.float32, 12)
     ref = plain.linear(a.double().cpu(), w.double().cpu(), bias.double().cpu())
-    variants = (1, 2, 3, 4, 5, 6) if M <= 64 else (1, 3, 4, 5, 6)  # tiles of 128 x 128, skinny, 256 x 256, 256 x 192, 64 x 128, 32 x 128
+    variants = (1, 2, 3, 4, 5, 6, 7) if M <= 64 else (1, 3, 4, 5, 6, 7)  # tiles of 128 x 128, skinny, 256 x 256, 256 x 192, 64 x 128, 32 x 128, 128 x 128 with eight waves
     for variant in variants:
         if mode == "accumulate":
             out = _rand((M, N), torch.float32, 13)
@@ -830,7 +830,7 @@ def test_gemm_bf16_reads_weights_kept_in_packed_order_only(M, N, K):
     packed = k.PackedWeight(w.clone(), keep_rows=False)
     assert packed.w is None and not packed.c.w
     ref = plain.linear(a.double().cpu(), w.double().cpu(), bias.double().cpu())
-    variants = [(v, None) for v in ((1, 2, 3, 4, 5, 6) if M <= 64 else (1, 3, 4, 5, 6))]
+    variants = [(v, None) for v in ((1, 2, 3, 4, 5, 6, 7) if M <= 64 else (1, 3, 4, 5, 6, 7))]
     if M > 16 and K >= 192:
         variants += [(1, 3), (5, 2), (6, 3), (0, 2)]  # K in parts
     variants.append((0, None))  # the library's own choice
@@ -1165,7 +1165,7 @@ def test_projection_scatters_keys_and_values(M, dtype, splits):
         assert torch.isnan(pool[page, 0, :, row + 1 :].float()).all()
 
 
-@pytest.mark.parametrize("variant", [0, 1, 3, 4, 5, 6])
+@pytest.mark.parametrize("variant", [0, 1, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("packed", [False, True])
 def test_tile_products_scatter_keys_and_values_themselves(variant, packed):
     """The many-row product writes keys and values into their pages from its own epilogue (every tile
