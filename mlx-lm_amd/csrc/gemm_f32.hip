@@ -1,5 +1,6 @@
 // Linear layer in true 32-bit: float operands, float products and sums
-// (v_mfma_f32_16x16x4_f32; no reduced-precision matrix mode, no splitting).
+// (v_mfma_f32_16x16x4_f32; no reduced-precision matrix mode, no float cut
+// into shorter pieces).
 //   out[m, n] = epilogue( sum_k A[m, k] * W[n, k] + bias[n] )
 // A is [M, K], W is [N, K], both contiguous along k.  Epilogues: plain,
 // tanh-GELU, or accumulate into the residual stream.  Any M, N; K % 4 == 0.
@@ -9,7 +10,8 @@
 // Up to 16 rows (decode steps) take a kernel of their own, which streams W
 // once through v_mfma_f32_16x16x4_f32, 16 features a block: a 64 x 64 tile
 // would spend its time on rows that are not there and leave most compute units
-// without a block.
+// without a block.  Where 16 features a block still give fewer blocks than
+// units, K goes in parts and a second kernel (the caller's) adds them up.
 #include "common.h"
 
 #define FLAG_GELU 1
