@@ -24,6 +24,7 @@ DEFINE_LAST_ERROR(mlxlm_last_error)
 #define GEMM_OUT_F32 4
 #define GEMM_KV 8
 #define DECODE_MAX_ROWS 16
+#define F32_FEW_ROWS 64  // rows that the 32-bit product's streaming kernel takes
 #define ROWS_MAX_ROWS 48  // up to here the kernel for 17 to 48 rows
 #define ATTN_ROW_MAX_HEAD_DIM 144
 #define READ_AHEAD_BYTES_PER_CU (160 * 1024)  // what an idle CU reads while decode attention runs
@@ -391,7 +392,7 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
     // Few rows of a narrow matrix give the kernel for them fewer blocks than there are compute
     // units: K goes in parts then, and the same second kernels add them up as for bfloat16.
     int n_splits = 1;
-    if ((variant == 0 || variant == 3) && M <= DECODE_MAX_ROWS) {
+    if ((variant == 0 || variant == 3) && M <= F32_FEW_ROWS) {
       if (splits == 0)
         QUERY(k_gemm_f32_splits, n_splits, M, N, K, ctx->force_splits);
       else

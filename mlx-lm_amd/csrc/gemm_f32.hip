@@ -7,7 +7,7 @@
 // The 32-bit twin of gemm_bf16.hip; replaces the same nn.Linear calls
 // (mlx_lm/models/gpt2.py:41-42,52,68,76-80,167).
 //
-// Up to 16 rows (decode steps) take a kernel of their own, which streams W
+// Up to 64 rows (decode steps) take a kernel of their own, which streams W
 // once through v_mfma_f32_16x16x4_f32, 16 features a block: a 64 x 64 tile
 // would spend its time on rows that are not there and leave most compute units
 // without a block.  Where 16 features a block still give fewer blocks than
@@ -154,23 +154,28 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs p) {
 #define SKF_WAVES_FEW 8   // waves a block where the blocks are fewer than the compute units
 #define SKF_WAVES_MANY 4  // and where every unit has a block or more (8: 12.1 us instead of 10.6 for 4,800 features of 1,600)
 #define SKF_MAX_WAVES 8
+#define SKF_MAX_ROWS 64
 #define SKF_SPLIT_FROM 5000000L  // elements of a matrix from which a split of K pays
 #define SKF_CHUNK 64                    // columns of a chunk
 #define SKF_STRIDE (SKF_CHUNK + 4)      // floats between a chunk's rows in LDS: no two of a load's lanes share a bank
 
-// Up to 16 rows.  A block owns 16 features and, where K is split over blockIdx.y, a run of
-// chunks of 64 columns; its waves take the run's chunks in turn, each wave on its own (no
-// barrier inside the loop).  A chunk of the weights comes from memory as 256 contiguous bytes a
-// feature, four features a load, goes through the wave's own piece of LDS and comes back in the
-// layout of v_mfma_f32_16x16x4_f32: lane l holds columns 4 * (l / 16) .. + 3 of each 16 of
-// feature l % 16.  The rows are the other operand, read in that layout from the L2, where they
-// stay.  The next chunk is asked for before this one is multiplied; other waves cover the rest
-// of the wait (a deeper queue was slower: 82 us against 72 for the vocabulary's matrix at 8
-// rows).  The same instructions run whatever the number of rows, so a row's result does not
-// depend on it.
+// Up to 64 rows, in RB blocks of 16.  A block owns 16 features and, where K is split over
+// blockIdx.y, a run of chunks of 64 columns; its waves take the run's chunks in turn, each wave on
+// its own (no barrier inside the loop).  A chunk of the weights comes from memory as 256
+// contiguous bytes a feature, four features a load, goes through the wave's own piece of LDS and
+// comes back in the layout of v_mfma_f32_16x16x4_f32: lane l holds columns 4 * (l / 16) .. + 3 of
+// each 16 of feature l % 16.  The rows are the other operand, read in that layout from the L2,
+// where they stay.  The next chunk is asked for before this one is multiplied; other waves cover
+// the rest of the wait (a deeper queue was slower: 82 us against 72 for the vocabulary's matrix
+// at 8 rows).  The same instructions run for every number of rows that fills the same blocks of
+// 16, and a block of rows is multiplied on its own, so a row's result does not depend on the
+// others.  With four blocks of rows the instructions bound the stream at some 4.8 TB/s.
+template <int RB>
 __global__ __launch_bounds__(64 * SKF_MAX_WAVES) void gemm_f32_skinny_kernel(GemmArgs p) {
   // (native vectors: a struct copied to LDS keeps what was loaded out of registers)
   __shared__ f32x4_t stage[SKF_MAX_WAVES][16 * SKF_STRIDE / 4];
+  static_assert(sizeof(float) * SKF_MAX_WAVES * RB * 256 <= sizeof(f32x4_t) * SKF_MAX_WAVES * (16 * SKF_STRIDE / 4),
+                "the waves' sums fit where the chunks were");
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n_waves = blockDim.x >> 6;
   const int n0 = blockIdx.x * 16;
   const int l16 = lane & 15, kq = lane >> 4;
@@ -178,60 +183,76 @@ __global__ __launch_bounds__(64 * SKF_MAX_WAVES) void gemm_f32_skinny_kernel(Gem
   const float* wsrc[4];  // load i: feature 4 * i + l / 16, columns 4 * (l % 16) .. + 3 of the chunk
 #pragma unroll
   for (int i = 0; i < 4; ++i) wsrc[i] = p.W + (size_t)min(n0 + 4 * i + kq, p.N - 1) * p.ldw;
-  const float* arow = p.A + (size_t)min(l16, p.M - 1) * p.lda;
+  const float* arow[RB];
+#pragma unroll
+  for (int b = 0; b < RB; ++b) arow[b] = p.A + (size_t)min(16 * b + l16, p.M - 1) * p.lda;
   f32x4_t* mine = stage[wave];
   const int n_chunks = (p.K + SKF_CHUNK - 1) / SKF_CHUNK;
   const int per_split = (n_chunks + p.n_splits - 1) / p.n_splits;
   const int c_end = min(n_chunks, (blockIdx.y + 1) * per_split);
 
-  f32x4_t wv[4], av[4];
+  f32x4_t wv[4], av[RB][4];
   // columns beyond K (in the last chunk) and chunks beyond the run (asked for ahead by the wave's
   // last round) are read from inside the matrix; the rows' values beyond K count as zero
   auto ask = [&](int c) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) wv[i] = *(const f32x4_t*)(wsrc[i] + min(c * SKF_CHUNK + 4 * l16, p.K - 4));
 #pragma unroll
-    for (int t = 0; t < 4; ++t) av[t] = *(const f32x4_t*)(arow + min(c * SKF_CHUNK + 16 * t + 4 * kq, p.K - 4));
+    for (int b = 0; b < RB; ++b)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        av[b][t] = *(const f32x4_t*)(arow[b] + min(c * SKF_CHUNK + 16 * t + 4 * kq, p.K - 4));
   };
-  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+  f32x4_t acc[RB];
+#pragma unroll
+  for (int b = 0; b < RB; ++b) acc[b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   int c = blockIdx.y * per_split + wave;
   ask(c);
   for (; c < c_end; c += n_waves) {
-    f32x4_t a[4];
+    f32x4_t a[RB][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) mine[(4 * i + kq) * (SKF_STRIDE / 4) + l16] = wv[i];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const float live = c * SKF_CHUNK + 16 * t + 4 * kq < p.K ? 1.f : 0.f;
-      a[t] = av[t] * live;
+#pragma unroll
+      for (int b = 0; b < RB; ++b) a[b][t] = av[b][t] * live;
     }
     ask(c + n_waves);
     __builtin_amdgcn_wave_barrier();  // (orders the compiler; a wave's LDS accesses run in order)
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const f32x4_t w = mine[l16 * (SKF_STRIDE / 4) + 4 * t + kq];
-      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t].x, w.x, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t].y, w.y, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t].z, w.z, acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t].w, w.w, acc, 0, 0, 0);
+#pragma unroll
+      for (int b = 0; b < RB; ++b) {
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[b][t].x, w.x, acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[b][t].y, w.y, acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[b][t].z, w.z, acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[b][t].w, w.w, acc[b], 0, 0, 0);
+      }
     }
     __builtin_amdgcn_wave_barrier();
   }
-  // accumulator r of lane l: row 4 * (l / 16) + r, feature l % 16.  The waves' sums are added
-  // in the order of the waves, one thread an output.
+  // accumulator r of lane l: row 4 * (l / 16) + r of its block of rows, feature l % 16.  The
+  // waves' sums are added in the order of the waves, one thread an output and block of rows.
   __syncthreads();  // the pieces of LDS are no longer read
-  float* parts = (float*)&stage[0][0];
+  float* parts = (float*)&stage[0][0];  // [wave][block of rows][row][feature]
 #pragma unroll
-  for (int r = 0; r < 4; ++r) parts[(wave * 16 + 4 * kq + r) * 16 + l16] = acc[r];
+  for (int b = 0; b < RB; ++b)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) parts[((wave * RB + b) * 16 + 4 * kq + r) * 16 + l16] = acc[b][r];
   __syncthreads();
   if (tid < 256) {
-    const int m = tid >> 4, n = n0 + (tid & 15);
-    if (m < p.M && n < p.N) {
-      float v = parts[tid];
-      for (int w = 1; w < n_waves; ++w) v += parts[w * 256 + tid];
+    const int n = n0 + (tid & 15);
+#pragma unroll
+    for (int b = 0; b < RB; ++b) {
+      const int m = 16 * b + (tid >> 4);
+      if (m >= p.M || n >= p.N) continue;
+      float v = parts[b * 256 + tid];
+      for (int w = 1; w < n_waves; ++w) v += parts[(w * RB + b) * 256 + tid];
       if (p.n_splits > 1) {
         p.ws[((size_t)blockIdx.y * p.M + m) * p.N + n] = v;  // added up, and finished, by the caller's second kernel
-        return;
+        continue;
       }
       if (p.bias) v += p.bias[n];
       const size_t idx = (size_t)m * p.ldo + n;
@@ -251,7 +272,7 @@ DEFINE_LAST_ERROR(mlxlm_last_error)
 // than the split gains.
 extern "C" int gemm_f32_splits(int M, int N, int K, int force) {
   const int n_chunks = (K + SKF_CHUNK - 1) / SKF_CHUNK;
-  if (M < 1 || M > 16) return 1;
+  if (M < 1 || M > SKF_MAX_ROWS) return 1;
   int want;
   if (force > 0) {
     want = force;
@@ -267,7 +288,7 @@ extern "C" int gemm_f32_splits(int M, int N, int K, int force) {
   return (n_chunks + per - 1) / per;  // no empty part
 }
 
-// variant: 0 = choose, 1 = 128x128 block tile, 2 = 64x64 block tile, 3 = the kernel for up to 16 rows.
+// variant: 0 = choose, 1 = 128x128 block tile, 2 = 64x64 block tile, 3 = the kernel for up to 64 rows.
 // n_splits > 1 (the kernel for few rows only): K in that many parts, whose sums go to
 // ws[part][M][N] (ws_floats floats at least) for sum_partials of gemm_bf16_decode.hip to add up
 // and finish; out is not written then.
@@ -296,13 +317,13 @@ extern "C" int gemm_f32(void* out, const void* A, const void* W, const float* bi
   if (M == 0) return 0;
   if (n_splits < 1) FAIL("gemm_f32: n_splits=%d", n_splits);
   if (n_splits > 1) {
-    if (variant == 0 && M <= 16) variant = 3;
-    if (variant != 3) FAIL("gemm_f32: only the kernel for up to 16 rows takes K in parts");
+    if (variant == 0 && M <= SKF_MAX_ROWS) variant = 3;
+    if (variant != 3) FAIL("gemm_f32: only the kernel for up to %d rows takes K in parts", SKF_MAX_ROWS);
     if (n_splits > (K + SKF_CHUNK - 1) / SKF_CHUNK) FAIL("gemm_f32: %d parts of K=%d", n_splits, K);
     if (!ws || ws_floats < (size_t)n_splits * M * N) FAIL("gemm_f32: the parts' workspace is too small");
     p.n_splits = n_splits, p.ws = ws;
   }
-  if (variant == 0) variant = M <= 16 ? 3 : (M <= 64 || (size_t)M * N < (size_t)128 * 128 * 128) ? 2 : 1;
+  if (variant == 0) variant = M <= SKF_MAX_ROWS ? 3 : (size_t)M * N < (size_t)128 * 128 * 128 ? 2 : 1;
   if (variant == 1) {
     dim3 grid((N + 127) / 128, (M + 127) / 128), block(256);
     hipLaunchKernelGGL(gemm_f32_kernel<4>, grid, block, 0, stream, p);
@@ -310,11 +331,19 @@ extern "C" int gemm_f32(void* out, const void* A, const void* W, const float* bi
     dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
     hipLaunchKernelGGL(gemm_f32_kernel<2>, grid, block, 0, stream, p);
   } else if (variant == 3) {
-    if (M > 16) FAIL("gemm_f32: the kernel for few rows takes at most 16, got %d", M);
+    if (M > SKF_MAX_ROWS) FAIL("gemm_f32: the kernel for few rows takes at most %d, got %d", SKF_MAX_ROWS, M);
     // where the blocks are fewer than the compute units, more waves each
     const int blocks = (N + 15) / 16;
     const int waves = blocks * p.n_splits < n_compute_units() ? SKF_WAVES_FEW : SKF_WAVES_MANY;
-    hipLaunchKernelGGL(gemm_f32_skinny_kernel, dim3(blocks, p.n_splits), dim3(64 * waves), 0, stream, p);
+    const dim3 grid(blocks, p.n_splits), block(64 * waves);
+    if (M <= 16)
+      hipLaunchKernelGGL(gemm_f32_skinny_kernel<1>, grid, block, 0, stream, p);
+    else if (M <= 32)
+      hipLaunchKernelGGL(gemm_f32_skinny_kernel<2>, grid, block, 0, stream, p);
+    else if (M <= 48)
+      hipLaunchKernelGGL(gemm_f32_skinny_kernel<3>, grid, block, 0, stream, p);
+    else
+      hipLaunchKernelGGL(gemm_f32_skinny_kernel<4>, grid, block, 0, stream, p);
   } else {
     FAIL("gemm_f32: unknown variant %d", variant);
   }

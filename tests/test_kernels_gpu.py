@@ -91,7 +91,7 @@ def test_gemm_f32(M, N, K, mode):
     w = _rand((N, K), torch.float32, 11, 0.1)
     bias = _rand((N,), torch.float32, 12)
     ref = plain.linear(a.double().cpu(), w.double().cpu(), bias.double().cpu())
-    for variant in (1, 2, 3) if M <= 16 else (1, 2):  # tiles of 128 and of 64, the kernel for few rows
+    for variant in (1, 2, 3) if M <= 64 else (1, 2):  # tiles of 128 and of 64, the kernel for few rows
         if mode == "accumulate":
             out = _rand((M, N), torch.float32, 13)
             want = out.double().cpu() + ref
@@ -107,17 +107,17 @@ def test_gemm_f32(M, N, K, mode):
 @pytest.mark.parametrize("N,K", [(1, 4), (7, 508), (9, 512), (17, 516), (40, 1024), (33, 1028), (100, 1600),
                                  (24, 2052), (4100, 520), (4097, 1600)])
 def test_gemm_f32_few_rows(N, K):
-    """The kernel for up to 16 rows at the edges of its chunks of 64 columns and of a block's 16
-    features, with 8 and with 12 waves a block (from 4,096 features on there is a block for every
-    compute unit), with K whole and in parts, and that a row's result does not depend on how many
-    other rows the step holds."""
+    """The kernel for up to 64 rows at the edges of its chunks of 64 columns, of a block's 16
+    features and of its blocks of 16 rows, with 8 and with 4 waves a block (from 4,096 features on
+    there is a block for every compute unit), with K whole and in parts, and that a row's result
+    does not depend on how many other rows the step holds."""
     k = _k()
     w = _rand((N, K), torch.float32, 21, 0.1)
     bias = _rand((N,), torch.float32, 22)
-    a_all = _rand((16, K + 4), torch.float32, 23)[:, :K]  # rows with a stride of their own
+    a_all = _rand((64, K + 4), torch.float32, 23)[:, :K]  # rows with a stride of their own
     alone = torch.empty(1, N, dtype=torch.float32, device=DEV)
     k.linear(alone, a_all[:1], w, bias, variant=3)
-    for M in (1, 2, 3, 4, 5, 8, 9, 16):
+    for M in (1, 2, 3, 4, 5, 8, 9, 16, 17, 32, 33, 47, 49, 64):
         a = a_all[:M]
         wide = torch.full((M, N + 3), float("nan"), dtype=torch.float32, device=DEV)
         out = wide[:, :N]
