@@ -682,21 +682,23 @@ struct Attention : Mixer {
     return 0;
   }
 
-  // (n_splits, n_waves) for the decode kernel whose blocks take 2 to 16 waves: few rows get many
-  // waves a block (a tile of 64 keys each); many rows few, each with several tiles.  Splits only
-  // where sixteen waves would take three tiles or more each and the splits' blocks still find a
-  // compute unit each at once.
+  // (n_splits, n_waves) for the decode kernel, whose waves take 32 keys at a time.  Eight waves a
+  // block (four where the rows' blocks alone are more than the CUs, or the keys no more than four
+  // waves' tiles): measured at 1 to 64 rows and contexts of 100 to 7,000, eight were level with or
+  // ahead of sixteen everywhere.  Splits need a second kernel to join them, which costs as much as
+  // a walk of some hundred keys a wave: only where a wave would walk 256 keys or more, as many as
+  // leave it 128, and no more than give every block a compute unit at once.
   void row_work(const EngCtx* ctx, int n_rows, long max_row_context, int* n_splits, int* n_waves) const {
-    const long c = window <= 0 ? max_row_context : (max_row_context < window + 63 ? max_row_context : window + 63);
-    const long tiles = c + 63 < 64 ? 1 : (c + 63) / 64;
+    const long c = window <= 0 ? max_row_context : (max_row_context < window + 31 ? max_row_context : window + 31);
+    const long tiles = c + 31 < 32 ? 1 : (c + 31) / 32;
     const long blocks = n_rows * n_heads < 1 ? 1 : (long)n_rows * n_heads;
-    const long want = (8L * ctx->n_compute_units + blocks - 1) / blocks;  // eight waves a CU in all
-    int nw = 2;
-    while (nw < 16 && nw < want && nw < tiles) nw *= 2;
-    const long rounds = (tiles + nw - 1) / nw;
+    int nw = blocks > ctx->n_compute_units ? 4 : 8;
+    const int fewest = head_dim > 128 ? 4 : 2;  // (the block's threads write a column of the head each)
+    while (nw > fewest && nw / 2 >= tiles) nw /= 2;
+    const long keys_a_wave = c / nw;
     long ns = 1;
-    if (rounds >= 3) {
-      ns = rounds;
+    if (keys_a_wave >= 256) {
+      ns = keys_a_wave / 128;
       if (ctx->n_compute_units / blocks < ns) ns = ctx->n_compute_units / blocks;
       if (ns > 64) ns = 64;
       if (ns < 1) ns = 1;
