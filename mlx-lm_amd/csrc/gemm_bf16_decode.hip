@@ -177,7 +177,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArg
   // weight fragments are not even zeroed when they lie outside the matrix:
   // every address is pulled into range, and what such a fragment meets is a
   // zero activation (k >= K) or an output that is never stored (n >= N).  So
-  // nothing has to wait for a weight before the MFMA that uses it.
+  // nothing has to wait for a weight before the MFMA that uses it.  (Whole
+  // k-blocks beyond the last are another matter: a wave skips them.)
   auto load_pass = [&](Frag (&w)[UU][2], int pass) {
     if (wave + NW * pass * UU >= n_chunks) return;  // the whole pass lies beyond K (uniform)
 #pragma unroll
