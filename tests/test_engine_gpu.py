@@ -164,12 +164,14 @@ def test_mixed_batches_with_few_pages(folders, dtype, name, sharp):
         _close(torch.cat(got[rid]), want, dtype, f"mixed, request {rid}")
 
 
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
 @pytest.mark.parametrize("name,sharp", [("B", 8.0), ("C", 0.0)])
 @pytest.mark.parametrize("use_graphs", [False, True])
-def test_split_sums_in_the_engine(folders, monkeypatch, name, sharp, use_graphs):
+def test_split_sums_in_the_engine(folders, monkeypatch, name, sharp, use_graphs, dtype):
     """Projections that split K (forced here: tiny layers would not) leave their sums into the
     residual stream pending between the parts; the next norm adds them.  Mixed batches and
-    recorded decode steps, against the plain implementation."""
+    recorded decode steps, against the plain implementation.  (In float32 only the kernel for up to
+    64 rows splits K.)"""
     from mlx_lm_amd.engine import Engine, StepEntry
     from mlx_lm_amd.ops import kernels
     from mlx_lm_amd.utils import load_model
@@ -179,8 +181,8 @@ def test_split_sums_in_the_engine(folders, monkeypatch, name, sharp, use_graphs)
     P = config["n_positions"]
     lengths = [min(P, n) for n in (100, 37, 128, 64, 90, 17)]
     tokens, steps = helpers.mixed_trace(config, seed=5, lengths=lengths)
-    model, _ = load_model(folder, dtype="bfloat16")
-    eng = Engine(model, dtype="bfloat16", page_size=16, n_pages=helpers.held(lengths, 4) // 16, max_requests=8,
+    model, _ = load_model(folder, dtype=dtype)
+    eng = Engine(model, dtype=dtype, page_size=16, n_pages=helpers.held(lengths, 4) // 16, max_requests=8,
                  use_graphs=use_graphs)
     got = {rid: [] for rid in tokens}
     for s in steps:
@@ -202,11 +204,11 @@ def test_split_sums_in_the_engine(folders, monkeypatch, name, sharp, use_graphs)
     before = eng.stats.settle_plain
     got["extra"] = [eng.step([StepEntry("extra", extra, [10])]).clone()]
     assert eng.stats.settle_plain == before + 1
-    want = _plain_logits(weights, config, extra, "bfloat16")[10:]
-    _close(got.pop("extra")[0], want, "bfloat16", "split sums, gathered rows")
+    want = _plain_logits(weights, config, extra, dtype)[10:]
+    _close(got.pop("extra")[0], want, dtype, "split sums, gathered rows")
     for rid, toks in tokens.items():
-        want = _plain_logits(weights, config, toks, "bfloat16")
-        _close(torch.cat(got[rid]), want, "bfloat16", f"split sums, request {rid}")
+        want = _plain_logits(weights, config, toks, dtype)
+        _close(torch.cat(got[rid]), want, dtype, f"split sums, request {rid}")
 
 
 @pytest.mark.parametrize("page_size", [16, 32, 64])
