@@ -52,9 +52,10 @@ struct DecodeArgs {
 
 #define MAX_WAVES 16
 
-// keys a wave takes at a time (with 64, a context of 530 gave nine of a block's waves a tile and
-// the others none: 9.3 us for 8 rows of 25 heads against 7.3 with 32)
-#define TILE 32
+// Keys a wave takes at a time: 32 or 64, the caller's choice.  With 64, a context of 530 gave nine
+// of a block's waves a tile and the others none: 9.3 us for 8 rows of 25 heads against 7.3 with 32.
+// Where rows x heads are several blocks a CU and the walk is long, the larger tile's sixteen
+// loads a lane in flight are ahead (32 rows at contexts of 512 to 1,022: 2 % of the step).
 
 // 16 bytes of a row as floats, and a float back as an element
 __device__ __forceinline__ void unpack(const uint4& v, float (&f)[8], const uint16_t*) {
@@ -70,8 +71,8 @@ __device__ __forceinline__ void unpack(const uint4& v, float (&f)[4], const floa
 __device__ __forceinline__ void put(uint16_t* at, float v) { *at = f32_to_bf16_bits(v); }
 __device__ __forceinline__ void put(float* at, float v) { *at = v; }
 
-// T: uint16_t (bfloat16 bits) or float.  CPK lanes per key: head_dim = EPL * CPK
-template <typename T, int CPK>
+// T: uint16_t (bfloat16 bits) or float.  CPK lanes per key: head_dim = EPL * CPK.  TILE: keys a wave at a time.
+template <typename T, int CPK, int TILE>
 __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void attn_decode_kernel(DecodeArgs p) {
   constexpr int EPL = 16 / sizeof(T);  // elements a lane holds of a key
   constexpr int HD = EPL * CPK;
@@ -262,7 +263,7 @@ __global__ void attn_decode_merge_kernel(DecodeArgs p) {
 DEFINE_LAST_ERROR(mlxlm_last_error)
 
 template <typename T, int CPK>
-static void launch(const DecodeArgs& p, int n_rows, int n_waves, hipStream_t stream) {
+static void launch(const DecodeArgs& p, int n_rows, int n_waves, int key_tile, hipStream_t stream) {
   // reading blocks for the CUs that the rows leave idle, if there are eight or more
   int extra_y = 0;
   if (p.ahead && p.ahead_chunks > 0) {
@@ -270,7 +271,11 @@ static void launch(const DecodeArgs& p, int n_rows, int n_waves, hipStream_t str
     if (extra_y * n_rows < 8) extra_y = 0;
   }
   const size_t lds = p.table_in_lds ? (size_t)p.max_blocks * sizeof(int) : 0;
-  hipLaunchKernelGGL((attn_decode_kernel<T, CPK>), dim3(n_rows, p.n_heads + extra_y, p.n_splits), dim3(64 * n_waves), lds, stream, p);
+  const dim3 grid(n_rows, p.n_heads + extra_y, p.n_splits), block(64 * n_waves);
+  if (key_tile == 64)
+    hipLaunchKernelGGL((attn_decode_kernel<T, CPK, 64>), grid, block, lds, stream, p);
+  else
+    hipLaunchKernelGGL((attn_decode_kernel<T, CPK, 32>), grid, block, lds, stream, p);
   if (p.n_splits > 1)
     hipLaunchKernelGGL((attn_decode_merge_kernel<T, CPK>), dim3(n_rows, p.n_heads), dim3(16 / sizeof(T) * CPK), 0, stream, p);
 }
@@ -279,14 +284,18 @@ static void launch(const DecodeArgs& p, int n_rows, int n_waves, hipStream_t str
 // item i of `rows` is row i and belongs to request i (every request of the step brings one token),
 // which saves the kernel two trips to memory.  dtype DT_BF16 with head_dim 32, 64 or 128, DT_F32
 // with 16, 32 or 64, and pages that hold whole loads (page_size a multiple of the keys in 1 KB).
+// key_tile: 32 or 64 keys a wave at a time (0: 32).
 extern "C" int attn_decode_rows(void* out, const void* q, int ldq, int ldo, const void* k_pages,
                                 const void* v_pages, size_t page_stride, const int* block_table,
                                 int max_blocks, const int* token_req, const int* positions,
                                 const int* rows, int n_rows, int n_heads, int n_kv_heads, int head_dim,
                                 int page_size, int window, float scale, int n_splits, float* part_o,
                                 float* part_ml, int n_waves, const void* ahead, size_t ahead_chunk_bytes,
-                                int ahead_chunks, int rows_are_requests, int dtype, hipStream_t stream) {
+                                int ahead_chunks, int rows_are_requests, int dtype, int key_tile,
+                                hipStream_t stream) {
   if (n_rows <= 0) return 0;
+  if (key_tile == 0) key_tile = 32;
+  if (key_tile != 32 && key_tile != 64) FAIL("attn_decode: a wave takes 32 or 64 keys at a time, not %d", key_tile);
   if (dtype != DT_F32 && dtype != DT_BF16) FAIL("attn_decode: unknown dtype code %d", dtype);
   const int epl = dtype == DT_F32 ? 4 : 8;  // elements in a lane's 16 bytes
   if (n_waves < 1 || n_waves > MAX_WAVES) FAIL("attn_decode: %d waves a block, must be 1 to %d", n_waves, MAX_WAVES);
@@ -324,18 +333,18 @@ extern "C" int attn_decode_rows(void* out, const void* q, int ldq, int ldo, cons
   p.table_in_lds = max_blocks > 0 && max_blocks <= 8192;  // (32 KB of LDS at most)
   if (dtype == DT_BF16) {
     if (cpk == 4)
-      launch<uint16_t, 4>(p, n_rows, n_waves, stream);
+      launch<uint16_t, 4>(p, n_rows, n_waves, key_tile, stream);
     else if (cpk == 8)
-      launch<uint16_t, 8>(p, n_rows, n_waves, stream);
+      launch<uint16_t, 8>(p, n_rows, n_waves, key_tile, stream);
     else
-      launch<uint16_t, 16>(p, n_rows, n_waves, stream);
+      launch<uint16_t, 16>(p, n_rows, n_waves, key_tile, stream);
   } else {
     if (cpk == 4)
-      launch<float, 4>(p, n_rows, n_waves, stream);
+      launch<float, 4>(p, n_rows, n_waves, key_tile, stream);
     else if (cpk == 8)
-      launch<float, 8>(p, n_rows, n_waves, stream);
+      launch<float, 8>(p, n_rows, n_waves, key_tile, stream);
     else
-      launch<float, 16>(p, n_rows, n_waves, stream);
+      launch<float, 16>(p, n_rows, n_waves, key_tile, stream);
   }
   CHECK_LAUNCH("attn_decode");
   return 0;

@@ -92,7 +92,7 @@ typedef int (*fn_attn_row)(void*, const void*, int, int, const void*, const void
                            float*, float*, int, hipStream_t);
 typedef int (*fn_attn_decode)(void*, const void*, int, int, const void*, const void*, size_t, const int*, int,
                               const int*, const int*, const int*, int, int, int, int, int, int, float, int,
-                              float*, float*, int, const void*, size_t, int, int, int, hipStream_t);
+                              float*, float*, int, const void*, size_t, int, int, int, int, hipStream_t);
 typedef int (*fn_attn_prefill)(void*, const void*, int, int, const void*, const void*, size_t, const int*,
                                int, const int*, const int*, const int*, int, int, int, int, int, int, float,
                                hipStream_t);
@@ -682,13 +682,16 @@ struct Attention : Mixer {
     return 0;
   }
 
-  // (n_splits, n_waves) for the decode kernel, whose waves take 32 keys at a time.  Eight waves a
-  // block (four where the rows' blocks alone are more than the CUs, or the keys no more than four
-  // waves' tiles): measured at 1 to 64 rows and contexts of 100 to 7,000, eight were level with or
-  // ahead of sixteen everywhere.  Splits need a second kernel to join them, which costs as much as
-  // a walk of some hundred keys a wave: only where a wave would walk 256 keys or more, as many as
-  // leave it 128, and no more than give every block a compute unit at once.
-  void row_work(const EngCtx* ctx, int n_rows, long max_row_context, int* n_splits, int* n_waves) const {
+  // (n_splits, n_waves, keys a wave at a time) for the decode kernel.  Eight waves a block (four
+  // where the rows' blocks alone are more than the CUs, or the keys no more than four waves'
+  // tiles): measured at 1 to 64 rows and contexts of 100 to 7,000, eight were level with or ahead
+  // of sixteen everywhere.  Tiles of 32 keys, so that every wave has some at a context of a few
+  // hundred; of 64 where the blocks are more than the CUs and the context is 640 or more (the
+  // larger tile keeps more loads in flight).  Splits need a second kernel to join them, which
+  // costs as much as a walk of some hundred keys a wave: only where a wave would walk 256 keys or
+  // more, as many as leave it 128, and no more than give every block a compute unit at once.
+  void row_work(const EngCtx* ctx, int n_rows, long max_row_context, int* n_splits, int* n_waves,
+                int* key_tile) const {
     const long c = window <= 0 ? max_row_context : (max_row_context < window + 31 ? max_row_context : window + 31);
     const long tiles = c + 31 < 32 ? 1 : (c + 31) / 32;
     const long blocks = n_rows * n_heads < 1 ? 1 : (long)n_rows * n_heads;
@@ -703,7 +706,15 @@ struct Attention : Mixer {
       if (ns > 64) ns = 64;
       if (ns < 1) ns = 1;
     }
-    *n_splits = (int)ns, *n_waves = nw;
+    *n_splits = (int)ns, *n_waves = nw, *key_tile = 32;
+    if (blocks > ctx->n_compute_units && c >= 640) {
+      // many rows and a long walk: tiles of 64 keys, and as many waves a block as make eight a CU
+      // (32 rows: four; 64 rows: two.  With four at 64 rows the step took 5.92 ms instead of 5.76.)
+      const long want = (8L * ctx->n_compute_units + blocks - 1) / blocks;
+      nw = fewest;
+      while (nw < 8 && nw < want) nw *= 2;
+      *n_waves = nw, *key_tile = 64;
+    }
   }
 
   // How many ways to split a row's keys so that the general row kernel's launch fills the GPU.
@@ -754,9 +765,9 @@ struct Attention : Mixer {
       const int key_bytes = head_dim * (bf16 ? 2 : 4);
       const bool fast = (key_bytes == 64 || key_bytes == 128 || key_bytes == 256) &&
                         kv.page_size % (1024 / key_bytes) == 0;
-      int n_splits = 1, n_waves = 4;
+      int n_splits = 1, n_waves = 4, key_tile = 32;
       if (fast)
-        row_work(ctx, n_rows, max_row_context, &n_splits, &n_waves);
+        row_work(ctx, n_rows, max_row_context, &n_splits, &n_waves, &key_tile);
       else
         n_splits = row_splits(ctx, n_rows, max_row_context);
       if (ctx->stats && n_splits > ctx->stats->key_splits_most) ctx->stats->key_splits_most = n_splits;
@@ -786,7 +797,7 @@ struct Attention : Mixer {
                kv.max_blocks, kv.token_req, kv.positions, rows, n_rows, n_heads, n_kv_heads, head_dim,
                kv.page_size, window, scale, n_splits, (float*)part_o.p, (float*)part_ml.p, n_waves,
                ahead ? ahead->packed : nullptr, ahead ? ahead->chunk_bytes : (size_t)0, chunks, rows_are_requests,
-               q.dtype, ctx->stream);
+               q.dtype, key_tile, ctx->stream);
       } else {
         KERNEL(k_attn_row, ctx, out.p, q.p, q.ld, out.ld, kv.k, kv.v, kv.page_stride, kv.block_table,
                kv.max_blocks, kv.token_req, kv.positions, rows, n_rows, n_heads, n_kv_heads, head_dim,

@@ -398,11 +398,13 @@ def test_attn_decode(case, n_splits, n_waves):
     rows = torch.arange(c.T, dtype=torch.int32, device=DEV)
     part_o = torch.empty(c.T * H * n_splits * hd, dtype=torch.float32, device=DEV)
     part_ml = torch.empty(c.T * H * n_splits * 2, dtype=torch.float32, device=DEV)
-    out = torch.full((c.T, H * hd), float("nan")).to(torch.bfloat16).to(DEV)
-    k.attn_decode(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, c.T, H,
-                  c.scale, window, n_splits, part_o, part_ml, n_waves)
-    err = (out.double().cpu() - c.reference()).abs().max().item()
-    assert err < _attn_tol(torch.bfloat16), err
+    want = c.reference()
+    for key_tile in (32, 64):  # keys a wave takes at a time
+        out = torch.full((c.T, H * hd), float("nan")).to(torch.bfloat16).to(DEV)
+        k.attn_decode(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, c.T, H,
+                      c.scale, window, n_splits, part_o, part_ml, n_waves, key_tile=key_tile)
+        err = (out.double().cpu() - want).abs().max().item()
+        assert err < _attn_tol(torch.bfloat16), (key_tile, err)
 
 
 @pytest.mark.parametrize("case", [c for c in ATTN_CASES if c[2] in (16, 32, 64)] + [
@@ -421,11 +423,13 @@ def test_attn_decode_float32(case, n_splits, n_waves):
     rows = torch.arange(c.T, dtype=torch.int32, device=DEV)
     part_o = torch.empty(c.T * H * n_splits * hd, dtype=torch.float32, device=DEV)
     part_ml = torch.empty(c.T * H * n_splits * 2, dtype=torch.float32, device=DEV)
-    out = torch.full((c.T, H * hd), float("nan"), dtype=torch.float32, device=DEV)
-    k.attn_decode(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, c.T, H,
-                  c.scale, window, n_splits, part_o, part_ml, n_waves)
-    err = (out.double().cpu() - c.reference()).abs().max().item()
-    assert err < _attn_tol(torch.float32), err
+    want = c.reference()
+    for key_tile in (32, 64):
+        out = torch.full((c.T, H * hd), float("nan"), dtype=torch.float32, device=DEV)
+        k.attn_decode(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, c.T, H,
+                      c.scale, window, n_splits, part_o, part_ml, n_waves, key_tile=key_tile)
+        err = (out.double().cpu() - want).abs().max().item()
+        assert err < _attn_tol(torch.float32), (key_tile, err)
 
 
 def test_attn_decode_takes_keys_of_64_to_256_bytes():
@@ -529,12 +533,12 @@ def test_attn_decode_far_key_stands_out(dtype):
         c.q[0, hd:] = (kf * (30.0 / (c.scale * float(kf.norm() ** 2)))).to(dtype)
         k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
         rows = torch.zeros(1, dtype=torch.int32, device=DEV)
-        for n_splits, n_waves in ((1, 4), (4, 4), (1, 16)):
+        for n_splits, n_waves, key_tile in ((1, 4, 32), (4, 4, 32), (1, 16, 32), (1, 4, 64), (3, 8, 64)):
             out = torch.empty(1, H * hd, dtype=dtype, device=DEV)
             po = torch.empty(H * n_splits * hd, dtype=torch.float32, device=DEV)
             pm = torch.empty(H * n_splits * 2, dtype=torch.float32, device=DEV)
             k.attn_decode(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, 1,
-                          H, c.scale, 0, n_splits, po, pm, n_waves)
+                          H, c.scale, 0, n_splits, po, pm, n_waves, key_tile=key_tile)
             v_far = c.v_full[0][far, 1].double()
             assert (out[0, hd:].double().cpu() - v_far).abs().max().item() < 0.1, (far, n_splits)
             assert (out.double().cpu() - c.reference()).abs().max().item() < _attn_tol(dtype)
