@@ -9,7 +9,7 @@
 // (mlx_lm/models/base.py:132-139 with mask=None, mlx_lm/generate.py:1414).
 //
 // Work split: grid (rows, heads, n_splits), 1 to 16 waves a block.  The row's
-// keys [k_lo, k_hi) are cut into tiles of 32; the tiles are dealt to the splits
+// keys [k_lo, k_hi) are cut into tiles of 32 or 64; the tiles are dealt to the splits
 // in runs and, inside a block, to the waves in turn.  With few rows in a step
 // it is the many waves of a block, joined through LDS, that give the GPU
 // enough to do: splits need a second kernel to join them, which at these sizes
