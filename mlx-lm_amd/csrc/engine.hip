@@ -686,8 +686,10 @@ struct Attention : Mixer {
   // where the rows' blocks alone are more than the CUs, or the keys no more than four waves'
   // tiles): measured at 1 to 64 rows and contexts of 100 to 7,000, eight were level with or ahead
   // of sixteen everywhere.  Tiles of 32 keys, so that every wave has some at a context of a few
-  // hundred; of 64 where the blocks are more than the CUs and the context is 640 or more (the
-  // larger tile keeps more loads in flight).  Splits need a second kernel to join them, which
+  // hundred; of 64 where the blocks are more than three a CU and the context is 640 or more (the
+  // larger tile keeps more loads in flight; a recorded step plans for the model's positions: at
+  // 1,024 of them, 12 to 30 rows were 1 to 3 % faster with 32 over contexts of 512 to 1,022, 32
+  // rows 2 % faster with 64).  Splits need a second kernel to join them, which
   // costs as much as a walk of some hundred keys a wave: only where a wave would walk 256 keys or
   // more, as many as leave it 128, and no more than give every block a compute unit at once.
   void row_work(const EngCtx* ctx, int n_rows, long max_row_context, int* n_splits, int* n_waves,
@@ -707,7 +709,7 @@ struct Attention : Mixer {
       if (ns < 1) ns = 1;
     }
     *n_splits = (int)ns, *n_waves = nw, *key_tile = 32;
-    if (blocks > ctx->n_compute_units && c >= 640) {
+    if (blocks > 3 * ctx->n_compute_units && c >= 640) {
       // many rows and a long walk: tiles of 64 keys, and as many waves a block as make eight a CU
       // (32 rows: four; 64 rows: two.  With four at 64 rows the step took 5.92 ms instead of 5.76.)
       const long want = (8L * ctx->n_compute_units + blocks - 1) / blocks;
