@@ -339,6 +339,7 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
     if (n_splits > 1) {
       const size_t most = ws ? ws_floats / ((size_t)M * N) : 0;
       if ((size_t)n_splits > most) n_splits = (int)most;
+      if (n_splits > 1) n_splits = split_count((K + 63) / 64, n_splits);  // (no part left empty by the cut)
       if (n_splits < 1) n_splits = 1;
     }
     int takes = 0;

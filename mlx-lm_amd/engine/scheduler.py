@@ -35,12 +35,21 @@ taken part in one step too many, whose result is dropped.  What can be known
 (``max_tokens``, the model's positions) is: such a request is left out.
 """
 
+import itertools
 import time
 from collections import deque
 from dataclasses import dataclass, field
 from typing import Any, Callable, List, Optional, Sequence
 
+from ..cache.manager import OutOfPages, OutOfSlots
 from .step import StepEntry
+
+# Every scheduler of the process has a number of its own.  An engine (and its cache manager) may
+# serve several schedulers at once -- the reference's ``BatchGenerator`` owns its caches and its
+# uid counter (mlx_lm/generate.py:1596-1607,1712-1731), so any number of them are live over one
+# model -- and each of them numbers its requests as it likes; the engine knows a request as
+# ``(scheduler's number, request_id)``.
+_scheduler_numbers = itertools.count()
 
 
 @dataclass(eq=False)
@@ -68,6 +77,9 @@ class Request:
     # row of the sampling call in flight that holds this request's newest token (not yet in ``generated``)
     inflight_row: Optional[int] = None
     live: bool = False  # the scheduler holds it (waiting or running)
+    # the name under which the engine and its cache manager know the request: unique over all
+    # schedulers that share the engine (``Scheduler.add`` sets it)
+    engine_id: Any = None
 
     @property
     def tokens(self):
@@ -158,6 +170,7 @@ class Scheduler:
         self.running: List[Request] = []
         self.stats = SchedulerStats()
         self._order = 0
+        self.number = next(_scheduler_numbers)
         self.pipelined = hasattr(sample, "launch") and hasattr(sample, "finish")
         self._inflight = None  # the sampling call whose tokens the host has not read yet
 
@@ -182,6 +195,7 @@ class Scheduler:
             raise ValueError(f"request id {request.request_id!r} is in use")
         request.order = self._order
         self._order += 1
+        request.engine_id = (self.number, request.request_id)
         if request.max_tokens == 0:
             # nothing to generate: finished as it comes, with no step run and no token sampled
             # (``generate_step`` yields nothing for it, mlx_lm/generate.py:448-461)
@@ -214,8 +228,14 @@ class Scheduler:
             self.running.remove(r)
         elif r in self.waiting:  # pre-empted, and finished by the token that was in flight
             self.waiting.remove(r)
-        if self.engine.has_request(r.request_id):
-            self.engine.end_request(r.request_id)
+        if self.engine.has_request(r.engine_id):
+            self.engine.end_request(r.engine_id)
+
+    def close(self):
+        """Take every request out and give back what they hold in the engine."""
+        self._inflight = None
+        for r in list(self.waiting) + list(self.running):
+            self._drop(r)
 
     def _ends_with_token_in_flight(self, r):
         """The token in flight is the request's last, whatever it is."""
@@ -233,8 +253,8 @@ class Scheduler:
     # -- decisions ---------------------------------------------------------------
 
     def _pages_for(self, r, n_new):
-        if self.engine.has_request(r.request_id):
-            return self.cache.pages_needed(r.request_id, n_new)
+        if self.engine.has_request(r.engine_id):
+            return self.cache.pages_needed(r.engine_id, n_new)
         return self.cache.blocks_for(n_new)
 
     def plan_step(self):
@@ -282,11 +302,22 @@ class Scheduler:
             whole = self.cache.blocks_for(min(r.num_tokens + 1, self.max_positions))
             if whole > free:
                 break
+            # The request leaves the queue only once the engine has it and its pages: whatever
+            # goes wrong before (another scheduler on the same engine holds the last slot) leaves
+            # it waiting, first in line.  The whole prompt's pages are taken now, so a request that
+            # was admitted can always finish reading its prompt.
+            try:
+                self.engine.add_request(r.engine_id)
+            except OutOfSlots:
+                break
+            try:
+                self.cache.reserve(r.engine_id, min(r.num_tokens + 1, self.max_positions))
+            except BaseException as e:
+                self.engine.end_request(r.engine_id)
+                if isinstance(e, OutOfPages):
+                    break
+                raise
             self.waiting.popleft()
-            self.engine.add_request(r.request_id)
-            # the whole prompt's pages are taken now, so a request that was
-            # admitted can always finish reading its prompt
-            self.cache.reserve(r.request_id, min(r.num_tokens + 1, self.max_positions))
             self.running.append(r)
             n = min(r.num_tokens, budget, self.prefill_step_size)
             free -= whole
@@ -297,8 +328,8 @@ class Scheduler:
     def _fit(self, r, n, free):
         """The longest portion of at most ``n`` tokens whose pages are free."""
         ps = self.cache.page_size
-        if self.engine.has_request(r.request_id):
-            rc = self.cache.requests[r.request_id]
+        if self.engine.has_request(r.engine_id):
+            rc = self.cache.requests[r.engine_id]
             room = self.cache.blocks_for(rc.reserved) * ps - rc.length
         else:
             room = 0
@@ -332,7 +363,7 @@ class Scheduler:
         if plan:
             logits = self._run(plan, prev)
         elif prev is None and self.has_work and not self.running:
-            raise RuntimeError("requests are waiting but none can be admitted")
+            raise RuntimeError(self._stuck())
         if prev is not None:
             outputs = self._finish(prev)  # the GPU is busy with this step meanwhile
         sampled = [p.request for p in plan if p.samples]
@@ -343,16 +374,25 @@ class Scheduler:
             self._inflight = job
         return outputs
 
+    def _stuck(self):
+        """Why nothing can run: requests wait, none runs here, and the first in line finds no room
+        (``add`` refused what could never fit, so others on the same engine hold the room)."""
+        others = [rid for rid in self.cache.requests
+                  if not (isinstance(rid, tuple) and len(rid) == 2 and rid[0] == self.number)]
+        return (f"requests are waiting but none can be admitted: {self.cache.free_pages()} of "
+                f"{self.cache.n_pages} pages are free and {len(others)} requests of other generators "
+                f"on this engine hold pages or slots; finish or close those first")
+
     def _run(self, plan, prev=None):
         """Launch the planned step; decoding requests whose token is in flight get it fed on the device."""
         entries = []
         for p in plan:
             r = p.request
             if r.inflight_row is not None:
-                entries.append(StepEntry(r.request_id, [0], [0] if p.samples else [], fed_row=r.inflight_row))
+                entries.append(StepEntry(r.engine_id, [0], [0] if p.samples else [], fed_row=r.inflight_row))
             else:
                 toks = r.tokens[r.num_computed : r.num_computed + p.n_tokens]
-                entries.append(StepEntry(r.request_id, toks, [p.n_tokens - 1] if p.samples else []))
+                entries.append(StepEntry(r.engine_id, toks, [p.n_tokens - 1] if p.samples else []))
         if prev is not None and any(e.fed_row >= 0 for e in entries):
             logits = self.engine.step(entries, fed=prev.tokens)
         else:
@@ -399,7 +439,7 @@ class Scheduler:
         plan = self.plan_step()
         if not plan:
             if self.has_work and not self.running:
-                raise RuntimeError("requests are waiting but none can be admitted")
+                raise RuntimeError(self._stuck())
             return []
         logits = self._run(plan)
         sampled = [p.request for p in plan if p.samples]

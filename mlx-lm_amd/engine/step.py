@@ -200,13 +200,19 @@ class Engine:
                 cm.rollback(rid, mark)
             raise
 
-        graph = self._recorded_step(entries) if self.use_graphs else None
-        if graph is not None:
-            logits = graph.run(entries)
-        else:
-            ctx = self._build_context(entries)
-            self.scratch.reset()
-            logits = self.decoder.forward(ctx)
+        try:
+            graph = self._recorded_step(entries) if self.use_graphs else None
+            if graph is not None:
+                logits = graph.run(entries)
+            else:
+                ctx = self._build_context(entries)
+                self.scratch.reset()
+                logits = self.decoder.forward(ctx)
+        except Exception:
+            # a step that raised has stored nothing that counts: its pages go back as above
+            for rid, mark in marks:
+                cm.rollback(rid, mark)
+            raise
         for e in entries:
             cm.commit(e.request_id, len(e.tokens))
         self.steps += 1

@@ -194,8 +194,7 @@ class _OneRequest:
                     self.progress(min(req.num_computed, len(self.prompt)), len(self.prompt))
                 yield from outs
         finally:
-            if self.engine.has_request(self.request_id):
-                sched.abort(self.request_id)
+            sched.close()  # (a generator dropped half-way gives its pages back here)
 
 
 def generate_step(prompt, model, *, max_tokens=256, sampler=None, logits_processors=None,
@@ -434,8 +433,16 @@ class BatchGenerator:
         self._requests = {}
 
     def close(self):
-        for uid in list(self._requests):
-            self.remove([uid])
+        """Drop every request; their pages and slots go back to the engine, which other
+        generators over the same model share."""
+        self._requests.clear()
+        self.scheduler.close()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
     @contextlib.contextmanager
     def stats(self, stats=None):

@@ -69,6 +69,12 @@ class DecoderModel:
         return want
 
     def load_tensors(self, tensors):
+        """Hand every part its device tensors.  The native twins keep the tensors' addresses, and
+        so do the steps an engine has recorded: once a twin exists, other weights need a new model."""
+        if self._native is not None or any(p._native is not None for p in self.parts()):
+            raise RuntimeError(
+                "this model has run (its native parts and recorded steps hold the addresses of its "
+                "weights): build a new model to load other weights")
         for part in self.parts():
             part.load(tensors)
 

@@ -167,6 +167,13 @@ def forward(weights, config, ids, dtype=torch.float64):
     mlx_lm/models/gpt2.py:125-151 (embeddings, blocks, final norm) and
     161-168 (tied head).  ``config`` is the dict of config.json.
     """
+    h = final_hidden(weights, config, ids, dtype)
+    return tied_head(h, weights["model.wte.weight"].to(dtype))
+
+
+def final_hidden(weights, config, ids, dtype=torch.float64):
+    """What the head is applied to, ``[L, D]``: embeddings, blocks, final norm
+    (mlx_lm/models/gpt2.py:125-151).  For tests that cannot afford the head at every position."""
     w = {k: v.to(dtype) for k, v in weights.items()}
     ids = torch.as_tensor(ids, dtype=torch.long)
     eps = config["layer_norm_epsilon"]
@@ -174,8 +181,7 @@ def forward(weights, config, ids, dtype=torch.float64):
     h = add_learned_positions(h, w["model.wpe.weight"], 0)
     for i in range(config["n_layer"]):
         h = block(h, w, i, config["n_head"], eps)
-    h = layer_norm(h, w["model.ln_f.weight"], w["model.ln_f.bias"], eps)
-    return tied_head(h, w["model.wte.weight"])
+    return layer_norm(h, w["model.ln_f.weight"], w["model.ln_f.bias"], eps)
 
 
 def log_softmax(logits):

@@ -216,3 +216,20 @@ def test_random_weights_from_the_command_line(tmp_path):
     a, b = load_file(str(tmp_path / "cli" / "model.safetensors")), load_file(str(tmp_path / "fn" / "model.safetensors"))
     assert sorted(a) == sorted(b) and all(torch.equal(a[k], b[k]) for k in a)
     assert json.loads((tmp_path / "cli" / "config.json").read_text()) == config
+
+
+def test_weights_cannot_be_swapped_under_a_model_that_has_run():
+    """The native twins of the parts (and the steps an engine recorded) hold the addresses of the
+    weights they were made from: a second load would leave them reading the old tensors."""
+    model = Model(ModelArgs.from_dict(helpers.TINY_A))
+    t = model.sanitize(Model.random_weights(model.args, 0, "a"))
+    placed = place_tensors(model.decoder.expected_tensors(), t, "float32", "cpu")
+    model.decoder.load_tensors(placed)
+    model.decoder.load_tensors(placed)  # nothing has been made from them yet: fine
+    part = model.decoder.final_norm
+    part._native = 1  # (stands for a twin; never handed to the library)
+    try:
+        with pytest.raises(RuntimeError, match="build a new model"):
+            model.decoder.load_tensors(placed)
+    finally:
+        part._native = None

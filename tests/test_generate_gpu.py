@@ -237,6 +237,67 @@ def test_many_interleaved_generators_keep_their_own_tokens(model_b, tiny):
     assert together == alone
 
 
+def test_two_batch_generators_and_a_generate_step_share_one_model(model_b, tiny):
+    """Any number of generators may be live over one model (mlx_lm/generate.py:1596-1607,
+    1712-1731: each ``BatchGenerator`` has caches and a uid counter of its own).  Here they share
+    the model's engine and its pages: both generators number their requests from 0, are stepped
+    in turn with a ``generate_step`` beside them, in a pool so small that requests wait or are
+    pre-empted; every request makes the tokens it makes alone."""
+    from mlx_lm_amd import generate_step
+    from mlx_lm_amd.engine import Engine
+    from mlx_lm_amd.generate import BatchGenerator
+
+    V = tiny["B"][1]["vocab_size"]
+    prompts_a = [helpers.random_tokens(n, V, seed=600 + n) for n in (40, 9, 23)]
+    prompts_b = [helpers.random_tokens(n, V, seed=700 + n) for n in (31, 17)]
+    prompt_c = helpers.random_tokens(12, V, seed=800)
+    limits_a, limits_b, limit_c = [30, 20, 25], [28, 35], 22
+    alone_a = [_single(model_b, p, max_tokens=m) for p, m in zip(prompts_a, limits_a)]
+    alone_b = [_single(model_b, p, max_tokens=m) for p, m in zip(prompts_b, limits_b)]
+    alone_c = _single(model_b, prompt_c, max_tokens=limit_c)
+    # 14 pages of 16 tokens: what the five requests of the two generators grow to needs 18
+    shared = Engine(model_b, dtype="float32", page_size=16, n_pages=14, max_requests=8)
+    a = BatchGenerator(model_b, engine=shared, prefill_step_size=16, completion_batch_size=4)
+    b = BatchGenerator(model_b, engine=shared, prefill_step_size=32, completion_batch_size=4)
+    uids_a, uids_b = a.insert(prompts_a, limits_a), b.insert(prompts_b, limits_b)
+    assert uids_a == [0, 1, 2] and uids_b == [0, 1]  # the same ids, and both live
+    got_a, got_b, got_c = {u: [] for u in uids_a}, {u: [] for u in uids_b}, []
+    c = generate_step(prompt_c, model_b, max_tokens=limit_c)  # on the model's own engine
+    held_back = 0
+    for _ in range(3000):
+        live = False
+        for gen, got in ((a, got_a), (b, got_b)):
+            if not gen.scheduler.has_work:
+                continue
+            live = True
+            try:
+                _, responses = gen.next()
+            except RuntimeError as e:  # the other generator holds every page just now
+                assert "other generators" in str(e)
+                held_back += 1
+                continue
+            for r in responses:
+                got[r.uid].append(r.token)
+        if len(got_c) < limit_c:
+            live = True
+            got_c.append(next(c)[0])
+        if not live:
+            break
+        shared.cache.check()
+    assert [got_a[u] for u in uids_a] == alone_a
+    assert [got_b[u] for u in uids_b] == alone_b
+    assert got_c == alone_c
+    assert a.scheduler.stats.preemptions + b.scheduler.stats.preemptions + held_back > 0
+    assert shared.cache.free_pages() == 14 and not shared.cache.requests
+    # a generator that is dropped with requests live gives their pages back
+    d = BatchGenerator(model_b, engine=shared, prefill_step_size=16)
+    d.insert(prompts_a[:1], [50])
+    d.next()
+    assert shared.cache.requests
+    d.close()
+    assert shared.cache.free_pages() == 14 and not shared.cache.requests
+
+
 def test_no_tokens_asked_for_none_made(model_b, tiny):
     """``max_tokens=0`` (mlx_lm/generate.py:448-461): nothing is yielded, and in a batch the
     request ends at once beside the others."""

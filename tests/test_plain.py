@@ -203,3 +203,115 @@ def test_penalties():
     assert plain.presence_penalty(x, [0, 0, 2], 0.5).tolist() == [0.5, -1.0, 1.5, 0.5]
     assert plain.frequency_penalty(x, [0, 0, 2], 0.5).tolist() == [0.0, -1.0, 1.5, 0.5]
     assert plain.frequency_penalty(x, [0, 0, 2], 0.5, context_size=1).tolist() == [1.0, -1.0, 1.5, 0.5]
+
+
+def _library_block(x, w, i, n_head, eps):
+    """One block put together from library routines only, in the order the reference's text
+    gives (mlx_lm/models/gpt2.py:98-108; inside attention :52-68, the MLP :71-80)."""
+    p = f"model.h.{i}."
+    D = x.shape[-1]
+    L = x.shape[0]
+    a = F.layer_norm(x, (D,), w[p + "ln_1.weight"], w[p + "ln_1.bias"], eps)
+    qkv = F.linear(a, w[p + "attn.c_attn.weight"], w[p + "attn.c_attn.bias"])
+    q, k, v = (t.reshape(L, n_head, D // n_head).transpose(0, 1)[None] for t in qkv.split(D, dim=-1))
+    o = F.scaled_dot_product_attention(q, k, v, is_causal=True)[0].transpose(0, 1).reshape(L, D)
+    h = x + F.linear(o, w[p + "attn.c_proj.weight"], w[p + "attn.c_proj.bias"])
+    m = F.layer_norm(h, (D,), w[p + "ln_2.weight"], w[p + "ln_2.bias"], eps)
+    m = F.gelu(F.linear(m, w[p + "mlp.c_fc.weight"], w[p + "mlp.c_fc.bias"]), approximate="tanh")
+    return h + F.linear(m, w[p + "mlp.c_proj.weight"], w[p + "mlp.c_proj.bias"])
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole_model_is_the_library_routines_in_the_reference_s_order(name):
+    config, w = _weights(name)
+    D, H, eps = config["n_embd"], config["n_head"], config["layer_norm_epsilon"]
+    ids = torch.tensor(helpers.random_tokens(23, config["vocab_size"], 6))
+    h = F.embedding(ids, w["model.wte.weight"]) + w["model.wpe.weight"][: len(ids)]
+    for i in range(config["n_layer"]):
+        want = _library_block(h, w, i, H, eps)
+        assert torch.allclose(plain.block(h, w, i, H, eps), want, atol=1e-11)
+        h = want
+    want = F.linear(F.layer_norm(h, (D,), w["model.ln_f.weight"], w["model.ln_f.bias"], eps), w["model.wte.weight"])
+    assert torch.allclose(plain.forward(w, config, ids), want, atol=1e-10)
+
+
+def test_block_wiring_by_invariants():
+    """What a mis-wired block would break: each sub-layer reads the *norm* of the stream (so its
+    contribution does not change when the stream is scaled), adds to the stream *unnormed*, the
+    attention sub-layer comes first with ``ln_1`` and the feed-forward reads its result with
+    ``ln_2``, and the last norm stands between the blocks and the head."""
+    config, w = _weights("B")
+    H, eps, D = config["n_head"], 0.0, config["n_embd"]  # (eps 0: the norm of c*x is the norm of x exactly)
+    x = torch.randn(9, D, dtype=torch.float64)
+    base = plain.block(x, w, 1, H, eps)
+    # pre-norm: block(c x) - c x == block(x) - x would hold only if the second sub-layer saw a
+    # scaled stream too; with the feed-forward's output projection off it is exact
+    off_mlp = dict(w)
+    off_mlp["model.h.1.mlp.c_proj.weight"] = torch.zeros_like(w["model.h.1.mlp.c_proj.weight"])
+    off_mlp["model.h.1.mlp.c_proj.bias"] = torch.zeros_like(w["model.h.1.mlp.c_proj.bias"])
+    d1 = plain.block(x, off_mlp, 1, H, eps) - x
+    assert torch.allclose(plain.block(3.0 * x, off_mlp, 1, H, eps) - 3.0 * x, d1, atol=1e-10)
+    assert d1.abs().max() > 1e-3
+    # the attention sub-layer uses ln_1, not ln_2: with the MLP off, ln_2 does not matter, ln_1 does
+    changed = dict(off_mlp)
+    changed["model.h.1.ln_2.weight"] = w["model.h.1.ln_2.weight"] * 1.7
+    assert torch.equal(plain.block(x, changed, 1, H, eps) - x, d1)
+    changed = dict(off_mlp)
+    changed["model.h.1.ln_1.bias"] = w["model.h.1.ln_1.bias"] + 0.3
+    assert (plain.block(x, changed, 1, H, eps) - x - d1).abs().max() > 1e-4
+    # attention off: what is left is x + mlp(ln_2(x)), row by row (no mixing of positions)
+    off_attn = dict(w)
+    off_attn["model.h.1.attn.c_proj.weight"] = torch.zeros_like(w["model.h.1.attn.c_proj.weight"])
+    off_attn["model.h.1.attn.c_proj.bias"] = torch.zeros_like(w["model.h.1.attn.c_proj.bias"])
+    d2 = plain.block(x, off_attn, 1, H, eps) - x
+    assert torch.allclose(plain.block(x[4:5], off_attn, 1, H, eps) - x[4:5], d2[4:5], atol=1e-12)
+    assert torch.allclose(plain.block(2.0 * x, off_attn, 1, H, eps) - 2.0 * x, d2, atol=1e-10)
+    # the feed-forward reads the stream *after* attention was added: both on is not the sum of each alone
+    assert ((base - x) - (d1 + d2)).abs().max() > 1e-4
+    # and attention does not read the feed-forward's output: the first row's attention term is
+    # the same whatever the feed-forward does (one key: the value itself)
+    moved = dict(w)
+    moved["model.h.1.mlp.c_proj.bias"] = w["model.h.1.mlp.c_proj.bias"] + 1.0
+    assert torch.allclose(plain.block(x, moved, 1, H, eps) - base, torch.ones_like(base), atol=1e-10)
+    # the final norm: scaling the last block's output stream leaves the logits unchanged, which
+    # holds only if ln_f stands before the head; its scale doubles them
+    cfg0 = dict(config, layer_norm_epsilon=0.0)
+    ids = helpers.random_tokens(7, config["vocab_size"], 8)
+    logits = plain.forward(w, cfg0, ids)
+    w2 = dict(w)
+    w2["model.ln_f.weight"], w2["model.ln_f.bias"] = 2 * w["model.ln_f.weight"], 2 * w["model.ln_f.bias"]
+    assert torch.allclose(plain.forward(w2, cfg0, ids), 2 * logits, atol=1e-9)
+
+
+def test_query_key_value_order_by_construction():
+    """Weights built so that the three thirds of ``c_attn`` can be told apart: the first third
+    makes queries that pick out, through the second third's keys, exactly one earlier position,
+    and the third third's values carry that position's marker.  Swapping any two thirds moves
+    the result (mlx_lm/models/gpt2.py:52-58: q, k, v in this order)."""
+    L, D = 6, 16
+    w = {k: torch.zeros(s, dtype=torch.float64) for k, s in {
+        "a.c_attn.weight": (3 * D, D), "a.c_attn.bias": (3 * D,), "a.c_proj.weight": (D, D), "a.c_proj.bias": (D,)}.items()}
+    # rows of x: one-hot of the position in columns 0..5, one-hot of the position to look at in 8..13
+    x = torch.zeros(L, D, dtype=torch.float64)
+    look = [0, 0, 1, 1, 3, 2]
+    for t in range(L):
+        x[t, t] = 1.0
+        x[t, 8 + look[t]] = 1.0
+    big = 60.0
+    mark = [9, 7, 12, 6, 15, 10]
+    for j in range(L):
+        w["a.c_attn.weight"][j, 8 + j] = big          # q_j = big * [looks at j]
+        w["a.c_attn.weight"][D + j, j] = 1.0          # k_j = [is position j]
+        w["a.c_attn.weight"][2 * D + mark[j], j] = 1.0  # v_j = position j's marker (not its key)
+    w["a.c_proj.weight"] = torch.eye(D, dtype=torch.float64)
+    out = plain.self_attention(x, w, "a.", 1)
+    want = torch.zeros(L, D, dtype=torch.float64)
+    for t in range(L):
+        want[t, mark[look[t]]] = 1.0
+    assert torch.allclose(out, want, atol=1e-6)
+    for a, b in ((0, 1), (0, 2), (1, 2)):
+        sw = dict(w)
+        m = w["a.c_attn.weight"].clone()
+        m[a * D:(a + 1) * D], m[b * D:(b + 1) * D] = w["a.c_attn.weight"][b * D:(b + 1) * D], w["a.c_attn.weight"][a * D:(a + 1) * D]
+        sw["a.c_attn.weight"] = m
+        assert (plain.self_attention(x, sw, "a.", 1) - want).abs().max() > 0.1, (a, b)

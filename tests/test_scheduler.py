@@ -29,17 +29,19 @@ class FakeEngine:
         return rid in self.cache.requests
 
     def step(self, entries, fed=None):
+        # the engine knows a request as (its scheduler's number, the scheduler's own id for it);
+        # the log and the rows name it as its scheduler does
         for e in entries:
             self.cache.reserve(e.request_id, len(e.tokens))
             if e.fed_row >= 0:  # the token comes from the sampling call in flight: the right row of it
-                assert fed is not None and fed[e.fed_row][0] == e.request_id and len(e.tokens) == 1
+                assert fed is not None and fed[e.fed_row][0] == e.request_id[1] and len(e.tokens) == 1
                 self.fed += 1
         rows = []
         for e in entries:
             start = self.cache.requests[e.request_id].length
             self.cache.commit(e.request_id, len(e.tokens))
-            rows += [(e.request_id, start + w, tuple(e.tokens)) for w in e.want]
-        self.log.append([(e.request_id, len(e.tokens), list(e.want)) for e in entries])
+            rows += [(e.request_id[1], start + w, tuple(e.tokens)) for w in e.want]
+        self.log.append([(e.request_id[1], len(e.tokens), list(e.want)) for e in entries])
         self.cache.check()
         return rows
 
@@ -283,5 +285,63 @@ def test_a_request_for_no_tokens_is_over_at_once(mode):
     assert r.finish_reason == "length" and not sched.has_work and not r.live
     sched.add(Request("one", [4, 5], 1))
     done = run_all(sched)
-    assert list(done) == ["one"] and r.generated == [] and not eng.has_request("none")
+    assert list(done) == ["one"] and r.generated == [] and not eng.cache.requests
     assert all(rid != "none" for step in eng.log for rid, _, _ in step)
+
+
+@pytest.mark.parametrize("mode", SAMPLERS)
+def test_two_schedulers_share_an_engine_with_the_same_request_ids(mode):
+    """Any number of generators may be live over one model, each numbering its requests from 0
+    (mlx_lm/generate.py:1596-1607,1712-1731): the engine keeps them apart, a scheduler that finds
+    the last slot or the pages taken leaves its request waiting (not lost), and each request makes
+    the tokens it makes alone."""
+    eng = FakeEngine(n_pages=7, max_positions=200, max_requests=3)
+    a = Scheduler(eng, SAMPLERS[mode](), max_num_seqs=4)
+    b = Scheduler(eng, SAMPLERS[mode](), max_num_seqs=4)
+    for s in (a, b):
+        s.add(Request(0, list(range(1, 31)), 30))  # 2 pages, grows to 4
+        s.add(Request(1, list(range(1, 10)), 20))  # 1 page, grows to 2
+    done = {id(a): {}, id(b): {}}
+    held_back = False
+    for _ in range(2000):
+        if not (a.has_work or b.has_work):
+            break
+        for s in (a, b):
+            if not s.has_work:
+                continue
+            try:
+                outs = s.step()
+            except RuntimeError as e:  # the other scheduler holds everything: said so, nothing lost
+                assert "other generators" in str(e)
+                assert len(s.waiting) + len(s.running) > 0
+                held_back = True
+                continue
+            for o in outs:
+                done[id(s)].setdefault(o.request_id, []).append(o.token)
+        eng.cache.check()
+    assert not (a.has_work or b.has_work)
+    for s in (a, b):
+        assert done[id(s)] == {0: [token_for(0, i) for i in range(30)], 1: [token_for(1, i) for i in range(20)]}
+    assert a.stats.preemptions + b.stats.preemptions >= 1 or held_back
+    assert eng.cache.free_pages() == 7 and not eng.cache.requests
+
+
+def test_admission_that_fails_keeps_the_request_first_in_line():
+    eng = FakeEngine(n_pages=16, max_requests=1)
+    a = Scheduler(eng, fake_sample)
+    b = Scheduler(eng, fake_sample)
+    a.add(Request("x", [1, 2, 3], 3))
+    a.step()  # takes the only slot
+    rb = b.add(Request("x", [4, 5], 2))
+    with pytest.raises(RuntimeError, match="1 requests of other generators"):
+        b.step()
+    assert list(b.waiting) == [rb] and rb.live and not b.running
+    run_all(a)
+    done = run_all(b)
+    assert [o.token for o in done["x"]] == [token_for("x", 0), token_for("x", 1)]
+    # a scheduler that is closed gives back what its requests hold
+    a.add(Request("y", list(range(1, 40)), 5))
+    a.step()
+    assert eng.cache.requests
+    a.close()
+    assert not eng.cache.requests and eng.cache.free_pages() == 16 and not a.has_work

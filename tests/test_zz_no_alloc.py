@@ -64,11 +64,14 @@ def test_split_product_without_a_workspace_twice_in_a_row():
         start = torch.randn(M, N, generator=g).to(dtype).cuda()
         want, got = start.clone(), start.clone()
         _existing(lib, want, a, w, bias, flags, n_splits)
-        before = torch.cuda.memory_allocated()
+        torch.cuda.synchronize()
+        # free bytes of the device as the driver counts them: a hipMalloc inside the call would
+        # show here (torch's own counters see only torch's allocator)
+        before = torch.cuda.mem_get_info()[0], torch.cuda.memory_reserved()
         rc = _static(lib, got, a, w, bias, flags, n_splits)
         assert rc == 0, lib.mlxlm_last_error().decode()
         torch.cuda.synchronize()
-        assert torch.cuda.memory_allocated() == before
+        assert (torch.cuda.mem_get_info()[0], torch.cuda.memory_reserved()) == before
         assert torch.equal(got, want), (M, N, K)
         ref = a.float() @ w.float().t() + bias
         if flags & 1:
@@ -90,3 +93,31 @@ def test_sizes_beyond_the_array_and_other_flags_are_refused():
     assert "flags" in lib.mlxlm_last_error().decode()
     assert _static(lib, out, a, w, None, 0, 8) == 0  # exactly what fits
     torch.cuda.synchronize()
+
+
+def test_the_call_can_be_captured_into_a_graph():
+    """Under stream capture (global mode) an allocating call is an error that ends the capture; this
+    one is recorded, and every replay gives what the eager entry points give."""
+    lib = _lib()
+    assert lib.gemm_bf16_decode_static_init() == 0, lib.mlxlm_last_error().decode()
+    g = torch.Generator().manual_seed(1)
+    M, N, K, n_splits, flags = 8, 1600, 1600, 4, 4
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
+    w = (0.05 * torch.randn(N, K, generator=g)).to(torch.bfloat16).cuda()
+    bias = torch.randn(N, generator=g).cuda()
+    want = torch.zeros(M, N, dtype=torch.float32, device="cuda")
+    got = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    assert _static(lib, got, a, w, bias, flags, n_splits) == 0  # warm-up: modules loaded, address looked up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, capture_error_mode="global"):
+        rc = _static(lib, got, a, w, bias, flags, n_splits)
+    assert rc == 0, lib.mlxlm_last_error().decode()
+    for trial in range(3):
+        a.copy_(torch.randn(M, K, generator=g).to(torch.bfloat16))  # eager work between the replays
+        _existing(lib, want, a, w, bias, flags, n_splits)
+        got.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), trial
