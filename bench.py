@@ -72,12 +72,13 @@ def _start(engine, sched, batch, prompt_len, vocab, seed, tag):
 
     g = torch.Generator().manual_seed(seed)
     prompts = torch.randint(0, vocab, (batch, prompt_len), generator=g).tolist()
-    rids = [(tag, batch, i) for i in range(batch)]
-    for i, rid in enumerate(rids):
-        sched.add(Request(rid, prompts[i], max_tokens=10**6, seed=i))  # greedy; the caller ends it
+    requests = [Request((tag, batch, i), prompts[i], max_tokens=10**6, seed=i)  # greedy; the caller ends it
+                for i in range(batch)]
+    for r in requests:
+        sched.add(r)
     while sched.waiting or not all(r.decoding for r in sched.running):
         sched.step()
-    return rids
+    return requests
 
 
 def run_decode(engine, batch, prompt_len, steps, warmup, vocab, seed):
@@ -88,17 +89,17 @@ def run_decode(engine, batch, prompt_len, steps, warmup, vocab, seed):
 
     sched = _scheduler(engine, batch, prompt_len)
     if warmup > 0:  # on requests of their own, so that the timed steps start at the prompt's end
-        rids = _start(engine, sched, batch, prompt_len, vocab, seed + 1000, "warm")
+        requests = _start(engine, sched, batch, prompt_len, vocab, seed + 1000, "warm")
         for _ in range(warmup):
             sched.step()
         torch.cuda.synchronize()
-        for rid in rids:
-            sched.abort(rid)
+        for r in requests:
+            sched.abort(r.request_id)
         while sched.has_work:
             sched.step()
-    rids = _start(engine, sched, batch, prompt_len, vocab, seed, "bench")
+    requests = _start(engine, sched, batch, prompt_len, vocab, seed, "bench")
     torch.cuda.synchronize()
-    ctx0 = engine.context_len(rids[0])
+    ctx0 = engine.context_len(requests[0].engine_id)
     t0 = time.perf_counter()
     n_out = 0
     for _ in range(steps):
@@ -107,9 +108,9 @@ def run_decode(engine, batch, prompt_len, steps, warmup, vocab, seed):
     dt = time.perf_counter() - t0
     if n_out != batch * steps:
         raise RuntimeError(f"{n_out} tokens came out of {steps} steps of {batch} requests")
-    for rid in rids:  # (a request that has reached the model's last position is over already)
-        if engine.has_request(rid):
-            sched.abort(rid)
+    for r in requests:  # (a request that has reached the model's last position is over already)
+        if r.live:
+            sched.abort(r.request_id)
     while sched.has_work:
         sched.step()
     # steps overlap: the first timed call launches the step at the prompt's end, and every call

@@ -48,9 +48,15 @@ struct DecodeArgs {
   // request brings one token), so neither `rows` nor `token_req` has to be read.
   // table_in_lds: the request's page numbers are copied to LDS once (max_blocks of them fit).
   int rows_are_requests, table_in_lds;
+  int out_head_dim;
 };
 
 #define MAX_WAVES 16
+
+// ldo == 0: out is in the packed order, tiles of 16 rows x 64 columns
+__device__ __forceinline__ size_t out_at(const DecodeArgs& p, int row, int col) {
+  return p.ldo != 0 ? (size_t)row * p.ldo + col : packed_at(row, col, (p.n_heads * p.out_head_dim + 63) / 64);
+}
 
 // Keys a wave takes at a time: 32 or 64, the caller's choice.  With 64, a context of 530 gave nine
 // of a block's waves a tile and the others none: 9.3 us for 8 rows of 25 heads against 7.3 with 32.
@@ -231,7 +237,7 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
   }
   if (tid < HD) {
     if (p.n_splits == 1) {
-      put((T*)p.out + (size_t)row * p.ldo + h * HD + tid, acc / L);
+      put((T*)p.out + out_at(p, row, h * HD + tid), acc / L);
     } else {
       const size_t base = ((size_t)item * p.n_heads + h) * p.n_splits + split;
       p.part_o[base * HD + tid] = acc;
@@ -257,7 +263,7 @@ __global__ void attn_decode_merge_kernel(DecodeArgs p) {
     L += p.part_ml[(base + s) * 2 + 1] * w;
     acc += p.part_o[(base + s) * HD + d] * w;
   }
-  put((T*)p.out + (size_t)row * p.ldo + h * HD + d, acc / L);
+  put((T*)p.out + out_at(p, row, h * HD + d), acc / L);
 }
 
 DEFINE_LAST_ERROR(mlxlm_last_error)
@@ -329,6 +335,8 @@ extern "C" int attn_decode_rows(void* out, const void* q, int ldq, int ldo, cons
     FAIL("attn_decode: what is read ahead must be chunks of 16-byte pieces");
   p.ahead = (const uint4*)ahead, p.ahead_pieces = ahead ? ahead_chunk_bytes / 16 : 0;
   p.ahead_chunks = ahead ? ahead_chunks : 0;
+  p.out_head_dim = head_dim;
+  if (ldo == 0 && dtype != DT_BF16) FAIL("attn_decode: the packed order (ldo == 0) is for a bfloat16 out");
   p.rows_are_requests = rows_are_requests ? 1 : 0;
   p.table_in_lds = max_blocks > 0 && max_blocks <= 8192;  // (32 KB of LDS at most)
   if (dtype == DT_BF16) {

@@ -203,3 +203,16 @@ static thread_local char g_err[512];
 
 #define DEFINE_LAST_ERROR(fn) \
   extern "C" const char* fn() { return g_err; }
+
+// Where element (m, n) of an activation matrix lies in the packed order: tiles of 16 rows x 64
+// columns, `kblocks` of them a tile row ((N + 63) / 64); in a tile the 8 values n = 16 g + 8 h + 0..7
+// of row f lie at ((4 h + g) * 16 + f) * 8, so that lane l of a wave (row l % 16, g = l / 16) reads
+// 16 bytes at l * 8 (h = 0) and at 512 + l * 8 (h = 1): a wave's load is 1 KB of consecutive bytes,
+// as with the packed weights.  Rows as an MFMA operand straight from a row-major matrix are
+// sixteen pieces of 64 bytes a load, which a CU fetches at a third of the speed.  Kernels that
+// make the rows of a product of 17 to 64 rows (the sum-and-norm, decode attention, that product's
+// own epilogue) write this order where the host asks for it.
+__device__ __forceinline__ size_t packed_at(int m, int n, int kblocks) {
+  const int kk = n & 63;
+  return ((size_t)(m >> 4) * kblocks + (n >> 6)) * 1024 + ((((kk >> 3) & 1) * 4 + (kk >> 4)) * 16 + (m & 15)) * 8 + (kk & 7);
+}

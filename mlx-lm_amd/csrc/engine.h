@@ -43,7 +43,10 @@ typedef struct {
   const float* gamma;
   const float* beta;
   float eps;
-  int pad_;
+  // packed != 0: m.p holds the bfloat16 rows in tiles of 16 rows x 64 columns, each tile in the
+  // order of the packed weights' tiles (what the product of 17 to 64 rows reads fastest); m.ld is
+  // not used then.  Only a part that asked for it (eng_wants_packed_rows) is handed such a value.
+  int packed;
 } EngValue;
 
 // Partial products that still have to be added into the residual stream.
@@ -191,16 +194,19 @@ typedef struct {
   const float* bias;
   const EngScatter* scatter;
   int gelu, accumulate, variant, splits;  // splits: 0 = the library chooses
+  int out_packed, pad_;  // out (bfloat16, [rows padded to 16][cols padded to 64]) in the packed order
 } EngLinear;
 int eng_linear(EngCtx* ctx, const EngLinear* call, EngPending* pending);
 // A pending sum outside a step's own: add it; whether the fused sum-and-norm takes it; add and norm.
 int eng_pending_settle(EngCtx* ctx, EngPending* pending);
 int eng_pending_can_norm(const EngPending* pending, const EngMat* x);
 int eng_pending_settle_normed(EngCtx* ctx, EngPending* pending, const EngMat* out, const float* gamma,
-                              const float* beta, float eps, const EngWeight* ahead);
+                              const float* beta, float eps, const EngWeight* ahead, int out_packed);
 int eng_read_ahead_pays(const EngCtx* ctx, const EngWeight* w, int n_rows, int with_norm);
 // 1 if the product of these sizes would norm a lazy input in its own prologue
 int eng_linear_norms_itself(const EngCtx* ctx, int M, int N, int K, int dtype, int splits);
+// 1 if the product of n_rows rows with w reads its rows fastest in the packed order (EngValue.packed)
+int eng_wants_packed_rows(const EngCtx* ctx, const EngWeight* w, int n_rows);
 
 #ifdef __cplusplus
 }

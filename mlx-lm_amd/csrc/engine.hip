@@ -25,7 +25,8 @@ DEFINE_LAST_ERROR(mlxlm_last_error)
 #define GEMM_KV 8
 #define DECODE_MAX_ROWS 16
 #define F32_FEW_ROWS 64  // rows that the 32-bit product's streaming kernel takes
-#define ROWS_MAX_ROWS 48  // up to here the kernel for 17 to 48 rows
+#define GEMM_OUT_PACKED 16
+#define ROWS_MAX_ROWS 64  // up to here the kernel for 17 to 64 rows
 #define ATTN_ROW_MAX_HEAD_DIM 144
 #define READ_AHEAD_BYTES_PER_CU (160 * 1024)  // what an idle CU reads while decode attention runs
 
@@ -81,7 +82,7 @@ typedef int (*fn_sum_partials)(void*, const float*, int, const float*, int, int,
                                size_t, const int*, int, const int*, const int*, int, int, int, int,
                                hipStream_t);
 typedef int (*fn_sum_partials_norm)(float*, int, const float*, int, const float*, const float*, const float*,
-                                    float, void*, int, int, int, const void*, size_t, int, hipStream_t);
+                                    float, void*, int, int, int, int, const void*, size_t, int, hipStream_t);
 typedef int (*fn_kv_write)(const void*, const void*, int, void*, void*, size_t, const int*, int, const int*,
                            const int*, int, int, int, int, int, hipStream_t);
 typedef int (*fn_attn_tile)(void*, const void*, int, int, const void*, const void*, size_t, const int*, int,
@@ -179,8 +180,8 @@ static inline bool waits_on(const EngPending& p, const EngMat& x) {
 }
 
 static int sum_partials(EngCtx* ctx, const EngMat& out, const float* ws, int n_splits, const float* bias,
-                        bool gelu, bool accumulate, const EngScatter* sc) {
-  int flags = (gelu ? GEMM_GELU : 0) | (accumulate ? GEMM_ACCUMULATE : 0);
+                        bool gelu, bool accumulate, const EngScatter* sc, bool out_packed = false) {
+  int flags = (gelu ? GEMM_GELU : 0) | (accumulate ? GEMM_ACCUMULATE : 0) | (out_packed ? GEMM_OUT_PACKED : 0);
   if (out.dtype == DT_F32) {
     if (!accumulate) flags |= GEMM_OUT_F32;
   } else if (accumulate) {
@@ -216,15 +217,22 @@ static int can_norm(const EngPending& p, const EngMat& x, bool* yes) {
 
 // Add what is pending into its target and write the LayerNorm of the new rows to `out`.
 static int settle_normed(EngCtx* ctx, EngPending* p, const EngMat& out, const float* gamma, const float* beta,
-                         float eps, const EngWeight* ahead) {
+                         float eps, const EngWeight* ahead, bool out_packed = false) {
   if (!p->target) FAIL("settle_normed: nothing is pending");
   float* h = p->target;
   p->target = nullptr;
-  if (out.rows != p->rows || out.cols != p->cols || out.ld != out.cols) FAIL("settle_normed: out's shape");
+  if (out.rows != p->rows || out.cols != p->cols || (!out_packed && out.ld != out.cols)) FAIL("settle_normed: out's shape");
   if (ctx->stats) ctx->stats->settle_normed++;
   KERNEL(k_sum_partials_norm, ctx, h, p->ld, p->ws, p->n_splits, p->bias, gamma, beta, eps, out.p, out.dtype,
-         p->rows, p->cols, ahead ? ahead->packed : nullptr, ahead ? ahead->chunk_bytes : (size_t)0,
-         ahead ? ahead->n_chunks : 0, ctx->stream);
+         out_packed ? 1 : 0, p->rows, p->cols, ahead ? ahead->packed : nullptr,
+         ahead ? ahead->chunk_bytes : (size_t)0, ahead ? ahead->n_chunks : 0, ctx->stream);
+  return 0;
+}
+
+// Memory for `rows` x `cols` bfloat16 values in the packed order: whole tiles of 16 rows x 64 columns.
+static int take_packed(EngCtx* ctx, int rows, int cols, EngMat* out) {
+  TRY(take(ctx, (rows + 15) / 16 * 16, (cols + 63) / 64 * 64, DT_BF16, out));
+  out->rows = rows, out->cols = cols, out->ld = 0;
   return 0;
 }
 
@@ -252,6 +260,7 @@ static int layernorm(EngCtx* ctx, const EngMat& out, const float* x, const float
 }
 
 static int materialize(EngCtx* ctx, const EngValue& v, EngMat* out) {
+  if (v.packed) FAIL("rows in the packed order were handed to a part that did not ask for them");
   if (!v.lazy) {
     *out = v.m;
     return 0;
@@ -289,19 +298,58 @@ extern "C" int eng_linear_norms_itself(const EngCtx* ctx, int M, int N, int K, i
 // goes into the residual stream and the caller allows that (the next norm adds it), otherwise
 // the second kernel adds the parts and runs the epilogue.
 static int finish_parts(EngCtx* ctx, const EngMat& out, float* ws, int n_splits, const float* bias, bool gelu,
-                        bool accumulate, const EngScatter* sc, EngPending* pending) {
+                        bool accumulate, const EngScatter* sc, EngPending* pending, bool out_packed = false) {
   if (accumulate && pending && pending->allowed) {
     pending->target = (float*)out.p, pending->rows = out.rows, pending->cols = out.cols, pending->ld = out.ld;
     pending->ws = ws, pending->n_splits = n_splits, pending->bias = bias;
     return 0;
   }
-  return sum_partials(ctx, out, ws, n_splits, bias, gelu, accumulate, sc);
+  return sum_partials(ctx, out, ws, n_splits, bias, gelu, accumulate, sc, out_packed);
+}
+
+// Whether the kernel for 17 to 64 rows takes the product of M rows with w, and with K in how many
+// parts (*n_splits; 0: it does not).
+// (A matrix of more blocks than two a CU, the vocabulary's, would take that kernel several rounds,
+// each with its own wait for memory: the tiles stream it 6 us faster.  Beyond 32 rows it wins
+// only where K is long enough for the tiles to split it: at widths 768 and 1,024 a decode
+// step of 48 rows is 4 to 5 % slower through it, at 1,280 the same, at 1,600 4 % faster.)
+static int rows_parts(const EngCtx* ctx, int M, const EngWeight& w, int variant, int splits, int* n_splits) {
+  *n_splits = 0;
+  const int N = w.N, K = w.K;
+  if (!(w.dtype == DT_BF16 && variant == 0 && M > DECODE_MAX_ROWS && M <= ROWS_MAX_ROWS && w.packed &&
+        (M <= 32 || K >= 1536) && (N + 31) / 32 <= 2 * ctx->n_compute_units))
+    return 0;
+  int n = 0;
+  if (splits == 0)
+    QUERY(k_rows_splits, n, M, N, K, ctx->force_splits);
+  else
+    n = split_count((K + 63) / 64, splits);
+  if (n > 1 && (!ctx->split_ws || (size_t)n > ctx->split_ws_floats / ((size_t)M * N))) n = 0;  // (the tiles then)
+  if (n >= 1) {
+    int takes = 0;
+    QUERY(k_rows_takes, takes, M, K, n);
+    if (!takes) n = 0;
+  }
+  *n_splits = n;
+  return 0;
+}
+
+// That product reads its rows fastest in the packed order: who makes the rows may write them so.
+static bool wants_packed(const EngCtx* ctx, int M, const EngWeight* w) {
+  int n = 0;
+  return w && rows_parts(ctx, M, *w, 0, 0, &n) == 0 && n >= 1;
+}
+
+extern "C" int eng_wants_packed_rows(const EngCtx* ctx, const EngWeight* w, int n_rows) {
+  return wants_packed(ctx, n_rows, w) ? 1 : 0;
 }
 
 static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWeight& w, const float* bias,
                   bool gelu, bool accumulate, int variant, const EngScatter* sc, int splits,
-                  EngPending* pending) {
+                  EngPending* pending, bool out_packed = false) {
   const int M = a.m.rows, K = a.m.cols, N = w.N;
+  if (a.packed && a.lazy) FAIL("linear: a norm not computed yet has no packed rows");
+  if (out_packed && (accumulate || sc || out.dtype != DT_BF16)) FAIL("linear: only a plain bfloat16 out can be packed");
   if (w.K != K) FAIL("linear: a is [%d,%d] but w is [%d,%d]", M, K, w.N, w.K);
   if (out.rows != M || out.cols != N) FAIL("linear: out is [%d,%d], want [%d,%d]", out.rows, out.cols, M, N);
   if (a.m.dtype != w.dtype || (w.dtype != DT_F32 && w.dtype != DT_BF16))
@@ -328,6 +376,11 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
   }
   float* ws = ctx->split_ws;
   const size_t ws_floats = ctx->split_ws_floats;
+  if (a.packed || out_packed) {
+    int n = 0;
+    if (M > 0) TRY(rows_parts(ctx, M, w, variant, splits, &n));
+    if (n < 1) FAIL("linear: rows in the packed order are for the product of 17 to 64 rows only");
+  }
 
   if (w.dtype == DT_BF16 && variant == 0 && M <= DECODE_MAX_ROWS) {
     const int with_norm = a.lazy ? 1 : 0;
@@ -359,34 +412,24 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
   }
 
   EngMat A;
-  TRY(materialize(ctx, a, &A));
-  // (a matrix of more blocks than two a CU, the vocabulary's, would take that kernel several rounds,
-  // each with its own wait for memory: the tiles stream it 6 us faster.  Beyond 32 rows it wins
-  // only where K is long enough for the tiles to split it: at widths 768 and 1,024 a decode
-  // step of 48 rows is 4 to 5 % slower through it, at 1,280 the same, at 1,600 4 % faster.)
-  if (w.dtype == DT_BF16 && variant == 0 && M > DECODE_MAX_ROWS && M <= ROWS_MAX_ROWS && w.packed &&
-      (M <= 32 || K >= 1536) && (N + 31) / 32 <= 2 * ctx->n_compute_units) {
-    // 17 to 48 rows: the kernel that holds a block's weights in registers, if the sizes fit it
+  if (a.packed)
+    A = a.m;
+  else
+    TRY(materialize(ctx, a, &A));
+  {
+    // 17 to 64 rows: the kernel that holds a block's weights in registers, if the sizes fit it
     int n_splits = 0;
-    if (splits == 0)
-      QUERY(k_rows_splits, n_splits, M, N, K, ctx->force_splits);
-    else
-      n_splits = split_count((K + 63) / 64, splits);
-    if (n_splits > 1 && (!ws || (size_t)n_splits > ws_floats / ((size_t)M * N))) n_splits = 0;  // (the tiles then)
-    if (n_splits >= 1) {
-      int takes = 0;
-      QUERY(k_rows_takes, takes, M, K, n_splits);
-      if (!takes) n_splits = 0;
-    }
+    TRY(rows_parts(ctx, M, w, variant, splits, &n_splits));
     if (n_splits >= 1) {
       if (n_splits > 1 && pending) TRY(settle(ctx, pending));  // the workspace is about to be written again
-      KERNEL(k_gemm_rows, ctx, out.p, A.p, A.ld, w.packed, bias, M, N, K, out.ld, flags | (sc ? GEMM_KV : 0),
+      KERNEL(k_gemm_rows, ctx, out.p, A.p, a.packed ? 0 : A.ld, w.packed, bias, M, N, K, out_packed ? 0 : out.ld,
+             flags | (sc ? GEMM_KV : 0) | (out_packed ? GEMM_OUT_PACKED : 0),
              sc ? sc->k : nullptr, sc ? sc->v : nullptr, sc ? sc->page_stride : (size_t)0,
              sc ? sc->block_table : nullptr, sc ? sc->max_blocks : 0, sc ? sc->token_req : nullptr,
              sc ? sc->positions : nullptr, sc ? sc->q_width : 0, sc ? sc->kv_width : 0, sc ? sc->head_dim : 0,
              sc ? sc->page_size : 0, n_splits, n_splits > 1 ? ws : nullptr, n_splits > 1 ? ws_floats : (size_t)0,
              ctx->stream);
-      return n_splits > 1 ? finish_parts(ctx, out, ws, n_splits, bias, gelu, accumulate, sc, pending) : 0;
+      return n_splits > 1 ? finish_parts(ctx, out, ws, n_splits, bias, gelu, accumulate, sc, pending, out_packed) : 0;
     }
   }
   if (w.dtype == DT_F32) {
@@ -453,7 +496,7 @@ static int linear(EngCtx* ctx, const EngMat& out, const EngValue& a, const EngWe
 
 extern "C" int eng_linear(EngCtx* ctx, const EngLinear* c, EngPending* pending) {
   return linear(ctx, c->out, c->a, c->w, c->bias, c->gelu != 0, c->accumulate != 0, c->variant, c->scatter,
-                c->splits, pending);
+                c->splits, pending, c->out_packed != 0);
 }
 
 // ---------------------------------------------------------------------------
@@ -478,8 +521,11 @@ struct Norm : EngPart {
   bool settles_pending = false, reads_ahead = false;
   Norm() : EngPart(KIND_NORM) {}
   // The norm of rows of the float32 stream `x` (all, or those listed in `rows`).
+  // `ahead`: the weights that the result meets first, if the caller knows them; `may_pack`: whoever
+  // takes the result takes it in the packed order too (EngValue.packed), where those weights'
+  // product reads it faster so.
   virtual int forward(EngCtx* ctx, const EngMat& x, const int* rows, int n_rows, bool lazy,
-                      const EngWeight* ahead, EngValue* out) = 0;
+                      const EngWeight* ahead, bool may_pack, EngValue* out) = 0;
 };
 
 struct Position : EngPart {
@@ -493,14 +539,14 @@ struct Position : EngPart {
 };
 
 struct Mixer : EngPart {
-  bool accepts_lazy = false;
+  bool accepts_lazy = false, accepts_packed = false;
   const EngWeight* first_weight = nullptr;
   Mixer() : EngPart(KIND_MIXER) {}
   virtual int forward(EngCtx* ctx, const EngValue& x, const EngMat& residual, int slot, bool writes) = 0;
 };
 
 struct FeedForward : EngPart {
-  bool accepts_lazy = false;
+  bool accepts_lazy = false, accepts_packed = false;
   const EngWeight* first_weight = nullptr;
   FeedForward() : EngPart(KIND_FFN) {}
   virtual int forward(EngCtx* ctx, const EngValue& x, const EngMat& residual) = 0;
@@ -529,7 +575,7 @@ struct PyNorm : Norm {
   PyNorm(int i, int flags) : id(i) {
     settles_pending = flags & ENG_SETTLES_PENDING, reads_ahead = false;
   }
-  int forward(EngCtx* ctx, const EngMat& x, const int* rows, int n_rows, bool, const EngWeight*,
+  int forward(EngCtx* ctx, const EngMat& x, const int* rows, int n_rows, bool, const EngWeight*, bool,
               EngValue* out) override {
     EngCall c = {};
     c.x = x, c.rows = rows, c.n_rows = n_rows;
@@ -624,7 +670,7 @@ struct LayerNorm : Norm {
     reads_ahead = true;      // takes the weights that its result meets first
   }
   int forward(EngCtx* ctx, const EngMat& x, const int* rows, int n_rows, bool lazy, const EngWeight* ahead,
-              EngValue* out) override {
+              bool may_pack, EngValue* out) override {
     if (x.cols != width || x.dtype != DT_F32) FAIL("layernorm: float32 rows of width %d", width);
     *out = EngValue{};
     EngPending* pending = &ctx->pending;
@@ -633,10 +679,16 @@ struct LayerNorm : Norm {
       if (!rows) TRY(can_norm(*pending, x, &fused));
       if (fused) {
         // the last projection split its sum: add the parts and norm the new rows in one kernel
-        TRY(take(ctx, x.rows, width, ctx->dtype, &out->m));
+        // (in the packed order, where the product that takes them reads that faster)
+        const bool pack = may_pack && ctx->dtype == DT_BF16 && wants_packed(ctx, x.rows, ahead);
+        if (pack)
+          TRY(take_packed(ctx, x.rows, width, &out->m));
+        else
+          TRY(take(ctx, x.rows, width, ctx->dtype, &out->m));
+        out->packed = pack ? 1 : 0;
         bool pays = false;
         if (ahead) TRY(read_ahead_pays(ctx, ahead, x.rows, false, &pays));
-        return settle_normed(ctx, pending, out->m, gamma, beta, eps, pays ? ahead : nullptr);
+        return settle_normed(ctx, pending, out->m, gamma, beta, eps, pays ? ahead : nullptr, pack);
       }
       TRY(settle(ctx, pending));
     }
@@ -666,7 +718,7 @@ struct Attention : Mixer {
   const float* out_b;
   Position* position;
 
-  Attention() { accepts_lazy = true; }
+  Attention() { accepts_lazy = true, accepts_packed = true; }
 
   int scatter_for(EngCtx* ctx, int slot, EngScatter* sc) const {
     if (slot < 0 || slot >= ctx->n_slots) FAIL("attention: cache slot %d of %d", slot, ctx->n_slots);
@@ -732,7 +784,17 @@ struct Attention : Mixer {
     return want < 1 ? 1 : (int)want;
   }
 
-  int attend(EngCtx* ctx, const EngMat& out, const EngMat& q, const EngScatter& kv) const {
+  // Whether the step's rows all go to the decode kernel, which can write its output in the
+  // packed order (the output projection of 17 to 64 rows reads that faster).
+  bool rows_only_fast(const EngCtx* ctx, const EngMat& q, const EngScatter& kv) const {
+    const int n_tiles = (int)ctx->counts[array_base + ARR_TILES] / 2;
+    const int n_rows = (int)ctx->counts[array_base + ARR_ROWS];
+    const int key_bytes = head_dim * (q.dtype == DT_BF16 ? 2 : 4);
+    return n_tiles == 0 && n_rows == q.rows && head_dim <= ATTN_ROW_MAX_HEAD_DIM &&
+           (key_bytes == 64 || key_bytes == 128 || key_bytes == 256) && kv.page_size % (1024 / key_bytes) == 0;
+  }
+
+  int attend(EngCtx* ctx, const EngMat& out, const EngMat& q, const EngScatter& kv, bool out_packed) const {
     const int* tiles = ctx->arrays[array_base + ARR_TILES];
     const int* rows = ctx->arrays[array_base + ARR_ROWS];
     const int* all_tiles = ctx->arrays[array_base + ARR_ALL_TILES];
@@ -796,7 +858,7 @@ struct Attention : Mixer {
         } else {
           ahead = nullptr;
         }
-        KERNEL(k_attn_decode, ctx, out.p, q.p, q.ld, out.ld, kv.k, kv.v, kv.page_stride, kv.block_table,
+        KERNEL(k_attn_decode, ctx, out.p, q.p, q.ld, out_packed ? 0 : out.ld, kv.k, kv.v, kv.page_stride, kv.block_table,
                kv.max_blocks, kv.token_req, kv.positions, rows, n_rows, n_heads, n_kv_heads, head_dim,
                kv.page_size, window, scale, n_splits, (float*)part_o.p, (float*)part_ml.p, n_waves,
                ahead ? ahead->packed : nullptr, ahead ? ahead->chunk_bytes : (size_t)0, chunks, rows_are_requests,
@@ -827,10 +889,14 @@ struct Attention : Mixer {
       if (writes) TRY(kv_write(ctx, k, v, kv));
     }
     EngMat out;
-    TRY(take(ctx, T, q_width, ctx->dtype, &out));
-    TRY(attend(ctx, out, q, kv));
+    const bool pack = ctx->dtype == DT_BF16 && wants_packed(ctx, T, &out_w) && rows_only_fast(ctx, q, kv);
+    if (pack)
+      TRY(take_packed(ctx, T, q_width, &out));
+    else
+      TRY(take(ctx, T, q_width, ctx->dtype, &out));
+    TRY(attend(ctx, out, q, kv, pack));
     EngValue o = {};
-    o.m = out;
+    o.m = out, o.packed = pack ? 1 : 0;
     return linear(ctx, residual, o, out_w, out_b, false, true, 0, nullptr, 0, &ctx->pending);
   }
 };
@@ -842,13 +908,20 @@ struct GeluMlp : FeedForward {
   EngWeight fc_w, proj_w;
   const float* fc_b;
   const float* proj_b;
-  GeluMlp() { accepts_lazy = true; }
+  GeluMlp() { accepts_lazy = true, accepts_packed = true; }
   int forward(EngCtx* ctx, const EngValue& x, const EngMat& residual) override {
     EngMat act;
-    TRY(take(ctx, x.m.rows, inner, ctx->dtype, &act));
-    TRY(linear(ctx, act, x, fc_w, fc_b, true, false, 0, nullptr, 0, &ctx->pending));
+    // (both products through the kernel for 17 to 64 rows: the first writes what the second reads
+    // in the packed order)
+    const int M = x.m.rows;
+    const bool pack = ctx->dtype == DT_BF16 && wants_packed(ctx, M, &fc_w) && wants_packed(ctx, M, &proj_w);
+    if (pack)
+      TRY(take_packed(ctx, M, inner, &act));
+    else
+      TRY(take(ctx, M, inner, ctx->dtype, &act));
+    TRY(linear(ctx, act, x, fc_w, fc_b, true, false, 0, nullptr, 0, &ctx->pending, pack));
     EngValue a = {};
-    a.m = act;
+    a.m = act, a.packed = pack ? 1 : 0;
     return linear(ctx, residual, a, proj_w, proj_b, false, true, 0, nullptr, 0, &ctx->pending);
   }
 };
@@ -865,21 +938,22 @@ struct PreNormBlock : Block {
   FeedForward* ffn;
   PreNormBlock() { handles_pending = true; }
 
-  static int normed(EngCtx* ctx, Norm* norm, const EngMat& h, bool lazy, const EngWeight* first, EngValue* x) {
+  static int normed(EngCtx* ctx, Norm* norm, const EngMat& h, bool lazy, bool may_pack, const EngWeight* first,
+                    EngValue* x) {
     if (!norm->settles_pending) TRY(settle(ctx, &ctx->pending));
-    return norm->forward(ctx, h, nullptr, 0, lazy, norm->reads_ahead ? first : nullptr, x);
+    return norm->forward(ctx, h, nullptr, 0, lazy, norm->reads_ahead ? first : nullptr, may_pack, x);
   }
 
   int forward(EngCtx* ctx, const EngMat& h, int slot, bool writes) override {
     const size_t mark = ctx->scratch->offset;
     EngValue x;
-    TRY(normed(ctx, mixer_norm, h, mixer->accepts_lazy, mixer->first_weight, &x));
+    TRY(normed(ctx, mixer_norm, h, mixer->accepts_lazy, mixer->accepts_packed, mixer->first_weight, &x));
     // (a mixer whose kernels leave CUs idle may have them read the weights that come after its own)
     ctx->read_ahead = ffn->first_weight;
     int rc = mixer->forward(ctx, x, h, slot, writes);
     ctx->read_ahead = nullptr;
     if (rc) return rc;
-    TRY(normed(ctx, ffn_norm, h, ffn->accepts_lazy, ffn->first_weight, &x));
+    TRY(normed(ctx, ffn_norm, h, ffn->accepts_lazy, ffn->accepts_packed, ffn->first_weight, &x));
     TRY(ffn->forward(ctx, x, h));
     ctx->scratch->offset = mark;
     return 0;
@@ -955,9 +1029,9 @@ struct Model : EngPart {
     if (ctx->n_wanted == 0) return 0;
     EngValue x;
     if (ctx->wants_every_row)
-      TRY(final_norm->forward(ctx, h, nullptr, 0, false, nullptr, &x));
+      TRY(final_norm->forward(ctx, h, nullptr, 0, false, nullptr, false, &x));
     else
-      TRY(final_norm->forward(ctx, h, ctx->wanted_rows, ctx->n_wanted, false, nullptr, &x));
+      TRY(final_norm->forward(ctx, h, ctx->wanted_rows, ctx->n_wanted, false, nullptr, false, &x));
     if (!ctx->logits || ctx->logits_rows < ctx->n_wanted) FAIL("the step's logits buffer is too small");
     const EngMat logits = {ctx->logits, ctx->n_wanted, vocab, vocab, DT_F32};
     return head->forward(ctx, x, logits);
@@ -1095,7 +1169,7 @@ extern "C" int eng_block_forward(EngPart* block, EngCtx* ctx, const EngMat* h, i
 extern "C" int eng_norm_forward(EngPart* norm, EngCtx* ctx, const EngMat* x, const int* rows, int n_rows,
                                 int lazy, const EngWeight* ahead, EngValue* out) {
   Norm* n = as<Norm>(norm, KIND_NORM, "eng_norm_forward");
-  return n ? n->forward(ctx, *x, rows, n_rows, lazy != 0, ahead, out) : 1;
+  return n ? n->forward(ctx, *x, rows, n_rows, lazy != 0, ahead, false, out) : 1;
 }
 
 extern "C" int eng_mixer_forward(EngPart* mixer, EngCtx* ctx, const EngValue* x, const EngMat* residual,
@@ -1137,8 +1211,8 @@ extern "C" int eng_pending_can_norm(const EngPending* pending, const EngMat* x) 
 }
 
 extern "C" int eng_pending_settle_normed(EngCtx* ctx, EngPending* pending, const EngMat* out, const float* gamma,
-                                         const float* beta, float eps, const EngWeight* ahead) {
-  return settle_normed(ctx, pending, *out, gamma, beta, eps, ahead);
+                                         const float* beta, float eps, const EngWeight* ahead, int out_packed) {
+  return settle_normed(ctx, pending, *out, gamma, beta, eps, ahead, out_packed != 0);
 }
 
 extern "C" int eng_read_ahead_pays(const EngCtx* ctx, const EngWeight* w, int n_rows, int with_norm) {

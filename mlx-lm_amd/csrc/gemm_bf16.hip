@@ -808,6 +808,7 @@ extern "C" int gemm_bf16_scatter(void* out, const void* A, const void* W, const 
       hipLaunchKernelGGL(gemm_bf16_skinny_kernel<4>, grid, block, 0, stream, p);
   } else if (variant == 7) {
     launch_tiles<Tile128x8>(p, stream);
+
   } else if (variant == 1 || variant == 3 || variant == 4 || variant == 5 || variant == 6) {
     if (variant == 1)
       launch_tiles<Tile128>(p, stream);

@@ -49,6 +49,7 @@
 #define FLAG_ACCUMULATE 2
 #define FLAG_OUT_F32 4
 #define FLAG_KV 8
+#define FLAG_OUT_PACKED 16  // a bfloat16 out in tiles of 16 rows x 64 columns, in the weights' packed order
 
 #define NW 8        // waves per block
 #define U 4         // k-blocks per pass and wave
@@ -79,9 +80,13 @@ struct DecodeGemmArgs {
   int rows;            // output features a block of the 16-row kernel owns (16, or 8 where features are few)
   float* ws;           // [n_splits][M][N] partial sums, when n_splits > 1
   int vec4;            // four outputs at a time: N, ldo and the scatter widths are multiples of 4, pointers aligned
+  int a_packed;        // rows kernel: A lies in tiles of 16 rows x 64 k in the weights' packed order (packed_at)
+  int row_groups;      // rows kernel: the rows go in this many groups of R_TILES tiles, a block each
+  int out_kblocks;     // FLAG_OUT_PACKED: tiles a tile row of out, (N + 63) / 64
 };
 
 __device__ __forceinline__ uint32_t pack2(float a, float b) { return pack_bf16x2(a, b); }
+
 
 union Frag {
   uint4 u;
@@ -104,7 +109,9 @@ __device__ __forceinline__ void finish(const DecodeGemmArgs& p, int m, int n, fl
     (is_v ? p.v_pages : p.k_pages)[dst] = f32_to_bf16_bits(v);
   } else {
     const size_t idx = (size_t)m * p.ldo + n;
-    if (p.flags & FLAG_ACCUMULATE)
+    if (p.flags & FLAG_OUT_PACKED)
+      ((uint16_t*)p.out)[packed_at(m, n, p.out_kblocks)] = f32_to_bf16_bits(v);
+    else if (p.flags & FLAG_ACCUMULATE)
       ((float*)p.out)[idx] += v;
     else if (p.flags & FLAG_OUT_F32)
       ((float*)p.out)[idx] = v;
@@ -134,7 +141,9 @@ __device__ __forceinline__ void finish4(const DecodeGemmArgs& p, int m, int n, f
     *(uint2*)((is_v ? p.v_pages : p.k_pages) + dst) = packed;
   } else {
     const size_t idx = (size_t)m * p.ldo + n;
-    if (p.flags & FLAG_ACCUMULATE) {
+    if (p.flags & FLAG_OUT_PACKED) {  // (four neighbouring columns from a multiple of four on stay together)
+      *(uint2*)((uint16_t*)p.out + packed_at(m, n, p.out_kblocks)) = packed;
+    } else if (p.flags & FLAG_ACCUMULATE) {
       float4* o = (float4*)((float*)p.out + idx);
       const float4 h = *o;
       *o = make_float4(h.x + v.x, h.y + v.y, h.z + v.z, h.w + v.w);
@@ -340,31 +349,45 @@ __global__ __launch_bounds__(NW * 64) void gemm_bf16_decode_kernel(DecodeGemmArg
 }
 
 // ---------------------------------------------------------------------------
-// 17 to 48 rows.  The weights still stream exactly once and all of a block's are in flight from
+// 17 to 64 rows.  The weights still stream exactly once and all of a block's are in flight from
 // its first instruction on: a block of four waves owns 32 output features (two packed chunks)
 // and a slice of K of at most 28 k-blocks; wave w takes the slice's k-blocks w, w + 4, ... and
 // holds their weights in registers (seven k-blocks of two chunks: 112 registers a lane).  The
 // activations are the MFMA's other operand, two or three tiles of 16 rows, read straight from
-// memory (the L2s: every block reads the same rows) a k-block ahead; no LDS on the way.  The four
-// waves' tiles are summed in their order through LDS and finished as in the kernel above.  The
-// tile kernels of gemm_bf16.hip need K split over some 220 blocks at these sizes and a second
-// kernel for the sum; here the wide products are one launch of 150 or 200 blocks, and the narrow
-// ones split K in two or four.  A decode step of GPT-2 XL's sizes at batch 17 / 24 / 32 / 40 / 48:
-// 2.93 / 3.23 / 3.52 / 3.97 / 4.44 ms instead of 3.34 / 3.64 / 3.91 / 4.23 / 4.64 through the
-// tiles.  (With four tiles of rows a block reads twice as many bytes of rows as of weights, and
-// at 56 to 64 rows the tiles are as fast or faster: 5.13 against 5.23 ms at batch 64.  A variant
-// with eight waves that held their k-blocks of rows as well as of weights, one trip to memory
-// for everything, was slower at every size.)
+// memory (the L2s: every block reads the same rows) a k-block ahead; no LDS on the way.  They
+// come row-major or, much faster, in the packed order (packed_at: a wave's load is then 1 KB of
+// consecutive bytes instead of sixteen pieces of 64: GPT-2 XL's four products at 48 rows took
+// 15.8 / 17.3 / 12.8 / 17.0 us from rows and 10.8 / 12.4 / 8.0 / 11.8 packed), which the kernels
+// that make these rows write where the host asks them to (the sum-and-norm, decode attention,
+// this kernel's own epilogue).  The four waves' tiles are summed in their order through LDS and
+// finished as in the kernel above.  The tile kernels of gemm_bf16.hip need K split over some 220
+// blocks at these sizes and a second kernel for the sum; here the wide products are one launch of
+// 150 or 200 blocks, and the narrow ones split K in two or four.  49 to 64 rows go as two groups
+// of two tiles, a block each, eight block ids apart: both on one die, so that the second finds
+// the weights in that die's L2 (the fetch counter shows them read from memory once).
+// (Other shapes measured at 64 rows of GPT-2 XL's sizes, packed rows, a decode step of twelve
+// layers: four tiles a block with 32 features and four or eight waves 1.34 and 1.29 ms, with 16
+// features 1.58, sixteen waves that hold everything after one trip to memory 1.65; two groups
+// 1.28; the tile kernels with K split and their second kernels 1.33.)
 #define RW 4          // waves a block
 #define R_FEATURES 32 // output features a block
 #define R_HELD 7      // k-blocks whose weights a wave holds
-#define ROWS_MAX_M 48
+#define ROWS_MAX_M 64
+#define ROWS_GROUP_FROM 49    // from this many rows on: groups of 32 rows, a block each
 #define ROWS_WANT_BLOCKS 100  // a split of K where the features give fewer blocks than this
-template <int R_TILES>  // tiles of 16 rows
-__global__ __launch_bounds__(RW * 64) void gemm_bf16_rows_kernel(DecodeGemmArgs p) {
-  __shared__ float red[RW][R_TILES * 2][256];
+// R_TILES: tiles of 16 rows; FT: chunks of 16 features a block; WAVES: waves a block; HELD: k-blocks a wave holds
+template <int R_TILES, int FT, int WAVES, int HELD>
+__global__ __launch_bounds__(WAVES * 64) void gemm_bf16_rows_kernel(DecodeGemmArgs p) {
+  __shared__ float red[WAVES][R_TILES * FT][256];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n0 = blockIdx.x * R_FEATURES;
+  // Blocks go to the dies in turn (block b to die b % 8).  The groups of rows that meet the same
+  // weights are eight block ids apart: on one die, one after the other, so that only the first
+  // fetches the weights from memory and the others find them in the die's L2.
+  const int within = blockIdx.x % (8 * p.row_groups);
+  const int group = within >> 3;
+  const int n0 = ((blockIdx.x / (8 * p.row_groups)) * 8 + (within & 7)) * (16 * FT);
+  const int t0 = group * R_TILES;  // this block's first tile of rows
+  if (n0 >= p.N) return;           // (the grid is padded to whole eights of feature blocks)
   const int n_chunks_all = (p.K + 63) / 64;
   const int c_begin = blockIdx.y * p.chunks_per_split;
   const int n_chunks = min(n_chunks_all, c_begin + p.chunks_per_split) - c_begin;
@@ -372,12 +395,12 @@ __global__ __launch_bounds__(RW * 64) void gemm_bf16_rows_kernel(DecodeGemmArgs 
   const int koff = (lane >> 4) * 16;
 
   // the weights, all at once (k-blocks beyond the slice repeat its last one and are not used)
-  Frag w[R_HELD][2][2];
+  Frag w[HELD][FT][2];
 #pragma unroll
-  for (int i = 0; i < R_HELD; ++i) {
-    const int c = c_begin + min(wave + RW * i, n_chunks - 1);
+  for (int i = 0; i < HELD; ++i) {
+    const int c = c_begin + min(wave + WAVES * i, n_chunks - 1);
 #pragma unroll
-    for (int ft = 0; ft < 2; ++ft) {
+    for (int ft = 0; ft < FT; ++ft) {
       const int fb = min((n0 >> 4) + ft, n_fb - 1);  // (a second chunk beyond the matrix repeats the first)
       const uint16_t* t = p.W + ((size_t)fb * n_chunks_all + c) * 1024 + lane * 8;
       w[i][ft][0].u = *(const uint4*)t;
@@ -388,23 +411,34 @@ __global__ __launch_bounds__(RW * 64) void gemm_bf16_rows_kernel(DecodeGemmArgs 
   // (l / 16) * 16 on (rows beyond M repeat the last; what they give is not stored)
   const uint16_t* arow[R_TILES];
 #pragma unroll
-  for (int rt = 0; rt < R_TILES; ++rt) arow[rt] = p.A + (size_t)min(rt * 16 + (lane & 15), p.M - 1) * p.lda;
+  for (int rt = 0; rt < R_TILES; ++rt) arow[rt] = p.A + (size_t)min((t0 + rt) * 16 + (lane & 15), p.M - 1) * p.lda;
+  const int m_tiles = (p.M + 15) / 16;
   auto load_a = [&](Frag (&a)[R_TILES][2], int i) {
-    const int k = (c_begin + min(wave + RW * i, n_chunks - 1)) * 64 + koff;
+    const int c = c_begin + min(wave + WAVES * i, n_chunks - 1);
+    const int k = c * 64 + koff;
+    if (p.a_packed) {
 #pragma unroll
-    for (int rt = 0; rt < R_TILES; ++rt) {
-      a[rt][0].u = *(const uint4*)(arow[rt] + min(k, p.K - 8));
-      a[rt][1].u = *(const uint4*)(arow[rt] + min(k + 8, p.K - 8));
+      for (int rt = 0; rt < R_TILES; ++rt) {
+        const uint16_t* t = p.A + ((size_t)min(t0 + rt, m_tiles - 1) * n_chunks_all + c) * 1024 + lane * 8;
+        a[rt][0].u = *(const uint4*)t;
+        a[rt][1].u = *(const uint4*)(t + 512);
+      }
+    } else {
+#pragma unroll
+      for (int rt = 0; rt < R_TILES; ++rt) {
+        a[rt][0].u = *(const uint4*)(arow[rt] + min(k, p.K - 8));
+        a[rt][1].u = *(const uint4*)(arow[rt] + min(k + 8, p.K - 8));
+      }
     }
   };
-  f32x4_t acc[R_TILES][2];
+  f32x4_t acc[R_TILES][FT];
 #pragma unroll
   for (int rt = 0; rt < R_TILES; ++rt)
 #pragma unroll
-    for (int ft = 0; ft < 2; ++ft) acc[rt][ft] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int ft = 0; ft < FT; ++ft) acc[rt][ft] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   auto multiply = [&](Frag (&a)[R_TILES][2], int i) {
-    if (wave + RW * i >= n_chunks) return;  // (uniform over the wave)
-    const int k = (c_begin + wave + RW * i) * 64 + koff;
+    if (wave + WAVES * i >= n_chunks) return;  // (uniform over the wave)
+    const int k = (c_begin + wave + WAVES * i) * 64 + koff;
     // columns beyond K meet zero weights (the packed order pads them), but must not be NaN
     const bool in0 = k < p.K, in1 = k + 8 < p.K;
 #pragma unroll
@@ -412,7 +446,7 @@ __global__ __launch_bounds__(RW * 64) void gemm_bf16_rows_kernel(DecodeGemmArgs 
       Frag a0, a1;
       a0.u = in0 ? a[rt][0].u : ZERO4, a1.u = in1 ? a[rt][1].u : ZERO4;
 #pragma unroll
-      for (int ft = 0; ft < 2; ++ft) {
+      for (int ft = 0; ft < FT; ++ft) {
         acc[rt][ft] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[i][ft][0].v, a0.v, acc[rt][ft], 0, 0, 0);
         acc[rt][ft] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[i][ft][1].v, a1.v, acc[rt][ft], 0, 0, 0);
       }
@@ -421,39 +455,37 @@ __global__ __launch_bounds__(RW * 64) void gemm_bf16_rows_kernel(DecodeGemmArgs 
   Frag a0[R_TILES][2], a1[R_TILES][2];
   load_a(a0, 0);
 #pragma unroll
-  for (int i = 0; i < R_HELD; i += 2) {
-    if (i + 1 < R_HELD) load_a(a1, i + 1);
+  for (int i = 0; i < HELD; i += 2) {
+    if (i + 1 < HELD) load_a(a1, i + 1);
     multiply(a0, i);
-    if (i + 2 < R_HELD) load_a(a0, i + 2);
-    if (i + 1 < R_HELD) multiply(a1, i + 1);
+    if (i + 2 < HELD) load_a(a0, i + 2);
+    if (i + 1 < HELD) multiply(a1, i + 1);
   }
 
   // ---- sum the waves' tiles in their order, then the epilogue -----------------
 #pragma unroll
   for (int rt = 0; rt < R_TILES; ++rt)
 #pragma unroll
-    for (int ft = 0; ft < 2; ++ft)
+    for (int ft = 0; ft < FT; ++ft)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) red[wave][rt * 2 + ft][lane * 4 + r] = acc[rt][ft][r];
+      for (int r = 0; r < 4; ++r) red[wave][rt * FT + ft][lane * 4 + r] = acc[rt][ft][r];
   __syncthreads();
-  // element tid = 4 * L + r of a tile: feature 4 * (L / 16) + r, row L % 16
-  const int L = tid >> 2, r = tid & 3;
+  // element e = 4 * L + r of a tile: feature 4 * (L / 16) + r, row L % 16; 256 threads a tile
+  const int e = tid & 255, L = e >> 2, r = e & 3;
+  for (int t = tid >> 8; t < R_TILES * FT; t += WAVES / 4) {
+    const int rt = t / FT, ft = t - rt * FT;
+    float v = 0.f;
 #pragma unroll
-  for (int rt = 0; rt < R_TILES; ++rt)
-#pragma unroll
-    for (int ft = 0; ft < 2; ++ft) {
-      float v = 0.f;
-#pragma unroll
-      for (int wv = 0; wv < RW; ++wv) v += red[wv][rt * 2 + ft][tid];
-      const int n = n0 + ft * 16 + 4 * (L >> 4) + r;
-      const int m = rt * 16 + (L & 15);
-      if (m < p.M && n < p.N) {
-        if (p.n_splits > 1)
-          p.ws[((size_t)blockIdx.y * p.M + m) * p.N + n] = v;  // summed, and finished, by sum_partials
-        else
-          finish(p, m, n, v);
-      }
+    for (int wv = 0; wv < WAVES; ++wv) v += red[wv][t][e];
+    const int n = n0 + ft * 16 + 4 * (L >> 4) + r;
+    const int m = (t0 + rt) * 16 + (L & 15);
+    if (m < p.M && n < p.N) {
+      if (p.n_splits > 1)
+        p.ws[((size_t)blockIdx.y * p.M + m) * p.N + n] = v;  // summed, and finished, by sum_partials
+      else
+        finish(p, m, n, v);
     }
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -498,6 +530,7 @@ struct SumNormArgs {
   void* out;
   float eps;
   int M, N, ldh, n_splits, out_dtype;
+  int out_packed;  // out (bfloat16) in the packed order of packed_at, for a product that takes its rows so
   // Blocks beyond the M rows read `ahead` (16-byte pieces) and drop it: the weights of the
   // product that comes next, which then finds them in the caches.  A row a block leaves nearly
   // every CU idle, and so does the memory.
@@ -599,7 +632,7 @@ __global__ __launch_bounds__(256) void sum_partials_norm_kernel(SumNormArgs q) {
     } else {
       uint2 o;
       o.x = pack2(y0, y1), o.y = pack2(y2, y3);
-      *(uint2*)((uint16_t*)q.out + (size_t)m * q.N + k) = o;
+      *(uint2*)((uint16_t*)q.out + (q.out_packed ? packed_at(m, k, (q.N + 63) / 64) : (size_t)m * q.N + k)) = o;
     }
   }
 }
@@ -661,6 +694,8 @@ static int fill_epilogue(DecodeGemmArgs& p, const char* who, void* out, const fl
   if (!out) FAIL("%s: null pointer", who);
   if ((flags & FLAG_ACCUMULATE) && (flags & (FLAG_GELU | FLAG_KV)))
     FAIL("%s: accumulate cannot be combined with GELU or the cache scatter", who);
+  if ((flags & FLAG_OUT_PACKED) && (flags & (FLAG_ACCUMULATE | FLAG_OUT_F32 | FLAG_KV)))
+    FAIL("%s: the packed order is for a bfloat16 out that is neither added to nor scattered", who);
   if (flags & FLAG_KV) {
     if (!k_pages || !v_pages || !block_table || !token_req || !positions)
       FAIL("%s: the cache scatter needs pages, block table, token_req and positions", who);
@@ -669,7 +704,7 @@ static int fill_epilogue(DecodeGemmArgs& p, const char* who, void* out, const fl
            q_width, kv_width, N, head_dim);
     if (flags & (FLAG_OUT_F32 | FLAG_GELU)) FAIL("%s: the cache scatter writes bfloat16, no GELU", who);
     if (ldo < q_width) FAIL("%s: ldo=%d smaller than q_width=%d", who, ldo, q_width);
-  } else if (ldo < N) {
+  } else if (ldo < N && !(flags & FLAG_OUT_PACKED)) {
     FAIL("%s: ldo=%d smaller than N=%d", who, ldo, N);
   }
   p.bias = bias, p.out = out, p.M = M, p.N = N, p.ldo = ldo, p.flags = flags;
@@ -677,6 +712,7 @@ static int fill_epilogue(DecodeGemmArgs& p, const char* who, void* out, const fl
   p.block_table = block_table, p.token_req = token_req, p.positions = positions;
   p.max_blocks = max_blocks, p.q_width = q_width, p.kv_width = kv_width;
   p.head_dim = head_dim, p.page_size = page_size;
+  p.out_kblocks = (N + 63) / 64;
   p.vec4 = N % 4 == 0 && ldo % 4 == 0 && aligned16(out) && aligned16(bias);
   if (flags & FLAG_KV)
     p.vec4 = p.vec4 && q_width % 4 == 0 && kv_width % 4 == 0 && head_dim % 4 == 0 && page_stride % 4 == 0 &&
@@ -772,8 +808,12 @@ extern "C" int gemm_bf16_rows_splits(int M, int N, int K, int force) {
   return gemm_bf16_rows_takes(M, K, n) ? n : 0;
 }
 
-// The product for 17 to 48 rows (see gemm_bf16_rows_kernel): W in the packed order only.  With
-// n_splits > 1 the partial sums go to `ws` and sum_partials or sum_partials_norm finishes.
+// The product for 17 to 64 rows (see gemm_bf16_rows_kernel): W in the packed order only; A
+// row-major, or with lda == 0 in the packed order of packed_at ([M, K] in tiles of 16 rows x 64
+// columns; what lies beyond row M or column K is never used and need not be written).  Flag 16
+// (with a bfloat16 out, no accumulate, no scatter) writes out in that order too, for the product
+// that reads it next; ldo is not used then.  With n_splits > 1 the partial sums go to `ws` and
+// sum_partials or sum_partials_norm finishes.
 extern "C" int gemm_bf16_rows(void* out, const void* A, int lda, const void* W, const float* bias, int M,
                               int N, int K, int ldo, int flags, void* k_pages, void* v_pages,
                               size_t page_stride, const int* block_table, int max_blocks,
@@ -785,13 +825,15 @@ extern "C" int gemm_bf16_rows(void* out, const void* A, int lda, const void* W, 
     FAIL("gemm_bf16_rows: M=%d K=%d in %d splits is outside what this kernel takes", M, K, n_splits);
   if (!A || !W) FAIL("gemm_bf16_rows: null pointer");
   if (!aligned16(W)) FAIL("gemm_bf16_rows: W must be 16-byte aligned");
-  if (lda % 8 != 0 || lda < K || !aligned16(A)) FAIL("gemm_bf16_rows: A rows must be 16-byte aligned");
+  if (lda != 0 && (lda % 8 != 0 || lda < K)) FAIL("gemm_bf16_rows: A rows must be 16-byte aligned");
+  if (!aligned16(A)) FAIL("gemm_bf16_rows: A must be 16-byte aligned");
   DecodeGemmArgs p = {};
   if (fill_epilogue(p, "gemm_bf16_rows", out, bias, M, N, ldo, flags, k_pages, v_pages, page_stride,
                     block_table, max_blocks, token_req, positions, q_width, kv_width, head_dim, page_size))
     return -1;
   p.W = (const uint16_t*)W, p.A = (const uint16_t*)A;
   p.K = K, p.lda = lda, p.ldw = 0;
+  p.a_packed = lda == 0;
   p.n_splits = n_splits, p.chunks_per_split = chunks_per_split(K, n_splits);
   p.ws = ws;
   if (n_splits > 1) {
@@ -799,11 +841,15 @@ extern "C" int gemm_bf16_rows(void* out, const void* A, int lda, const void* W, 
     if (ws_floats < (size_t)n_splits * M * N)
       FAIL("gemm_bf16_rows: workspace of %zu floats is too small for %d splits of %d x %d", ws_floats, n_splits, M, N);
   }
-  const dim3 grid((N + R_FEATURES - 1) / R_FEATURES, n_splits), block(RW * 64);
-  if (M <= 32)
-    hipLaunchKernelGGL(gemm_bf16_rows_kernel<2>, grid, block, 0, stream, p);
+  p.row_groups = M >= ROWS_GROUP_FROM ? (M + 31) / 32 : 1;
+  // (the grid holds whole eights of feature blocks, so that a group's blocks and the next group's
+  // are on the same dies; the surplus blocks return at once)
+  const int fbs = ((N + R_FEATURES - 1) / R_FEATURES + 7) / 8 * 8;
+  const dim3 grid(fbs * p.row_groups, n_splits), block(RW * 64);
+  if (M <= 32 || p.row_groups > 1)
+    hipLaunchKernelGGL((gemm_bf16_rows_kernel<2, 2, RW, R_HELD>), grid, block, 0, stream, p);
   else
-    hipLaunchKernelGGL(gemm_bf16_rows_kernel<3>, grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gemm_bf16_rows_kernel<3, 2, RW, R_HELD>), grid, block, 0, stream, p);
   CHECK_LAUNCH("gemm_bf16_rows");
   return 0;
 }
@@ -831,11 +877,12 @@ extern "C" int sum_partials(void* out, const float* ws, int n_splits, const floa
 // 1 if sum_partials_norm takes this width
 extern "C" int sum_partials_norm_takes(int N, int ldh) { return N > 0 && N % 4 == 0 && N <= 8192 && ldh % 4 == 0; }
 
-// h[m] += bias + sum of the partial products;  out[m] = LayerNorm(h[m]) (float32 or bfloat16, [M][N])
+// h[m] += bias + sum of the partial products;  out[m] = LayerNorm(h[m]) (float32 or bfloat16, [M][N];
+// with out_packed a bfloat16 out in the packed order that gemm_bf16_rows reads fastest)
 extern "C" int sum_partials_norm(float* h, int ldh, const float* ws, int n_splits, const float* bias,
                                  const float* gamma, const float* beta, float eps, void* out,
-                                 int out_dtype, int M, int N, const void* ahead, size_t ahead_chunk_bytes,
-                                 int ahead_chunks, hipStream_t stream) {
+                                 int out_dtype, int out_packed, int M, int N, const void* ahead,
+                                 size_t ahead_chunk_bytes, int ahead_chunks, hipStream_t stream) {
   if (M == 0) return 0;
   if (ahead && (!aligned16(ahead) || ahead_chunk_bytes % 16 != 0 || ahead_chunks < 0))
     FAIL("sum_partials_norm: what is read ahead must be chunks of 16-byte pieces");
@@ -845,7 +892,9 @@ extern "C" int sum_partials_norm(float* h, int ldh, const float* ws, int n_split
   if (!aligned16(h) || !aligned16(ws) || !aligned16(bias) || !aligned16(gamma) || !aligned16(beta) || !aligned16(out))
     FAIL("sum_partials_norm: pointers must be 16-byte aligned");
   if (out_dtype != DT_F32 && out_dtype != DT_BF16) FAIL("sum_partials_norm: unknown dtype code %d", out_dtype);
+  if (out_packed && out_dtype != DT_BF16) FAIL("sum_partials_norm: the packed order is for a bfloat16 out");
   SumNormArgs q;
+  q.out_packed = out_packed ? 1 : 0;
   q.h = h, q.ws = ws, q.bias = bias, q.gamma = gamma, q.beta = beta, q.out = out, q.eps = eps;
   q.M = M, q.N = N, q.ldh = ldh, q.n_splits = n_splits, q.out_dtype = out_dtype;
   q.ahead = (const uint4*)ahead, q.ahead_pieces = ahead ? ahead_chunk_bytes / 16 : 0;

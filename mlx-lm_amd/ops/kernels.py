@@ -221,6 +221,52 @@ class PackedWeight:
                                   w.stride(0) if keep_rows else 0, DT[w.dtype], self.chunk_bytes, self.n_chunks, 0)
 
 
+class PackedRows:
+    """bfloat16 activations ``[M, K]`` in the order in which the product of 17 to 64 rows reads them
+    fastest: tiles of 16 rows by 64 columns, each laid out like a tile of ``PackedWeight``.  What
+    lies beyond row ``M`` or column ``K`` in the last tiles is never used.
+
+    ``PackedRows.empty(M, K, device)`` makes room for a kernel to write into
+    (``sum_partials_norm(..., out=...)``, ``attn_decode``, ``linear(out=...)``);
+    ``PackedRows.of(a)`` packs a row-major matrix and ``.rows()`` gives it back (tests)."""
+
+    def __init__(self, data, shape):
+        self.data, self.shape = data, tuple(shape)
+        self.dtype, self.device = data.dtype, data.device
+
+    @classmethod
+    def empty(cls, M, K, device):
+        n = (M + 15) // 16 * ((K + 63) // 64) * 1024
+        return cls(torch.zeros(n, dtype=torch.bfloat16, device=device), (M, K))
+
+    @classmethod
+    def of(cls, a):
+        _need(a.dtype == torch.bfloat16 and a.dim() == 2, "PackedRows: a 2-D bfloat16 matrix")
+        M, K = a.shape
+        Mp, Kp = (M + 15) // 16 * 16, (K + 63) // 64 * 64
+        padded = torch.zeros((Mp, Kp), dtype=a.dtype, device=a.device)
+        padded[:M, :K] = a
+        t = padded.view(Mp // 16, 16, Kp // 64, 4, 2, 8).permute(0, 2, 4, 3, 1, 5)
+        return cls(t.contiguous().view(-1), (M, K))
+
+    def rows(self):
+        M, K = self.shape
+        Mp, Kp = (M + 15) // 16 * 16, (K + 63) // 64 * 64
+        t = self.data.view(Mp // 16, Kp // 64, 2, 4, 16, 8).permute(0, 4, 1, 3, 2, 5)
+        return t.reshape(Mp, Kp)[:M, :K].contiguous()
+
+    def data_ptr(self):
+        return self.data.data_ptr()
+
+
+def wants_packed_rows(w, n_rows):
+    """Whether the product of ``n_rows`` rows with ``w`` (a ``PackedWeight``) reads its rows fastest
+    as ``PackedRows``: the kernel that holds a block's weights in registers takes it."""
+    if not isinstance(w, PackedWeight):
+        return False
+    return bool(native.lib().eng_wants_packed_rows(ctypes.byref(bare_context()), ctypes.byref(w.c), int(n_rows)))
+
+
 def weight_struct(w):
     """The native description of a weight matrix (a ``PackedWeight`` or a 2-D tensor ``[N, K]``)."""
     if isinstance(w, PackedWeight):
@@ -309,12 +355,17 @@ class PendingSum:
     def settle_normed(self, out, gamma, beta, eps, ahead=None):
         """Add what is pending into its target and write the LayerNorm of the new rows to ``out``.
 
-        ``ahead``: the weights of the product that reads ``out`` (see ``sum_partials_norm``)."""
-        _need(out.is_contiguous(), "settle_normed: out must be contiguous")
-        m = native.mat(out)
+        ``ahead``: the weights of the product that reads ``out`` (see ``sum_partials_norm``);
+        ``out`` may be a ``PackedRows`` where that product reads its rows fastest so."""
+        packed = isinstance(out, PackedRows)
+        if packed:
+            m = native.EngMat(out.data_ptr(), out.shape[0], out.shape[1], 0, DT[out.dtype])
+        else:
+            _need(out.is_contiguous(), "settle_normed: out must be contiguous")
+            m = native.mat(out)
         native.check(native.lib().eng_pending_settle_normed(
             ctypes.byref(self._native()), ctypes.byref(self.c), ctypes.byref(m), native.ptr(gamma),
-            native.ptr(beta), float(eps), ctypes.byref(ahead.c) if ahead is not None else None))
+            native.ptr(beta), float(eps), ctypes.byref(ahead.c) if ahead is not None else None, 1 if packed else 0))
 
     def can_norm(self, x):
         if not self.waits_on(x) or x.stride(1) != 1:
@@ -365,15 +416,20 @@ def sum_partials_norm(h, ws, n_splits, bias, gamma, beta, eps, out, ahead=None):
     M, N = h.shape
     _dev(h, "h", torch.float32)
     _dev(ws, "ws", torch.float32)
-    _dev(out, "out")
-    _need(out.dtype in DT and tuple(out.shape) == (M, N) and out.is_contiguous(), "sum_partials_norm: out")
+    packed = isinstance(out, PackedRows)
+    if packed:
+        _need(out.shape == (M, N), "sum_partials_norm: out's shape")
+    else:
+        _dev(out, "out")
+        _need(out.dtype in DT and tuple(out.shape) == (M, N) and out.is_contiguous(), "sum_partials_norm: out")
     _need(ws.numel() >= n_splits * M * N, "sum_partials_norm: workspace too small")
     for name, v in (("bias", bias), ("gamma", gamma), ("beta", beta)):
         if v is not None:
             _dev(v, name, torch.float32)
             v.numel() == N or _fail(f"sum_partials_norm: {name} has {v.numel()} elements, width is {N}")
     rc = lib.sum_partials_norm(_ptr(h), _c_int(_rows2d(h, "h")), _ptr(ws), _c_int(n_splits), _ptr(bias),
-                               _ptr(gamma), _ptr(beta), _c_float(eps), _ptr(out), _c_int(DT[out.dtype]),
+                               _ptr(gamma), _ptr(beta), _c_float(eps), _ptr(out.data if packed else out),
+                               _c_int(DT[out.dtype]), _c_int(1 if packed else 0),
                                _c_int(M), _c_int(N), _ptr(ahead.packed if ahead is not None else None),
                                _c_size_t(ahead.chunk_bytes if ahead is not None else 0),
                                _c_int(ahead.n_chunks if ahead is not None else 0), _stream())
@@ -415,9 +471,16 @@ def linear(out, a, w, bias=None, gelu=False, accumulate=False, variant=0, scatte
         call.a.lazy, call.a.ldx = 1, a.x.stride(0)
         call.a.m = native.EngMat(None, a.shape[0], a.shape[1], a.shape[1], DT[a.dtype])
         call.a.x, call.a.gamma, call.a.beta, call.a.eps = a.x.data_ptr(), native.ptr(a.gamma), native.ptr(a.beta), a.eps
+    elif isinstance(a, PackedRows):
+        call.a.m = native.EngMat(a.data_ptr(), a.shape[0], a.shape[1], 0, DT[a.dtype])
+        call.a.packed = 1
     else:
         call.a.m = native.mat(a)
-    call.out = native.mat(out)
+    if isinstance(out, PackedRows):
+        call.out = native.EngMat(out.data_ptr(), out.shape[0], out.shape[1], 0, DT[out.dtype])
+        call.out_packed = 1
+    else:
+        call.out = native.mat(out)
     if bias is not None:
         _dev(bias, "bias", torch.float32)
         _need(bias.numel() == N, "linear: bias length")
@@ -587,10 +650,13 @@ def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_h
     ``rows_are_requests``: item ``i`` of ``rows`` is row ``i`` of request ``i`` (the caller says so).
     ``key_tile``: 32 or 64 keys a wave at a time."""
     lib = build.load("attention_decode")
-    ldq, ldo = _rows2d(q, "q"), _rows2d(out, "out")
+    packed_out = isinstance(out, PackedRows)  # (the order that the product after attention reads fastest)
+    ldq, ldo = _rows2d(q, "q"), 0 if packed_out else _rows2d(out, "out")
     _need(q.dtype in (torch.bfloat16, torch.float32), "attn_decode: bfloat16 or float32")
     _need(q.shape[1] == n_heads * kv.head_dim, "attn_decode: q width must be n_heads*head_dim")
     _need(out.shape[1] == n_heads * kv.head_dim and out.dtype == q.dtype, "attn_decode: out shape/dtype")
+    if packed_out:
+        _need(out.shape[0] >= q.shape[0], "attn_decode: out has fewer rows than q")
     _attn_common(q, kv, block_table, token_req, positions)
     _dev(rows, "rows", torch.int32)
     _need(rows.numel() >= n_rows, "attn_decode: row list too short")
@@ -602,7 +668,7 @@ def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_h
     if rows_are_requests:
         _need(n_rows <= block_table.shape[0], "attn_decode: more rows than requests")
     rc = lib.attn_decode_rows(
-        _ptr(out), _ptr(q), _c_int(ldq), _c_int(ldo), _ptr(kv.k), _ptr(kv.v),
+        _ptr(out.data if packed_out else out), _ptr(q), _c_int(ldq), _c_int(ldo), _ptr(kv.k), _ptr(kv.v),
         _c_size_t(kv.page_stride), _ptr(block_table), _c_int(block_table.shape[1]),
         _ptr(token_req), _ptr(positions), _ptr(rows), _c_int(n_rows), _c_int(n_heads),
         _c_int(kv.n_kv_heads), _c_int(kv.head_dim), _c_int(kv.page_size), _c_int(window),

@@ -40,7 +40,7 @@ class EngWeight(Structure):
 
 class EngValue(Structure):
     _fields_ = [("m", EngMat), ("lazy", c_int), ("ldx", c_int), ("x", c_void_p), ("gamma", c_void_p),
-                ("beta", c_void_p), ("eps", c_float), ("pad_", c_int)]
+                ("beta", c_void_p), ("eps", c_float), ("packed", c_int)]
 
 
 class EngPending(Structure):
@@ -94,7 +94,7 @@ class EngScatter(Structure):
 class EngLinear(Structure):
     _fields_ = [("out", EngMat), ("a", EngValue), ("w", EngWeight), ("bias", c_void_p),
                 ("scatter", POINTER(EngScatter)), ("gelu", c_int), ("accumulate", c_int), ("variant", c_int),
-                ("splits", c_int)]
+                ("splits", c_int), ("out_packed", c_int), ("pad_", c_int)]
 
 
 _RESOLVER = ctypes.CFUNCTYPE(c_void_p, c_char_p, c_char_p)
@@ -172,8 +172,9 @@ def lib():
         "eng_pending_settle": (c_int, [POINTER(EngCtx), POINTER(EngPending)]),
         "eng_pending_can_norm": (c_int, [POINTER(EngPending), POINTER(EngMat)]),
         "eng_pending_settle_normed": (c_int, [POINTER(EngCtx), POINTER(EngPending), POINTER(EngMat), P, P,
-                                              c_float, POINTER(EngWeight)]),
+                                              c_float, POINTER(EngWeight), c_int]),
         "eng_read_ahead_pays": (c_int, [POINTER(EngCtx), POINTER(EngWeight), c_int, c_int]),
+        "eng_wants_packed_rows": (c_int, [POINTER(EngCtx), POINTER(EngWeight), c_int]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)

@@ -846,7 +846,7 @@ def test_gemm_bf16_reads_weights_kept_in_packed_order_only(M, N, K):
             outs.append(out)
         # (left to itself the library takes another kernel for 17 to 64 rows of packed weights,
         # which adds in another order)
-        if variant != 0 or not 16 < M <= 48:
+        if variant != 0 or not 16 < M <= 64:
             assert torch.equal(outs[0], outs[1]), (variant, splits)
         assert torch.allclose(outs[1].double().cpu(), plain.gelu_tanh(ref), rtol=2**-7, atol=1e-3), (variant, splits)
 
@@ -856,10 +856,10 @@ def test_gemm_bf16_reads_weights_kept_in_packed_order_only(M, N, K):
 @pytest.mark.parametrize("mode", ["plain", "gelu", "accumulate", "f32out"])
 @pytest.mark.parametrize("packed", [False, True])
 def test_gemm_bf16_17_to_64_rows(M, N, K, mode, packed):
-    """17 to 64 rows, the library's own choice of kernel and parts: up to 48 rows of packed weights
-    the kernel that holds a block's weights in registers (32 features a block; K in parts where
-    that gives few blocks or a part would be longer than a block holds), otherwise tiles of
-    32 x 128 and 64 x 128 with K split over blocks."""
+    """17 to 64 rows, the library's own choice of kernel and parts: with packed weights the kernel
+    that holds a block's weights in registers (32 features a block; K in parts where that gives
+    few blocks or a part would be longer than a block holds; from 49 rows on two groups of rows,
+    a block each), otherwise tiles of 32 x 128 and 64 x 128 with K split over blocks."""
     k = _k()
     a = _rand((M, K), torch.bfloat16, 10)
     w = _rand((N, K), torch.bfloat16, 11, 0.1)
@@ -890,7 +890,7 @@ def test_gemm_bf16_17_to_64_rows(M, N, K, mode, packed):
 @pytest.mark.parametrize("M,N,K", [(17, 48, 1024), (48, 1600, 6400), (24, 333, 1608), (33, 4800, 1600), (32, 1000, 1792),
                                    (41, 72, 136), (20, 100, 1856)])
 def test_gemm_bf16_rows_kernel_in_parts_and_with_the_cache_scatter(M, N, K):
-    """The kernel for 17 to 48 rows, asked for directly: whole and with K in 2, 3 and 8 parts (the
+    """The kernel for 17 to 64 rows, asked for directly: whole and with K in 2, 3 and 8 parts (the
     same bits run after run), at the longest slice it holds (28 k-blocks), refusing a longer one,
     and with keys and values going to their pages from its epilogue or from the second kernel."""
     k = _k()
@@ -899,7 +899,7 @@ def test_gemm_bf16_rows_kernel_in_parts_and_with_the_cache_scatter(M, N, K):
     lib = build.load("gemm_bf16_decode")
     n_blocks = (K + 63) // 64
     assert lib.gemm_bf16_rows_takes(M, K, 1) == (1 if n_blocks <= 28 else 0)
-    assert lib.gemm_bf16_rows_takes(16, K, 1) == 0 and lib.gemm_bf16_rows_takes(49, K, 1) == 0
+    assert lib.gemm_bf16_rows_takes(16, K, 1) == 0 and lib.gemm_bf16_rows_takes(65, K, 1) == 0
     auto = lib.gemm_bf16_rows_splits(M, N, K, 0)
     assert auto >= 1 and (n_blocks + auto - 1) // auto <= 28
     a = _rand((M, K), torch.bfloat16, 10)
@@ -948,6 +948,100 @@ def test_gemm_bf16_rows_kernel_in_parts_and_with_the_cache_scatter(M, N, K):
                 assert torch.allclose(c.pool[written].float(), want_pool[written].float(), rtol=2**-6, atol=2e-3)
             assert torch.isnan(out[:, qw:].float()).all()
             assert written.any() and torch.isnan(c.pool[~written].float()).all()
+
+
+@pytest.mark.parametrize("M,N,K", [(17, 48, 64), (33, 257, 1536), (64, 4800, 1600), (40, 1600, 6400), (49, 333, 1608),
+                                   (48, 80, 1600), (20, 100, 520), (32, 4800, 1600), (63, 1600, 1792), (50, 6400, 1600)])
+def test_rows_in_the_packed_order_into_and_out_of_the_product_of_17_to_64_rows(M, N, K):
+    """The product of 17 to 64 rows takes its rows row-major or in tiles of 16 rows x 64 columns laid
+    out like the packed weights' tiles, and writes a bfloat16 result in that order where asked: the
+    same bits either way, whole and with K in parts (the second kernel then writes the order), and
+    whatever lies in the tiles beyond the last row and column (NaN here)."""
+    k = _k()
+    a = _rand((M, K), torch.bfloat16, 10)
+    w = k.PackedWeight(_rand((N, K), torch.bfloat16, 11, 0.1), keep_rows=False)
+    bias = _rand((N,), torch.float32, 12)
+    # (beyond 32 rows that kernel takes a product only where K is long: 1,536 columns or more)
+    assert k.wants_packed_rows(w, M) and not k.wants_packed_rows(w, 16) and not k.wants_packed_rows(w, 65)
+    assert k.wants_packed_rows(w, 33) == (K >= 1536)
+    pa = k.PackedRows.of(a)
+    assert torch.equal(pa.rows(), a)
+    # what the tiles hold beyond the matrix must not matter
+    Mp, Kp = (M + 15) // 16 * 16, (K + 63) // 64 * 64
+    junk = torch.full((Mp, Kp), float("nan"), dtype=torch.bfloat16, device=DEV)
+    junk[:M, :K] = a
+    pa = k.PackedRows(k.PackedRows.of(junk).data, (M, K))
+    n_blocks = (K + 63) // 64
+    for splits in (None, 2, 3):
+        if splits is not None and (splits > n_blocks or (n_blocks + splits - 1) // splits > 28):
+            continue
+        for gelu in (False, True):
+            want = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+            k.linear(want, a, w, bias, gelu=gelu, splits=splits)
+            got = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+            k.linear(got, pa, w, bias, gelu=gelu, splits=splits)
+            assert torch.equal(got, want), (splits, gelu)
+            out = k.PackedRows.empty(M, N, DEV)
+            out.data.fill_(float("nan"))
+            k.linear(out, pa, w, bias, gelu=gelu, splits=splits)
+            assert torch.equal(out.rows(), want), (splits, gelu)
+        h = _rand((M, N), torch.float32, 13)
+        h2 = h.clone()
+        k.linear(h, a, w, bias, accumulate=True, splits=splits)
+        k.linear(h2, pa, w, bias, accumulate=True, splits=splits)
+        assert torch.equal(h, h2), splits
+    ref = plain.linear(a.double().cpu(), w_rows(w, N, K).double().cpu(), bias.double().cpu())
+    assert torch.allclose(want.double().cpu(), plain.gelu_tanh(ref), rtol=2**-7, atol=1e-3)
+    # elsewhere the order is refused, not misread
+    few = k.PackedRows.of(a[:8].contiguous())
+    with pytest.raises(RuntimeError, match="packed order"):
+        k.linear(torch.empty(8, N, dtype=torch.bfloat16, device=DEV), few, w, bias)
+
+
+def w_rows(w, N, K):
+    """A ``PackedWeight``'s matrix back in rows."""
+    k = _k()
+    return k.PackedRows(w.packed, (N, K)).rows()
+
+
+def test_the_sum_and_norm_and_decode_attention_write_the_packed_order():
+    k = _k()
+    M, N, K = 40, 1600, 1792
+    a = _rand((M, K), torch.bfloat16, 1)
+    w = k.PackedWeight(_rand((N, K), torch.bfloat16, 2, 0.1), keep_rows=False)
+    bias, gamma, beta = _rand((N,), torch.float32, 3), 1 + _rand((N,), torch.float32, 4, 0.1), _rand((N,), torch.float32, 5, 0.1)
+    h0 = _rand((M, N), torch.float32, 6)
+    outs = []
+    for packed in (False, True):
+        h = h0.clone()
+        pending = k.PendingSum()
+        pending.allowed = True
+        k.linear(h, a, w, bias, accumulate=True, splits=4, pending=pending)
+        assert pending.waits_on(h) and pending.can_norm(h)
+        y = k.PackedRows.empty(M, N, DEV) if packed else torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        pending.settle_normed(y, gamma, beta, 1e-5)
+        outs.append((h, y.rows() if packed else y))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    want = plain.layer_norm(outs[0][0].double().cpu(), gamma.double().cpu(), beta.double().cpu(), 1e-5)
+    assert torch.allclose(outs[0][1].double().cpu(), want, atol=2e-2, rtol=2e-2)
+    # decode attention: 37 rows of 5 heads of 64, each a request of its own
+    H, hd, n = 5, 64, 37
+    c = PagedCase(torch.bfloat16, H, H, hd, 16, [3 + 11 * i for i in range(n)], [1] * n, seed=8)
+    k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
+    rows = torch.arange(c.T, dtype=torch.int32, device=DEV)
+    plain_out = torch.empty(c.T, H * hd, dtype=torch.bfloat16, device=DEV)
+    k.attn_decode(plain_out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, c.T, H, c.scale)
+    for n_splits in (1, 3):
+        packed_out = k.PackedRows.empty(c.T, H * hd, DEV)
+        part_o = torch.empty(c.T * H * n_splits * hd, device=DEV)
+        part_ml = torch.empty(c.T * H * n_splits * 2, device=DEV)
+        k.attn_decode(packed_out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, c.T, H, c.scale,
+                      n_splits=n_splits, part_o=part_o, part_ml=part_ml)
+        if n_splits == 1:
+            assert torch.equal(packed_out.rows(), plain_out)
+        else:
+            assert torch.allclose(packed_out.rows().float(), plain_out.float(), rtol=2**-6, atol=2e-3)
+    assert torch.allclose(plain_out.double().cpu(), c.reference(), rtol=2**-6, atol=3e-3)
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 48, 1024), (8, 1600, 6400), (16, 80, 200), (16, 1600, 6400), (11, 333, 1608),
