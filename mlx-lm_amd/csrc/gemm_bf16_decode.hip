@@ -470,20 +470,31 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_rows_kernel(DecodeGemmAr
 #pragma unroll
       for (int r = 0; r < 4; ++r) red[wave][rt * FT + ft][lane * 4 + r] = acc[rt][ft][r];
   __syncthreads();
-  // element e = 4 * L + r of a tile: feature 4 * (L / 16) + r, row L % 16; 256 threads a tile
-  const int e = tid & 255, L = e >> 2, r = e & 3;
-  for (int t = tid >> 8; t < R_TILES * FT; t += WAVES / 4) {
+  // elements 4 * L .. 4 * L + 3 of a tile: features 4 * (L / 16) + 0..3 of row L % 16; a wave a tile
+  const int L = lane;
+  for (int t = wave; t < R_TILES * FT; t += WAVES) {
     const int rt = t / FT, ft = t - rt * FT;
-    float v = 0.f;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-    for (int wv = 0; wv < WAVES; ++wv) v += red[wv][t][e];
-    const int n = n0 + ft * 16 + 4 * (L >> 4) + r;
+    for (int wv = 0; wv < WAVES; ++wv) {
+      const float4 x = *(const float4*)&red[wv][t][4 * L];
+      v.x += x.x, v.y += x.y, v.z += x.z, v.w += x.w;
+    }
+    const int n = n0 + ft * 16 + 4 * (L >> 4);
     const int m = (t0 + rt) * 16 + (L & 15);
-    if (m < p.M && n < p.N) {
-      if (p.n_splits > 1)
-        p.ws[((size_t)blockIdx.y * p.M + m) * p.N + n] = v;  // summed, and finished, by sum_partials
-      else
-        finish(p, m, n, v);
+    if (m >= p.M || n >= p.N) continue;
+    const float vs[4] = {v.x, v.y, v.z, v.w};
+    if (p.n_splits > 1) {  // summed, and finished, by sum_partials
+      float* dst = p.ws + ((size_t)blockIdx.y * p.M + m) * p.N + n;
+      if ((p.N & 3) == 0) {
+        *(float4*)dst = v;
+      } else {
+        for (int j = 0; j < 4 && n + j < p.N; ++j) dst[j] = vs[j];
+      }
+    } else if (p.vec4) {
+      finish4(p, m, n, v);
+    } else {
+      for (int j = 0; j < 4 && n + j < p.N; ++j) finish(p, m, n + j, vs[j]);
     }
   }
 }
@@ -846,10 +857,15 @@ extern "C" int gemm_bf16_rows(void* out, const void* A, int lda, const void* W, 
   // are on the same dies; the surplus blocks return at once)
   const int fbs = ((N + R_FEATURES - 1) / R_FEATURES + 7) / 8 * 8;
   const dim3 grid(fbs * p.row_groups, n_splits), block(RW * 64);
-  if (M <= 32 || p.row_groups > 1)
+  // (eight waves of four k-blocks each where a block takes all the rows: a wave's trips to the L2s for
+  // its rows follow one another, and four are fewer than seven; a decode step of GPT-2 XL's sizes
+  // at 32 and at 48 rows 2 and 4 % shorter, with the groups of 49 to 64 rows 3 % longer)
+  if (p.row_groups > 1)
     hipLaunchKernelGGL((gemm_bf16_rows_kernel<2, 2, RW, R_HELD>), grid, block, 0, stream, p);
+  else if (M <= 32)
+    hipLaunchKernelGGL((gemm_bf16_rows_kernel<2, 2, 2 * RW, 4>), grid, dim3(2 * RW * 64), 0, stream, p);
   else
-    hipLaunchKernelGGL((gemm_bf16_rows_kernel<3, 2, RW, R_HELD>), grid, block, 0, stream, p);
+    hipLaunchKernelGGL((gemm_bf16_rows_kernel<3, 2, 2 * RW, 4>), grid, dim3(2 * RW * 64), 0, stream, p);
   CHECK_LAUNCH("gemm_bf16_rows");
   return 0;
 }
