@@ -7,7 +7,8 @@ mlx_lm/models/cache.py:325-407) or per layer and batch (``BatchKVCache``,
 cut into pages of ``page_size`` tokens instead:
 
 * Cache slots (one per layer run that writes a cache) whose mixers want the
-  same thing -- same key heads, head size and window -- form a *group*.  A
+  same thing -- same key heads, widths of a key and of a value, and window --
+  form a *group*.  A
   group has one pool of pages; page ``p`` of the group is one page in every
   slot of the group, so a request has one block table per group.
 * A request's block table lists, for block ``b`` (positions ``b*page_size ..``),
@@ -51,7 +52,9 @@ class _Group:
         self.need = need
         self.slots: List[int] = []
         self.pool = PagePool(n_pages)
-        self.storage = None  # [n_slots, n_pages, 2, n_kv_heads, page_size, head_dim]
+        # keys [n_slots, n_pages, n_kv_heads, page_size, head_dim] and values [.., value_dim]: where both
+        # have one width they are the two halves of every page of one tensor, keys first
+        self.keys = self.values = None
 
 
 class CacheManager:
@@ -97,11 +100,15 @@ class CacheManager:
 
         for g in self.groups:
             n = g.need
-            g.storage = torch.zeros(
-                (len(g.slots), self.n_pages, 2, n.n_kv_heads, self.page_size, n.head_dim),
-                dtype=self.dtype,
-                device=self.device,
-            )
+            shape = (len(g.slots), self.n_pages, n.n_kv_heads, self.page_size)
+            if n.value_dim == n.head_dim:
+                # a page's keys and values side by side: one stride for both, which the attention
+                # kernels here ask for
+                both = torch.zeros((*shape[:2], 2, *shape[2:], n.head_dim), dtype=self.dtype, device=self.device)
+                g.keys, g.values = both[:, :, 0], both[:, :, 1]
+            else:
+                g.keys = torch.zeros((*shape, n.head_dim), dtype=self.dtype, device=self.device)
+                g.values = torch.zeros((*shape, n.value_dim), dtype=self.dtype, device=self.device)
         for slot, need in self.state_needs.items():
             self.state_storage[slot] = torch.zeros(
                 (self.max_requests, *need.shape), dtype=getattr(torch, need.dtype), device=self.device
@@ -117,7 +124,8 @@ class CacheManager:
         import torch
 
         size = torch.empty((), dtype=self.dtype).element_size() if self.dtype is not None else 0
-        return sum(2 * g.need.n_kv_heads * g.need.head_dim * len(g.slots) * size for g in self.groups)
+        return sum(g.need.n_kv_heads * (g.need.head_dim + g.need.value_dim) * len(g.slots) * size
+                   for g in self.groups)
 
     def free_pages(self):
         """Free pages of the group that has fewest."""
@@ -256,10 +264,10 @@ class CacheManager:
         return self.requests[request_id].blocks[group]
 
     def kv(self, slot):
-        """``(keys, values)`` of cache slot ``slot``, each ``[n_pages, n_kv_heads, page, head_dim]``."""
+        """``(keys, values)`` of cache slot ``slot``: ``[n_pages, n_kv_heads, page, head_dim]`` and
+        ``[.., value_dim]``."""
         g, i = self.slot_group[slot]
-        s = self.groups[g].storage[i]
-        return s[:, 0], s[:, 1]
+        return self.groups[g].keys[i], self.groups[g].values[i]
 
     def state(self, slot):
         """State tensor of cache slot ``slot``: ``[max_requests, *shape]``."""
@@ -270,9 +278,10 @@ class CacheManager:
         import torch
 
         for g in self.groups:
-            free = torch.tensor(sorted(g.pool._free), dtype=torch.long, device=g.storage.device)
+            free = torch.tensor(sorted(g.pool._free), dtype=torch.long, device=g.keys.device)
             if free.numel():
-                g.storage[:, free] = value
+                g.keys[:, free] = value
+                g.values[:, free] = value
 
     def check(self):
         """No page lost, held twice or free while in a block table."""

@@ -50,8 +50,13 @@ class CacheNeed:
     """Paged keys and values that a mixer wants for one cache slot."""
 
     n_kv_heads: int
-    head_dim: int
+    head_dim: int  # width of a head's key
     window: int = 0  # 0: every earlier token; n: the last n tokens
+    v_head_dim: int = 0  # width of a head's value; 0: as the key's
+
+    @property
+    def value_dim(self):
+        return self.v_head_dim or self.head_dim
 
 
 @dataclass(frozen=True)

@@ -644,6 +644,9 @@ static int allow_lds(const char* who, const void* kernel, size_t bytes) {
 
 // items: n_tiles pairs (first flat row, number of rows 1..16); the rows of a
 // tile are consecutive tokens of one request at consecutive positions.
+// The most queries a tile of attn_tile's list may hold: who makes the lists asks here.
+extern "C" int attn_tile_queries(void) { return QT; }
+
 extern "C" int attn_tile(void* out, const void* q, int ldq, int ldo, const void* k_pages,
                          const void* v_pages, size_t page_stride, const int* block_table,
                          int max_blocks, const int* token_req, const int* positions,

@@ -314,6 +314,9 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
 
 DEFINE_LAST_ERROR(mlxlm_last_error)
 
+// The most queries a tile of attn_prefill's list may hold: who makes the lists asks here.
+extern "C" int attn_prefill_tile_queries(void) { return BQ; }
+
 // tiles: n_tiles pairs (first flat row, number of rows 1..128); the rows of a
 // tile are consecutive tokens of one request at consecutive positions.
 // bfloat16 only, head_dim 32, 64 or 128.

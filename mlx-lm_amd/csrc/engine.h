@@ -62,9 +62,10 @@ typedef struct {
 typedef struct {
   void* k;
   void* v;
-  size_t page_stride;  // elements
+  size_t page_stride;    // elements from a page's keys to the next page's
+  size_t v_page_stride;  // the same for values (the built-in attention asks for equal strides and widths)
   int n_kv_heads, head_dim, page_size, dtype;
-  int group, pad_;     // index of the slot's block table in a step; -1: no pages
+  int group, v_head_dim;  // group: index of the slot's block table in a step; -1: no pages
 } EngSlot;
 
 // Scratch memory of a step: a bump allocator over one device buffer.  The

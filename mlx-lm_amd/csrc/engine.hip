@@ -727,6 +727,9 @@ struct Attention : Mixer {
     if (s.n_kv_heads != n_kv_heads || s.head_dim != head_dim)
       FAIL("attention: cache slot %d holds %d heads of %d, the mixer has %d of %d", slot, s.n_kv_heads,
            s.head_dim, n_kv_heads, head_dim);
+    if (s.v_head_dim != s.head_dim || s.v_page_stride != s.page_stride)
+      FAIL("attention: cache slot %d holds values of width %d beside keys of %d; this mixer's kernels take one width",
+           slot, s.v_head_dim, s.head_dim);
     sc->k = s.k, sc->v = s.v, sc->page_stride = s.page_stride;
     sc->n_kv_heads = s.n_kv_heads, sc->head_dim = s.head_dim, sc->page_size = s.page_size, sc->dtype = s.dtype;
     sc->block_table = ctx->block_tables[s.group], sc->max_blocks = ctx->table_width[s.group];

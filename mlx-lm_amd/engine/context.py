@@ -100,12 +100,16 @@ class _DeviceArray:
 
 
 class CacheView:
-    """One cache slot as a mixer sees it in a step."""
+    """One cache slot as a mixer sees it in a step: ``keys``/``values`` are the slot's pages
+    (``[n_pages, n_kv_heads, page, width]`` each, of widths of their own), ``kv`` the same for the
+    attention kernels here where both have one width, ``block_table`` the requests' page numbers,
+    ``state`` a slot of fixed-size state."""
 
-    __slots__ = ("kv", "block_table", "state", "slot")
+    __slots__ = ("kv", "keys", "values", "block_table", "state", "slot")
 
-    def __init__(self, slot, kv=None, block_table=None, state=None):
+    def __init__(self, slot, kv=None, block_table=None, state=None, keys=None, values=None):
         self.slot, self.kv, self.block_table, self.state = slot, kv, block_table, state
+        self.keys, self.values = keys, values
 
 
 class HostBatch:
@@ -288,7 +292,9 @@ class StepContext:
                 from ..ops.kernels import PagedKV
 
                 g, _ = cm.slot_group[slot]
-                v = CacheView(slot, kv=PagedKV(*cm.kv(slot)), block_table=self.block_tables[g])
+                keys, values = cm.kv(slot)
+                v = CacheView(slot, kv=PagedKV(keys, values) if keys.shape == values.shape else None,
+                              block_table=self.block_tables[g], keys=keys, values=values)
             elif slot in cm.state_needs:
                 v = CacheView(slot, state=cm.state(slot))
             else:

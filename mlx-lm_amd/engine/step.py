@@ -53,6 +53,10 @@ class Engine:
             n_pages = (max_tokens + page_size - 1) // page_size
         self.cache = CacheManager(self.decoder.cache_needs(), page_size, n_pages, max_requests,
                                   dtype=self.dtype, device=self.device)
+        if len(self.cache.groups) > native.MAX_GROUPS:
+            raise ValueError(
+                f"the model's cache slots fall into {len(self.cache.groups)} groups of different needs; "
+                f"a step carries at most {native.MAX_GROUPS} block tables (ENG_MAX_GROUPS in csrc/engine.h)")
         self.scratch = Scratch(self.device)
         self._eager = EagerStore(self.device)
         self._logits = None
@@ -90,8 +94,9 @@ class Engine:
                 g, _ = cm.slot_group[slot]
                 k, v = cm.kv(slot)
                 need = cm.groups[g].need
-                s.k, s.v, s.page_stride = k.data_ptr(), v.data_ptr(), k.stride(0)
+                s.k, s.v, s.page_stride, s.v_page_stride = k.data_ptr(), v.data_ptr(), k.stride(0), v.stride(0)
                 s.n_kv_heads, s.head_dim, s.page_size = need.n_kv_heads, need.head_dim, cm.page_size
+                s.v_head_dim = need.value_dim
                 s.dtype, s.group = native.DT[k.dtype], g
         return table
 

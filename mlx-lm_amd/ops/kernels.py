@@ -602,7 +602,17 @@ def attn_row(out, q, kv, block_table, token_req, positions, rows, n_rows, n_head
     return out
 
 
-ATTN_PREFILL_TILE = 128  # queries per tile of attn_prefill
+_TILE_SIZES = None
+
+
+def attn_tile_sizes():
+    """``(queries a tile of attn_tile, queries a tile of attn_prefill)``: what the kernels were
+    compiled with, asked of their libraries (the one place these sizes are written is the source)."""
+    global _TILE_SIZES
+    if _TILE_SIZES is None:
+        _TILE_SIZES = (int(build.load("attention").attn_tile_queries()),
+                       int(build.load("attention_prefill").attn_prefill_tile_queries()))
+    return _TILE_SIZES
 
 
 def attn_prefill_takes(q_dtype, kv):

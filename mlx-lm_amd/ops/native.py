@@ -49,8 +49,9 @@ class EngPending(Structure):
 
 
 class EngSlot(Structure):
-    _fields_ = [("k", c_void_p), ("v", c_void_p), ("page_stride", c_size_t), ("n_kv_heads", c_int),
-                ("head_dim", c_int), ("page_size", c_int), ("dtype", c_int), ("group", c_int), ("pad_", c_int)]
+    _fields_ = [("k", c_void_p), ("v", c_void_p), ("page_stride", c_size_t), ("v_page_stride", c_size_t),
+                ("n_kv_heads", c_int), ("head_dim", c_int), ("page_size", c_int), ("dtype", c_int),
+                ("group", c_int), ("v_head_dim", c_int)]
 
 
 class EngScratch(Structure):

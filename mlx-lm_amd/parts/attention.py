@@ -7,8 +7,8 @@ from ..ops import kernels, native
 from .base import POSITION_ENCODINGS, Mixer, TensorSpec, build_part, register_mixer, value_of
 
 ROW_KERNEL_MAX_Q = 4  # requests with at most this many tokens in a step take the row kernels
-TILE_Q = 16  # queries per tile of the general tile kernel
-BIG_TILE_Q = 128  # queries per tile of the matrix-core prefill kernel
+# (how many queries a tile of the general kernel and of the matrix-core prefill kernel holds is the
+# kernels' own business: ``kernels.attn_tile_sizes()`` asks their libraries)
 
 
 class CausalSelfAttention(Mixer):
@@ -91,14 +91,15 @@ class CausalSelfAttention(Mixer):
         """Which of the step's rows go to which attention kernel.
 
         Requests that bring at most ``ROW_KERNEL_MAX_Q`` tokens are handled row by row (``rows``;
-        keys split over blocks); longer portions in tiles of ``TILE_Q`` consecutive queries
-        (``tiles``: first flat row and number of rows each), and the same portions in tiles of
-        ``BIG_TILE_Q`` for the matrix-core kernel (``big_tiles``, the tile with the most keys
-        first).  ``all_tiles`` covers every row with tiles, for head sizes the row kernels do
+        keys split over blocks); longer portions in tiles of consecutive queries, as many as the
+        general tile kernel takes (``tiles``: first flat row and number of rows each), and the
+        same portions in the larger tiles of the matrix-core kernel (``big_tiles``, the tile with
+        the most keys first).  ``all_tiles`` covers every row with tiles, for head sizes the row kernels do
         not take.  ``max_row_context``: the most keys that a row of ``rows`` sees, which decides
         how its keys are split; in a step that is recorded, the model's positions.
         ``rows_are_requests``: 1 if every request brings one token, so that item ``i`` of ``rows``
         is row ``i`` of request ``i`` (the decode kernel then need not look either up)."""
+        TILE_Q, BIG_TILE_Q = kernels.attn_tile_sizes()
         tiles, rows, all_tiles, big = [], [], [], []
         longest = 0
         for q0, n, length in zip(batch.q_starts, batch.q_lens, batch.context_lens):

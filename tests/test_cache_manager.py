@@ -202,3 +202,31 @@ def test_rollback_gives_back_what_was_taken_since_the_mark_and_nothing_else():
     assert rc.blocks[0] == held and rc.reserved == 60 and rc.length == 10
     assert cm.free_pages() == 8 - len(held)
     cm.check()
+
+
+def test_keys_and_values_may_differ_in_width():
+    """A mixer may keep values of another width than its keys (``CacheNeed.v_head_dim``): such slots
+    form a group of their own, keys and values are tensors of their own there, and both widths count
+    in the bytes of a token.  With one width a page's keys and values lie side by side under one
+    page stride, which the attention kernels ask for."""
+    import torch
+
+    same, narrow = CacheNeed(2, 32, 0), CacheNeed(2, 32, 0, v_head_dim=16)
+    assert same != narrow and same.value_dim == 32 and narrow.value_dim == 16
+    cm = CacheManager([same, narrow, narrow, same], 16, 5, 2, dtype=torch.bfloat16, device="cpu")
+    assert len(cm.groups) == 2 and cm.slot_group[1][0] == cm.slot_group[2][0] != cm.slot_group[0][0]
+    k, v = cm.kv(0)
+    assert k.shape == v.shape == (5, 2, 16, 32) and k.stride(0) == v.stride(0) == 2 * 2 * 16 * 32
+    assert v.data_ptr() - k.data_ptr() == 2 * 16 * 32 * 2  # the values follow the page's keys
+    k, v = cm.kv(2)
+    assert k.shape == (5, 2, 16, 32) and v.shape == (5, 2, 16, 16) and k.stride(0) != v.stride(0)
+    assert cm.bytes_per_token() == 2 * (2 * 2 * (32 + 32) + 2 * 2 * (32 + 16))
+    cm.add("r")
+    cm.reserve("r", 20)
+    cm.commit("r", 20)
+    cm.poison_free_pages(7.0)
+    held = set(cm.block_table("r", cm.slot_group[2][0]))
+    k, v = cm.kv(2)
+    for p in range(5):
+        assert bool((k[p] == 7).all()) == (p not in held) and bool((v[p] == 7).all()) == (p not in held)
+    cm.check()

@@ -492,7 +492,7 @@ def test_attn_prefill(case):
     c = PagedCase(torch.bfloat16, H, Hkv, hd, ps, ctx, ql, seed=hd + H + 3, window=window)
     assert k.attn_prefill_takes(torch.bfloat16, c.kv)
     k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
-    tiles = c.tiles(k.ATTN_PREFILL_TILE)
+    tiles = c.tiles(k.attn_tile_sizes()[1])
     out = torch.full((c.T, H * hd), float("nan")).to(torch.bfloat16).to(DEV)
     k.attn_prefill(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, tiles,
                    tiles.shape[0], H, c.scale, window)
@@ -512,7 +512,7 @@ def test_attn_prefill_far_key_stands_out():
         kf = c.k_full[0][far[i], 0].float()
         c.q[i, :hd] = (kf * (30.0 / (c.scale * float(kf.norm() ** 2)))).to(torch.bfloat16)
     k.kv_write(c.k_new.to(DEV), c.v_new.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions)
-    tiles = c.tiles(k.ATTN_PREFILL_TILE)
+    tiles = c.tiles(k.attn_tile_sizes()[1])
     out = torch.empty(n, H * hd, dtype=torch.bfloat16, device=DEV)
     k.attn_prefill(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, tiles,
                    tiles.shape[0], H, c.scale, 0)

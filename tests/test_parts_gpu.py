@@ -687,3 +687,141 @@ def test_a_window_under_recorded_steps(tmp_path, dtype):
     for r, toks in seqs.items():
         _close(results[True][r], plain_logits(toks[: results[True][r].shape[0]]), dtype, f"a window under recorded steps, request {r}")
         assert torch.equal(results[True][r], results[False][r]), r
+
+
+# ---------------------------------------------------------------------------
+# a mixer whose values are narrower than its keys: the cache slot's layout is the mixer's choice
+
+
+def _register_narrow_values():
+    from mlx_lm_amd.config import BaseModelArgs, CacheNeed, LayerSpec, ModelPlan, PartSpec, RunEntry, register_model
+    from mlx_lm_amd.parts import DecoderModel, Mixer, TensorSpec, register_mixer
+
+    class NarrowValueAttention(Mixer):
+        """One head; keys of ``key_dim`` columns, values of ``value_dim`` (written with torch ops
+        over the slot's pages, which it reaches through the step's block table)."""
+
+        def __init__(self, width, key_dim, value_dim, prefix=""):
+            super().__init__(prefix)
+            self.width, self.key_dim, self.value_dim = width, key_dim, value_dim
+
+        def cache_need(self):
+            return CacheNeed(1, self.key_dim, 0, v_head_dim=self.value_dim)
+
+        def tensors(self):
+            n = self._name
+            return {n("q"): TensorSpec((self.key_dim, self.width), "matrix"),
+                    n("k"): TensorSpec((self.key_dim, self.width), "matrix"),
+                    n("v"): TensorSpec((self.value_dim, self.width), "matrix"),
+                    n("o"): TensorSpec((self.width, self.value_dim), "matrix")}
+
+        def load(self, tensors):
+            self.q, self.k, self.v, self.o = (tensors[self._name(t)] for t in "qkvo")
+
+        def forward(self, ctx, x, residual, cache, writes_cache=True):
+            assert cache.kv is None and cache.keys.shape[-1] == self.key_dim and cache.values.shape[-1] == self.value_dim
+            ps = cache.keys.shape[2]
+            xf = x.float()
+            q, k, v = xf @ self.q.float().t(), xf @ self.k.float().t(), xf @ self.v.float().t()
+            pos, req = ctx.positions.long(), ctx.token_req.long()
+            pages = cache.block_table[req, pos // ps].long()
+            cache.keys[pages, 0, pos % ps] = k.to(cache.keys.dtype)
+            cache.values[pages, 0, pos % ps] = v.to(cache.values.dtype)
+            for t in range(x.shape[0]):
+                n = int(pos[t]) + 1
+                pg = cache.block_table[req[t], : (n + ps - 1) // ps].long()
+                keys = cache.keys[pg, 0].reshape(-1, self.key_dim)[:n].float()
+                values = cache.values[pg, 0].reshape(-1, self.value_dim)[:n].float()
+                p = torch.softmax(keys @ q[t] * self.key_dim**-0.5, 0)
+                residual[t] += (p @ values) @ self.o.float().t()
+
+    register_mixer("toy_narrow_values", NarrowValueAttention)
+
+    @dataclass
+    class NarrowArgs(BaseModelArgs):
+        model_type: str
+        width: int
+        vocab: int
+        max_len: int
+        key_dim: int
+        value_dim: int
+        inner: int
+
+    class NarrowModel:
+        def __init__(self, args):
+            self.args, self.model_type = args, args.model_type
+            self.decoder = DecoderModel(self.plan(args))
+
+        @property
+        def layers(self):
+            return self.decoder.layers
+
+        @staticmethod
+        def plan(a):
+            def norm(p):
+                return PartSpec("layernorm", {"width": a.width, "eps": 1e-5}, p)
+
+            layers = [LayerSpec("pre_norm", dict(
+                mixer_norm=norm(f"l{i}.n1."),
+                mixer=PartSpec("toy_narrow_values", {"width": a.width, "key_dim": a.key_dim, "value_dim": a.value_dim}, f"l{i}.mix."),
+                ffn_norm=norm(f"l{i}.n2."), ffn=PartSpec("gelu_mlp", {"width": a.width, "inner": a.inner}, f"l{i}.ff.")))
+                for i in range(2)]
+            return ModelPlan(width=a.width, vocab_size=a.vocab, max_positions=a.max_len,
+                             embedding=PartSpec("token", {"vocab_size": a.vocab, "width": a.width}, "emb."),
+                             embedding_positions=None, layers=layers, schedule=[RunEntry(0, 0), RunEntry(1, 1)],
+                             final_norm=norm("nf."),
+                             head=PartSpec("linear", {"vocab_size": a.vocab, "width": a.width, "weight_name": "emb.weight"}))
+
+    register_model("toy_narrow", NarrowModel, NarrowArgs)
+    return NarrowModel, NarrowArgs
+
+
+def test_a_mixer_whose_values_are_narrower_than_its_keys(tmp_path):
+    """``CacheNeed(v_head_dim=...)``: the manager keeps keys and values of such a slot as tensors of
+    their own widths and the step hands both to the mixer; whole, in portions and token by token
+    give the plain computation, with pages used again."""
+    from safetensors.torch import save_file
+
+    from mlx_lm_amd.engine import Engine, StepEntry
+    from mlx_lm_amd.utils import load_model
+
+    cfg = dict(model_type="toy_narrow", width=48, vocab=97, max_len=96, key_dim=32, value_dim=16, inner=64)
+    Model, Args = _register_narrow_values()
+    g = torch.Generator().manual_seed(3)
+    tensors = {}
+    for name, spec in Model(Args.from_dict(cfg)).decoder.expected_tensors().items():
+        if spec.role == "vector":
+            tensors[name] = torch.ones(spec.shape) if name.endswith("weight") else torch.zeros(spec.shape)
+        else:
+            tensors[name] = torch.randn(spec.shape, generator=g) * (0.4 if name.endswith((".q", ".k")) else 0.1)
+    json.dump(cfg, open(os.path.join(tmp_path, "config.json"), "w"))
+    save_file(tensors, os.path.join(tmp_path, "model.safetensors"))
+    model, _ = load_model(str(tmp_path), dtype="float32")
+    eng = Engine(model, dtype="float32", page_size=16, n_pages=8, max_requests=2)
+    assert len(eng.cache.groups) == 1 and eng.cache.kv(1)[1].shape[-1] == 16
+
+    w = {k: v.double() for k, v in tensors.items()}
+    ids = helpers.random_tokens(70, cfg["vocab"], 5)
+
+    def ln(x, p):
+        return plain.layer_norm(x, w[p + "weight"], w[p + "bias"], 1e-5)
+
+    h = plain.embed_tokens(w["emb.weight"], torch.tensor(ids))
+    for i in range(2):
+        x = ln(h, f"l{i}.n1.")
+        q, k, v = (plain.linear(x, w[f"l{i}.mix.{t}"]) for t in "qkv")
+        o = plain.attention(q[None], k[None], v[None], cfg["key_dim"] ** -0.5, plain.causal_mask(len(ids)))[0]
+        h = h + plain.linear(o, w[f"l{i}.mix.o"])
+        h = h + plain.mlp(ln(h, f"l{i}.n2."), w, f"l{i}.ff.")
+    want = plain.tied_head(ln(h, "nf."), w["emb.weight"])
+    for cuts in ([70], [33, 2, 1, 1, 20, 13], [64] + [1] * 6):
+        eng.add_request("r")
+        eng.cache.poison_free_pages()
+        rows, i = [], 0
+        for n in cuts:
+            rows.append(eng.step([StepEntry("r", ids[i : i + n], list(range(n)))]).clone())
+            i += n
+        eng.end_request("r")
+        _close(torch.cat(rows), want, "float32", f"portions {cuts}")
+    eng.cache.check()
+    assert eng.cache.free_pages() == 8
