@@ -58,14 +58,16 @@ typedef struct {
   int allowed, pad_;
 } EngPending;
 
-// One cache slot: pages of keys and values, or a state tensor, or nothing.
+// One cache slot: pages of keys and values, or a state tensor, or nothing.  A slot of per-request
+// state (group == -2) has the tensor [max_requests, ...] at k, the elements a request's row holds
+// in page_stride and the element type in dtype; a request's row is EngCtx.slot_ids[request].
 typedef struct {
   void* k;
   void* v;
   size_t page_stride;    // elements from a page's keys to the next page's
   size_t v_page_stride;  // the same for values (the built-in attention asks for equal strides and widths)
   int n_kv_heads, head_dim, page_size, dtype;
-  int group, v_head_dim;  // group: index of the slot's block table in a step; -1: no pages
+  int group, v_head_dim;  // group: index of the slot's block table in a step; -1: nothing; -2: a state tensor
 } EngSlot;
 
 // Scratch memory of a step: a bump allocator over one device buffer.  The
@@ -208,6 +210,30 @@ int eng_read_ahead_pays(const EngCtx* ctx, const EngWeight* w, int n_rows, int w
 int eng_linear_norms_itself(const EngCtx* ctx, int M, int N, int K, int dtype, int splits);
 // 1 if the product of n_rows rows with w reads its rows fastest in the packed order (EngValue.packed)
 int eng_wants_packed_rows(const EngCtx* ctx, const EngWeight* w, int n_rows);
+
+// The host's own routines, for a native part that lives in a library of its own (engine_parts.h).
+// Each returns 0, or non-zero with the text kept where mlxlm_last_error() of the host finds it.
+typedef struct EngHost {
+  // rows x cols values of dtype in the step's scratch memory (freed when the block is done)
+  int (*take)(EngCtx* ctx, int rows, int cols, int dtype, EngMat* out);
+  // a value as a matrix: a norm not computed yet is computed now
+  int (*materialize)(EngCtx* ctx, const EngValue* v, EngMat* out);
+  // out = epilogue(a @ w^T + bias): eng_linear
+  int (*linear)(EngCtx* ctx, const EngLinear* call, EngPending* pending);
+  // add a pending sum into its target (eng_pending_settle); the step's own is &ctx->pending
+  int (*settle)(EngCtx* ctx, EngPending* pending);
+  // where the keys and values of cache slot `slot` go and come from in this step
+  int (*slot_pages)(EngCtx* ctx, int slot, int q_width, int kv_width, EngScatter* out);
+  // keys and values of this step's tokens into their pages
+  int (*kv_write)(EngCtx* ctx, const EngMat* k, const EngMat* v, const EngScatter* sc);
+  // an entry point of csrc/<library>.hip's library (built at first use), or null
+  void* (*kernel)(const char* library, const char* symbol);
+  // a launch was made (the step's counters)
+  void (*launched)(EngCtx* ctx);
+  // keep a message as the error of the call under way; returns 1
+  int (*fail)(const char* format, ...);
+} EngHost;
+const EngHost* eng_host(void);
 
 #ifdef __cplusplus
 }

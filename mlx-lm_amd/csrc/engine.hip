@@ -11,7 +11,9 @@
 // launches.
 #include "common.h"
 #include "engine.h"
+#include "engine_parts.h"
 
+#include <stdarg.h>
 #include <string.h>
 
 #include <memory>
@@ -502,71 +504,11 @@ extern "C" int eng_linear(EngCtx* ctx, const EngLinear* c, EngPending* pending) 
 // ---------------------------------------------------------------------------
 // parts
 
-enum { KIND_NORM = ENG_NORM, KIND_MIXER = ENG_MIXER, KIND_FFN = ENG_FFN, KIND_BLOCK = ENG_BLOCK, KIND_POSITION = ENG_POSITION,
-       KIND_EMBEDDING = ENG_EMBEDDING, KIND_HEAD = ENG_HEAD, KIND_MODEL = ENG_MODEL };
-
-struct EngPart {
-  int kind;
-  explicit EngPart(int k) : kind(k) {}
-  virtual ~EngPart() {}
-};
-
 static int call_python(int part_id, int method, EngCtx* ctx, EngCall* call) {
   if (!g_callback) FAIL("a part that lives in Python was called, and no callback is set");
   if (ctx->stats) ctx->stats->callbacks++;
   return g_callback(part_id, method, ctx, call) != 0 ? 2 : 0;
 }
-
-struct Norm : EngPart {
-  bool settles_pending = false, reads_ahead = false;
-  Norm() : EngPart(KIND_NORM) {}
-  // The norm of rows of the float32 stream `x` (all, or those listed in `rows`).
-  // `ahead`: the weights that the result meets first, if the caller knows them; `may_pack`: whoever
-  // takes the result takes it in the packed order too (EngValue.packed), where those weights'
-  // product reads it faster so.
-  virtual int forward(EngCtx* ctx, const EngMat& x, const int* rows, int n_rows, bool lazy,
-                      const EngWeight* ahead, bool may_pack, EngValue* out) = 0;
-};
-
-struct Position : EngPart {
-  Position() : EngPart(KIND_POSITION) {}
-  virtual int embedding_term(EngCtx* ctx, EngMat* table, const int** index) {
-    table->p = nullptr, *index = nullptr;
-    return 0;
-  }
-  virtual int rotate(EngCtx*, const EngMat&, const EngMat&) { return 0; }
-  virtual bool rotates() const { return false; }
-};
-
-struct Mixer : EngPart {
-  bool accepts_lazy = false, accepts_packed = false;
-  const EngWeight* first_weight = nullptr;
-  Mixer() : EngPart(KIND_MIXER) {}
-  virtual int forward(EngCtx* ctx, const EngValue& x, const EngMat& residual, int slot, bool writes) = 0;
-};
-
-struct FeedForward : EngPart {
-  bool accepts_lazy = false, accepts_packed = false;
-  const EngWeight* first_weight = nullptr;
-  FeedForward() : EngPart(KIND_FFN) {}
-  virtual int forward(EngCtx* ctx, const EngValue& x, const EngMat& residual) = 0;
-};
-
-struct Block : EngPart {
-  bool handles_pending = false;
-  Block() : EngPart(KIND_BLOCK) {}
-  virtual int forward(EngCtx* ctx, const EngMat& h, int slot, bool writes) = 0;
-};
-
-struct Embedding : EngPart {
-  Embedding() : EngPart(KIND_EMBEDDING) {}
-  virtual int forward(EngCtx* ctx, const EngMat& out, const EngMat& add_table, const int* add_index) = 0;
-};
-
-struct Head : EngPart {
-  Head() : EngPart(KIND_HEAD) {}
-  virtual int forward(EngCtx* ctx, const EngValue& x, const EngMat& out) = 0;
-};
 
 // -- parts that live in Python ------------------------------------------------
 
@@ -720,23 +662,7 @@ struct Attention : Mixer {
 
   Attention() { accepts_lazy = true, accepts_packed = true; }
 
-  int scatter_for(EngCtx* ctx, int slot, EngScatter* sc) const {
-    if (slot < 0 || slot >= ctx->n_slots) FAIL("attention: cache slot %d of %d", slot, ctx->n_slots);
-    const EngSlot& s = ctx->slots[slot];
-    if (s.group < 0 || !s.k) FAIL("attention: cache slot %d holds no pages", slot);
-    if (s.n_kv_heads != n_kv_heads || s.head_dim != head_dim)
-      FAIL("attention: cache slot %d holds %d heads of %d, the mixer has %d of %d", slot, s.n_kv_heads,
-           s.head_dim, n_kv_heads, head_dim);
-    if (s.v_head_dim != s.head_dim || s.v_page_stride != s.page_stride)
-      FAIL("attention: cache slot %d holds values of width %d beside keys of %d; this mixer's kernels take one width",
-           slot, s.v_head_dim, s.head_dim);
-    sc->k = s.k, sc->v = s.v, sc->page_stride = s.page_stride;
-    sc->n_kv_heads = s.n_kv_heads, sc->head_dim = s.head_dim, sc->page_size = s.page_size, sc->dtype = s.dtype;
-    sc->block_table = ctx->block_tables[s.group], sc->max_blocks = ctx->table_width[s.group];
-    sc->token_req = ctx->token_req, sc->positions = ctx->positions;
-    sc->q_width = q_width, sc->kv_width = kv_width;
-    return 0;
-  }
+  int scatter_for(EngCtx* ctx, int slot, EngScatter* sc) const;
 
   // (n_splits, n_waves, keys a wave at a time) for the decode kernel.  Eight waves a block (four
   // where the rows' blocks alone are more than the CUs, or the keys no more than four waves'
@@ -904,6 +830,16 @@ struct Attention : Mixer {
   }
 };
 
+static int host_slot_pages(EngCtx* ctx, int slot, int q_width, int kv_width, EngScatter* sc);
+
+int Attention::scatter_for(EngCtx* ctx, int slot, EngScatter* sc) const {
+  TRY(host_slot_pages(ctx, slot, q_width, kv_width, sc));
+  if (sc->n_kv_heads != n_kv_heads || sc->head_dim != head_dim)
+    FAIL("attention: cache slot %d holds %d heads of %d, the mixer has %d of %d", slot, sc->n_kv_heads,
+         sc->head_dim, n_kv_heads, head_dim);
+  return 0;
+}
+
 // -- feed-forward ---------------------------------------------------------------
 
 struct GeluMlp : FeedForward {
@@ -1040,6 +976,54 @@ struct Model : EngPart {
     return head->forward(ctx, x, logits);
   }
 };
+
+// ---------------------------------------------------------------------------
+// the host's routines for parts in libraries of their own
+
+static int host_materialize(EngCtx* ctx, const EngValue* v, EngMat* out) { return materialize(ctx, *v, out); }
+
+static int host_slot_pages(EngCtx* ctx, int slot, int q_width, int kv_width, EngScatter* sc) {
+  if (slot < 0 || slot >= ctx->n_slots) FAIL("cache slot %d of %d", slot, ctx->n_slots);
+  const EngSlot& s = ctx->slots[slot];
+  if (s.group < 0 || !s.k) FAIL("cache slot %d holds no pages", slot);
+  if (s.v_head_dim != s.head_dim || s.v_page_stride != s.page_stride)
+    FAIL("cache slot %d holds values of width %d beside keys of %d: no one description fits both", slot,
+         s.v_head_dim, s.head_dim);
+  sc->k = s.k, sc->v = s.v, sc->page_stride = s.page_stride;
+  sc->n_kv_heads = s.n_kv_heads, sc->head_dim = s.head_dim, sc->page_size = s.page_size, sc->dtype = s.dtype;
+  sc->block_table = ctx->block_tables[s.group], sc->max_blocks = ctx->table_width[s.group];
+  sc->token_req = ctx->token_req, sc->positions = ctx->positions;
+  sc->q_width = q_width, sc->kv_width = kv_width;
+  return 0;
+}
+
+static int host_kv_write(EngCtx* ctx, const EngMat* k, const EngMat* v, const EngScatter* sc) {
+  return kv_write(ctx, *k, *v, *sc);
+}
+
+static void* host_kernel(const char* library, const char* symbol) {
+  return g_resolver ? g_resolver(library, symbol) : nullptr;
+}
+
+static void host_launched(EngCtx* ctx) {
+  if (ctx->stats) ctx->stats->launches++;
+}
+
+static int host_fail(const char* format, ...) {
+  va_list args;
+  va_start(args, format);
+  vsnprintf(g_err, sizeof(g_err), format, args);
+  va_end(args);
+  return 1;
+}
+
+extern "C" int eng_linear(EngCtx* ctx, const EngLinear* c, EngPending* pending);
+
+extern "C" const EngHost* eng_host(void) {
+  static const EngHost host = {take, host_materialize, eng_linear, settle, host_slot_pages, host_kv_write,
+                               host_kernel, host_launched, host_fail};
+  return &host;
+}
 
 // ---------------------------------------------------------------------------
 // C entry points

@@ -98,6 +98,11 @@ class Engine:
                 s.n_kv_heads, s.head_dim, s.page_size = need.n_kv_heads, need.head_dim, cm.page_size
                 s.v_head_dim = need.value_dim
                 s.dtype, s.group = native.DT[k.dtype], g
+            elif slot in cm.state_needs:
+                # per-request state: the tensor, and how many elements a request's row holds
+                state = cm.state(slot)
+                s.k, s.page_stride = state.data_ptr(), state.stride(0)
+                s.dtype, s.group = native.DT.get(state.dtype, -1), -2
         return table
 
     # -- buffers ---------------------------------------------------------------

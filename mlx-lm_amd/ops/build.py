@@ -69,10 +69,32 @@ def _readonly_lib_dir():
     return os.path.join(_PKG, "_lib")
 
 
+def _source(name):
+    """The path of the source called ``name``: one of ``csrc/``, or one registered with ``add_source``."""
+    return _extra_sources.get(name) or os.path.join(CSRC, name + ".hip")
+
+
+_extra_sources = {}
+
+
+def add_source(path):
+    """Make a ``.hip`` file outside ``csrc/`` known (a native part of a library of its own, which
+    includes ``engine_parts.h``): ``load(name)`` then builds and loads it like the others, its
+    library beside its source under ``_lib/``.  Returns the name (the file's, without ``.hip``)."""
+    path = os.path.abspath(path)
+    name = os.path.splitext(os.path.basename(path))[0]
+    if name in SOURCES:
+        raise ExtensionError(f"'{name}' is the name of one of the package's own sources")
+    if not os.path.exists(path):
+        raise ExtensionError(f"no such source: {path}")
+    _extra_sources[name] = path
+    return name
+
+
 def _digest(name):
     h = hashlib.sha256()
     headers = sorted(f for f in os.listdir(CSRC) if f.endswith(".h"))
-    for f in [os.path.join(CSRC, name + ".hip")] + [os.path.join(CSRC, h) for h in headers]:
+    for f in [_source(name)] + [os.path.join(CSRC, h) for h in headers]:
         with open(f, "rb") as fh:
             h.update(fh.read())
     h.update(" ".join(HIPCC_FLAGS).encode())
@@ -92,10 +114,10 @@ def compile_one(name, out_dir=None, verbose=True):
     hipcc = _hipcc()
     if hipcc is None:
         raise ExtensionError(f"hipcc not found; cannot build the '{name}' kernels")
-    out_dir = out_dir or _lib_dir()
+    out_dir = out_dir or _out_dir(name)
     so = os.path.join(out_dir, name + ".so")
     tmp = f"{so}.{os.getpid()}.tmp"
-    cmd = [hipcc, *HIPCC_FLAGS, "-I", CSRC, os.path.join(CSRC, name + ".hip"), "-o", tmp]
+    cmd = [hipcc, *HIPCC_FLAGS, "-I", CSRC, _source(name), "-o", tmp]
     t0 = time.time()
     if verbose:
         print(f"[mlx_lm_amd] compiling {name}.hip for gfx950 ...", file=sys.stderr, flush=True)
@@ -125,10 +147,27 @@ def compile_one(name, out_dir=None, verbose=True):
     return so
 
 
+def _out_dir(name):
+    """Where the library of source ``name`` goes: the package's ``_lib/``, or for a source
+    registered with ``add_source`` a ``_lib/`` beside it (the temporary folder if neither can be written)."""
+    if name not in _extra_sources:
+        return _lib_dir()
+    d = os.path.join(os.path.dirname(_extra_sources[name]), "_lib")
+    try:
+        os.makedirs(d, exist_ok=True)
+        probe = os.path.join(d, f".w{os.getpid()}")
+        with open(probe, "w"):
+            pass
+        os.unlink(probe)
+        return d
+    except OSError:
+        return _lib_dir()
+
+
 def build_all(verbose=True):
     """Compile every source, whether or not a built library is there."""
     d = _lib_dir()
-    return [compile_one(n, d, verbose) for n in SOURCES]
+    return [compile_one(n, d, verbose) for n in SOURCES] + [compile_one(n, None, verbose) for n in _extra_sources]
 
 
 def load(name):
@@ -137,10 +176,13 @@ def load(name):
         lib = _loaded.get(name)
         if lib is not None:
             return lib
-        if name not in SOURCES:
+        if name not in SOURCES and name not in _extra_sources:
             raise ExtensionError(f"no kernel source named '{name}'")
         so = None
-        for d in (_readonly_lib_dir(), _lib_dir()):
+        dirs = (_readonly_lib_dir(), _lib_dir())
+        if name in _extra_sources:
+            dirs = (os.path.join(os.path.dirname(_extra_sources[name]), "_lib"),) + dirs
+        for d in dirs:
             cand = os.path.join(d, name + ".so")
             if _is_current(cand, name):
                 so = cand
@@ -156,7 +198,8 @@ def load(name):
             lib = ctypes.CDLL(so)
         except OSError as e:
             raise ExtensionError(f"cannot load {so}: {e}") from e
-        lib.mlxlm_last_error.restype = ctypes.c_char_p
+        if hasattr(lib, "mlxlm_last_error"):  # (a part of a library of its own reports through the host's)
+            lib.mlxlm_last_error.restype = ctypes.c_char_p
         _loaded[name] = lib
         return lib
 

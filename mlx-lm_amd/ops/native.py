@@ -176,6 +176,7 @@ def lib():
                                               c_float, POINTER(EngWeight), c_int]),
         "eng_read_ahead_pays": (c_int, [POINTER(EngCtx), POINTER(EngWeight), c_int, c_int]),
         "eng_wants_packed_rows": (c_int, [POINTER(EngCtx), POINTER(EngWeight), c_int]),
+        "eng_host": (P, []),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -201,6 +202,12 @@ def check(rc, what="the native host"):
         raise e
     if rc != 0:
         raise NativeError(lib().mlxlm_last_error().decode() or f"{what} failed")
+
+
+def host():
+    """The host's table of routines (``EngHost`` of csrc/engine.h), for the maker of a native part
+    that lives in a library of its own (csrc/engine_parts.h)."""
+    return lib().eng_host()
 
 
 def made(handle, what):

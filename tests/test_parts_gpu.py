@@ -475,6 +475,25 @@ def _register_running_sum():
 
     register_mixer("toy_running_sum", RunningSum)
 
+    class NativeRunningSum(RunningSum):
+        """The same mixer with a native twin in a library of its own (tests/native_parts/
+        running_sum.hip, which includes csrc/engine_parts.h): the native walk calls it without a
+        trip through Python, and no file of the framework names it."""
+
+        def make_native(self):
+            import ctypes
+
+            from mlx_lm_amd.ops import build, native
+
+            lib = build.load(build.add_source(os.path.join(os.path.dirname(__file__), "native_parts", "running_sum.hip")))
+            lib.make_running_sum.restype, lib.make_running_sum.argtypes = ctypes.c_void_p, [ctypes.c_void_p, ctypes.c_int]
+            return native.made(lib.make_running_sum(native.host(), self.width), "running sum")
+
+        def forward(self, ctx, x, residual, cache, writes_cache=True):
+            raise AssertionError("the native twin runs, not this")
+
+    register_mixer("toy_running_sum_native", NativeRunningSum)
+
     @dataclass
     class SumArgs(BaseModelArgs):
         model_type: str
@@ -482,6 +501,7 @@ def _register_running_sum():
         vocab: int
         max_len: int
         inner: int
+        mixer: str = "toy_running_sum"
 
     class SumModel:
         def __init__(self, args):
@@ -499,7 +519,7 @@ def _register_running_sum():
 
             layers = [
                 LayerSpec("pre_norm", dict(
-                    mixer_norm=norm("l0.n1."), mixer=PartSpec("toy_running_sum", {"width": a.width}, "l0.mix."),
+                    mixer_norm=norm("l0.n1."), mixer=PartSpec(a.mixer, {"width": a.width}, "l0.mix."),
                     ffn_norm=norm("l0.n2."), ffn=PartSpec("gelu_mlp", {"width": a.width, "inner": a.inner}, "l0.ff."))),
                 LayerSpec("pre_norm", dict(
                     mixer_norm=norm("l1.n1."),
@@ -517,16 +537,19 @@ def _register_running_sum():
     return SumModel, SumArgs
 
 
+@pytest.mark.parametrize("mixer", ["toy_running_sum", "toy_running_sum_native"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_recorded_step_takes_its_tokens_once(tmp_path, dtype):
+def test_a_recorded_step_takes_its_tokens_once(tmp_path, dtype, mixer):
     """Steps of a model whose mixer keeps state, replayed from graphs, against the same steps
-    run eagerly, bit for bit: the step that records a graph counts once, like any other."""
+    run eagerly, bit for bit: the step that records a graph counts once, like any other.  The
+    mixer is a Python part that launches kernels only, or a native part in a library of its own
+    that the native walk calls directly (both give the same logits up to the order of a sum)."""
     from safetensors.torch import save_file
 
     from mlx_lm_amd.engine import Engine, StepEntry
     from mlx_lm_amd.utils import load_model
 
-    cfg = dict(model_type="toy_sum", width=64, vocab=97, max_len=96, inner=80)
+    cfg = dict(model_type="toy_sum", width=64, vocab=97, max_len=96, inner=80, mixer=mixer)
     SumModel, SumArgs = _register_running_sum()
     g = torch.Generator().manual_seed(3)
     tensors = {}
@@ -559,6 +582,17 @@ def test_a_recorded_step_takes_its_tokens_once(tmp_path, dtype):
         states[use_graphs] = eng.cache.state(0)[[eng.cache.requests[r].state_slot for r in seqs]].clone()
     assert torch.equal(states[True], states[False])
     assert torch.equal(results[True], results[False])
+    if mixer == "toy_running_sum_native":
+        assert eng.stats.callbacks == 0  # no part of this model is called back in Python
+        assert model.layers[0].mixer._native is not None
+    _SUM_RESULTS[dtype, mixer] = results[False].float().cpu()
+    other = _SUM_RESULTS.get((dtype, "toy_running_sum" if mixer.endswith("native") else "toy_running_sum_native"))
+    if other is not None:
+        tol = 1e-4 if dtype == "float32" else 5e-2
+        assert (other - _SUM_RESULTS[dtype, mixer]).abs().max().item() <= tol * other.abs().max().item()
+
+
+_SUM_RESULTS = {}
 
 
 # ---------------------------------------------------------------------------
