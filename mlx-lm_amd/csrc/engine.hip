@@ -243,7 +243,9 @@ static int take_packed(EngCtx* ctx, int rows, int cols, EngMat* out) {
 // on die j % 8), for few enough rows that most CUs have none.
 static int read_ahead_pays(const EngCtx* ctx, const EngWeight* w, int n_rows, bool with_norm, bool* yes) {
   *yes = false;
-  if (!w || !w->packed || n_rows <= 0 || n_rows > DECODE_MAX_ROWS || w->n_chunks < 150) return 0;
+  // (a matrix of fewer chunks than three fifths of the CUs is read by blocks of eight features, whose
+  // chunks are not the reading blocks')
+  if (!w || !w->packed || n_rows <= 0 || n_rows > DECODE_MAX_ROWS || w->n_chunks < ctx->n_compute_units * 3 / 5) return 0;
   int takes = 0, splits = 0;
   QUERY(k_decode_takes, takes, n_rows, w->K, with_norm ? 1 : 0, 1);
   if (!takes) return 0;

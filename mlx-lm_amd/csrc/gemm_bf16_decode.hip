@@ -651,7 +651,13 @@ __global__ __launch_bounds__(256) void sum_partials_norm_kernel(SumNormArgs q) {
 DEFINE_LAST_ERROR(mlxlm_last_error)
 
 #define MAX_LDS_BYTES (120 * 1024)
-#define FEW_BLOCKS 150  // fewer blocks of 16 features than this leave many CUs idle
+// Fewer blocks of 16 features than this leave many CUs idle: three fifths of the device's CUs
+// (150 of 256).  The thresholds below are fractions of the CU count and a time, not sizes: they
+// were measured at widths 768 to 2,048 on 256 CUs and move with the device, not with one model.
+static int few_blocks() { return n_compute_units() * 3 / 5; }
+// A CU draws some 30 GB/s of a matrix that comes from memory; a second kernel costs some 5 us.
+#define CU_STREAM_BYTES_PER_US 30000.0
+#define SECOND_KERNEL_US 1.3  // a matrix that streams in less than this gains nothing from a split
 
 // LDS row stride: rows of 16-byte reads from 16 lanes must fall on distinct
 // banks, which holds when the stride in 32-bit words is 4 mod 32.
@@ -678,10 +684,12 @@ extern "C" int gemm_bf16_decode_splits(int M, int N, int K, int with_norm, int f
     want = force;
   } else {
     const int n_blocks = (N + 15) / 16;
-    if (n_blocks >= 200 || M < 4) return 1;  // (one to three rows: the next projection's norm prologue is cheaper than a second kernel)
+    // enough blocks as it is (four fifths of the CUs; 200 of 256), or one to three rows: the next
+    // projection's norm prologue is cheaper than a second kernel
+    if (n_blocks >= n_compute_units() * 4 / 5 || M < 4) return 1;
     // a small matrix streams in less time than the second kernel costs (measured at N = 1600:
-    // K = 1600 loses 2 us by the split, K = 6400 gains 4)
-    if ((long)N * K < 5000000L) return 1;
+    // K = 1600, 5 MB, loses 2 us by the split; K = 6400, 20 MB, gains 4)
+    if (2.0 * N * K / (CU_STREAM_BYTES_PER_US * n_compute_units()) < SECOND_KERNEL_US) return 1;
     // one and a half blocks a CU (N = 1600, K = 6400: four parts; with six, two blocks a CU, a decode step of
     // GPT-2 XL's sizes at batch 8 took 2.25 ms instead of 2.22, the parts' sum being read by the next kernel;
     // three parts are more k-blocks than a wave holds at once, 2.41 ms)
@@ -762,7 +770,7 @@ extern "C" int gemm_bf16_decode(
   p.K = K, p.lda = lda, p.ldx = ldx, p.ldw = ldw;
   // Few features and no split of K: blocks of eight features (half of each MFMA
   // tile is idle, which costs nothing here) put twice as many CUs to work.
-  p.rows = (n_splits == 1 && (N + 15) / 16 < FEW_BLOCKS) ? 8 : 16;
+  p.rows = (n_splits == 1 && (N + 15) / 16 < few_blocks()) ? 8 : 16;
   p.n_splits = n_splits, p.chunks_per_split = chunks_per_split(K, n_splits);
   p.ws = ws;
   if (n_splits > 1) {
