@@ -23,6 +23,7 @@
 //  * attn_row: one query per block, its keys split over the block's four
 //    waves and over `n_splits` blocks; attn_merge joins the splits.
 #include "common.h"
+#include "attention_tiles.h"
 
 struct AttnArgs {
   void* out;          // [n_tokens, n_heads*head_dim]
@@ -45,7 +46,7 @@ struct AttnArgs {
 };
 
 #define KT 64   // keys per tile
-#define QT 16   // queries per block in attn_tile
+#define QT ATTN_TILE_QUERIES  // queries per block in attn_tile
 
 template <typename T>
 struct Vec;
@@ -644,9 +645,6 @@ static int allow_lds(const char* who, const void* kernel, size_t bytes) {
 
 // items: n_tiles pairs (first flat row, number of rows 1..16); the rows of a
 // tile are consecutive tokens of one request at consecutive positions.
-// The most queries a tile of attn_tile's list may hold: who makes the lists asks here.
-extern "C" int attn_tile_queries(void) { return QT; }
-
 extern "C" int attn_tile(void* out, const void* q, int ldq, int ldo, const void* k_pages,
                          const void* v_pages, size_t page_stride, const int* block_table,
                          int max_blocks, const int* token_req, const int* positions,

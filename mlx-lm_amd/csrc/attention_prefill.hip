@@ -23,6 +23,7 @@
 //    eight 32-bit words (two keys each).
 //  * Online softmax in 32-bit per lane; outputs leave as O^T accumulators.
 #include "common.h"
+#include "attention_tiles.h"
 #include <type_traits>
 
 struct PrefillArgs {
@@ -41,7 +42,7 @@ struct PrefillArgs {
   float scale;
 };
 
-#define BQ 128  // queries per block
+#define BQ ATTN_PREFILL_TILE_QUERIES  // queries per block
 #define KT 64   // keys per tile
 #define VT_STRIDE (KT + 8)  // 144 bytes a row: 16-byte reads of 32 rows fall on distinct banks
 
@@ -313,9 +314,6 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
 }
 
 DEFINE_LAST_ERROR(mlxlm_last_error)
-
-// The most queries a tile of attn_prefill's list may hold: who makes the lists asks here.
-extern "C" int attn_prefill_tile_queries(void) { return BQ; }
 
 // tiles: n_tiles pairs (first flat row, number of rows 1..128); the rows of a
 // tile are consecutive tokens of one request at consecutive positions.

@@ -136,6 +136,8 @@ typedef void* (*eng_resolver_t)(const char*, const char*);
 void eng_set_hooks(eng_resolver_t resolver, eng_callback_t callback);
 int eng_struct_sizes(long* out, int n);  // for the Python side's check of its mirrored layouts
 int eng_compute_units(void);
+// queries a tile of attn_tile's and of attn_prefill's work lists holds (attention_tiles.h)
+void eng_attn_tile_sizes(int* tile, int* prefill_tile);
 
 // flags of a callback part
 #define ENG_ACCEPTS_LAZY 1

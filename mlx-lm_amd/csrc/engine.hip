@@ -12,6 +12,7 @@
 #include "common.h"
 #include "engine.h"
 #include "engine_parts.h"
+#include "attention_tiles.h"
 
 #include <stdarg.h>
 #include <string.h>
@@ -44,6 +45,10 @@ extern "C" void eng_set_hooks(eng_resolver_t resolver, eng_callback_t callback) 
 }
 
 extern "C" int eng_compute_units(void) { return n_compute_units(); }
+
+extern "C" void eng_attn_tile_sizes(int* tile, int* prefill_tile) {
+  *tile = ATTN_TILE_QUERIES, *prefill_tile = ATTN_PREFILL_TILE_QUERIES;
+}
 
 template <typename F>
 struct Entry {

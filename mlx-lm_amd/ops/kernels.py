@@ -606,12 +606,14 @@ _TILE_SIZES = None
 
 
 def attn_tile_sizes():
-    """``(queries a tile of attn_tile, queries a tile of attn_prefill)``: what the kernels were
-    compiled with, asked of their libraries (the one place these sizes are written is the source)."""
+    """``(queries a tile of attn_tile, queries a tile of attn_prefill)``: what the kernels are
+    compiled with (``csrc/attention_tiles.h``, the one place these sizes are written), asked of
+    the native host, which includes the same header."""
     global _TILE_SIZES
     if _TILE_SIZES is None:
-        _TILE_SIZES = (int(build.load("attention").attn_tile_queries()),
-                       int(build.load("attention_prefill").attn_prefill_tile_queries()))
+        a, b = ctypes.c_int(), ctypes.c_int()
+        native.lib().eng_attn_tile_sizes(ctypes.byref(a), ctypes.byref(b))
+        _TILE_SIZES = (a.value, b.value)
     return _TILE_SIZES
 
 

@@ -177,6 +177,7 @@ def lib():
         "eng_read_ahead_pays": (c_int, [POINTER(EngCtx), POINTER(EngWeight), c_int, c_int]),
         "eng_wants_packed_rows": (c_int, [POINTER(EngCtx), POINTER(EngWeight), c_int]),
         "eng_host": (P, []),
+        "eng_attn_tile_sizes": (None, [POINTER(c_int), POINTER(c_int)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
