@@ -113,6 +113,7 @@ static Entry<fn_gemm_bf16> k_gemm_bf16("gemm_bf16", "gemm_bf16_scatter");
 static Entry<fn_int5> k_gemm_bf16_splits("gemm_bf16", "gemm_bf16_splits");
 static Entry<fn_gemm_decode> k_gemm_decode("gemm_bf16_decode", "gemm_bf16_decode");
 static Entry<fn_int4> k_decode_takes("gemm_bf16_decode", "gemm_bf16_decode_takes");
+static Entry<int (*)()> k_decode_few_blocks("gemm_bf16_decode", "gemm_bf16_decode_few_blocks");
 static Entry<fn_int5> k_decode_splits("gemm_bf16_decode", "gemm_bf16_decode_splits");
 static Entry<fn_gemm_rows> k_gemm_rows("gemm_bf16_decode", "gemm_bf16_rows");
 static Entry<fn_int4> k_rows_splits("gemm_bf16_decode", "gemm_bf16_rows_splits");
@@ -248,9 +249,11 @@ static int take_packed(EngCtx* ctx, int rows, int cols, EngMat* out) {
 // on die j % 8), for few enough rows that most CUs have none.
 static int read_ahead_pays(const EngCtx* ctx, const EngWeight* w, int n_rows, bool with_norm, bool* yes) {
   *yes = false;
-  // (a matrix of fewer chunks than three fifths of the CUs is read by blocks of eight features, whose
-  // chunks are not the reading blocks')
-  if (!w || !w->packed || n_rows <= 0 || n_rows > DECODE_MAX_ROWS || w->n_chunks < ctx->n_compute_units * 3 / 5) return 0;
+  // (a matrix of few chunks is read by blocks of eight features, whose chunks are not the reading
+  // blocks': the decode kernels' library says from how many on it is sixteen)
+  int few = 0;
+  QUERY(k_decode_few_blocks, few);
+  if (!w || !w->packed || n_rows <= 0 || n_rows > DECODE_MAX_ROWS || w->n_chunks < few) return 0;
   int takes = 0, splits = 0;
   QUERY(k_decode_takes, takes, n_rows, w->K, with_norm ? 1 : 0, 1);
   if (!takes) return 0;

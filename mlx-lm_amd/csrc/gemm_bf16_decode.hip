@@ -651,10 +651,11 @@ __global__ __launch_bounds__(256) void sum_partials_norm_kernel(SumNormArgs q) {
 DEFINE_LAST_ERROR(mlxlm_last_error)
 
 #define MAX_LDS_BYTES (120 * 1024)
-// Fewer blocks of 16 features than this leave many CUs idle: three fifths of the device's CUs
+// Fewer blocks of 16 features than this leave many CUs idle: 75/128 of the device's CUs
 // (150 of 256).  The thresholds below are fractions of the CU count and a time, not sizes: they
 // were measured at widths 768 to 2,048 on 256 CUs and move with the device, not with one model.
-static int few_blocks() { return n_compute_units() * 3 / 5; }
+static int few_blocks() { return n_compute_units() * 75 / 128; }
+extern "C" int gemm_bf16_decode_few_blocks(void) { return few_blocks(); }
 // A CU draws some 30 GB/s of a matrix that comes from memory; a second kernel costs some 5 us.
 #define CU_STREAM_BYTES_PER_US 30000.0
 #define SECOND_KERNEL_US 1.3  // a matrix that streams in less than this gains nothing from a split
