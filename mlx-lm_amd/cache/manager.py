@@ -19,6 +19,8 @@ cut into pages of ``page_size`` tokens instead:
   out of their reach.
 * Every request also gets a state slot: a row in each fixed-size state tensor
   (zeroed when the request starts), whether or not any mixer asks for one.
+* What a request computed can be kept beyond its end (``detach``) for a later
+  request to go on from (``attach``): its pages simply stay held.
 """
 
 from dataclasses import dataclass, field
@@ -45,6 +47,20 @@ class RequestCache:
     blocks: List[List[int]] = field(default_factory=list)  # per group: page of each block or -1
     serial: int = 0  # unique over the manager's life, unlike the id
     version: int = 0  # counts the edits of ``blocks``: who keeps a copy of a table compares it
+
+
+@dataclass
+class KeptPages:
+    """What a request had computed, taken out of the list of live requests but not given back:
+    its pages stay held (no other request gets them), its state rows are copied.  ``attach``
+    makes a live request of it again, ``drop`` gives everything back.  (The reference keeps a
+    request's arrays as its prompt cache, mlx_lm/models/cache.py:15-43; with pages nothing is copied.)"""
+
+    length: int
+    reserved: int
+    blocks: List[List[int]]
+    state: Dict[int, object] = field(default_factory=dict)  # cache slot -> the request's row of that state tensor
+    live: bool = True  # False once attached again or dropped
 
 
 class _Group:
@@ -92,6 +108,7 @@ class CacheManager:
                 raise TypeError(f"cache slot {slot}: unknown need {need!r}")
         self._free_state_slots = list(range(max_requests - 1, -1, -1))
         self.requests: Dict[object, RequestCache] = {}
+        self.kept: List[KeptPages] = []  # detached and neither attached again nor dropped
         if device is not None:
             self._allocate()
 
@@ -254,6 +271,102 @@ class CacheManager:
             g.pool.give_back([p for p in rc.blocks[gi] if p >= 0])
         self._free_state_slots.append(rc.state_slot)
 
+    # -- keeping what a request computed ----------------------------------------
+
+    def detach(self, request_id):
+        """Take a request out and keep what it holds: its pages stay held, its state rows are
+        copied, its request slot goes back.  Returns the ``KeptPages``."""
+        rc = self.requests.pop(request_id)
+        state = {slot: storage[rc.state_slot].clone() for slot, storage in self.state_storage.items()}
+        self._free_state_slots.append(rc.state_slot)
+        kept = KeptPages(rc.length, rc.reserved, rc.blocks, state)
+        self.kept.append(kept)
+        return kept
+
+    def attach(self, request_id, kept):
+        """A live request that goes on from what ``kept`` holds (which is used up by this)."""
+        if not kept.live or not any(k is kept for k in self.kept):
+            raise ValueError("these kept pages are not this cache manager's, or were used already")
+        rc = self.add(request_id)
+        rc.length, rc.reserved, rc.blocks = kept.length, kept.reserved, kept.blocks
+        rc.version += 1
+        for slot, row in kept.state.items():
+            self.state_storage[slot][rc.state_slot].copy_(row)
+        self._forget(kept)
+        return rc
+
+    def fork(self, kept):
+        """A second ``KeptPages`` with the same tokens in pages of its own (their contents are
+        copied on the device), so that two requests can go on from one point.  All or nothing:
+        ``OutOfPages`` if a group is short."""
+        if not kept.live:
+            raise ValueError("these kept pages were used already")
+        n_blocks = self.blocks_for(kept.length)
+        taken = []
+        for gi, g in enumerate(self.groups):
+            old = kept.blocks[gi][:n_blocks]
+            new = g.pool.take(sum(p >= 0 for p in old))
+            if new is None:
+                for gj, pages in taken:
+                    self.groups[gj].pool.give_back(pages)
+                raise OutOfPages(f"a copy of {kept.length} kept tokens needs {sum(p >= 0 for p in old)} pages "
+                                 f"of group {gi}; {g.pool.n_free} are free")
+            taken.append((gi, new))
+        blocks = []
+        for (gi, new), g in zip(taken, self.groups):
+            old = kept.blocks[gi][:n_blocks]
+            fresh = iter(new)
+            blocks.append([next(fresh) if p >= 0 else -1 for p in old])
+            src = [p for p in old if p >= 0]
+            if g.keys is not None and src:
+                import torch
+
+                i_src = torch.tensor(src, device=g.keys.device)
+                i_dst = torch.tensor(new, device=g.keys.device)
+                g.keys.index_copy_(1, i_dst, g.keys.index_select(1, i_src))
+                g.values.index_copy_(1, i_dst, g.values.index_select(1, i_src))
+        state = {slot: row.clone() for slot, row in kept.state.items()}
+        copy = KeptPages(kept.length, n_blocks * self.page_size, blocks, state)
+        self.kept.append(copy)
+        return copy
+
+    def set_state(self, request_id, state=None):
+        """A live request's rows of the state tensors: as ``state`` (cache slot -> row) has them, or zero."""
+        rc = self.requests[request_id]
+        for slot, storage in self.state_storage.items():
+            if state is None:
+                storage[rc.state_slot].zero_()
+            else:
+                storage[rc.state_slot].copy_(state[slot])
+
+    def drop(self, kept):
+        """Give back the pages of a ``KeptPages`` that nobody goes on from."""
+        if not kept.live:
+            return
+        for gi, g in enumerate(self.groups):
+            g.pool.give_back([p for p in kept.blocks[gi] if p >= 0])
+        self._forget(kept)
+
+    def _forget(self, kept):
+        kept.live = False
+        self.kept = [k for k in self.kept if k is not kept]
+
+    def truncate_kept(self, kept, new_length):
+        """``truncate`` for pages that are kept: forget the tokens from ``new_length`` on.  (State rows
+        cannot be taken back; whether a model's state allows a cut is the caller's to know.)"""
+        if not kept.live:
+            raise ValueError("these kept pages were used already")
+        # (through a request of a moment: the rules are truncate's)
+        name = ("kept", id(kept))
+        rc = RequestCache(name, -1, kept.length, kept.reserved, kept.blocks)
+        self.requests[name] = rc
+        try:
+            self.truncate(name, new_length)
+        finally:
+            del self.requests[name]
+        kept.length, kept.reserved, kept.blocks = rc.length, rc.reserved, rc.blocks
+        return kept
+
     def release_all(self):
         for rid in list(self.requests):
             self.release(rid)
@@ -288,17 +401,17 @@ class CacheManager:
         for gi, g in enumerate(self.groups):
             g.pool.check()
             seen = {}
-            for rc in self.requests.values():
-                for p in rc.blocks[gi]:
+            holders = [(rc.request_id, rc.blocks) for rc in self.requests.values()]
+            holders += [(("kept", i), k.blocks) for i, k in enumerate(self.kept)]
+            for holder, blocks in holders:
+                for p in blocks[gi]:
                     if p < 0:
                         continue
                     if p in seen:
-                        raise AssertionError(
-                            f"group {gi}: page {p} held by {seen[p]!r} and {rc.request_id!r}"
-                        )
+                        raise AssertionError(f"group {gi}: page {p} held by {seen[p]!r} and {holder!r}")
                     if not g.pool._held[p]:
                         raise AssertionError(f"group {gi}: page {p} in a block table but free")
-                    seen[p] = rc.request_id
+                    seen[p] = holder
             if len(seen) != g.pool.n_held:
                 raise AssertionError(
                     f"group {gi}: {g.pool.n_held} pages held but {len(seen)} in block tables"

@@ -80,6 +80,11 @@ class Request:
     # the name under which the engine and its cache manager know the request: unique over all
     # schedulers that share the engine (``Scheduler.add`` sets it)
     engine_id: Any = None
+    # A kept cache (``prompt_cache.PromptCache``) that the request goes on from and leaves what it
+    # computed in: the prompt then holds only the tokens that come on top of the cache's, which
+    # are ``offset`` (set when the request is added).
+    kept: Any = None
+    offset: int = 0
 
     @property
     def tokens(self):
@@ -88,6 +93,11 @@ class Request:
     @property
     def num_tokens(self):
         return len(self.prompt) + len(self.generated)
+
+    @property
+    def context(self):
+        """Tokens of the whole sequence so far, a kept cache's included."""
+        return self.offset + len(self.prompt) + len(self.generated)
 
     @property
     def decoding(self):
@@ -181,11 +191,16 @@ class Scheduler:
             raise ValueError("a request needs a prompt of at least one token")
         if request.max_tokens < 0:
             raise ValueError("max_tokens must not be negative")
-        if len(request.prompt) > self.max_positions:
+        if request.kept is not None and request.kept.in_use:
+            raise ValueError("the request's prompt cache is in use by another live request")
+        request.offset = request.kept.offset if request.kept is not None else 0
+        if request.offset + len(request.prompt) > self.max_positions:
             raise ValueError(
-                f"the prompt has {len(request.prompt)} tokens, the model has {self.max_positions} positions"
+                f"the prompt has {len(request.prompt)} tokens"
+                + (f" on top of the {request.offset} of its cache" if request.offset else "")
+                + f", the model has {self.max_positions} positions"
             )
-        most = min(len(request.prompt) + request.max_tokens, self.max_positions)
+        most = min(request.offset + len(request.prompt) + request.max_tokens, self.max_positions)
         if self.cache.blocks_for(most) > self.cache.n_pages:
             raise ValueError(
                 f"request {request.request_id!r} can reach {most} tokens, the cache holds "
@@ -205,8 +220,10 @@ class Scheduler:
         self.waiting.append(request)
         return request
 
-    def abort(self, request_id):
-        """Take a request out, wherever it is (``remove`` of mlx_lm/generate.py:1777-1802)."""
+    def abort(self, request_id, keep=None):
+        """Take a request out, wherever it is (``remove`` of mlx_lm/generate.py:1777-1802).
+        ``keep``: an empty kept cache that takes what the request has computed (a request that
+        came with a kept cache leaves it there anyway)."""
         for r in list(self.waiting):
             if r.request_id == request_id:
                 self.waiting.remove(r)
@@ -214,6 +231,8 @@ class Scheduler:
                 return r
         for r in self.running:
             if r.request_id == request_id:
+                if keep is not None and r.kept is None:
+                    r.kept, keep.in_use = keep, True
                 self._drop(r)
                 return r
         raise KeyError(f"request {request_id!r} is not known")
@@ -228,8 +247,30 @@ class Scheduler:
             self.running.remove(r)
         elif r in self.waiting:  # pre-empted, and finished by the token that was in flight
             self.waiting.remove(r)
-        if self.engine.has_request(r.engine_id):
+        if not self.engine.has_request(r.engine_id):
+            return
+        if r.kept is None:
             self.engine.end_request(r.engine_id)
+        else:
+            self._keep(r)
+
+    def _keep(self, r):
+        """The request is over and its cache is kept: the cache is to hold exactly the tokens that
+        the host knows, the last generated one included (mlx_lm/generate.py:444-461 feeds it
+        before it stops).  A token still in flight when the request was taken out is forgotten;
+        tokens that were never fed (the last one, which ends a request before it is read back)
+        go through the model now, with no logits asked for."""
+        eid = r.engine_id
+        known = r.offset + len(r.prompt) + len(r.generated)
+        have = self.engine.context_len(eid)
+        try:
+            if have > known:
+                r.kept.rewind(self.engine, eid, known)
+            elif have < known and r.finish_reason is not None:
+                missing = (r.prompt + r.generated)[have - r.offset:]
+                self.engine.step([StepEntry(eid, missing, [])])
+        finally:
+            r.kept.checkin(self.engine, eid)
 
     def close(self):
         """Take every request out and give back what they hold in the engine."""
@@ -240,9 +281,13 @@ class Scheduler:
     def _ends_with_token_in_flight(self, r):
         """The token in flight is the request's last, whatever it is."""
         return r.inflight_row is not None and (
-            len(r.generated) + 1 >= r.max_tokens or r.num_tokens + 1 >= self.max_positions)
+            len(r.generated) + 1 >= r.max_tokens or r.context + 1 >= self.max_positions)
 
     def _preempt(self, r):
+        if r.kept is not None and self.engine.has_request(r.engine_id):
+            # back to what the kept cache held when the request came: only its own tokens are read again
+            r.kept.rewind(self.engine, r.engine_id)
+            r.kept.checkin(self.engine, r.engine_id)
         self._drop(r)
         r.num_computed = 0
         r.preemptions += 1
@@ -299,7 +344,9 @@ class Scheduler:
             r = self.waiting[0]
             if r.inflight_row is not None:
                 break  # pre-empted with a token in flight: it is read as a prompt once that token is known
-            whole = self.cache.blocks_for(min(r.num_tokens + 1, self.max_positions))
+            # (a kept cache brings the pages of its tokens with it)
+            n_new = min(r.num_tokens + 1, self.max_positions - r.offset)
+            whole = self.cache.blocks_for(r.offset + n_new) - self.cache.blocks_for(r.offset)
             if whole > free:
                 break
             # The request leaves the queue only once the engine has it and its pages: whatever
@@ -307,13 +354,19 @@ class Scheduler:
             # it waiting, first in line.  The whole prompt's pages are taken now, so a request that
             # was admitted can always finish reading its prompt.
             try:
-                self.engine.add_request(r.engine_id)
+                if r.kept is not None:
+                    r.kept.checkout(self.engine, r.engine_id)
+                else:
+                    self.engine.add_request(r.engine_id)
             except OutOfSlots:
                 break
             try:
-                self.cache.reserve(r.engine_id, min(r.num_tokens + 1, self.max_positions))
+                self.cache.reserve(r.engine_id, n_new)
             except BaseException as e:
-                self.engine.end_request(r.engine_id)
+                if r.kept is not None:
+                    r.kept.checkin(self.engine, r.engine_id)
+                else:
+                    self.engine.end_request(r.engine_id)
                 if isinstance(e, OutOfPages):
                     break
                 raise
@@ -379,9 +432,11 @@ class Scheduler:
         (``add`` refused what could never fit, so others on the same engine hold the room)."""
         others = [rid for rid in self.cache.requests
                   if not (isinstance(rid, tuple) and len(rid) == 2 and rid[0] == self.number)]
+        kept = sum(len(pages) for k in getattr(self.cache, "kept", ()) for pages in k.blocks)
         return (f"requests are waiting but none can be admitted: {self.cache.free_pages()} of "
-                f"{self.cache.n_pages} pages are free and {len(others)} requests of other generators "
-                f"on this engine hold pages or slots; finish or close those first")
+                f"{self.cache.n_pages} pages are free, {len(others)} requests of other generators "
+                f"on this engine hold pages or slots and kept prompt caches hold {kept} pages; "
+                f"finish, close or free those first")
 
     def _run(self, plan, prev=None):
         """Launch the planned step; decoding requests whose token is in flight get it fed on the device."""
@@ -425,7 +480,7 @@ class Scheduler:
         # "length" at max_tokens or when the model's positions are used up;
         # "stop" is checked second and wins (mlx_lm/generate.py:1501-1514)
         reason = None
-        if len(r.generated) >= r.max_tokens or r.num_tokens >= self.max_positions:
+        if len(r.generated) >= r.max_tokens or r.context >= self.max_positions:
             reason = "length"
         if stops(r.generated, r.stop_sequences):
             reason = "stop"

@@ -120,6 +120,17 @@ class Engine:
     def end_request(self, request_id):
         self.cache.release(request_id)
 
+    def detach_request(self, request_id):
+        """End a request but keep what it computed (its pages stay held): ``KeptPages`` that
+        ``attach_request`` makes a request of again and ``drop_kept`` gives back."""
+        return self.cache.detach(request_id)
+
+    def attach_request(self, request_id, kept):
+        return self.cache.attach(request_id, kept)
+
+    def drop_kept(self, kept):
+        self.cache.drop(kept)
+
     def has_request(self, request_id):
         return request_id in self.cache.requests
 

@@ -131,7 +131,7 @@ def make_sample_fn():
 
 
 _UNSUPPORTED = {
-    "max_kv_size": None, "prompt_cache": None, "kv_bits": None, "input_embeddings": None,
+    "max_kv_size": None, "kv_bits": None, "input_embeddings": None,
     "draft_model": None,
 }
 
@@ -154,18 +154,23 @@ class _OneRequest:
     The prompt is read in portions of ``prefill_step_size`` (under ``max_num_batched_tokens``
     a step); then one token per step.  ``stop_tokens`` end the request with reason ``"stop"``,
     ``max_tokens`` or the model's positions with ``"length"``; its pages go back at once.
-    ``page_size``/``num_pages`` choose the cache that the model's engine is made with.
+    ``page_size``/``num_pages`` choose the cache that the model's engine is made with; ``engine``
+    names an engine instead (by default the one whose pool ``prompt_cache`` lies in, if it holds tokens).
+    ``prompt_cache`` (a ``PromptCache``): the prompt comes on top of the tokens that the cache
+    holds, and when the request ends the cache holds the prompt and all generated tokens as well.
     """
 
     def __init__(self, model, prompt, max_tokens, sampler=None, logits_processors=None,
                  prefill_step_size=2048, prompt_progress_callback=None, seed=None, stop_tokens=(),
                  want_logprobs=True, page_size=16, num_pages=None, max_num_seqs=1,
-                 max_num_batched_tokens=None):
+                 max_num_batched_tokens=None, prompt_cache=None, engine=None):
         self.prompt = [int(t) for t in (prompt.tolist() if hasattr(prompt, "tolist") else prompt)]
         if len(self.prompt) == 0:
             raise ValueError("Either input_embeddings or prompt (or both) must be provided.")
-        self.engine = engine_for(model, page_size=page_size,
-                                 max_cache_tokens=None if num_pages is None else num_pages * page_size)
+        if engine is None and prompt_cache is not None:
+            engine = prompt_cache.engine  # a cache that holds tokens holds them in one engine's pool
+        self.engine = engine or engine_for(
+            model, page_size=page_size, max_cache_tokens=None if num_pages is None else num_pages * page_size)
         self.scheduler = Scheduler(self.engine, make_sample_fn(), max_num_seqs=max(1, max_num_seqs),
                                    max_num_batched_tokens=max_num_batched_tokens or prefill_step_size,
                                    prefill_step_size=prefill_step_size)
@@ -177,7 +182,7 @@ class _OneRequest:
             seed = sample_utils.default_seed()
         self.request = Request(self.request_id, self.prompt, max_tokens, sampler=sampler,
                                logits_processors=logits_processors, seed=seed, want_logprobs=want_logprobs,
-                               stop_sequences=[[int(t)] for t in stop_tokens])
+                               stop_sequences=[[int(t)] for t in stop_tokens], kept=prompt_cache)
         self.progress = prompt_progress_callback
         self.scheduler.add(self.request)
 
@@ -198,15 +203,20 @@ class _OneRequest:
 
 
 def generate_step(prompt, model, *, max_tokens=256, sampler=None, logits_processors=None,
-                  prefill_step_size=2048, prompt_progress_callback=None, seed=None, **kwargs):
+                  prefill_step_size=2048, prompt_progress_callback=None, seed=None, prompt_cache=None,
+                  **kwargs):
     """Yield ``(token, logprobs)`` for one prompt (mlx_lm/generate.py:298-461).
+
+    ``prompt_cache`` (``make_prompt_cache(model)``): what earlier calls computed; the prompt is
+    read on top of it and the cache is updated in place (mlx_lm/generate.py:306,329-331), so a
+    later call goes on from prompt and generated tokens with only its own tokens to read.
 
     The prompt is read in portions of ``prefill_step_size``; then one token
     per step.  ``logprobs`` is a float32 device tensor ``[vocab]``.  Exactly
     ``max_tokens`` tokens are yielded unless the model's positions run out.
     Beyond the reference's options: ``seed`` keys the draws; ``page_size``,
     ``num_pages``, ``max_num_seqs`` and ``max_num_batched_tokens`` shape the
-    cache and the scheduler.
+    cache and the scheduler; ``engine`` names the engine to run on.
     """
     _refuse_unsupported(kwargs)
     geometry = {k: kwargs.pop(k) for k in _ENGINE_OPTIONS if k in kwargs}
@@ -214,12 +224,12 @@ def generate_step(prompt, model, *, max_tokens=256, sampler=None, logits_process
         raise TypeError(f"unknown options: {sorted(kwargs)}")
     run = _OneRequest(model, prompt, max_tokens, sampler=sampler, logits_processors=logits_processors,
                       prefill_step_size=prefill_step_size, prompt_progress_callback=prompt_progress_callback,
-                      seed=seed, **geometry)
+                      seed=seed, prompt_cache=prompt_cache, **geometry)
     for out in run:
         yield out.token, out.logprobs
 
 
-_ENGINE_OPTIONS = ("page_size", "num_pages", "max_num_seqs", "max_num_batched_tokens")
+_ENGINE_OPTIONS = ("page_size", "num_pages", "max_num_seqs", "max_num_batched_tokens", "engine")
 
 
 @dataclass
@@ -411,7 +421,7 @@ class BatchGenerator:
     def __init__(self, model, *, max_tokens=128, stop_tokens=None, sampler=None,
                  logits_processors=None, completion_batch_size=32, prefill_batch_size=8,
                  prefill_step_size=2048, max_kv_size=None, stream=None, seed=None,
-                 want_logprobs=True, engine=None):
+                 want_logprobs=True, engine=None, return_prompt_caches=False):
         if max_kv_size is not None:
             raise ValueError("'max_kv_size' is not supported by this engine")
         self.model = model
@@ -431,12 +441,17 @@ class BatchGenerator:
             prefill_step_size=prefill_step_size)
         self._uid_count = 0
         self._requests = {}
+        # every finished request's response carries what it computed as a ``PromptCache``
+        self.return_prompt_caches = return_prompt_caches
 
     def close(self):
         """Drop every request; their pages and slots go back to the engine, which other
         generators over the same model share."""
-        self._requests.clear()
+        live, self._requests = list(self._requests.values()), {}
         self.scheduler.close()
+        for r in live:
+            if r.kept is not None:
+                r.kept.free()
 
     def __del__(self):
         try:
@@ -468,10 +483,13 @@ class BatchGenerator:
 
         ``stop_matchers[i]`` is a list of token-id sequences that stop request
         ``i``.  ``seeds[i]`` keys its random draws (default: the generator's
-        seed plus the uid).
+        seed plus the uid).  ``caches[i]``: a ``PromptCache`` that request ``i`` goes on from: its
+        prompt comes on top of the cache's tokens.  As in the reference, which merges the given
+        caches into its batch (mlx_lm/generate.py:1107-1120), the cache given stays as it is:
+        the request works on a copy (pages of its own), which its last response carries.
         """
-        if caches is not None and any(c is not None for c in caches):
-            raise ValueError("re-inserting prompt caches is not supported")
+        from .prompt_cache import PromptCache
+
         uids = []
         for i, p in enumerate(prompts):
             uid = self._uid_count
@@ -485,7 +503,9 @@ class BatchGenerator:
                 stop_sequences=(stop_matchers[i] if stop_matchers and stop_matchers[i] is not None
                                 else self.stop_tokens),
                 seed=(seeds[i] if seeds else self.seed + uid),
-                want_logprobs=self.want_logprobs)
+                want_logprobs=self.want_logprobs,
+                kept=(caches[i].copy() if caches and caches[i] is not None
+                      else PromptCache(self.model) if self.return_prompt_caches else None))
             self.scheduler.add(req)
             if req.finish_reason is None:  # (a request for no tokens at all is over already)
                 self._requests[uid] = req
@@ -493,14 +513,24 @@ class BatchGenerator:
         return uids
 
     def remove(self, uids, return_prompt_caches=False):
+        """Drop requests; with ``return_prompt_caches`` a dict from uid to the ``PromptCache`` of
+        what the request had computed (mlx_lm/generate.py:1777-1802)."""
+        from .prompt_cache import PromptCache
+
+        caches = {}
         for uid in uids:
             if uid in self._requests:
+                r = self._requests.pop(uid)
+                keep = PromptCache(self.model) if return_prompt_caches and r.kept is None else None
                 try:
-                    self.scheduler.abort(uid)
+                    self.scheduler.abort(uid, keep=keep)
                 except KeyError:
                     pass
-                del self._requests[uid]
-        return {} if return_prompt_caches else None
+                if return_prompt_caches and r.kept is not None:
+                    caches[uid] = r.kept
+                elif r.kept is not None:
+                    r.kept.free()  # the request's own copy: nobody goes on from it
+        return caches if return_prompt_caches else None
 
     def _next(self):
         before = {uid: r.num_computed for uid, r in self._requests.items() if not r.generated}
@@ -514,7 +544,8 @@ class BatchGenerator:
         responses = []
         for o in outs:
             r = self._requests[o.request_id]
-            responses.append(self.Response(o.request_id, o.token, o.logprobs, o.finish_reason, None,
+            responses.append(self.Response(o.request_id, o.token, o.logprobs, o.finish_reason,
+                                           r.kept if o.finish_reason else None,
                                            r.tokens if o.finish_reason else None, o.logprob))
             if o.finish_reason is not None:
                 del self._requests[o.request_id]
@@ -539,11 +570,9 @@ def batch_generate(model, tokenizer, prompts, prompt_caches=None, max_tokens=128
     The tokenizer's end tokens stop a request; the token that stops it is not part of its
     result.  ``kwargs`` go to ``BatchGenerator``.
     """
-    if prompt_caches is not None or return_prompt_caches:
-        raise ValueError("prompt caches are not supported")
     tokenizer = tokenizer if tokenizer is not None else IdTokenizer()
     gen = BatchGenerator(model, stop_tokens=[[t] for t in tokenizer.eos_token_ids],
-                         want_logprobs=False, **kwargs)
+                         want_logprobs=False, return_prompt_caches=return_prompt_caches, **kwargs)
     limits = [max_tokens] * len(prompts) if isinstance(max_tokens, int) else list(max_tokens)
     total, finished = len(prompts), 0
 
@@ -553,8 +582,9 @@ def batch_generate(model, tokenizer, prompts, prompt_caches=None, max_tokens=128
                   end=end)
 
     progress()
-    uids = gen.insert(prompts, limits)
+    uids = gen.insert(prompts, limits, caches=prompt_caches)
     kept = {uid: ([], []) for uid in uids}  # tokens and their log-probabilities
+    caches = {}
     with gen.stats() as stats:
         while True:
             responses = gen.next_generated()
@@ -566,15 +596,21 @@ def batch_generate(model, tokenizer, prompts, prompt_caches=None, max_tokens=128
                     kept[r.uid][1].append(r.token_logprob)
                 if r.finish_reason is not None:
                     finished += 1
+                    caches[r.uid] = r.prompt_cache
                     progress()
     gen.close()
+    if not return_prompt_caches:
+        for c in caches.values():
+            if c is not None:
+                c.free()
     progress(end="\n")
     if verbose:
         print(f"[batch_generate] Prompt: {stats.prompt_tokens} tokens, {stats.prompt_tps:.3f} tokens-per-sec")
         print(f"[batch_generate] Generation: {stats.generation_tokens} tokens, "
               f"{stats.generation_tps:.3f} tokens-per-sec")
         print(f"[batch_generate] Peak memory: {stats.peak_memory:.3f} GB")
-    return BatchResponse([tokenizer.decode(kept[uid][0]) for uid in uids], stats, None,
+    return BatchResponse([tokenizer.decode(kept[uid][0]) for uid in uids], stats,
+                         [caches.get(uid) for uid in uids] if return_prompt_caches else None,
                          [kept[uid][0] for uid in uids] if return_token_ids else None,
                          [kept[uid][1] for uid in uids] if return_logprobs else None)
 

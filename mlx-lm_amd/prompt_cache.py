@@ -1,0 +1,136 @@
+"""What a request has computed, kept for a later request to go on from.
+
+The reference keeps a list of per-layer caches (``make_prompt_cache``,
+mlx_lm/models/cache.py:15-43) that ``generate_step(..., prompt_cache=...)``
+fills and updates in place (mlx_lm/generate.py:306,329-331,362-385), that
+``trim_prompt_cache`` shortens (mlx_lm/models/cache.py:88-111) and that
+``BatchGenerator`` takes and hands back per request
+(mlx_lm/generate.py:1689-1731,1777-1802).  Here a kept cache is one object for
+the whole model: the pages that the request held in the engine's pool, which
+simply stay held, and the request's row of every state tensor.  Nothing is
+copied when a request goes on from it.  Saving one to a file is not offered.
+"""
+
+
+class PromptCache:
+    """Keys, values and state of the tokens that went through it, in the pool of one engine.
+
+    A request is given it as ``prompt_cache`` (``generate_step``, ``stream_generate``) or in
+    ``caches`` (``BatchGenerator.insert``); it then reads only the tokens it brings, on top
+    of what the cache holds, and when it ends the cache holds those tokens and all the
+    generated ones as well.  While a request uses it, nobody else can.  ``offset`` is the
+    number of tokens held.  The pages count against the engine's pool until ``free()`` (or
+    until the object goes away).
+    """
+
+    def __init__(self, model=None):
+        self.model = model
+        self._engine = None
+        self._kept = None
+        self._at_checkout = (0, None)
+        self.in_use = False
+
+    @property
+    def offset(self):
+        return self._kept.length if self._kept is not None else 0
+
+    @property
+    def engine(self):
+        """The engine in whose pool the tokens lie (``None`` while the cache is empty and was never used)."""
+        return self._engine if (self._kept is not None or self.in_use) else None
+
+    def __len__(self):
+        return self.offset
+
+    # -- what the scheduler calls ------------------------------------------------
+
+    def checkout(self, engine, engine_id):
+        """A live request ``engine_id`` of ``engine`` that holds what this cache holds."""
+        if self.in_use:
+            raise ValueError("this prompt cache is in use by a live request")
+        if self._kept is not None and self._engine is not engine:
+            raise ValueError("this prompt cache holds pages of another engine (another cache geometry or model)")
+        self._engine, self.in_use = engine, True
+        self._at_checkout = (self.offset, self._kept.state if self._kept is not None else None)
+        if self._kept is None:
+            engine.add_request(engine_id)
+        else:
+            kept, self._kept = self._kept, None
+            try:
+                engine.attach_request(engine_id, kept)
+            except Exception:
+                self._kept, self.in_use = kept, False
+                raise
+
+    def rewind(self, engine, engine_id, length=None):
+        """Cut the live request back to ``length`` tokens, or to what the cache held when the request
+        took it.  Per-request state cannot be cut: a model that has some goes all the way back,
+        its state rows as they were then."""
+        offset, state = self._at_checkout
+        if length is None or (engine.cache.state_needs and length != engine.context_len(engine_id)):
+            length = offset
+            if engine.cache.state_needs:
+                engine.cache.set_state(engine_id, state)
+        engine.truncate(engine_id, length)
+
+    def checkin(self, engine, engine_id):
+        """The request ends: what it holds is this cache's from now on."""
+        self._engine = engine
+        engine.truncate(engine_id, engine.context_len(engine_id))  # pages taken ahead of the tokens go back
+        self._kept = engine.detach_request(engine_id)
+        self.in_use = False
+
+    # -- what callers use ----------------------------------------------------------
+
+    def is_trimmable(self):
+        return not self.in_use and (self._engine is None or not self._engine.cache.state_needs)
+
+    def trim(self, n_tokens):
+        """Forget the last ``n_tokens`` tokens (at most all); returns how many went."""
+        if self.in_use:
+            raise ValueError("this prompt cache is in use by a live request")
+        n = max(0, min(int(n_tokens), self.offset))
+        if n:
+            self._engine.cache.truncate_kept(self._kept, self.offset - n)
+        return n
+
+    def copy(self):
+        """A second cache with the same tokens, in pages of its own (``OutOfPages`` if the pool is short)."""
+        if self.in_use:
+            raise ValueError("this prompt cache is in use by a live request")
+        other = PromptCache(self.model)
+        if self._kept is not None:
+            other._engine = self._engine
+            other._kept = self._engine.cache.fork(self._kept)
+        return other
+
+    def free(self):
+        """Give the pages back to the engine's pool; the cache is empty afterwards."""
+        if self._kept is not None and not self.in_use:
+            self._engine.drop_kept(self._kept)
+            self._kept = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:  # noqa: BLE001 (the interpreter may be shutting down)
+            pass
+
+
+def make_prompt_cache(model=None, max_kv_size=None):
+    """An empty cache for ``model`` (``make_prompt_cache`` of mlx_lm/models/cache.py:15-43)."""
+    if max_kv_size is not None:
+        raise ValueError("'max_kv_size' is not supported by this engine")
+    return PromptCache(model)
+
+
+def can_trim_prompt_cache(cache):
+    """mlx_lm/models/cache.py:88-92."""
+    return cache.is_trimmable()
+
+
+def trim_prompt_cache(cache, num_tokens):
+    """Trim in place; returns the number of tokens trimmed (mlx_lm/models/cache.py:95-111)."""
+    if not can_trim_prompt_cache(cache):
+        return 0
+    return cache.trim(num_tokens)

@@ -114,10 +114,37 @@ def test_truncate_gives_whole_pages_back():
 def test_random_orders_keep_every_page_accounted(seed, window):
     rng = random.Random(seed)
     cm = _manager(n_pages=12, window=window, max_requests=5)
-    live, n = {}, 0
+    live, n, kept = {}, 0, []
     for _ in range(600):
         op = rng.random()
-        if op < 0.2 and len(live) < 5:
+        if op < 0.08 and live:  # a request's pages are kept aside ...
+            rid = rng.choice(list(live))
+            kept.append((cm.detach(rid), live.pop(rid)))
+            assert rid not in cm.requests
+        elif op < 0.16 and kept:  # ... and go on under a new name, are cut back, or are given back
+            k, length = kept.pop(rng.randrange(len(kept)))
+            what = rng.random()
+            if what < 0.5 and len(live) < 5:
+                rid = f"r{n}"
+                n += 1
+                assert cm.attach(rid, k).length == length
+                live[rid] = length
+                with pytest.raises(ValueError):
+                    cm.attach("again", k)
+            elif what < 0.75 and window == 0:
+                new = rng.randint(0, length)
+                cm.truncate_kept(k, new)
+                kept.append((k, new))
+            elif what < 0.85:
+                kept.append((k, length))
+                try:
+                    kept.append((cm.fork(k), length))
+                except OutOfPages:
+                    pass
+            else:
+                cm.drop(k)
+                cm.drop(k)  # a second time is nothing
+        elif op < 0.3 and len(live) < 5:
             rid = f"r{n}"
             n += 1
             cm.add(rid)
@@ -155,7 +182,11 @@ def test_random_orders_keep_every_page_accounted(seed, window):
                 first = 0 if g.need.window == 0 else lo // 16
                 assert all(p >= 0 for p in rc.blocks[gi][first : cm.blocks_for(length)])
     cm.release_all()
-    assert all(g.pool.n_free == 12 for g in cm.groups)
+    assert all(g.pool.n_free == 12 - sum(sum(p >= 0 for p in k.blocks[gi]) for k, _ in kept)
+               for gi, g in enumerate(cm.groups))
+    for k, _ in kept:
+        cm.drop(k)
+    assert all(g.pool.n_free == 12 for g in cm.groups) and not cm.kept
     cm.check()
 
 
@@ -230,3 +261,47 @@ def test_keys_and_values_may_differ_in_width():
     for p in range(5):
         assert bool((k[p] == 7).all()) == (p not in held) and bool((v[p] == 7).all()) == (p not in held)
     cm.check()
+
+
+def test_kept_pages_carry_contents_and_state():
+    """``detach``/``attach`` move nothing but the state rows; ``fork`` copies the pages' contents into
+    pages of its own (a window's missing pages stay missing) and fails whole when the pool is short."""
+    import torch
+
+    needs = [CacheNeed(2, 16, 0), CacheNeed(1, 16, 24, v_head_dim=32), StateNeed((3,))]
+    cm = CacheManager(needs, 16, 9, 3, dtype=torch.float32, device="cpu")
+    cm.add("a")
+    cm.reserve("a", 70)
+    cm.commit("a", 70)  # five blocks; the window of 24 has passed the first two
+    rc = cm.requests["a"]
+    assert rc.blocks[1][:2] == [-1, -1] and all(p >= 0 for p in rc.blocks[0])
+    for gi, g in enumerate(cm.groups):
+        for b, p in enumerate(rc.blocks[gi]):
+            if p >= 0:
+                g.keys[:, p] = 100 * gi + b + 1
+                g.values[:, p] = -(100 * gi + b + 1)
+    cm.state(2)[rc.state_slot] = torch.tensor([1.0, 2.0, 3.0])
+    kept = cm.detach("a")
+    cm.add("b")  # takes the state row that "a" had
+    cm.state(2)[cm.requests["b"].state_slot] = 7.0
+    with pytest.raises(OutOfPages, match="a copy of 70 kept tokens"):
+        cm.fork(kept)  # group 0 has 4 pages left, five are needed
+    assert [g.pool.n_free for g in cm.groups] == [4, 6]
+    cm.truncate_kept(kept, 60)  # four blocks
+    copy = cm.fork(kept)
+    assert [g.pool.n_free for g in cm.groups] == [1, 5] and copy.length == 60  # a page each came back by the cut
+    assert copy.blocks[1][:2] == [-1, -1] and not set(copy.blocks[0]) & set(kept.blocks[0])
+    cm.drop(kept)  # the original goes; the copy stands alone
+    rc = cm.attach("c", copy)
+    for gi, g in enumerate(cm.groups):
+        for b, p in enumerate(rc.blocks[gi]):
+            if p >= 0:
+                assert (g.keys[:, p] == 100 * gi + b + 1).all() and (g.values[:, p] == -(100 * gi + b + 1)).all()
+    assert cm.state(2)[rc.state_slot].tolist() == [1.0, 2.0, 3.0]
+    cm.set_state("c")
+    assert cm.state(2)[rc.state_slot].tolist() == [0.0, 0.0, 0.0]
+    cm.set_state("c", {2: torch.tensor([4.0, 5.0, 6.0])})
+    assert cm.state(2)[rc.state_slot].tolist() == [4.0, 5.0, 6.0]
+    cm.check()
+    cm.release_all()
+    assert [g.pool.n_free for g in cm.groups] == [9, 9] and not cm.kept

@@ -28,6 +28,21 @@ class FakeEngine:
     def has_request(self, rid):
         return rid in self.cache.requests
 
+    def context_len(self, rid):
+        return self.cache.requests[rid].length
+
+    def truncate(self, rid, new_length):
+        return self.cache.truncate(rid, new_length).length
+
+    def detach_request(self, rid):
+        return self.cache.detach(rid)
+
+    def attach_request(self, rid, kept):
+        return self.cache.attach(rid, kept)
+
+    def drop_kept(self, kept):
+        self.cache.drop(kept)
+
     def step(self, entries, fed=None):
         # the engine knows a request as (its scheduler's number, the scheduler's own id for it);
         # the log and the rows name it as its scheduler does
@@ -54,7 +69,7 @@ def fake_sample(rows, requests):
     assert len(rows) == len(requests)
     out = []
     for (rid, pos, _), r in zip(rows, requests):
-        assert rid == r.request_id and pos == r.num_tokens - 1  # the row of the newest token
+        assert rid == r.request_id and pos == r.offset + r.num_tokens - 1  # the row of the newest token
         out.append((token_for(rid, len(r.generated)), -1.0, None))
     return out
 
@@ -345,3 +360,80 @@ def test_admission_that_fails_keeps_the_request_first_in_line():
     assert eng.cache.requests
     a.close()
     assert not eng.cache.requests and eng.cache.free_pages() == 16 and not a.has_work
+
+
+@pytest.mark.parametrize("mode", SAMPLERS)
+def test_a_request_goes_on_from_a_kept_cache_and_leaves_its_tokens_there(mode):
+    """``generate_step(..., prompt_cache=c)`` of the reference updates the cache in place: after
+    the call it holds the prompt and every generated token, the last one too
+    (mlx_lm/generate.py:306,329-331,444-461; tests/test_prompt_cache.py:184-204), and the next
+    call reads only its own tokens on top.  Here the request's pages simply stay held."""
+    from mlx_lm_amd.prompt_cache import PromptCache, can_trim_prompt_cache, trim_prompt_cache
+
+    eng = FakeEngine(n_pages=8, max_positions=64)
+    c = PromptCache()
+    s = Scheduler(eng, SAMPLERS[mode]())
+    prompt = list(range(1, 21))
+    s.add(Request("a", prompt, 3, kept=c))
+    done = run_all(s)
+    first = [o.token for o in done["a"]]
+    assert first == [token_for("a", i) for i in range(3)]
+    assert c.offset == 23 and not c.in_use and not eng.cache.requests  # prompt and all three tokens
+    assert eng.cache.free_pages() == 8 - 2 and len(eng.cache.kept) == 1
+    # the token that ended the request went through the model with no logits asked for
+    assert eng.log[-1] == [("a", 1, [])] or mode == "overlapped"
+    eng.cache.check()
+    # the next request brings one token and starts at position 23
+    s2 = Scheduler(eng, SAMPLERS[mode]())
+    r = s2.add(Request("a", [777], 2, kept=c))
+    assert r.offset == 23 and c.offset == 23
+    before = len(eng.log)
+    early = s2.step()
+    with pytest.raises(ValueError, match="in use"):  # a cache serves one live request at a time
+        s2.add(Request("b", [5], 1, kept=c))
+    done = run_all(s2)
+    assert eng.log[before] == [("a", 1, [0])]  # only its own token is read
+    assert c.offset == 23 + 1 + 2 and len(early) + len(done["a"]) == 2
+    # what does not fit the positions on top of the cache is refused
+    with pytest.raises(ValueError, match="on top of the 26 of its cache"):
+        Scheduler(eng, fake_sample).add(Request("x", list(range(1, 60)), 1, kept=c))
+    # trimming, then giving the pages back
+    assert can_trim_prompt_cache(c) and trim_prompt_cache(c, 10) == 10 and c.offset == 16
+    assert eng.cache.free_pages() == 8 - 1
+    eng.cache.check()
+    c.free()
+    assert eng.cache.free_pages() == 8 and not eng.cache.kept and c.offset == 0
+
+
+@pytest.mark.parametrize("mode", SAMPLERS)
+def test_kept_caches_under_preemption_and_abort(mode):
+    from mlx_lm_amd.prompt_cache import PromptCache
+
+    eng = FakeEngine(n_pages=6, max_positions=200)
+    c = PromptCache()
+    s = Scheduler(eng, SAMPLERS[mode](), max_num_seqs=4)
+    s.add(Request("seed", list(range(1, 18)), 1, kept=c))  # 17 + 1 tokens: two pages kept
+    run_all(s)
+    assert c.offset == 18
+    # "old" grows until the pool is full; "new", on top of the kept cache, is the victim: it goes
+    # back to the 18 tokens of its cache and reads only its own tokens again
+    s.add(Request("old", list(range(1, 31)), 20))
+    s.add(Request("new", list(range(1, 11)), 30, kept=c))
+    done = run_all(s)
+    assert s.stats.preemptions >= 1
+    assert [o.token for o in done["new"]] == [token_for("new", i) for i in range(30)]
+    assert [o.token for o in done["old"]] == [token_for("old", i) for i in range(20)]
+    assert c.offset == 18 + 10 + 30 and eng.cache.free_pages() == 6 - 4
+    reread = [e for st in eng.log for e in st if e[0] == "new" and e[1] > 10]
+    assert reread and all(e[1] <= 10 + 30 for e in reread)  # never the cache's own 18 tokens
+    eng.cache.check()
+    # taken out half-way with an empty cache to keep what it computed
+    s.add(Request("cut", list(range(1, 21)), 5))
+    s.max_num_batched_tokens = s.prefill_step_size = 16
+    s.step()
+    half = PromptCache()
+    s.abort("cut", keep=half)
+    assert half.offset == 16 and not s.has_work
+    half.free()
+    c.free()
+    assert eng.cache.free_pages() == 6 and not eng.cache.kept
