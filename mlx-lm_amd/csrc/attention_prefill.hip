@@ -57,7 +57,8 @@ __device__ __forceinline__ int key_of_row(int rho) {
   return 16 * (j >> 1) + 8 * g + 4 * (j & 1) + i;
 }
 
-template <int HD>
+// POW2: the page size is a power of two (a key's page and row are a shift and a mask)
+template <int HD, bool POW2>
 __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(PrefillArgs p) {
   constexpr int KS_STRIDE = HD + 8;
   constexpr int DC = HD / 16;           // 16-column chunks of a head (QK contraction steps)
@@ -81,7 +82,7 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
   const int kv_head = h / (p.n_heads / p.n_kv_heads);
   const int pos0 = p.positions[row0];
   const int* table = p.block_table + (size_t)p.token_req[row0] * p.max_blocks;
-  const size_t head_off = (size_t)kv_head * p.page_size * HD;
+  const uint32_t head_off = (uint32_t)(kv_head * p.page_size * HD);  // (within a page: below its stride)
 
   const int ql = lane & 31, g = lane >> 5;
   const int qi = wave * 32 + ql;         // this lane's query within the tile
@@ -132,15 +133,22 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_prefill_kernel(Pre
   // Loads are never predicated and never zeroed: a key outside [k_lo, k_hi) is
   // read from the nearest key inside (a valid address with finite numbers);
   // its score is masked below, so its probability is zero.
+  // An address is a dozen integer instructions, four times a thread and tile, in a kernel whose
+  // time is its vector instructions: a division by a run-time page size alone costs thirty, and
+  // choosing between it and a shift at run time put a branch around every address.  So the
+  // choice is the kernel's template argument, and everything but the page's start is 32-bit.
   const uint32_t stride32 = (uint32_t)p.page_stride;
+  const int shift = p.page_shift, row_mask = p.page_size - 1;
   auto address = [&](int key, int col) __attribute__((always_inline)) -> size_t {
     const int kk = min(max(key, k_lo), k_hi - 1);
-    // (a division by a run-time number costs some thirty instructions, and there are four
-    // addresses a thread and tile: page sizes that are powers of two take a shift instead)
-    const int idx = p.page_shift >= 0 ? kk >> p.page_shift : kk / p.page_size;
-    const int row = kk - idx * p.page_size;
-    // (page number and page stride are 32-bit: one multiply-add instead of a 64-bit product's four)
-    return (size_t)(uint32_t)page_of[idx - pg0] * stride32 + (head_off + (size_t)(row * HD + col));
+    int idx, row;
+    if constexpr (POW2) {
+      idx = kk >> shift, row = kk & row_mask;
+    } else {
+      idx = kk / p.page_size, row = kk - idx * p.page_size;
+    }
+    const uint32_t within = head_off + (uint32_t)(row * HD + col);
+    return (size_t)(uint32_t)page_of[idx - pg0] * stride32 + within;
   };
   auto fetch = [&](int kt, const int set) __attribute__((always_inline)) {
 #pragma unroll
@@ -354,12 +362,18 @@ extern "C" int attn_prefill(void* out, const void* q, int ldq, int ldo, const vo
   if (max_blocks > 7168)
     FAIL("attn_prefill: block tables of %d pages a request do not fit beside the tiles (at most 7168)", max_blocks);
   const size_t lds = (size_t)max_blocks * sizeof(int);
-  if (head_dim == 32)
-    hipLaunchKernelGGL(attn_prefill_kernel<32>, grid, block, lds, stream, p);
-  else if (head_dim == 64)
-    hipLaunchKernelGGL(attn_prefill_kernel<64>, grid, block, lds, stream, p);
-  else
-    hipLaunchKernelGGL(attn_prefill_kernel<128>, grid, block, lds, stream, p);
+  const bool pow2 = p.page_shift >= 0;
+#define LAUNCH_PREFILL(HD)                                                                    \
+  if (pow2) hipLaunchKernelGGL((attn_prefill_kernel<HD, true>), grid, block, lds, stream, p); \
+  else hipLaunchKernelGGL((attn_prefill_kernel<HD, false>), grid, block, lds, stream, p)
+  if (head_dim == 32) {
+    LAUNCH_PREFILL(32);
+  } else if (head_dim == 64) {
+    LAUNCH_PREFILL(64);
+  } else {
+    LAUNCH_PREFILL(128);
+  }
+#undef LAUNCH_PREFILL
   CHECK_LAUNCH("attn_prefill");
   return 0;
 }
