@@ -193,6 +193,9 @@ class Scheduler:
             raise ValueError("max_tokens must not be negative")
         if request.kept is not None and request.kept.in_use:
             raise ValueError("the request's prompt cache is in use by another live request")
+        if request.kept is not None and getattr(request.kept, "engine", None) not in (None, self.engine):
+            raise ValueError("the request's prompt cache holds pages of another engine (another cache "
+                             "geometry, dtype or model): it goes on only where it was made")
         request.offset = request.kept.offset if request.kept is not None else 0
         if request.offset + len(request.prompt) > self.max_positions:
             raise ValueError(

@@ -490,6 +490,10 @@ class BatchGenerator:
         """
         from .prompt_cache import PromptCache
 
+        for c in caches or ():
+            if c is not None and c.engine not in (None, self.engine):
+                raise ValueError("a prompt cache in 'caches' holds pages of another engine than this "
+                                 "generator's: it goes on only where it was made")
         uids = []
         for i, p in enumerate(prompts):
             uid = self._uid_count

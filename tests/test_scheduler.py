@@ -397,6 +397,9 @@ def test_a_request_goes_on_from_a_kept_cache_and_leaves_its_tokens_there(mode):
     # what does not fit the positions on top of the cache is refused
     with pytest.raises(ValueError, match="on top of the 26 of its cache"):
         Scheduler(eng, fake_sample).add(Request("x", list(range(1, 60)), 1, kept=c))
+    # a cache goes on only in the engine whose pool holds it
+    with pytest.raises(ValueError, match="another engine"):
+        Scheduler(FakeEngine(n_pages=8, max_positions=64), fake_sample).add(Request("y", [1], 1, kept=c))
     # trimming, then giving the pages back
     assert can_trim_prompt_cache(c) and trim_prompt_cache(c, 10) == 10 and c.offset == 16
     assert eng.cache.free_pages() == 8 - 1
