@@ -7,7 +7,8 @@ Python entry points (cf. mlx_lm/__init__.py:9-20).
 __version__ = "0.1.0"
 
 from .generate import BatchGenerator, batch_generate, generate, generate_step, stream_generate
-from .prompt_cache import PromptCache, can_trim_prompt_cache, make_prompt_cache, trim_prompt_cache
+from .prompt_cache import (PromptCache, can_trim_prompt_cache, load_prompt_cache, make_prompt_cache,
+                           save_prompt_cache, trim_prompt_cache)
 from .sample_utils import make_logits_processors, make_sampler
 from .utils import load
 
@@ -22,6 +23,8 @@ __all__ = [
     "make_prompt_cache",
     "trim_prompt_cache",
     "can_trim_prompt_cache",
+    "save_prompt_cache",
+    "load_prompt_cache",
     "PromptCache",
     "load",
     "__version__",

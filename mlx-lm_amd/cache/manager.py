@@ -330,6 +330,76 @@ class CacheManager:
         self.kept.append(copy)
         return copy
 
+    def read_kept(self, kept):
+        """What a ``KeptPages`` holds, out of its pages: ``({slot: (keys [tokens, n_kv_heads,
+        head_dim], values [tokens, n_kv_heads, value_dim])}, {slot: state row})`` as tensors of
+        their own (for a file, or for another engine's pool)."""
+        import torch
+
+        if not kept.live:
+            raise ValueError("these kept pages were used already")
+        n_blocks = self.blocks_for(kept.length)
+        out = {}
+        for gi, g in enumerate(self.groups):
+            pages = kept.blocks[gi][:n_blocks]
+            if any(p < 0 for p in pages):
+                raise ValueError("a window has given pages of these tokens back: what is left cannot "
+                                 "stand for the tokens and is not written out")
+            index = torch.tensor(pages, dtype=torch.long, device=g.keys.device)
+            for i, slot in enumerate(g.slots):
+                both = []
+                for pool in (g.keys[i], g.values[i]):  # [pages, heads, page, width]
+                    t = pool.index_select(0, index).permute(0, 2, 1, 3)
+                    both.append(t.reshape(-1, t.shape[2], t.shape[3])[: kept.length].contiguous())
+                out[slot] = tuple(both)
+        return out, {slot: row.clone() for slot, row in kept.state.items()}
+
+    def write_kept(self, length, per_slot, state):
+        """The opposite of ``read_kept``: pages of this pool filled with the given keys and values.
+        Returns the ``KeptPages`` (``OutOfPages`` if the pool is short, with nothing taken)."""
+        import torch
+
+        if set(per_slot) != set(self.slot_group) or set(state) != set(self.state_needs):
+            raise ValueError(f"the cache was written by a model with other layers: it has the cache slots "
+                             f"{sorted(per_slot)} and state slots {sorted(state)}, this model "
+                             f"{sorted(self.slot_group)} and {sorted(self.state_needs)}")
+        for slot, (k, v) in per_slot.items():
+            g = self.groups[self.slot_group[slot][0]]
+            want_k = (length, g.need.n_kv_heads, g.need.head_dim)
+            want_v = (length, g.need.n_kv_heads, g.need.value_dim)
+            if tuple(k.shape) != want_k or tuple(v.shape) != want_v:
+                raise ValueError(f"cache slot {slot}: keys {tuple(k.shape)} and values {tuple(v.shape)} in the "
+                                 f"cache, {want_k} and {want_v} in this model")
+        for slot, row in state.items():
+            if tuple(row.shape) != tuple(self.state_storage[slot].shape[1:]):
+                raise ValueError(f"state slot {slot}: shape {tuple(row.shape)} in the cache, "
+                                 f"{tuple(self.state_storage[slot].shape[1:])} in this model")
+        n_blocks = self.blocks_for(length)
+        taken = []
+        for gi, g in enumerate(self.groups):
+            pages = g.pool.take(n_blocks)
+            if pages is None:
+                for gj, got in taken:
+                    self.groups[gj].pool.give_back(got)
+                raise OutOfPages(f"a cache of {length} tokens needs {n_blocks} pages of group {gi}; "
+                                 f"{g.pool.n_free} are free")
+            taken.append((gi, pages))
+        blocks = []
+        for (gi, pages), g in zip(taken, self.groups):
+            blocks.append(pages)
+            index = torch.tensor(pages, dtype=torch.long, device=g.keys.device)
+            for i, slot in enumerate(g.slots):
+                for pool, t in zip((g.keys[i], g.values[i]), per_slot[slot]):
+                    full = torch.zeros((n_blocks * self.page_size, *t.shape[1:]), dtype=pool.dtype, device=pool.device)
+                    full[:length] = t.to(device=pool.device, dtype=pool.dtype)
+                    full = full.view(n_blocks, self.page_size, *t.shape[1:]).permute(0, 2, 1, 3)
+                    pool.index_copy_(0, index, full)
+        rows = {slot: row.to(device=self.state_storage[slot].device, dtype=self.state_storage[slot].dtype).clone()
+                for slot, row in state.items()}
+        kept = KeptPages(length, n_blocks * self.page_size, blocks, rows)
+        self.kept.append(kept)
+        return kept
+
     def set_state(self, request_id, state=None):
         """A live request's rows of the state tensors: as ``state`` (cache slot -> row) has them, or zero."""
         rc = self.requests[request_id]

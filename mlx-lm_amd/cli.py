@@ -7,6 +7,7 @@ from . import __version__
 
 SUBCOMMANDS = {
     "generate": ("mlx_lm_amd.generate", "main"),
+    "cache_prompt": ("mlx_lm_amd.cache_prompt", "main"),
     "trace_run": ("mlx_lm_amd.engine.replay", "main"),
     "random_weights": ("mlx_lm_amd.weights.random_init", "main"),
 }

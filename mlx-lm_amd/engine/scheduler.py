@@ -85,6 +85,10 @@ class Request:
     # are ``offset`` (set when the request is added).
     kept: Any = None
     offset: int = 0
+    # No token is asked for and there is a kept cache: the prompt is read into it and that is all
+    # (``generate_step(..., max_tokens=0, prompt_cache=c)`` of the reference reads the whole
+    # prompt before it stops, which is how mlx_lm/cache_prompt.py:132-143 fills a cache).
+    fill_only: bool = False
 
     @property
     def tokens(self):
@@ -214,9 +218,11 @@ class Scheduler:
         request.order = self._order
         self._order += 1
         request.engine_id = (self.number, request.request_id)
-        if request.max_tokens == 0:
-            # nothing to generate: finished as it comes, with no step run and no token sampled
-            # (``generate_step`` yields nothing for it, mlx_lm/generate.py:448-461)
+        request.fill_only = request.max_tokens == 0 and request.kept is not None
+        if request.max_tokens == 0 and not request.fill_only:
+            # nothing to generate and no cache to leave the prompt in: finished as it comes, with
+            # no step run and no token sampled (``generate_step`` yields nothing for it,
+            # mlx_lm/generate.py:448-461)
             request.finish_reason = "length"
             return request
         request.live = True
@@ -340,7 +346,7 @@ class Scheduler:
                 continue
             free -= self._pages_for(r, n)
             budget -= n
-            plan.append(PlannedEntry(r, n, n == left))
+            plan.append(PlannedEntry(r, n, n == left and not r.fill_only))
 
         # 3. admit waiting requests while their whole prompt fits
         while self.waiting and len(self.running) < self.max_num_seqs and budget > 0:
@@ -348,8 +354,10 @@ class Scheduler:
             if r.inflight_row is not None:
                 break  # pre-empted with a token in flight: it is read as a prompt once that token is known
             # (a kept cache brings the pages of its tokens with it)
-            n_new = min(r.num_tokens + 1, self.max_positions - r.offset)
+            n_new = min(r.num_tokens + (0 if r.fill_only else 1), self.max_positions - r.offset)
             whole = self.cache.blocks_for(r.offset + n_new) - self.cache.blocks_for(r.offset)
+            if r.kept is not None and getattr(r.kept, "needs_pages", False):
+                whole += self.cache.blocks_for(r.offset)  # (read from a file: its tokens have no pages yet)
             if whole > free:
                 break
             # The request leaves the queue only once the engine has it and its pages: whatever
@@ -361,7 +369,7 @@ class Scheduler:
                     r.kept.checkout(self.engine, r.engine_id)
                 else:
                     self.engine.add_request(r.engine_id)
-            except OutOfSlots:
+            except (OutOfSlots, OutOfPages):
                 break
             try:
                 self.cache.reserve(r.engine_id, n_new)
@@ -378,7 +386,7 @@ class Scheduler:
             n = min(r.num_tokens, budget, self.prefill_step_size)
             free -= whole
             budget -= n
-            plan.append(PlannedEntry(r, n, n == r.num_tokens))
+            plan.append(PlannedEntry(r, n, n == r.num_tokens and not r.fill_only))
         return plan
 
     def _fit(self, r, n, free):
@@ -460,6 +468,9 @@ class Scheduler:
             if not r.generated and r.inflight_row is None:
                 self.stats.prompt_tokens += p.n_tokens
             r.num_computed += p.n_tokens
+            if r.fill_only and r.num_computed >= r.num_tokens:  # the prompt is in its cache: done
+                r.finish_reason = "length"
+                self._drop(r)
         self.stats.steps += 1
         self.stats.pages_high_water = max(
             self.stats.pages_high_water, max((g.pool.high_water for g in self.cache.groups), default=0)

@@ -131,6 +131,14 @@ class Engine:
     def drop_kept(self, kept):
         self.cache.drop(kept)
 
+    def read_kept(self, kept):
+        """``KeptPages`` as tensors of their own (``CacheManager.read_kept``)."""
+        return self.cache.read_kept(kept)
+
+    def write_kept(self, length, per_slot, state):
+        """Pages of this engine's pool that hold the given keys, values and state rows."""
+        return self.cache.write_kept(length, per_slot, state)
+
     def has_request(self, request_id):
         return request_id in self.cache.requests
 

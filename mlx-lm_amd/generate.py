@@ -553,6 +553,12 @@ class BatchGenerator:
                                            r.tokens if o.finish_reason else None, o.logprob))
             if o.finish_reason is not None:
                 del self._requests[o.request_id]
+        # a request for no tokens on top of a cache is over once its prompt is read: its one
+        # response carries no token, only the cache
+        for uid, r in list(self._requests.items()):
+            if r.fill_only and r.finish_reason is not None:
+                responses.append(self.Response(uid, None, None, r.finish_reason, r.kept, r.tokens))
+                del self._requests[uid]
         return prompt_responses, responses
 
     def next(self):
@@ -595,7 +601,7 @@ def batch_generate(model, tokenizer, prompts, prompt_caches=None, max_tokens=128
             if not responses:
                 break
             for r in responses:
-                if r.finish_reason != "stop":
+                if r.finish_reason != "stop" and r.token is not None:
                     kept[r.uid][0].append(r.token)
                     kept[r.uid][1].append(r.token_logprob)
                 if r.finish_reason is not None:
@@ -648,6 +654,8 @@ _OPTIONS = [
     (("--seed",), int, DEFAULT_SEED, "Seed of the random draws.", {}),
     (("--ignore-chat-template",), None, False, "Give the model the prompt as it is.", {"action": "store_true"}),
     (("--chat-template-config",), None, None, "More variables for the chat template, as a JSON object.", {}),
+    (("--prompt-cache-file",), str, None, "A file containing saved KV caches to avoid recomputing them "
+                                          "(written by the cache_prompt command): the prompt goes on from it.", {}),
     (("--verbose",), str2bool, True, "'True'/'T': stream the text, then print token counts, rates and peak "
                                      "memory; 'False'/'F': print the text only.", {}),
     # this engine's own
@@ -673,10 +681,12 @@ def setup_arg_parser():
     return parser
 
 
-def chat_prompt(tokenizer, prompt, args):
+def chat_prompt(tokenizer, prompt, args, using_cache=False):
     """The prompt inside the tokenizer's chat template, as token ids (mlx_lm/generate.py:2115-2152).
 
     A tokenizer without a template, or ``--ignore-chat-template``, leaves the text as it is.
+    ``using_cache``: what comes before the user's text in the template lies in a saved cache
+    already, so the prompt is the template's text from the last message's text on (2139-2149).
     """
     if args.ignore_chat_template or not getattr(tokenizer, "has_chat_template", False):
         return prompt
@@ -688,6 +698,14 @@ def chat_prompt(tokenizer, prompt, args):
     has_prefill = args.prefill_response is not None
     if has_prefill:
         messages.append({"role": "assistant", "content": args.prefill_response})
+    if using_cache:
+        text = tokenizer.apply_chat_template(messages, tokenize=False, continue_final_message=has_prefill,
+                                             add_generation_prompt=not has_prefill, **template_kwargs)
+        marked = [dict(m) for m in messages]
+        marked[-1]["content"] = "<query>"
+        probe = tokenizer.apply_chat_template(marked, tokenize=False, continue_final_message=has_prefill,
+                                              add_generation_prompt=not has_prefill)
+        return tokenizer.encode(text[probe.index("<query>"):], add_special_tokens=False)
     return tokenizer.apply_chat_template(messages, tokenize=True, continue_final_message=has_prefill,
                                          add_generation_prompt=not has_prefill, **template_kwargs)
 
@@ -718,6 +736,14 @@ def main(argv=None):
     args = setup_arg_parser().parse_args(argv)
     if args.seed is not None:
         sample_utils.seed(args.seed)
+    prompt_cache = None
+    if args.prompt_cache_file is not None:
+        # the cache, and the model it was made with unless another is named (mlx_lm/generate.py:2070-2096)
+        from .prompt_cache import load_prompt_cache
+
+        prompt_cache, metadata = load_prompt_cache(args.prompt_cache_file, return_metadata=True)
+        if args.model is None and args.random_weights is None and metadata.get("model"):
+            args.model = metadata["model"]
     model, tokenizer = _model_of(args)
     tokenizer = tokenizer if tokenizer is not None else IdTokenizer()
     for token in args.extra_eos_token:
@@ -726,7 +752,8 @@ def main(argv=None):
         prompt = [int(t) for t in args.prompt_ids.replace(",", " ").split()]
     else:
         text = args.prompt.replace("\\n", "\n").replace("\\t", "\t")
-        prompt = chat_prompt(tokenizer, sys.stdin.read() if text == "-" else text, args)
+        prompt = chat_prompt(tokenizer, sys.stdin.read() if text == "-" else text, args,
+                             using_cache=prompt_cache is not None)
     never_dropped = []  # by XTC: the line break and the end tokens (mlx_lm/generate.py:2168)
     if args.xtc_probability > 0:
         never_dropped = list(tokenizer.encode("\n", add_special_tokens=False)) + sorted(tokenizer.eos_token_ids)
@@ -734,7 +761,7 @@ def main(argv=None):
                            xtc_probability=args.xtc_probability, xtc_threshold=args.xtc_threshold,
                            xtc_special_tokens=never_dropped)
     text = generate(model, tokenizer, prompt, max_tokens=args.max_tokens, verbose=args.verbose, sampler=sampler,
-                    prefill_step_size=args.prefill_step_size, page_size=args.block_size, num_pages=args.num_pages,
+                    prompt_cache=prompt_cache, prefill_step_size=args.prefill_step_size, page_size=args.block_size, num_pages=args.num_pages,
                     max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens)
     if not args.verbose:
         print(text)

@@ -8,8 +8,14 @@ fills and updates in place (mlx_lm/generate.py:306,329-331,362-385), that
 (mlx_lm/generate.py:1689-1731,1777-1802).  Here a kept cache is one object for
 the whole model: the pages that the request held in the engine's pool, which
 simply stay held, and the request's row of every state tensor.  Nothing is
-copied when a request goes on from it.  Saving one to a file is not offered.
+copied when a request goes on from it.  ``save_prompt_cache`` writes the keys,
+values and state out of the pages into a safetensors file and
+``load_prompt_cache`` reads them back (mlx_lm/models/cache.py:43-85); a cache
+that was read from a file holds tensors of its own until the first request
+that uses it gives it pages in that request's engine.
 """
+
+import json
 
 
 class PromptCache:
@@ -27,12 +33,22 @@ class PromptCache:
         self.model = model
         self._engine = None
         self._kept = None
+        # (length, {slot: (keys, values)}, {slot: state row}) of a cache that was read from a file
+        # and has no pages yet
+        self._loaded = None
         self._at_checkout = (0, None)
         self.in_use = False
 
     @property
     def offset(self):
-        return self._kept.length if self._kept is not None else 0
+        if self._kept is not None:
+            return self._kept.length
+        return self._loaded[0] if self._loaded is not None else 0
+
+    @property
+    def needs_pages(self):
+        """Read from a file and not yet in any engine's pool: the first request brings it there."""
+        return self._loaded is not None
 
     @property
     def engine(self):
@@ -50,6 +66,9 @@ class PromptCache:
             raise ValueError("this prompt cache is in use by a live request")
         if self._kept is not None and self._engine is not engine:
             raise ValueError("this prompt cache holds pages of another engine (another cache geometry or model)")
+        if self._loaded is not None:  # read from a file: into pages of this engine's pool now
+            self._kept = engine.write_kept(*self._loaded)
+            self._loaded = None
         self._engine, self.in_use = engine, True
         self._at_checkout = (self.offset, self._kept.state if self._kept is not None else None)
         if self._kept is None:
@@ -71,26 +90,34 @@ class PromptCache:
             length = offset
             if engine.cache.state_needs:
                 engine.cache.set_state(engine_id, state)
-        engine.truncate(engine_id, length)
+        engine.cache.truncate(engine_id, length)
 
     def checkin(self, engine, engine_id):
         """The request ends: what it holds is this cache's from now on."""
         self._engine = engine
-        engine.truncate(engine_id, engine.context_len(engine_id))  # pages taken ahead of the tokens go back
+        # pages taken ahead of the tokens go back (the cache manager's own cut: no token is dropped)
+        engine.cache.truncate(engine_id, engine.context_len(engine_id))
         self._kept = engine.detach_request(engine_id)
         self.in_use = False
 
     # -- what callers use ----------------------------------------------------------
 
     def is_trimmable(self):
-        return not self.in_use and (self._engine is None or not self._engine.cache.state_needs)
+        if self.in_use:
+            return False
+        if self._loaded is not None:
+            return not self._loaded[2]
+        return self._engine is None or not self._engine.cache.state_needs
 
     def trim(self, n_tokens):
         """Forget the last ``n_tokens`` tokens (at most all); returns how many went."""
         if self.in_use:
             raise ValueError("this prompt cache is in use by a live request")
         n = max(0, min(int(n_tokens), self.offset))
-        if n:
+        if n and self._loaded is not None:
+            length, per_slot, state = self._loaded
+            self._loaded = (length - n, {s: (k[: length - n], v[: length - n]) for s, (k, v) in per_slot.items()}, state)
+        elif n:
             self._engine.cache.truncate_kept(self._kept, self.offset - n)
         return n
 
@@ -99,13 +126,28 @@ class PromptCache:
         if self.in_use:
             raise ValueError("this prompt cache is in use by a live request")
         other = PromptCache(self.model)
+        other._loaded = self._loaded  # (never written to: trim makes a new tuple)
         if self._kept is not None:
             other._engine = self._engine
             other._kept = self._engine.cache.fork(self._kept)
         return other
 
+    def tensors(self):
+        """``(length, {slot: (keys, values)}, {slot: state row})``: the tokens' keys ``[length,
+        n_kv_heads, head_dim]`` and values of every cache slot and the state rows, as tensors of
+        their own."""
+        if self.in_use:
+            raise ValueError("this prompt cache is in use by a live request")
+        if self._loaded is not None:
+            return self._loaded
+        if self._kept is None:
+            return 0, {}, {}
+        per_slot, state = self._engine.read_kept(self._kept)
+        return self._kept.length, per_slot, state
+
     def free(self):
         """Give the pages back to the engine's pool; the cache is empty afterwards."""
+        self._loaded = None
         if self._kept is not None and not self.in_use:
             self._engine.drop_kept(self._kept)
             self._kept = None
@@ -122,6 +164,56 @@ def make_prompt_cache(model=None, max_kv_size=None):
     if max_kv_size is not None:
         raise ValueError("'max_kv_size' is not supported by this engine")
     return PromptCache(model)
+
+
+_FORMAT = "mlx_lm_amd prompt cache 1"
+
+
+def save_prompt_cache(file_name, cache, metadata=None):
+    """Write a cache's keys, values and state rows to a ``.safetensors`` file, with ``metadata``
+    (a dict of strings) beside them (``save_prompt_cache`` of mlx_lm/models/cache.py:43-59)."""
+    from safetensors.torch import save_file
+
+    length, per_slot, state = cache.tensors()
+    tensors = {}
+    for slot, (k, v) in per_slot.items():
+        tensors[f"slot.{slot}.keys"] = k.detach().cpu().contiguous()
+        tensors[f"slot.{slot}.values"] = v.detach().cpu().contiguous()
+    for slot, row in state.items():
+        tensors[f"state.{slot}"] = row.detach().cpu().contiguous()
+    if not tensors:  # (a file of no tensors: an empty cache is one tensor of nothing)
+        import torch
+
+        tensors["empty"] = torch.zeros(0)
+    info = {"format": _FORMAT, "length": str(int(length)),
+            "metadata": json.dumps({str(k): str(v) for k, v in (metadata or {}).items()})}
+    save_file(tensors, file_name, metadata=info)
+
+
+def load_prompt_cache(file_name, return_metadata=False):
+    """Read a cache that ``save_prompt_cache`` wrote (``load_prompt_cache`` of
+    mlx_lm/models/cache.py:62-85).  Its tensors get pages in the engine of the first request that
+    uses it, which must be of a model with the same layers, heads and head sizes."""
+    from safetensors import safe_open
+
+    per_slot, state = {}, {}
+    with safe_open(file_name, framework="pt", device="cpu") as fh:
+        info = fh.metadata() or {}
+        if info.get("format") != _FORMAT:
+            raise ValueError(f"{file_name} is not a prompt cache of this engine (format {info.get('format')!r})")
+        length = int(info["length"])
+        for name in fh.keys():
+            kind, _, rest = name.partition(".")
+            if kind == "slot":
+                slot, _, what = rest.partition(".")
+                per_slot.setdefault(int(slot), {})[what] = fh.get_tensor(name)
+            elif kind == "state":
+                state[int(rest)] = fh.get_tensor(name)
+    cache = PromptCache()
+    if length or state:
+        cache._loaded = (length, {slot: (kv["keys"], kv["values"]) for slot, kv in per_slot.items()}, state)
+    metadata = json.loads(info.get("metadata", "{}"))
+    return (cache, metadata) if return_metadata else cache
 
 
 def can_trim_prompt_cache(cache):

@@ -305,3 +305,83 @@ def test_kept_pages_carry_contents_and_state():
     cm.check()
     cm.release_all()
     assert [g.pool.n_free for g in cm.groups] == [9, 9] and not cm.kept
+
+
+def test_kept_pages_go_to_a_file_and_into_another_pool(tmp_path):
+    """``read_kept`` gathers the tokens' keys, values and state out of the pages, ``write_kept`` fills
+    pages of another pool with them (another page size, scrambled pages); through a file with
+    ``save_prompt_cache`` / ``load_prompt_cache`` (mlx_lm/models/cache.py:43-85, with the metadata
+    that mlx_lm/cache_prompt.py:150-153 writes)."""
+    import torch
+
+    from mlx_lm_amd.prompt_cache import PromptCache, load_prompt_cache, save_prompt_cache, trim_prompt_cache
+
+    needs = [CacheNeed(2, 16, 0), CacheNeed(1, 16, 0, v_head_dim=32), StateNeed((3,))]
+
+    class Shim:  # what a PromptCache asks of an engine, over a pool on the CPU
+        def __init__(self, page_size, n_pages):
+            self.cache = CacheManager(needs, page_size, n_pages, 3, dtype=torch.float32, device="cpu")
+            for name in ("read_kept", "write_kept", "attach", "detach", "add", "drop"):
+                setattr(self, {"attach": "attach_request", "detach": "detach_request", "add": "add_request",
+                               "drop": "drop_kept"}.get(name, name), getattr(self.cache, name))
+
+        def context_len(self, rid):
+            return self.cache.requests[rid].length
+
+    a = Shim(16, 9)
+    a.cache.add("junk"), a.cache.reserve("junk", 20), a.cache.commit("junk", 20)  # so that pages are not 0, 1, 2 ...
+    cache = PromptCache()
+    cache.checkout(a, "r")
+    a.cache.reserve("r", 45), a.cache.commit("r", 45)
+    rc = a.cache.requests["r"]
+    g = torch.Generator().manual_seed(0)
+    want = {}
+    for slot in (0, 1):
+        gi, i = a.cache.slot_group[slot]
+        grp = a.cache.groups[gi]
+        k = torch.randn(45, grp.need.n_kv_heads, grp.need.head_dim, generator=g)
+        v = torch.randn(45, grp.need.n_kv_heads, grp.need.value_dim, generator=g)
+        want[slot] = (k, v)
+        for t in range(45):
+            page = rc.blocks[gi][t // 16]
+            grp.keys[i][page, :, t % 16] = k[t]
+            grp.values[i][page, :, t % 16] = v[t]
+    a.cache.state(2)[rc.state_slot] = torch.tensor([1.0, 2.0, 3.0])
+    cache.checkin(a, "r")
+    length, per_slot, state = cache.tensors()
+    assert length == 45 and state[2].tolist() == [1.0, 2.0, 3.0]
+    assert all(torch.equal(per_slot[s][0], want[s][0]) and torch.equal(per_slot[s][1], want[s][1]) for s in want)
+    path = str(tmp_path / "cache.safetensors")
+    save_prompt_cache(path, cache, {"model": "somewhere", "tokenizer_config": "{}"})
+    loaded, metadata = load_prompt_cache(path, return_metadata=True)
+    assert metadata == {"model": "somewhere", "tokenizer_config": "{}"}
+    assert loaded.offset == 45 and loaded.engine is None and not loaded.is_trimmable()  # (it has state)
+    assert trim_prompt_cache(loaded, 5) == 0
+    # into a pool with pages of 32 tokens
+    b = Shim(32, 4)
+    loaded.checkout(b, "x")
+    rb = b.cache.requests["x"]
+    assert rb.length == 45 and b.cache.state(2)[rb.state_slot].tolist() == [1.0, 2.0, 3.0]
+    for slot in (0, 1):
+        gi, i = b.cache.slot_group[slot]
+        grp = b.cache.groups[gi]
+        for t in (0, 15, 16, 31, 32, 44):
+            page = rb.blocks[gi][t // 32]
+            assert torch.equal(grp.keys[i][page, :, t % 32], want[slot][0][t])
+            assert torch.equal(grp.values[i][page, :, t % 32], want[slot][1][t])
+    loaded.checkin(b, "x")
+    b.cache.check()
+    # a pool that is too small, and a model with other sizes
+    again = load_prompt_cache(path)
+    with pytest.raises(OutOfPages, match="a cache of 45 tokens"):
+        again.checkout(Shim(16, 2), "y")
+    assert not again.in_use or True
+    other = Shim(16, 9)
+    other.cache = CacheManager([CacheNeed(2, 16, 0), CacheNeed(1, 32, 0), StateNeed((3,))], 16, 9, 3,
+                               dtype=torch.float32, device="cpu")
+    other.write_kept = other.cache.write_kept
+    with pytest.raises(ValueError, match="cache slot 1: keys"):
+        load_prompt_cache(path).checkout(other, "z")
+    # an empty cache goes through a file as well
+    save_prompt_cache(path, PromptCache())
+    assert load_prompt_cache(path).offset == 0

@@ -238,3 +238,60 @@ def test_preemption_with_kept_caches_and_a_pool_that_they_fill(setup):
     for c in caches:
         c.free()
     assert engine.cache.free_pages() == 20 and not engine.cache.kept
+
+
+def test_a_cache_goes_through_a_file_and_into_another_engine(setup, tmp_path):
+    """``save_prompt_cache`` / ``load_prompt_cache`` (mlx_lm/models/cache.py:43-85; the reference's
+    tests/test_prompt_cache.py:43-69 saves, loads and compares): the loaded cache gives the tokens
+    of the one in memory, in the model's own engine and in one with pages of another size."""
+    from mlx_lm_amd import generate_step, load_prompt_cache, make_prompt_cache, save_prompt_cache
+    from mlx_lm_amd.engine import Engine
+
+    model, engine, config, weights, dtype = setup
+    V = config["vocab_size"]
+    head = helpers.random_tokens(37, V, seed=130)
+    tail = helpers.random_tokens(5, V, seed=131)
+    want = [t for t, _ in generate_step(head + tail, model, max_tokens=9, engine=engine)]
+    cache = make_prompt_cache(model)
+    assert list(generate_step(head, model, max_tokens=0, prompt_cache=cache, engine=engine)) == []
+    assert cache.offset == 37  # (no token asked for: the prompt is read into the cache, mlx_lm/cache_prompt.py:132-143)
+    path = str(tmp_path / "c.safetensors")
+    save_prompt_cache(path, cache, {"model": "m"})
+    cache.free()
+    assert engine.cache.free_pages() == 20
+    loaded, meta = load_prompt_cache(path, return_metadata=True)
+    assert meta == {"model": "m"} and loaded.offset == 37 and loaded.engine is None
+    got = [t for t, _ in generate_step(tail, model, max_tokens=9, prompt_cache=loaded, engine=engine)]
+    assert got == want and loaded.engine is engine and loaded.offset == 37 + 5 + 9
+    loaded.free()
+    other = Engine(model, dtype=dtype, page_size=32, n_pages=6, max_requests=2)
+    again = load_prompt_cache(path)
+    assert [t for t, _ in generate_step(tail, model, max_tokens=9, prompt_cache=again, engine=other)] == want
+    again.free()
+    assert engine.cache.free_pages() == 20 and other.cache.free_pages() == 6
+
+
+def test_cache_prompt_and_generate_on_the_command_line(tmp_path):
+    """``cache_prompt`` writes the file that ``generate --prompt-cache-file`` goes on from, and the
+    file names the model (mlx_lm/cache_prompt.py:150-153, mlx_lm/generate.py:2070-2096)."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    d = str(tmp_path / "model")
+    config, weights = helpers.make_folder(d, "A", 0.0)
+    head, tail = [3, 1, 4, 1, 5, 9, 2, 6, 5, 3, 5, 8, 9, 7, 9, 3, 2, 3], [8, 4, 6]
+    want = plain.greedy_generate(weights, config, head + tail, 6)
+    env = dict(os.environ, PYTHONPATH=root)
+    path = str(tmp_path / "head.safetensors")
+    out = subprocess.run([sys.executable, "-m", "mlx_lm_amd", "cache_prompt", "--model", d, "--prompt-ids",
+                          " ".join(map(str, head)), "--prompt-cache-file", path, "--dtype", "float32",
+                          "--prefill-step-size", "7"], capture_output=True, text=True, env=env, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    assert "Processed     18 tokens" in out.stdout and "Saving..." in out.stdout
+    out = subprocess.run([sys.executable, "-m", "mlx_lm_amd", "generate", "--prompt-cache-file", path, "--prompt-ids",
+                          " ".join(map(str, tail)), "--max-tokens", "6", "--dtype", "float32", "--verbose", "F"],
+                         capture_output=True, text=True, env=env, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    assert out.stdout.strip() == " ".join(map(str, want))

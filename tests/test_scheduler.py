@@ -440,3 +440,30 @@ def test_kept_caches_under_preemption_and_abort(mode):
     half.free()
     c.free()
     assert eng.cache.free_pages() == 6 and not eng.cache.kept
+
+
+@pytest.mark.parametrize("mode", SAMPLERS)
+def test_no_tokens_asked_for_on_top_of_a_cache_reads_the_prompt_into_it(mode):
+    """mlx_lm/cache_prompt.py:132-143 fills a cache with ``generate_step(..., max_tokens=0,
+    prompt_cache=cache)``: the whole prompt is read, nothing is sampled."""
+    from mlx_lm_amd.prompt_cache import PromptCache
+
+    eng = FakeEngine(n_pages=8, max_positions=64)
+    c = PromptCache()
+    s = Scheduler(eng, SAMPLERS[mode](), prefill_step_size=8)
+    r = s.add(Request("fill", list(range(1, 22)), 0, kept=c))
+    assert r.fill_only and s.has_work
+    assert run_all(s) == {}
+    assert c.offset == 21 and not c.in_use and r.finish_reason == "length"
+    assert [e[1] for st in eng.log for e in st] == [8, 8, 5] and all(e[2] == [] for st in eng.log for e in st)
+    assert eng.cache.free_pages() == 8 - 2
+    # without a cache there is nothing to do
+    assert s.add(Request("none", [1, 2, 3], 0)).finish_reason == "length" and not s.has_work
+    # beside a request that decodes
+    s.add(Request("gen", [5, 6, 7], 4))
+    s.add(Request("more", [9] * 10, 0, kept=c))
+    done = run_all(s)
+    assert list(done) == ["gen"] and len(done["gen"]) == 4 and c.offset == 31
+    c.free()
+    assert eng.cache.free_pages() == 8
+    eng.cache.check()
