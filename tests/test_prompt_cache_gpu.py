@@ -295,3 +295,89 @@ def test_cache_prompt_and_generate_on_the_command_line(tmp_path):
                          capture_output=True, text=True, env=env, timeout=300)
     assert out.returncode == 0, out.stderr[-2000:]
     assert out.stdout.strip() == " ".join(map(str, want))
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_random_chains_of_requests_over_kept_caches(setup, seed):
+    """Conversations of several turns in one generator over a pool that is too small for them all:
+    each turn goes on from the cache that the turn before left (or from a copy that was cut back,
+    or from one that went through ``remove`` half-way), requests are pre-empted, caches are freed
+    at random.  In 32-bit every turn's tokens are those of one uncached request over all the
+    conversation's tokens so far."""
+    import random
+
+    from mlx_lm_amd.generate import BatchGenerator, generate_step
+
+    model, engine, config, _, dtype = setup
+    if dtype != "float32":
+        pytest.skip("token-for-token equality is a 32-bit matter")
+    rng = random.Random(seed)
+    V = config["vocab_size"]
+    gen = BatchGenerator(model, engine=engine, prefill_step_size=16, prefill_batch_size=2, completion_batch_size=4,
+                         return_prompt_caches=True)
+    talks = []  # [tokens so far, cache or None]
+    live = {}   # uid -> (talk index, tokens before this turn, prompt, limit)
+    checked = turns = 0
+    for _ in range(400):
+        if len(live) < 5 and turns < 24 and rng.random() < 0.5:
+            free_tokens = engine.cache.free_pages() * 16
+            if talks and rng.random() < 0.6:
+                i = rng.randrange(len(talks))
+                if any(t[0] == i for t in live.values()) or talks[i][1] is None:
+                    continue
+            else:
+                talks.append([[], None])
+                i = len(talks) - 1
+            so_far, cache = talks[i]
+            prompt = helpers.random_tokens(rng.randint(1, 30), V, seed=rng.randrange(10**6))
+            limit = rng.randint(1, 12)
+            if len(so_far) + len(prompt) + limit > 150 or len(so_far) + len(prompt) + limit + 16 > free_tokens:
+                continue
+            if cache is not None and rng.random() < 0.3 and cache.offset > 3:  # cut the conversation back
+                cut = rng.randint(1, 3)
+                assert cache.trim(cut) == cut
+                so_far = talks[i][0] = so_far[:-cut]
+            uid = gen.insert([prompt], [limit], caches=[cache] if cache is not None else None)[0]
+            live[uid] = (i, list(so_far), prompt, limit)
+            turns += 1
+        if not gen.scheduler.has_work:
+            if turns >= 24 and not live:
+                break
+            continue
+        if live and rng.random() < 0.04:  # taken out half-way: what it had computed goes on as the cache
+            uid = rng.choice(list(live))
+            i, before, prompt, limit = live.pop(uid)
+            got = gen.remove([uid], return_prompt_caches=True)[uid]
+            if talks[i][1] is not None:
+                talks[i][1].free()
+            known = before + prompt
+            assert got.offset <= len(known) + limit
+            # (the tokens that it had generated are not known here: go on from the prompt's part)
+            keep = min(got.offset, len(known))
+            got.trim(got.offset - keep)
+            talks[i] = [known[:keep], got]
+            continue
+        _, responses = gen.next()
+        for r in responses:
+            if r.finish_reason is None:
+                continue
+            i, before, prompt, limit = live.pop(r.uid)
+            made = r.all_tokens[len(prompt):]
+            # (alone, on the model's own engine: the small pool is full of conversations)
+            want = [t for t, _ in generate_step(before + prompt, model, max_tokens=limit)]
+            assert made == want, (seed, r.uid)
+            checked += 1
+            if talks[i][1] is not None:
+                talks[i][1].free()  # (the turn worked on a copy)
+            talks[i] = [before + prompt + made, r.prompt_cache]
+            assert r.prompt_cache.offset == len(talks[i][0])
+            if rng.random() < 0.2:
+                r.prompt_cache.free()
+                talks[i][1] = None
+        engine.cache.check()
+    assert checked >= 8 and not live
+    gen.close()
+    for _, cache in talks:
+        if cache is not None:
+            cache.free()
+    assert engine.cache.free_pages() == 20 and not engine.cache.kept and not engine.cache.requests
