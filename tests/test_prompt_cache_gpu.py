@@ -381,3 +381,32 @@ def test_random_chains_of_requests_over_kept_caches(setup, seed):
         if cache is not None:
             cache.free()
     assert engine.cache.free_pages() == 20 and not engine.cache.kept and not engine.cache.requests
+
+
+def test_a_batch_of_prompts_is_read_into_caches_without_a_token(setup):
+    """``max_tokens=0`` with a cache in a ``BatchGenerator``: the prompts are read beside a request
+    that decodes, each gives one response without a token that carries the cache, and a later
+    request goes on from it."""
+    from mlx_lm_amd import make_prompt_cache
+    from mlx_lm_amd.generate import BatchGenerator, generate_step
+
+    model, engine, config, _, dtype = setup
+    V = config["vocab_size"]
+    heads = [helpers.random_tokens(n, V, seed=150 + n) for n in (19, 40)]
+    tail = helpers.random_tokens(4, V, seed=160)
+    want = [[t for t, _ in generate_step(h + tail, model, max_tokens=5, engine=engine)] for h in heads]
+    gen = BatchGenerator(model, engine=engine, prefill_step_size=16)
+    uids = gen.insert(heads + [tail], [0, 0, 6], caches=[make_prompt_cache(model), make_prompt_cache(model), None])
+    caches, tokens = {}, []
+    while responses := gen.next_generated():
+        for r in responses:
+            if r.uid in uids[:2]:
+                assert r.token is None and r.finish_reason == "length"
+                caches[r.uid] = r.prompt_cache
+            else:
+                tokens.append(r.token)
+    assert len(tokens) == 6 and [caches[u].offset for u in uids[:2]] == [19, 40]
+    for u, w in zip(uids[:2], want):
+        assert [t for t, _ in generate_step(tail, model, max_tokens=5, prompt_cache=caches[u])] == w
+        caches[u].free()
+    assert engine.cache.free_pages() == 20
