@@ -131,7 +131,7 @@ def test_thousands_of_keys_split_over_blocks(tmp_path, monkeypatch, dtype, use_g
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,sharp", [("A", 8.0), ("B", 8.0), ("C", 0.0)])
+@pytest.mark.parametrize("name,sharp", [("A", 8.0), ("B", 8.0), ("C", 0.0), ("C", 8.0)])
 def test_mixed_batches_with_few_pages(folders, dtype, name, sharp):
     from mlx_lm_amd.engine import StepEntry
 
