@@ -197,6 +197,10 @@ class Scheduler:
             raise ValueError("max_tokens must not be negative")
         if request.kept is not None and request.kept.in_use:
             raise ValueError("the request's prompt cache is in use by another live request")
+        if request.kept is not None and any(g.need.window > 0 for g in self.cache.groups):
+            # (pre-emption and removal take a request back to what its cache held; pages that a
+            # window has passed are gone, so that state cannot be had again)
+            raise ValueError("prompt caches are not offered for a model whose attention has a window")
         if request.kept is not None and getattr(request.kept, "engine", None) not in (None, self.engine):
             raise ValueError("the request's prompt cache holds pages of another engine (another cache "
                              "geometry, dtype or model): it goes on only where it was made")

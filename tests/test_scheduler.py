@@ -467,3 +467,16 @@ def test_no_tokens_asked_for_on_top_of_a_cache_reads_the_prompt_into_it(mode):
     c.free()
     assert eng.cache.free_pages() == 8
     eng.cache.check()
+
+
+def test_a_model_with_a_window_takes_no_prompt_cache():
+    from mlx_lm_amd.config.plan import CacheNeed
+    from mlx_lm_amd.prompt_cache import PromptCache
+
+    eng = FakeEngine(n_pages=8, max_positions=64)
+    eng.cache = CacheManager([CacheNeed(2, 16, 24)], 16, 8, 4)
+    s = Scheduler(eng, fake_sample)
+    with pytest.raises(ValueError, match="window"):
+        s.add(Request("w", [1, 2, 3], 2, kept=PromptCache()))
+    s.add(Request("w", [1, 2, 3], 2))  # without one it runs
+    assert len(run_all(s)["w"]) == 2
