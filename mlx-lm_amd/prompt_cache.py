@@ -68,18 +68,14 @@ class PromptCache:
             raise ValueError("this prompt cache holds pages of another engine (another cache geometry or model)")
         if self._loaded is not None:  # read from a file: into pages of this engine's pool now
             self._kept = engine.write_kept(*self._loaded)
-            self._loaded = None
-        self._engine, self.in_use = engine, True
-        self._at_checkout = (self.offset, self._kept.state if self._kept is not None else None)
+            self._loaded, self._engine = None, engine
+        at_checkout = (self.offset, self._kept.state if self._kept is not None else None)
         if self._kept is None:
-            engine.add_request(engine_id)
+            engine.add_request(engine_id)  # (may find no request slot free: nothing has changed then)
         else:
-            kept, self._kept = self._kept, None
-            try:
-                engine.attach_request(engine_id, kept)
-            except Exception:
-                self._kept, self.in_use = kept, False
-                raise
+            engine.attach_request(engine_id, self._kept)
+            self._kept = None
+        self._engine, self.in_use, self._at_checkout = engine, True, at_checkout
 
     def rewind(self, engine, engine_id, length=None):
         """Cut the live request back to ``length`` tokens, or to what the cache held when the request

@@ -382,6 +382,25 @@ def test_kept_pages_go_to_a_file_and_into_another_pool(tmp_path):
     other.write_kept = other.cache.write_kept
     with pytest.raises(ValueError, match="cache slot 1: keys"):
         load_prompt_cache(path).checkout(other, "z")
+    # no request slot free: the cache stays as it was and can be used later
+    full = Shim(16, 9)
+    held = load_prompt_cache(path)
+    for name in ("p", "q", "r"):
+        full.cache.add(name)
+    from mlx_lm_amd.cache import OutOfSlots
+
+    with pytest.raises(OutOfSlots):
+        held.checkout(full, "s")
+    assert not held.in_use and held.offset == 45
+    full.cache.release("p")
+    held.checkout(full, "s")
+    assert held.in_use and full.cache.requests["s"].length == 45
+    held.checkin(full, "s")
+    fresh = PromptCache()
+    full.cache.add("p")
+    with pytest.raises(OutOfSlots):
+        fresh.checkout(full, "t")
+    assert not fresh.in_use
     # an empty cache goes through a file as well
     save_prompt_cache(path, PromptCache())
     assert load_prompt_cache(path).offset == 0
