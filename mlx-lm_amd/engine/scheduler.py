@@ -237,6 +237,8 @@ class Scheduler:
         """Take a request out, wherever it is (``remove`` of mlx_lm/generate.py:1777-1802).
         ``keep``: an empty kept cache that takes what the request has computed (a request that
         came with a kept cache leaves it there anyway)."""
+        if keep is not None and any(g.need.window > 0 for g in self.cache.groups):
+            raise ValueError("prompt caches are not offered for a model whose attention has a window")
         for r in list(self.waiting):
             if r.request_id == request_id:
                 self.waiting.remove(r)
