@@ -85,6 +85,10 @@ class Request:
     # are ``offset`` (set when the request is added).
     kept: Any = None
     offset: int = 0
+    # Tokens that the kept cache knows but that have not gone through the model yet (the last
+    # token of the request before, which ended it before it was fed): this request reads them
+    # ahead of its prompt.  Set when the request is added.
+    prefix: List[int] = field(default_factory=list)
     # No token is asked for and there is a kept cache: the prompt is read into it and that is all
     # (``generate_step(..., max_tokens=0, prompt_cache=c)`` of the reference reads the whole
     # prompt before it stops, which is how mlx_lm/cache_prompt.py:132-143 fills a cache).
@@ -95,8 +99,13 @@ class Request:
         return self.prompt + self.generated
 
     @property
+    def feed_tokens(self):
+        """What goes through the model for this request, in order."""
+        return self.prefix + self.prompt + self.generated
+
+    @property
     def num_tokens(self):
-        return len(self.prompt) + len(self.generated)
+        return len(self.prefix) + len(self.prompt) + len(self.generated)
 
     @property
     def context(self):
@@ -195,8 +204,8 @@ class Scheduler:
             raise ValueError("a request needs a prompt of at least one token")
         if request.max_tokens < 0:
             raise ValueError("max_tokens must not be negative")
-        if request.kept is not None and request.kept.in_use:
-            raise ValueError("the request's prompt cache is in use by another live request")
+        if request.kept is not None and (request.kept.in_use or getattr(request.kept, "claimed", False)):
+            raise ValueError("the request's prompt cache is in use by another request")
         if request.kept is not None and any(g.need.window > 0 for g in self.cache.groups):
             # (pre-emption and removal take a request back to what its cache held; pages that a
             # window has passed are gone, so that state cannot be had again)
@@ -204,14 +213,16 @@ class Scheduler:
         if request.kept is not None and getattr(request.kept, "engine", None) not in (None, self.engine):
             raise ValueError("the request's prompt cache holds pages of another engine (another cache "
                              "geometry, dtype or model): it goes on only where it was made")
-        request.offset = request.kept.offset if request.kept is not None else 0
-        if request.offset + len(request.prompt) > self.max_positions:
+        request.prefix = list(request.kept.pending) if request.kept is not None else []
+        request.offset = request.kept.offset - len(request.prefix) if request.kept is not None else 0
+        before = request.offset + len(request.prefix)
+        if before + len(request.prompt) > self.max_positions:
             raise ValueError(
                 f"the prompt has {len(request.prompt)} tokens"
-                + (f" on top of the {request.offset} of its cache" if request.offset else "")
+                + (f" on top of the {before} of its cache" if before else "")
                 + f", the model has {self.max_positions} positions"
             )
-        most = min(request.offset + len(request.prompt) + request.max_tokens, self.max_positions)
+        most = min(before + len(request.prompt) + request.max_tokens, self.max_positions)
         if self.cache.blocks_for(most) > self.cache.n_pages:
             raise ValueError(
                 f"request {request.request_id!r} can reach {most} tokens, the cache holds "
@@ -230,6 +241,8 @@ class Scheduler:
             request.finish_reason = "length"
             return request
         request.live = True
+        if request.kept is not None:
+            request.kept.claimed = True  # (this request's from now on, until it is over)
         self.waiting.append(request)
         return request
 
@@ -243,6 +256,8 @@ class Scheduler:
             if r.request_id == request_id:
                 self.waiting.remove(r)
                 r.live = False
+                if r.kept is not None:
+                    r.kept.claimed = False
                 return r
         for r in self.running:
             if r.request_id == request_id:
@@ -262,6 +277,8 @@ class Scheduler:
             self.running.remove(r)
         elif r in self.waiting:  # pre-empted, and finished by the token that was in flight
             self.waiting.remove(r)
+        if r.kept is not None:
+            r.kept.claimed = False
         if not self.engine.has_request(r.engine_id):
             return
         if r.kept is None:
@@ -271,21 +288,25 @@ class Scheduler:
 
     def _keep(self, r):
         """The request is over and its cache is kept: the cache is to hold exactly the tokens that
-        the host knows, the last generated one included (mlx_lm/generate.py:444-461 feeds it
-        before it stops).  A token still in flight when the request was taken out is forgotten;
-        tokens that were never fed (the last one, which ends a request before it is read back)
-        go through the model now, with no logits asked for."""
+        the host knows, the last generated one included (the reference feeds it before it stops,
+        mlx_lm/generate.py:444-461).  A token still in flight when the request was taken out is
+        forgotten.  The token that ended the request was never fed: the cache keeps it as
+        ``pending`` and the next request reads it ahead of its prompt (a step of its own for one
+        token would cost every finished request a whole decode step)."""
         eid = r.engine_id
-        known = r.offset + len(r.prompt) + len(r.generated)
+        known = r.context
         have = self.engine.context_len(eid)
         try:
             if have > known:
                 r.kept.rewind(self.engine, eid, known)
-            elif have < known and r.finish_reason is not None:
-                missing = (r.prompt + r.generated)[have - r.offset:]
-                self.engine.step([StepEntry(eid, missing, [])])
+                have = self.engine.context_len(eid)
         finally:
             r.kept.checkin(self.engine, eid)
+        fed = have - r.offset  # of prefix + prompt + generated
+        if r.finish_reason is not None:
+            r.kept.pending = r.feed_tokens[fed:]
+        else:  # taken out half-way: what was computed, and of the cache's own pending tokens those not yet read
+            r.kept.pending = r.prefix[fed:]
 
     def close(self):
         """Take every request out and give back what they hold in the engine."""
@@ -303,11 +324,14 @@ class Scheduler:
             # back to what the kept cache held when the request came: only its own tokens are read again
             r.kept.rewind(self.engine, r.engine_id)
             r.kept.checkin(self.engine, r.engine_id)
+            r.kept.pending = list(r.prefix)
         self._drop(r)
         r.num_computed = 0
         r.preemptions += 1
         self.stats.preemptions += 1
         r.live = True
+        if r.kept is not None:
+            r.kept.claimed = True
         self.waiting.appendleft(r)
 
     # -- decisions ---------------------------------------------------------------
@@ -382,6 +406,7 @@ class Scheduler:
             except BaseException as e:
                 if r.kept is not None:
                     r.kept.checkin(self.engine, r.engine_id)
+                    r.kept.pending = list(r.prefix)
                 else:
                     self.engine.end_request(r.engine_id)
                 if isinstance(e, OutOfPages):
@@ -463,7 +488,7 @@ class Scheduler:
             if r.inflight_row is not None:
                 entries.append(StepEntry(r.engine_id, [0], [0] if p.samples else [], fed_row=r.inflight_row))
             else:
-                toks = r.tokens[r.num_computed : r.num_computed + p.n_tokens]
+                toks = r.feed_tokens[r.num_computed : r.num_computed + p.n_tokens]
                 entries.append(StepEntry(r.engine_id, toks, [p.n_tokens - 1] if p.samples else []))
         if prev is not None and any(e.fed_row >= 0 for e in entries):
             logits = self.engine.step(entries, fed=prev.tokens)

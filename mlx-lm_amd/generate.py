@@ -196,7 +196,8 @@ class _OneRequest:
             while sched.has_work:
                 outs = sched.step()
                 if self.progress is not None and not req.generated:
-                    self.progress(min(req.num_computed, len(self.prompt)), len(self.prompt))
+                    read = max(0, req.num_computed - len(req.prefix))  # (of the prompt itself)
+                    self.progress(min(read, len(self.prompt)), len(self.prompt))
                 yield from outs
         finally:
             sched.close()  # (a generator dropped half-way gives its pages back here)
@@ -543,8 +544,8 @@ class BatchGenerator:
         for uid, done in before.items():
             r = self._requests[uid]
             if r.num_computed != done:
-                n = len(r.prompt)
-                prompt_responses.append(self.PromptResponse(uid, (min(r.num_computed, n), n), r.num_computed >= n))
+                n, read = len(r.prompt), max(0, r.num_computed - len(r.prefix))
+                prompt_responses.append(self.PromptResponse(uid, (min(read, n), n), read >= n))
         responses = []
         for o in outs:
             r = self._requests[o.request_id]

@@ -24,8 +24,9 @@ class PromptCache:
     A request is given it as ``prompt_cache`` (``generate_step``, ``stream_generate``) or in
     ``caches`` (``BatchGenerator.insert``); it then reads only the tokens it brings, on top
     of what the cache holds, and when it ends the cache holds those tokens and all the
-    generated ones as well.  While a request uses it, nobody else can.  ``offset`` is the
-    number of tokens held.  The pages count against the engine's pool until ``free()`` (or
+    generated ones as well (the very last one as ``pending``: it has not gone through the model,
+    the next request reads it first).  While a request uses it, nobody else can.  ``offset`` is
+    the number of tokens held.  The pages count against the engine's pool until ``free()`` (or
     until the object goes away).
     """
 
@@ -37,13 +38,21 @@ class PromptCache:
         # and has no pages yet
         self._loaded = None
         self._at_checkout = (0, None)
-        self.in_use = False
+        self.in_use = False    # a live request holds the pages
+        self.claimed = False   # a request that waits or runs will go on from this cache
+        # Tokens that belong to the cache but have not gone through the model: the token that
+        # ended the request before (it ends a request before it is fed).  The next request reads
+        # them ahead of its prompt.
+        self.pending = []
 
     @property
     def offset(self):
+        """Tokens held, the pending ones included."""
         if self._kept is not None:
-            return self._kept.length
-        return self._loaded[0] if self._loaded is not None else 0
+            in_pages = self._kept.length
+        else:
+            in_pages = self._loaded[0] if self._loaded is not None else 0
+        return in_pages + len(self.pending)
 
     @property
     def needs_pages(self):
@@ -69,13 +78,14 @@ class PromptCache:
         if self._loaded is not None:  # read from a file: into pages of this engine's pool now
             self._kept = engine.write_kept(*self._loaded)
             self._loaded, self._engine = None, engine
-        at_checkout = (self.offset, self._kept.state if self._kept is not None else None)
+        at_checkout = (self.offset - len(self.pending), self._kept.state if self._kept is not None else None)
         if self._kept is None:
             engine.add_request(engine_id)  # (may find no request slot free: nothing has changed then)
         else:
             engine.attach_request(engine_id, self._kept)
             self._kept = None
         self._engine, self.in_use, self._at_checkout = engine, True, at_checkout
+        self.pending = []  # (the request has them: it reads them ahead of its prompt)
 
     def rewind(self, engine, engine_id, length=None):
         """Cut the live request back to ``length`` tokens, or to what the cache held when the request
@@ -99,7 +109,7 @@ class PromptCache:
     # -- what callers use ----------------------------------------------------------
 
     def is_trimmable(self):
-        if self.in_use:
+        if self.in_use or self.claimed:
             return False
         if self._loaded is not None:
             return not self._loaded[2]
@@ -107,14 +117,17 @@ class PromptCache:
 
     def trim(self, n_tokens):
         """Forget the last ``n_tokens`` tokens (at most all); returns how many went."""
-        if self.in_use:
-            raise ValueError("this prompt cache is in use by a live request")
+        if self.in_use or self.claimed:
+            raise ValueError("this prompt cache is in use by a request")
         n = max(0, min(int(n_tokens), self.offset))
-        if n and self._loaded is not None:
+        first = min(n, len(self.pending))  # the tokens that are not in pages yet go first
+        self.pending = self.pending[: len(self.pending) - first]
+        rest = n - first
+        if rest and self._loaded is not None:
             length, per_slot, state = self._loaded
-            self._loaded = (length - n, {s: (k[: length - n], v[: length - n]) for s, (k, v) in per_slot.items()}, state)
-        elif n:
-            self._engine.cache.truncate_kept(self._kept, self.offset - n)
+            self._loaded = (length - rest, {s: (k[: length - rest], v[: length - rest]) for s, (k, v) in per_slot.items()}, state)
+        elif rest:
+            self._engine.cache.truncate_kept(self._kept, self._kept.length - rest)
         return n
 
     def copy(self):
@@ -122,6 +135,7 @@ class PromptCache:
         if self.in_use:
             raise ValueError("this prompt cache is in use by a live request")
         other = PromptCache(self.model)
+        other.pending = list(self.pending)
         other._loaded = self._loaded  # (never written to: trim makes a new tuple)
         if self._kept is not None:
             other._engine = self._engine
@@ -144,6 +158,8 @@ class PromptCache:
     def free(self):
         """Give the pages back to the engine's pool; the cache is empty afterwards."""
         self._loaded = None
+        if not self.in_use:
+            self.pending = []
         if self._kept is not None and not self.in_use:
             self._engine.drop_kept(self._kept)
             self._kept = None
@@ -181,7 +197,7 @@ def save_prompt_cache(file_name, cache, metadata=None):
         import torch
 
         tensors["empty"] = torch.zeros(0)
-    info = {"format": _FORMAT, "length": str(int(length)),
+    info = {"format": _FORMAT, "length": str(int(length)), "pending": json.dumps([int(t) for t in cache.pending]),
             "metadata": json.dumps({str(k): str(v) for k, v in (metadata or {}).items()})}
     save_file(tensors, file_name, metadata=info)
 
@@ -208,6 +224,7 @@ def load_prompt_cache(file_name, return_metadata=False):
     cache = PromptCache()
     if length or state:
         cache._loaded = (length, {slot: (kv["keys"], kv["values"]) for slot, kv in per_slot.items()}, state)
+    cache.pending = [int(t) for t in json.loads(info.get("pending", "[]"))]
     metadata = json.loads(info.get("metadata", "{}"))
     return (cache, metadata) if return_metadata else cache
 

@@ -263,7 +263,17 @@ def test_a_cache_goes_through_a_file_and_into_another_engine(setup, tmp_path):
     assert meta == {"model": "m"} and loaded.offset == 37 and loaded.engine is None
     got = [t for t, _ in generate_step(tail, model, max_tokens=9, prompt_cache=loaded, engine=engine)]
     assert got == want and loaded.engine is engine and loaded.offset == 37 + 5 + 9
+    # the token that ended that request has not gone through the model: it travels with the file
+    assert loaded.pending == [want[-1]]
+    more = helpers.random_tokens(3, V, seed=132)
+    want_more = [t for t, _ in generate_step(head + tail + want + more, model, max_tokens=4, engine=engine)]
+    path2 = str(tmp_path / "c2.safetensors")
+    save_prompt_cache(path2, loaded)
     loaded.free()
+    second = load_prompt_cache(path2)
+    assert second.offset == 51 and second.pending == [want[-1]]
+    assert [t for t, _ in generate_step(more, model, max_tokens=4, prompt_cache=second, engine=engine)] == want_more
+    second.free()
     other = Engine(model, dtype=dtype, page_size=32, n_pages=6, max_requests=2)
     again = load_prompt_cache(path)
     assert [t for t, _ in generate_step(tail, model, max_tokens=9, prompt_cache=again, engine=other)] == want

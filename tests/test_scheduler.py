@@ -379,21 +379,22 @@ def test_a_request_goes_on_from_a_kept_cache_and_leaves_its_tokens_there(mode):
     first = [o.token for o in done["a"]]
     assert first == [token_for("a", i) for i in range(3)]
     assert c.offset == 23 and not c.in_use and not eng.cache.requests  # prompt and all three tokens
+    # the token that ended the request has not gone through the model: the cache keeps it for the
+    # next request to read first
+    assert c.pending == [first[-1]] and eng.cache.kept[0].length == 22
     assert eng.cache.free_pages() == 8 - 2 and len(eng.cache.kept) == 1
-    # the token that ended the request went through the model with no logits asked for
-    assert eng.log[-1] == [("a", 1, [])] or mode == "overlapped"
     eng.cache.check()
     # the next request brings one token and starts at position 23
     s2 = Scheduler(eng, SAMPLERS[mode]())
     r = s2.add(Request("a", [777], 2, kept=c))
-    assert r.offset == 23 and c.offset == 23
+    assert r.offset == 22 and r.prefix == [first[-1]] and c.offset == 23 and c.claimed
+    with pytest.raises(ValueError, match="in use"):  # a cache serves one request at a time
+        s2.add(Request("b", [5], 1, kept=c))
     before = len(eng.log)
     early = s2.step()
-    with pytest.raises(ValueError, match="in use"):  # a cache serves one live request at a time
-        s2.add(Request("b", [5], 1, kept=c))
     done = run_all(s2)
-    assert eng.log[before] == [("a", 1, [0])]  # only its own token is read
-    assert c.offset == 23 + 1 + 2 and len(early) + len(done["a"]) == 2
+    assert eng.log[before] == [("a", 2, [1])]  # the pending token and its own, nothing else
+    assert c.offset == 23 + 1 + 2 and len(early) + len(done["a"]) == 2 and not c.claimed
     # what does not fit the positions on top of the cache is refused
     with pytest.raises(ValueError, match="on top of the 26 of its cache"):
         Scheduler(eng, fake_sample).add(Request("x", list(range(1, 60)), 1, kept=c))
