@@ -12,8 +12,8 @@
 // keys [k_lo, k_hi) are cut into tiles of 32 or 64; the tiles are dealt to the splits
 // in runs and, inside a block, to the waves in turn.  With few rows in a step
 // it is the many waves of a block, joined through LDS, that give the GPU
-// enough to do: splits need a second kernel to join them, which at these sizes
-// costs as much as the attention itself.  A wave reads a tile as
+// enough to do; the parts of splits are joined by the block of a (row, head) that
+// finishes last, or by a second kernel.  A wave reads a tile as
 // CPK-lane groups: lane l holds 16 bytes (EPL = 8 bfloat16 or 4 float columns)
 // l % CPK of key l / CPK of each load, where CPK = head_dim / EPL lanes cover
 // one key.  One load instruction therefore reads 64 / CPK whole keys that lie
@@ -49,6 +49,9 @@ struct DecodeArgs {
   // table_in_lds: the request's page numbers are copied to LDS once (max_blocks of them fit).
   int rows_are_requests, table_in_lds;
   int out_head_dim;
+  // the blocks that share a row's keys join their sums themselves: the one that arrives last at
+  // the (row, head)'s counter adds them in the order of the parts (no second kernel)
+  int join_here;
 };
 
 #define MAX_WAVES 16
@@ -77,6 +80,33 @@ __device__ __forceinline__ void unpack(const uint4& v, float (&f)[4], const floa
 __device__ __forceinline__ void put(uint16_t* at, float v) { *at = f32_to_bf16_bits(v); }
 __device__ __forceinline__ void put(float* at, float v) { *at = v; }
 
+// Joining a row's parts inside the kernel.  The parts' sums pass between blocks on different
+// dies, whose L2s do not see each other's lines: they are written and read at agent scope (past
+// the die's L2), and a counter a (row, head) says when all are there.  The counters are zero
+// between launches (the block that arrives last puts its counter back); all launches on a GPU
+// share them, so launches that overlap on one GPU race.
+#define JOIN_MAX_ITEMS 65536
+static __device__ unsigned join_counters[JOIN_MAX_ITEMS];
+__device__ __forceinline__ void put_shared(float* at, float v) {
+  __hip_atomic_store(at, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float get_shared(const float* at) {
+  return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Called by every thread of the block after its put_shared calls; true in all threads of the
+// block that arrives last of `n_parts` at `counter`.  No block waits for another.
+__device__ __forceinline__ bool last_to_arrive(unsigned* counter, unsigned n_parts, int* s_last) {
+  __builtin_amdgcn_s_waitcnt(0);  // this thread's sums have been taken
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const unsigned before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *s_last = before == n_parts - 1;
+    if (*s_last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  return *s_last != 0;
+}
+
 // T: uint16_t (bfloat16 bits) or float.  CPK lanes per key: head_dim = EPL * CPK.  TILE: keys a wave at a time.
 template <typename T, int CPK, int TILE>
 __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void attn_decode_kernel(DecodeArgs p) {
@@ -86,6 +116,7 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
   constexpr int NL = TILE / KPL;   // loads per tile (= CPK)
   __shared__ float Ms[MAX_WAVES], Ls[MAX_WAVES];
   __shared__ float Os[MAX_WAVES][HD];
+  __shared__ int s_last;
   extern __shared__ int page_of[];  // [max_blocks] with table_in_lds
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -147,7 +178,16 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
   const int k_lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
   const int kt0 = (k_lo / TILE) * TILE;
   const int n_tiles = (k_hi - kt0 + TILE - 1) / TILE;
-  const int per_split = (n_tiles + p.n_splits - 1) / p.n_splits;
+  // Joined here, a row may take fewer splits than the launch has: as many as leave a wave a tile
+  // of 32 keys, and one if a wave has fewer than 96 keys anyway (joining costs about a tile's
+  // time).  Blocks of the splits it does not take have nothing to do.
+  int n_splits = p.n_splits;
+  if (p.join_here == 2) {
+    const int keys_a_wave = (k_hi - kt0) / n_waves;
+    n_splits = keys_a_wave >= 96 ? min(n_splits, keys_a_wave / 32) : 1;
+    if (split >= n_splits) return;  // (the whole block)
+  }
+  const int per_split = (n_tiles + n_splits - 1) / n_splits;
   const int t_begin = split * per_split;
   const int t_end = min(n_tiles, t_begin + per_split);
 
@@ -235,8 +275,37 @@ __global__ __launch_bounds__(64 * (CPK >= 16 ? MAX_WAVES / 2 : MAX_WAVES)) void 
     L += Ls[i] * w;
     if (tid < HD) acc += Os[i][tid] * w;
   }
+  if (n_splits > 1 && p.join_here) {  // (uniform over the block)
+    const size_t first = ((size_t)item * p.n_heads + h) * p.n_splits;
+    if (tid < HD) put_shared(p.part_o + (first + split) * HD + tid, acc);
+    if (tid == 0) put_shared(p.part_ml + (first + split) * 2, M), put_shared(p.part_ml + (first + split) * 2 + 1, L);
+    if (!last_to_arrive(join_counters + (size_t)item * p.n_heads + h, (unsigned)n_splits, &s_last)) return;
+    if (tid < HD) {  // the parts in their order, whoever arrived when
+      float Mj = -INFINITY, Lj = 0.f, aj = 0.f;
+      for (int s0 = 0; s0 < n_splits; s0 += 4) {
+        float ms[4], ls[4], os[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {  // four parts' values on their way at a time
+          const size_t at = first + min(s0 + j, n_splits - 1);
+          ms[j] = get_shared(p.part_ml + at * 2), ls[j] = get_shared(p.part_ml + at * 2 + 1);
+          os[j] = get_shared(p.part_o + at * HD + tid);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (s0 + j >= n_splits || ms[j] == -INFINITY) continue;  // (a part without a tile)
+          const float M2 = fmaxf(Mj, ms[j]);
+          const float wa = __expf(Mj - M2), wb = __expf(ms[j] - M2);
+          Lj = Lj * wa + ls[j] * wb;
+          aj = aj * wa + os[j] * wb;
+          Mj = M2;
+        }
+      }
+      put((T*)p.out + out_at(p, row, h * HD + tid), aj / Lj);
+    }
+    return;
+  }
   if (tid < HD) {
-    if (p.n_splits == 1) {
+    if (n_splits == 1) {
       put((T*)p.out + out_at(p, row, h * HD + tid), acc / L);
     } else {
       const size_t base = ((size_t)item * p.n_heads + h) * p.n_splits + split;
@@ -282,7 +351,7 @@ static void launch(const DecodeArgs& p, int n_rows, int n_waves, int key_tile, h
     hipLaunchKernelGGL((attn_decode_kernel<T, CPK, 64>), grid, block, lds, stream, p);
   else
     hipLaunchKernelGGL((attn_decode_kernel<T, CPK, 32>), grid, block, lds, stream, p);
-  if (p.n_splits > 1)
+  if (p.n_splits > 1 && !p.join_here)
     hipLaunchKernelGGL((attn_decode_merge_kernel<T, CPK>), dim3(n_rows, p.n_heads), dim3(16 / sizeof(T) * CPK), 0, stream, p);
 }
 
@@ -290,7 +359,11 @@ static void launch(const DecodeArgs& p, int n_rows, int n_waves, int key_tile, h
 // item i of `rows` is row i and belongs to request i (every request of the step brings one token),
 // which saves the kernel two trips to memory.  dtype DT_BF16 with head_dim 32, 64 or 128, DT_F32
 // with 16, 32 or 64, and pages that hold whole loads (page_size a multiple of the keys in 1 KB).
-// key_tile: 32 or 64 keys a wave at a time (0: 32).
+// key_tile: 32 or 64 keys a wave at a time (0: 32).  join_in_kernel: 0, a second kernel joins the
+// n_splits parts of a (row, head); 1, the block that finishes a (row, head) last does (up to
+// 65,536 (row, head)s; part_o and part_ml are still where the parts pass through); 2, the same,
+// and n_splits is only the most a row takes: a short row takes fewer, by its own length.
+// Launches that join in the kernel and overlap on one GPU race (they share the counters).
 extern "C" int attn_decode_rows(void* out, const void* q, int ldq, int ldo, const void* k_pages,
                                 const void* v_pages, size_t page_stride, const int* block_table,
                                 int max_blocks, const int* token_req, const int* positions,
@@ -298,7 +371,7 @@ extern "C" int attn_decode_rows(void* out, const void* q, int ldq, int ldo, cons
                                 int page_size, int window, float scale, int n_splits, float* part_o,
                                 float* part_ml, int n_waves, const void* ahead, size_t ahead_chunk_bytes,
                                 int ahead_chunks, int rows_are_requests, int dtype, int key_tile,
-                                hipStream_t stream) {
+                                int join_in_kernel, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (key_tile == 0) key_tile = 32;
   if (key_tile != 32 && key_tile != 64) FAIL("attn_decode: a wave takes 32 or 64 keys at a time, not %d", key_tile);
@@ -338,6 +411,9 @@ extern "C" int attn_decode_rows(void* out, const void* q, int ldq, int ldo, cons
   p.out_head_dim = head_dim;
   if (ldo == 0 && dtype != DT_BF16) FAIL("attn_decode: the packed order (ldo == 0) is for a bfloat16 out");
   p.rows_are_requests = rows_are_requests ? 1 : 0;
+  // (more (row, head)s than counters: the second kernel joins the parts)
+  if (join_in_kernel < 0 || join_in_kernel > 2) FAIL("attn_decode: join_in_kernel %d is not 0, 1 or 2", join_in_kernel);
+  p.join_here = n_splits > 1 && (long)n_rows * n_heads <= JOIN_MAX_ITEMS ? join_in_kernel : 0;
   p.table_in_lds = max_blocks > 0 && max_blocks <= 8192;  // (32 KB of LDS at most)
   if (dtype == DT_BF16) {
     if (cpk == 4)

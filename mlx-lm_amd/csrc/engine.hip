@@ -100,7 +100,7 @@ typedef int (*fn_attn_row)(void*, const void*, int, int, const void*, const void
                            float*, float*, int, hipStream_t);
 typedef int (*fn_attn_decode)(void*, const void*, int, int, const void*, const void*, size_t, const int*, int,
                               const int*, const int*, const int*, int, int, int, int, int, int, float, int,
-                              float*, float*, int, const void*, size_t, int, int, int, int, hipStream_t);
+                              float*, float*, int, const void*, size_t, int, int, int, int, int, hipStream_t);
 typedef int (*fn_attn_prefill)(void*, const void*, int, int, const void*, const void*, size_t, const int*,
                                int, const int*, const int*, const int*, int, int, int, int, int, int, float,
                                hipStream_t);
@@ -681,9 +681,12 @@ struct Attention : Mixer {
   // hundred; of 64 where the blocks are more than three a CU and the context is 640 or more (the
   // larger tile keeps more loads in flight; a recorded step plans for the model's positions: at
   // 1,024 of them, 12 to 30 rows were 1 to 3 % faster with 32 over contexts of 512 to 1,022, 32
-  // rows 2 % faster with 64).  Splits need a second kernel to join them, which
-  // costs as much as a walk of some hundred keys a wave: only where a wave would walk 256 keys or
-  // more, as many as leave it 128, and no more than give every block a compute unit at once.
+  // rows 2 % faster with 64).  The block that finishes a (row, head) last joins its splits, which
+  // costs about as much as a tile of keys: splits only where a wave would walk 96 keys or more, as
+  // many as leave it a tile, and no more than give every block a compute unit at once (one row at
+  // 1,000 keys: 9.4 us unsplit, 7.3 in four; at 7,000: 44 unsplit, 13.6 in eight, 15.9 in twelve).
+  // This is the most a row takes; the kernel gives a shorter row fewer by the same rule, so a
+  // recorded step, planned for the model's positions, splits only the rows that are long.
   void row_work(const EngCtx* ctx, int n_rows, long max_row_context, int* n_splits, int* n_waves,
                 int* key_tile) const {
     const long c = window <= 0 ? max_row_context : (max_row_context < window + 31 ? max_row_context : window + 31);
@@ -694,8 +697,8 @@ struct Attention : Mixer {
     while (nw > fewest && nw / 2 >= tiles) nw /= 2;
     const long keys_a_wave = c / nw;
     long ns = 1;
-    if (keys_a_wave >= 256) {
-      ns = keys_a_wave / 128;
+    if (keys_a_wave >= 96) {
+      ns = keys_a_wave / 32;
       if (ctx->n_compute_units / blocks < ns) ns = ctx->n_compute_units / blocks;
       if (ns > 64) ns = 64;
       if (ns < 1) ns = 1;
@@ -801,7 +804,7 @@ struct Attention : Mixer {
                kv.max_blocks, kv.token_req, kv.positions, rows, n_rows, n_heads, n_kv_heads, head_dim,
                kv.page_size, window, scale, n_splits, (float*)part_o.p, (float*)part_ml.p, n_waves,
                ahead ? ahead->packed : nullptr, ahead ? ahead->chunk_bytes : (size_t)0, chunks, rows_are_requests,
-               q.dtype, key_tile, ctx->stream);
+               q.dtype, key_tile, 2, ctx->stream);
       } else {
         KERNEL(k_attn_row, ctx, out.p, q.p, q.ld, out.ld, kv.k, kv.v, kv.page_stride, kv.block_table,
                kv.max_blocks, kv.token_req, kv.positions, rows, n_rows, n_heads, n_kv_heads, head_dim,

@@ -653,14 +653,16 @@ def attn_decode_takes(q_dtype, kv):
 
 def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_heads, scale,
                 window=0, n_splits=1, part_o=None, part_ml=None, n_waves=4, ahead=None, ahead_chunks=0,
-                rows_are_requests=False, key_tile=32):
+                rows_are_requests=False, key_tile=32, join_in_kernel=0):
     """``attn_row`` for keys of 64, 128 or 256 bytes (bfloat16 with head_dim 32, 64 or 128, float32
     with 16, 32 or 64): keys stream into registers.
 
     ``ahead``: a ``PackedWeight`` whose first ``ahead_chunks`` chunks the CUs without a row read
     meanwhile, each the chunks that a block on its own die will ask for (``sum_partials_norm``).
     ``rows_are_requests``: item ``i`` of ``rows`` is row ``i`` of request ``i`` (the caller says so).
-    ``key_tile``: 32 or 64 keys a wave at a time."""
+    ``key_tile``: 32 or 64 keys a wave at a time.  ``join_in_kernel``: 0, a second kernel joins
+    the ``n_splits`` parts of a (row, head); 1, the block that finishes it last does; 2, the same,
+    and a short row takes fewer than ``n_splits`` by its own length."""
     lib = build.load("attention_decode")
     packed_out = isinstance(out, PackedRows)  # (the order that the product after attention reads fastest)
     ldq, ldo = _rows2d(q, "q"), 0 if packed_out else _rows2d(out, "out")
@@ -688,7 +690,8 @@ def attn_decode(out, q, kv, block_table, token_req, positions, rows, n_rows, n_h
         _ptr(ahead.packed if ahead is not None else None),
         _c_size_t(ahead.chunk_bytes if ahead is not None else 0),
         _c_int(min(ahead_chunks, ahead.n_chunks) if ahead is not None else 0),
-        _c_int(1 if rows_are_requests else 0), _c_int(DT[q.dtype]), _c_int(key_tile), _stream(),
+        _c_int(1 if rows_are_requests else 0), _c_int(DT[q.dtype]), _c_int(key_tile),
+        _c_int(int(join_in_kernel)), _stream(),
     )
     build.check(lib, rc, "attn_decode")
     return out

@@ -399,12 +399,14 @@ def test_attn_decode(case, n_splits, n_waves):
     part_o = torch.empty(c.T * H * n_splits * hd, dtype=torch.float32, device=DEV)
     part_ml = torch.empty(c.T * H * n_splits * 2, dtype=torch.float32, device=DEV)
     want = c.reference()
-    for key_tile in (32, 64):  # keys a wave takes at a time
+    for key_tile, here in ((32, 0), (64, 0), (32, 1), (64, 1), (32, 1), (32, 2), (64, 2)):
+        # keys a wave takes at a time; the parts joined by a second kernel (0) or by the block that
+        # arrives last (1; twice in a row: its counters are back at zero), short rows in fewer parts (2)
         out = torch.full((c.T, H * hd), float("nan")).to(torch.bfloat16).to(DEV)
         k.attn_decode(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, c.T, H,
-                      c.scale, window, n_splits, part_o, part_ml, n_waves, key_tile=key_tile)
+                      c.scale, window, n_splits, part_o, part_ml, n_waves, key_tile=key_tile, join_in_kernel=here)
         err = (out.double().cpu() - want).abs().max().item()
-        assert err < _attn_tol(torch.bfloat16), (key_tile, err)
+        assert err < _attn_tol(torch.bfloat16), (key_tile, here, err)
 
 
 @pytest.mark.parametrize("case", [c for c in ATTN_CASES if c[2] in (16, 32, 64)] + [
@@ -424,12 +426,12 @@ def test_attn_decode_float32(case, n_splits, n_waves):
     part_o = torch.empty(c.T * H * n_splits * hd, dtype=torch.float32, device=DEV)
     part_ml = torch.empty(c.T * H * n_splits * 2, dtype=torch.float32, device=DEV)
     want = c.reference()
-    for key_tile in (32, 64):
+    for key_tile, here in ((32, 0), (64, 0), (32, 1), (64, 1), (32, 2)):
         out = torch.full((c.T, H * hd), float("nan"), dtype=torch.float32, device=DEV)
         k.attn_decode(out, c.q.to(DEV), c.kv, c.block_table_dev, c.token_req, c.positions, rows, c.T, H,
-                      c.scale, window, n_splits, part_o, part_ml, n_waves, key_tile=key_tile)
+                      c.scale, window, n_splits, part_o, part_ml, n_waves, key_tile=key_tile, join_in_kernel=here)
         err = (out.double().cpu() - want).abs().max().item()
-        assert err < _attn_tol(torch.float32), (key_tile, err)
+        assert err < _attn_tol(torch.float32), (key_tile, here, err)
 
 
 def test_attn_decode_takes_keys_of_64_to_256_bytes():
