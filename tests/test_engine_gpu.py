@@ -109,7 +109,8 @@ def test_first_tokens_and_long_decode(folders, dtype):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("use_graphs", [False, True])
 def test_thousands_of_keys_split_over_blocks(tmp_path, monkeypatch, dtype, use_graphs):
-    """A prompt of 3,300 tokens in two portions, then 40 decoded tokens whose keys several blocks share."""
+    """A prompt of 3,300 tokens in two portions, then 40 decoded tokens whose keys several blocks share,
+    beside a request of a few dozen tokens."""
     from mlx_lm_amd.engine import Engine, StepEntry
     from mlx_lm_amd.ops import kernels
     from mlx_lm_amd.utils import load_model
@@ -119,15 +120,22 @@ def test_thousands_of_keys_split_over_blocks(tmp_path, monkeypatch, dtype, use_g
     tokens = helpers.random_tokens(n, config["vocab_size"], seed=31)
     want = _plain_logits(weights, config, tokens, dtype)
     model, _ = load_model(str(tmp_path), dtype=dtype)
-    eng = Engine(model, dtype=dtype, page_size=16, n_pages=(n + 63) // 64 * 4, max_requests=2, use_graphs=use_graphs)
+    eng = Engine(model, dtype=dtype, page_size=16, n_pages=(n + 63) // 64 * 4 + 5, max_requests=2, use_graphs=use_graphs)
     eng.add_request("r")
     first = eng.step([StepEntry("r", tokens[:2000], [1999])])
     _close(first, want[1999:2000], dtype, "the first portion's last row")
     rows = [eng.step([StepEntry("r", tokens[2000:n_prompt], [n_prompt - 2001])]).clone()]
+    # a short request decodes beside the long one: in one launch its rows take one part and the long one's several
+    short = helpers.random_tokens(70, config["vocab_size"], seed=32)
+    want_short = _plain_logits(weights, config, short, dtype)
+    eng.add_request("s")
+    short_rows = [eng.step([StepEntry("s", short[:30], [29])]).clone()]
     for i in range(n_prompt, n):
-        rows.append(eng.step([StepEntry("r", tokens[i : i + 1], [0])]).clone())
+        both = eng.step([StepEntry("r", tokens[i : i + 1], [0]), StepEntry("s", short[i - n_prompt + 30 : i - n_prompt + 31], [0])])
+        rows.append(both[:1].clone()), short_rows.append(both[1:].clone())
     assert eng.stats.key_splits_most > 1, "no step split a row's keys"
     _close(torch.cat(rows), want[n_prompt - 1 :], dtype, "decoded after 3,300 tokens")
+    _close(torch.cat(short_rows), want_short[29:], dtype, "the short request beside it")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
