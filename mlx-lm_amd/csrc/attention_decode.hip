@@ -49,8 +49,9 @@ struct DecodeArgs {
   // table_in_lds: the request's page numbers are copied to LDS once (max_blocks of them fit).
   int rows_are_requests, table_in_lds;
   int out_head_dim;
-  // the blocks that share a row's keys join their sums themselves: the one that arrives last at
-  // the (row, head)'s counter adds them in the order of the parts (no second kernel)
+  // 1 or 2: the blocks that share a row's keys join their sums themselves: the one that arrives
+  // last at the (row, head)'s counter adds them in the order of the parts (no second kernel);
+  // 2: n_splits is the most a row takes, and a row takes as many as its own length calls for
   int join_here;
 };
 
