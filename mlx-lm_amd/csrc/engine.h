@@ -138,6 +138,8 @@ int eng_struct_sizes(long* out, int n);  // for the Python side's check of its m
 int eng_compute_units(void);
 // queries a tile of attn_tile's and of attn_prefill's work lists holds (attention_tiles.h)
 void eng_attn_tile_sizes(int* tile, int* prefill_tile);
+// The context length from which a decode step may split a row's keys over blocks.
+int eng_rows_split_from(void);
 
 // flags of a callback part
 #define ENG_ACCEPTS_LAZY 1

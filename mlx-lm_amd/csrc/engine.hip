@@ -46,6 +46,15 @@ extern "C" void eng_set_hooks(eng_resolver_t resolver, eng_callback_t callback) 
 
 extern "C" int eng_compute_units(void) { return n_compute_units(); }
 
+// The decode kernel's waves a block where rows are few, and the keys a wave from which a row's keys
+// are split over blocks (the kernel narrows a launch's splits row by row with the same number).
+#define ROW_WAVES 8
+#define ROW_SPLIT_KEYS_A_WAVE 96
+
+// The context length from which a decode step may split a row's keys over blocks (what a recorded
+// step's planning length is chosen by: below it no step launches splits).
+extern "C" int eng_rows_split_from(void) { return ROW_WAVES * ROW_SPLIT_KEYS_A_WAVE; }
+
 extern "C" void eng_attn_tile_sizes(int* tile, int* prefill_tile) {
   *tile = ATTN_TILE_QUERIES, *prefill_tile = ATTN_PREFILL_TILE_QUERIES;
 }
@@ -692,12 +701,12 @@ struct Attention : Mixer {
     const long c = window <= 0 ? max_row_context : (max_row_context < window + 31 ? max_row_context : window + 31);
     const long tiles = c + 31 < 32 ? 1 : (c + 31) / 32;
     const long blocks = n_rows * n_heads < 1 ? 1 : (long)n_rows * n_heads;
-    int nw = blocks > ctx->n_compute_units ? 4 : 8;
+    int nw = blocks > ctx->n_compute_units ? 4 : ROW_WAVES;
     const int fewest = head_dim > 128 ? 4 : 2;  // (the block's threads write a column of the head each)
     while (nw > fewest && nw / 2 >= tiles) nw /= 2;
     const long keys_a_wave = c / nw;
     long ns = 1;
-    if (keys_a_wave >= 96) {
+    if (keys_a_wave >= ROW_SPLIT_KEYS_A_WAVE) {
       ns = keys_a_wave / 32;
       if (ctx->n_compute_units / blocks < ns) ns = ctx->n_compute_units / blocks;
       if (ns > 64) ns = 64;

@@ -119,7 +119,9 @@ class HostBatch:
     ``q_starts[r]``, ``q_lens[r]`` say where request ``r``'s tokens lie in the flat batch,
     ``context_lens[r]`` how many tokens it held before.  ``static``: the arrays are for a step
     that is recorded and replayed, so nothing about the launches (how many ways keys are split)
-    may depend on the lengths; ``max_positions`` is then the length to plan for.
+    may depend on the lengths; ``max_positions`` is then the length to plan for (the model's
+    positions, or fewer where the parts put recorded steps into classes of length,
+    ``length_class``).
     """
 
     __slots__ = ("q_starts", "q_lens", "context_lens", "state_slots", "n_tokens", "static", "max_positions")

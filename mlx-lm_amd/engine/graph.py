@@ -47,11 +47,11 @@ def _recording(graph):
 class StepGraph:
     """A recorded step of one shape (tokens per request, number of wanted places)."""
 
-    def __init__(self, engine):
+    def __init__(self, engine, plan_positions=None):
         # (a weak reference: the engine owns its graphs, and without a cycle they are freed
         # the moment the engine is dropped, not whenever the collector next runs)
         self.engine = weakref.proxy(engine)
-        self.store = StaticStore(engine.device)
+        self.store = StaticStore(engine.device, plan_positions)
         self.graph = None
         self.logits = None
         self.failed = False

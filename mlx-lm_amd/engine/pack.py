@@ -68,8 +68,9 @@ class StaticStore:
 
     static = True
 
-    def __init__(self, device):
+    def __init__(self, device, plan_positions=None):
         self.device = device
+        self.plan_positions = plan_positions  # the length the step is planned for (None: the model's positions)
         self.host = self.host_np = self.dev = None
         self.total = None
         self.copied = None  # recorded after the copy that reads the host buffer was queued
@@ -120,7 +121,8 @@ def pack(engine, entries, store):
         q_starts.append(s)
         s += n
     static = store.static
-    batch = HostBatch(q_starts, q_lens, context_lens, state_slots, static, dec.max_positions)
+    batch = HostBatch(q_starts, q_lens, context_lens, state_slots, static,
+                      getattr(store, "plan_positions", None) or dec.max_positions)
 
     if T == R:  # one token a request: no repeats to spell out
         token_ids = [e.tokens[0] for e in entries]

@@ -75,6 +75,7 @@ class Engine:
         # decode steps are recorded as graphs where every part launches kernels only
         self.use_graphs = use_graphs and all(getattr(p, "graph_safe", False) for p in self.decoder.parts())
         self._graphs = {}
+        self._length_classers = None  # the parts that put recorded decode steps into classes of length
         # Other steps whose shape keeps coming back (portions of prompts of the scheduler's size, with
         # or without decoding requests beside them) are recorded too, if asked for.
         self.record_prompt_steps = bool(record_prompt_steps) and self.use_graphs
@@ -261,11 +262,16 @@ class Engine:
         every = n_wanted == sum(q_lens) and all(list(e.want) == list(range(len(e.tokens))) for e in entries)
         decode = every and n_wanted == len(entries)
         if decode:
-            graph = self._graphs.get(len(entries))
+            # one recorded step for each number of requests and class of length: a step is planned
+            # for the longest request of its class, not for the model's positions
+            longest = max(self.cache.requests[e.request_id].length for e in entries) + 1
+            classes, plan_positions = self._length_class(longest)
+            key = (len(entries), classes)
+            graph = self._graphs.get(key)
             if graph is None:
                 from .graph import StepGraph
 
-                graph = self._graphs[len(entries)] = StepGraph(self)
+                graph = self._graphs[key] = StepGraph(self, plan_positions)
             return None if graph.failed else graph
         if not self.record_prompt_steps:
             return None
@@ -287,6 +293,24 @@ class Engine:
         while len(self._step_graphs) > self.MAX_RECORDED:
             self._step_graphs.popitem(last=False)
         return graph
+
+    def _length_class(self, longest):
+        """``(classes, length to plan for)`` of a recorded decode step whose longest request holds
+        ``longest`` tokens: what the parts that have a ``length_class`` say (one answer a kind of
+        part), and the largest of their lengths, at most the model's positions."""
+        if self._length_classers is None:
+            kinds = {}
+            for p in self.decoder.parts():
+                if hasattr(p, "length_class"):
+                    kinds.setdefault(type(p), p)
+            self._length_classers = list(kinds.values())
+        classes, plan = [], 0
+        for p in self._length_classers:
+            c, n = p.length_class(longest)
+            classes.append(c)
+            plan = max(plan, n)
+        P = self.decoder.max_positions
+        return tuple(classes), (min(plan, P) if classes else P)
 
     def _build_context(self, entries):
         """The context of an eager step: its arrays packed and on their way to the device, tokens

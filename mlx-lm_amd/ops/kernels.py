@@ -617,6 +617,12 @@ def attn_tile_sizes():
     return _TILE_SIZES
 
 
+def rows_split_from():
+    """The context length from which a decode step may split a row's keys over blocks (the native
+    host's policy; recorded decode steps are kept apart by it)."""
+    return int(native.lib().eng_rows_split_from())
+
+
 def attn_prefill_takes(q_dtype, kv):
     """Whether the matrix-core prefill kernel takes this cache geometry."""
     return q_dtype == torch.bfloat16 and kv.head_dim in (32, 64, 128)

@@ -178,6 +178,7 @@ def lib():
         "eng_wants_packed_rows": (c_int, [POINTER(EngCtx), POINTER(EngWeight), c_int]),
         "eng_host": (P, []),
         "eng_attn_tile_sizes": (None, [POINTER(c_int), POINTER(c_int)]),
+        "eng_rows_split_from": (c_int, []),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)

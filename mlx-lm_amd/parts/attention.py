@@ -96,7 +96,7 @@ class CausalSelfAttention(Mixer):
         same portions in the larger tiles of the matrix-core kernel (``big_tiles``, the tile with
         the most keys first).  ``all_tiles`` covers every row with tiles, for head sizes the row kernels do
         not take.  ``max_row_context``: the most keys that a row of ``rows`` sees, which decides
-        how its keys are split; in a step that is recorded, the model's positions.
+        how its keys are split; in a step that is recorded, the length it is planned for.
         ``rows_are_requests``: 1 if every request brings one token, so that item ``i`` of ``rows``
         is row ``i`` of request ``i`` (the decode kernel then need not look either up)."""
         TILE_Q, BIG_TILE_Q = kernels.attn_tile_sizes()
@@ -120,6 +120,20 @@ class CausalSelfAttention(Mixer):
         return {"tiles": tiles, "rows": rows, "all_tiles": all_tiles,
                 "big_tiles": [v for _, r0, m in big for v in (r0, m)], "max_row_context": longest,
                 "rows_are_requests": int(all(n == 1 for n in batch.q_lens))}
+
+    @staticmethod
+    def length_class(longest):
+        """``(class, length to plan for)`` of a recorded decode step whose longest request sees
+        ``longest`` keys.  Class 0 is every length below the one from which the decode kernel may
+        split a row's keys over blocks, class 1 up to twice that, class 2 up to four times, and a
+        step is planned for the longest of its class.  (Planned for the model's positions, a step
+        of requests that are nowhere near that long would launch the blocks of splits that no row
+        takes and leave fewer CUs to read weights ahead.)"""
+        base = kernels.rows_split_from()
+        if longest < base:
+            return 0, base - 1
+        c = (longest // base).bit_length()
+        return c, base * (1 << c) - 1
 
     # -- the native twin ---------------------------------------------------------
 

@@ -128,3 +128,8 @@ def mixed_trace(config, seed, lengths, n_live=4):
 
 def held(lengths, n_live):
     return sum(sorted(((n + 63) // 64 * 64 for n in lengths), reverse=True)[:n_live])
+
+
+def decode_graphs(engine, n_requests):
+    """The engine's recorded decode steps of ``n_requests`` requests (one a class of length)."""
+    return [g for (n, _), g in engine._graphs.items() if n == n_requests]

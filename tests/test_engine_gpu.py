@@ -139,6 +139,31 @@ def test_thousands_of_keys_split_over_blocks(tmp_path, monkeypatch, dtype, use_g
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recorded_decode_steps_by_class_of_length(tmp_path, dtype):
+    """Decoding across the length from which a row's keys may be split: the recorded step of the
+    shorter lengths is planned without splits, the next one with, and the logits do not notice."""
+    from mlx_lm_amd.engine import Engine, StepEntry
+    from mlx_lm_amd.ops import kernels
+    from mlx_lm_amd.utils import load_model
+
+    config, weights = helpers.make_folder(str(tmp_path), "LONG", 8.0)
+    edge = kernels.rows_split_from()
+    n_prompt, n = edge - 8, edge + 8
+    tokens = helpers.random_tokens(n, config["vocab_size"], seed=33)
+    want = _plain_logits(weights, config, tokens, dtype)
+    model, _ = load_model(str(tmp_path), dtype=dtype)
+    eng = Engine(model, dtype=dtype, page_size=16, n_pages=(n + 15) // 16 + 1, max_requests=2, use_graphs=True)
+    eng.add_request("r")
+    rows = [eng.step([StepEntry("r", tokens[:n_prompt], [n_prompt - 1])]).clone()]
+    for i in range(n_prompt, n):
+        rows.append(eng.step([StepEntry("r", tokens[i : i + 1], [0])]).clone())
+    graphs = helpers.decode_graphs(eng, 1)
+    assert len(graphs) == 2 and all(g.graph is not None for g in graphs)
+    assert sorted(g.store.plan_positions for g in graphs) == [edge - 1, 2 * edge - 1]
+    _close(torch.cat(rows), want[n_prompt - 1 :], dtype, "decoded across the edge of a class of length")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name,sharp", [("A", 8.0), ("B", 8.0), ("C", 0.0), ("C", 8.0)])
 def test_mixed_batches_with_few_pages(folders, dtype, name, sharp):
     from mlx_lm_amd.engine import StepEntry
@@ -386,7 +411,7 @@ def test_recorded_decode_steps_equal_eager_ones(folders, dtype):
                 live.append("d")
             eng.cache.check()
         if use_graphs:
-            assert sorted(eng._graphs) == [1, 2, 3, 4] and all(g.graph is not None for g in eng._graphs.values())
+            assert sorted({n for n, _ in eng._graphs}) == [1, 2, 3, 4] and all(g.graph is not None for g in eng._graphs.values())
         results[use_graphs] = {r: torch.cat(v) for r, v in got.items()}
     for r, toks in seqs.items():
         want = _plain_logits(weights, config, toks, dtype)
@@ -462,8 +487,8 @@ def test_a_dropped_engine_frees_its_graphs_at_once(folders):
             eng.step([StepEntry("a", [1 + at, 2 + at, 3 + at], [2])])
         for t in range(3):
             eng.step([StepEntry("a", [20 + t], [0])])
-        refs = [weakref.ref(eng), weakref.ref(eng._graphs[1])] + [weakref.ref(g) for g in eng._step_graphs.values()]
-        assert len(refs) == 3 and eng._graphs[1].graph is not None
+        refs = [weakref.ref(eng), weakref.ref(helpers.decode_graphs(eng, 1)[0])] + [weakref.ref(g) for g in eng._step_graphs.values()]
+        assert len(refs) == 3 and helpers.decode_graphs(eng, 1)[0].graph is not None
         del eng
         assert all(r() is None for r in refs)
     finally:
@@ -568,7 +593,7 @@ def test_trim_and_regenerate_across_a_page_edge(folders, dtype, use_graphs):
     got_b += [eng.step([StepEntry("b", [b[i]], [0])]).clone() for i in range(10, 40)]
     _close(torch.cat(got_b), want_b, dtype, "the request that took the page")
     if use_graphs:
-        assert eng._graphs[1].graph is not None
+        assert all(g.graph is not None for g in helpers.decode_graphs(eng, 1)) and helpers.decode_graphs(eng, 1)
     # trimming more than there is drops everything (tests/test_prompt_cache.py:259-264)
     assert eng.trim("a", 1000) == 56 and eng.context_len("a") == 0
     eng.end_request("a")

@@ -576,7 +576,7 @@ def test_a_recorded_step_takes_its_tokens_once(tmp_path, dtype, mixer):
         for i in range(3):  # (recorded at the third sighting of the shape)
             out.append(eng.step([StepEntry("a", seqs["a"][33 + 2 * i : 35 + 2 * i], [0, 1])]).clone())
         if use_graphs:
-            assert eng._graphs[2].graph is not None
+            assert helpers.decode_graphs(eng, 2)[0].graph is not None
             assert any(sg.graph is not None for sg in eng._step_graphs.values())
         results[use_graphs] = torch.cat(out)
         states[use_graphs] = eng.cache.state(0)[[eng.cache.requests[r].state_slot for r in seqs]].clone()
@@ -716,7 +716,7 @@ def test_a_window_under_recorded_steps(tmp_path, dtype):
         for i in range(80, 90):
             got["b"].append(eng.step([StepEntry("b", [seqs["b"][i]], [0])]).clone())
         if use_graphs:
-            assert all(eng._graphs[n].graph is not None for n in (1, 2))
+            assert all(helpers.decode_graphs(eng, n)[0].graph is not None for n in (1, 2))
         results[use_graphs] = {r: torch.cat(v) for r, v in got.items()}
     for r, toks in seqs.items():
         _close(results[True][r], plain_logits(toks[: results[True][r].shape[0]]), dtype, f"a window under recorded steps, request {r}")
